@@ -1,0 +1,137 @@
+/*
+ * paged_attn.h — C ABI of libpaged_attn.so: paged flash attention for AMD
+ * Instinct MI355X (gfx950), hand-written HIP kernels.
+ *
+ * Role relative to the reference (aws-neuron/nkipy): these entry points stand
+ * where the reference runs its attention math on the device, i.e. the body of
+ *   examples/models/qwen3/kernels/attention.py:108-144   (repeat_kv, QK^T/sqrt(d),
+ *   causal mask, softmax, PV), its multi-token-at-offset variant
+ *   examples/models/gpt_oss/kernels/attention.py:102-150, and the execute call
+ *   that launches it, spike/src/spike/spike_model.py:248-288 -> spike/src/model.cpp:90-110
+ *   (NrtModel::execute).  The reference has no paged/block-table form; the
+ *   block-table gather is the np.take form of nkipy/src/nkipy/core/tensor.py:575-640
+ *   applied to a pool laid out [num_blocks, block_size, Hkv, D].
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller (the reference's
+ *     ownership rule: caller allocates inputs and outputs,
+ *     nkipy/src/nkipy/runtime/device_tensor.py:51-74); nothing is allocated,
+ *     freed or retained by the library;
+ *   - calls are asynchronous on `stream` (a hipStream_t passed as void*; NULL is
+ *     the default stream) and never synchronise;
+ *   - return 0 = launched; negative = argument error found on the host before
+ *     any launch (pa_last_error() holds the text); positive = hipError_t;
+ *   - thread-safe and re-entrant: no mutable global state except the debug and
+ *     profiling switches below, which are meant for tests and benchmarks;
+ *   - dtype codes: PA_F32 = 0, PA_BF16 = 1, PA_FP8_E4M3FN = 2 (OCP e4m3fn,
+ *     KV cache only, with one float scale per (block, kv head)).
+ *
+ * Tensor layouts (row-major, contiguous)
+ *   q, out (decode)      [B, Hq, D]
+ *   q, out (prefill)     [B, T, Hq, D]; rows t >= query_lens[b] are padding
+ *   k_cache, v_cache     [num_blocks, block_size, Hkv, D]
+ *   k_scale, v_scale     [num_blocks, Hkv] float (fp8 KV only, else NULL)
+ *   block_tables         [B, max_blocks_per_seq] int32, logical -> physical block
+ *   seq_lens             [B] int32, keys visible to the last query token
+ *   query_lens           [B] int32, new tokens of each sequence (<= T, <= seq_lens[b])
+ * q head h reads kv head h / (Hq / Hkv)   (attention.py:15-22 repeat_kv).
+ */
+#ifndef PAGED_ATTN_H_
+#define PAGED_ATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { PA_F32 = 0, PA_BF16 = 1, PA_FP8_E4M3FN = 2 };
+
+/* Library version: major * 10000 + minor * 100 + patch. */
+int pa_version(void);
+
+/* Text of the calling thread's most recent error ("" if none).  Mirrors the
+ * status strings of spike/src/include/error.h:23-43. */
+const char* pa_last_error(void);
+
+/* Bytes of scratch pa_decode needs for split-K partials: per (sequence, q head,
+ * partition) D floats of normalised partial output plus (max, sum).  Zero when
+ * max_seq_len fits one partition. */
+size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int partition_size);
+
+/*
+ * Paged decode attention: one query token per sequence.
+ *   out[b, h, :] = softmax(q[b, h, :] . K_b^T * scale) V_b,  K_b/V_b = the first
+ *   seq_lens[b] rows gathered through block_tables[b]   (the decode branch of
+ *   examples/models/qwen3/kernels/attention.py:103-144, start_pos = seq_len - 1).
+ * Contexts longer than partition_size are split into partitions (split-K) whose
+ * partial results go through `workspace` and are merged by a second kernel.
+ * max_seq_len: upper bound of seq_lens (sizes the grid; 0 = max_blocks_per_seq *
+ * block_size).  seq_lens[b] == 0 yields zeros.
+ * q_dtype / kv_dtype: (F32, F32), (BF16, BF16) or (BF16, FP8_E4M3FN).
+ */
+int pa_decode(const void* q, const void* k_cache, const void* v_cache,
+              const float* k_scale, const float* v_scale,
+              const int32_t* block_tables, const int32_t* seq_lens,
+              void* out, void* workspace, size_t workspace_bytes,
+              int B, int Hq, int Hkv, int D, int block_size,
+              int max_blocks_per_seq, int num_blocks, int max_seq_len,
+              float scale, int partition_size, int q_dtype, int kv_dtype,
+              void* stream);
+
+/*
+ * Paged chunked prefill with a cached prefix, causal: query token i of sequence
+ * b (i < query_lens[b]) sees keys j <= seq_lens[b] - query_lens[b] + i
+ * (examples/models/gpt_oss/kernels/attention.py:85,127-135: "query at
+ * start_pos+i attends to keys <= start_pos+i").  The new tokens' K/V are
+ * already in the pool.  dtype: BF16 for q/k/v/out.
+ */
+int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
+               const int32_t* block_tables, const int32_t* seq_lens,
+               const int32_t* query_lens, void* out,
+               int B, int T, int Hq, int Hkv, int D, int block_size,
+               int max_blocks_per_seq, int num_blocks,
+               float scale, int dtype, void* stream);
+
+/*
+ * Block-sparse causal prefill over dense q [B, S, Hq, D], k/v [B, S, Hkv, D]:
+ * q block i attends k block j iff j <= i and (i - j < local_blocks or
+ * (j + h % vert_stride) % vert_stride == 0), token-causal inside a block.
+ * Equals the dense causal prefill of attention.py:112-144 under that mask.
+ * `block` must be 64.  dtype: BF16.
+ */
+int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* out,
+                           int B, int S, int Hq, int Hkv, int D,
+                           int block, int local_blocks, int vert_stride,
+                           float scale, int dtype, void* stream);
+
+/*
+ * Test hook: materialise the block-table gather.  out [B, max_seq_len, Hkv, D]
+ * (elem_bytes per element, bits copied verbatim); rows >= seq_lens[b] are zero.
+ * Bit-exact counterpart of np.take(pool, table, axis=0)
+ * (nkipy/src/nkipy/core/tensor.py:575-640).
+ */
+int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,
+                 void* out, int B, int Hkv, int D, int block_size,
+                 int max_blocks_per_seq, int num_blocks, int max_seq_len,
+                 int elem_bytes, void* stream);
+
+/* Debug switches (process-wide; tests only).  key 0: decode kernel choice
+ * (0 = automatic, 1 = force the scalar-ALU kernel, 2 = force the MFMA kernel);
+ * key 1: waves per workgroup of the MFMA decode kernel (0 = default). */
+int pa_debug_set(int key, int value);
+
+/* Kernel timing for benchmarks: when enabled, every launch of the main kernel
+ * of pa_decode / pa_prefill / pa_blocksparse_prefill is bracketed by HIP events
+ * on its own stream.  pa_profile_collect synchronises those events, writes up
+ * to `cap` durations (milliseconds, oldest first) and clears the list; returns
+ * the number written.  The counterpart of the reference's device-side timing,
+ * spike/src/spike/spike_model.py:290-363. */
+int pa_profile_enable(int on);
+int pa_profile_collect(float* ms, int cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PAGED_ATTN_H_ */

@@ -1,0 +1,63 @@
+"""ctypes binding of libpaged_attn.so (the C ABI declared in include/paged_attn.h).
+
+torch is imported first on purpose: the library links the HIP runtime by soname
+and must share the one instance torch has already loaded, so that device
+pointers and stream handles mean the same thing on both sides.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch  # noqa: F401  (loads the HIP runtime this library binds to)
+
+from .build import LIB_PATH
+
+_lock = threading.Lock()
+_lib = None
+
+c_int, c_float, c_void_p, c_size_t = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+
+SIGNATURES = {
+    "pa_version": (c_int, []),
+    "pa_last_error": (ctypes.c_char_p, []),
+    "pa_decode_workspace_bytes": (c_size_t, [c_int] * 5),
+    "pa_decode": (c_int, [c_void_p] * 9 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p]),
+    "pa_prefill": (c_int, [c_void_p] * 7 + [c_int] * 8 + [c_float, c_int, c_void_p]),
+    "pa_blocksparse_prefill": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_float, c_int, c_void_p]),
+    "pa_gather_kv": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_void_p]),
+    "pa_debug_set": (c_int, [c_int, c_int]),
+    "pa_profile_enable": (c_int, [c_int]),
+    "pa_profile_collect": (c_int, [ctypes.POINTER(c_float), c_int]),
+}
+
+
+class PagedAttnLibraryError(RuntimeError):
+    """The native library is missing or failed to load (no fallback exists)."""
+
+
+def load():
+    """Load the shared library once.  Raises if it has not been built."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise PagedAttnLibraryError(
+                f"{LIB_PATH} not found: build it with `python -m nkipy_amd.build` "
+                "(there is no CPU or PyTorch fallback for these ops)")
+        try:
+            lib = ctypes.CDLL(LIB_PATH)
+        except OSError as e:  # pragma: no cover - depends on the machine
+            raise PagedAttnLibraryError(f"cannot load {LIB_PATH}: {e}") from e
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+        return _lib
+
+
+def last_error() -> str:
+    return load().pa_last_error().decode("utf-8", "replace")

@@ -1,0 +1,55 @@
+"""Builds libpaged_attn.so (HIP kernels + C ABI) for gfx950 with hipcc.
+
+The library has no Python or torch dependency; it links only the HIP runtime.
+Run `python -m nkipy_amd.build` or call `build()`.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libpaged_attn.so")
+
+SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # hipcc must not form packed-fp32 instructions from float code on these machines
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _compile(src: str, extra) -> str:
+    obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(extra_flags=(), jobs: int = 4) -> str:
+    """Compile every HIP source and link the shared library; returns its path."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(extra_flags=sys.argv[1:]))

@@ -1,0 +1,268 @@
+// extern "C" surface of libpaged_attn.so: argument validation on the host,
+// kernel selection, launch.  See include/paged_attn.h for the contract.
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "pa_common.h"
+
+namespace pa {
+
+static thread_local char tl_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(tl_error, sizeof(tl_error), fmt, ap);
+  va_end(ap);
+}
+
+int fail_arg(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(tl_error, sizeof(tl_error), fmt, ap);
+  va_end(ap);
+  return -1;
+}
+
+int check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return 0;
+  set_error("%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+  return (int)e > 0 ? (int)e : 1;
+}
+
+// ---- debug switches ------------------------------------------------------------
+static std::atomic<int> g_decode_impl{0};
+static std::atomic<int> g_decode_waves{0};
+
+// ---- profiling: event pairs around the main kernel of each op ----------------
+static std::atomic<int> g_profile{0};
+static std::mutex g_prof_mu;
+static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
+static thread_local hipEvent_t tl_start = nullptr;
+
+void profile_begin(hipStream_t s) {
+  if (!g_profile.load(std::memory_order_relaxed)) return;
+  hipEvent_t a = nullptr;
+  if (hipEventCreate(&a) != hipSuccess) return;
+  (void)hipEventRecord(a, s);
+  tl_start = a;
+}
+
+void profile_end(hipStream_t s) {
+  if (!tl_start) return;
+  hipEvent_t b = nullptr;
+  if (hipEventCreate(&b) != hipSuccess) { (void)hipEventDestroy(tl_start); tl_start = nullptr; return; }
+  (void)hipEventRecord(b, s);
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof_events.emplace_back(tl_start, b);
+  tl_start = nullptr;
+}
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+static int ilog2_exact(int v) {
+  if (v <= 0 || (v & (v - 1))) return -1;
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+extern "C" {
+
+int pa_version(void) { return 100; }
+
+const char* pa_last_error(void) { return tl_error; }
+
+int pa_debug_set(int key, int value) {
+  if (key == 0) { g_decode_impl = value; return 0; }
+  if (key == 1) { g_decode_waves = value; return 0; }
+  return fail_arg("pa_debug_set: unknown key %d", key);
+}
+
+int pa_profile_enable(int on) {
+  g_profile = on ? 1 : 0;
+  return 0;
+}
+
+int pa_profile_collect(float* ms, int cap) {
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> ev;
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ev.swap(g_prof_events);
+  }
+  int n = 0;
+  for (auto& pr : ev) {
+    float t = 0.f;
+    if (hipEventSynchronize(pr.second) == hipSuccess &&
+        hipEventElapsedTime(&t, pr.first, pr.second) == hipSuccess && ms && n < cap)
+      ms[n++] = t;
+    (void)hipEventDestroy(pr.first);
+    (void)hipEventDestroy(pr.second);
+  }
+  return n;
+}
+
+static int num_partitions_for(int max_seq_len, int partition_size) {
+  if (max_seq_len <= 0) return 1;
+  return (max_seq_len + partition_size - 1) / partition_size;
+}
+
+size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int partition_size) {
+  if (B <= 0 || Hq <= 0 || D <= 0 || partition_size <= 0) return 0;
+  const int np = num_partitions_for(max_seq_len, partition_size);
+  if (np <= 1) return 0;
+  return (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+}
+
+int pa_decode(const void* q, const void* k_cache, const void* v_cache,
+              const float* k_scale, const float* v_scale,
+              const int32_t* block_tables, const int32_t* seq_lens,
+              void* out, void* workspace, size_t workspace_bytes,
+              int B, int Hq, int Hkv, int D, int block_size,
+              int max_blocks_per_seq, int num_blocks, int max_seq_len,
+              float scale, int partition_size, int q_dtype, int kv_dtype,
+              void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_decode: bad sizes B=%d Hq=%d Hkv=%d D=%d", B, Hq, Hkv, D);
+  if (Hq % Hkv) return fail_arg("pa_decode: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0)
+    return fail_arg("pa_decode: bad paging sizes block_size=%d max_blocks_per_seq=%d num_blocks=%d",
+                    block_size, max_blocks_per_seq, num_blocks);
+  if (partition_size <= 0) return fail_arg("pa_decode: partition_size=%d must be positive", partition_size);
+  if (!(q_dtype == PA_F32 && kv_dtype == PA_F32) && !(q_dtype == PA_BF16 && kv_dtype == PA_BF16) &&
+      !(q_dtype == PA_BF16 && kv_dtype == PA_FP8_E4M3FN))
+    return fail_arg("pa_decode: unsupported dtype pair q=%d kv=%d", q_dtype, kv_dtype);
+  if (D != 32 && D != 64 && D != 128 && D != 256) return fail_arg("pa_decode: head_dim %d not in {32,64,128,256}", D);
+  if (B == 0) return 0;
+  if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !out) return fail_arg("pa_decode: null pointer argument");
+  if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_decode: fp8 KV needs k_scale and v_scale");
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return fail_arg("pa_decode: q, k_cache, v_cache and out must be 16-byte aligned");
+  const long cap = (long)max_blocks_per_seq * block_size;
+  if (max_seq_len <= 0 || max_seq_len > cap) max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
+
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
+  p.block_tables = block_tables; p.seq_lens = seq_lens; p.out = out;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
+  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
+  p.block_shift = ilog2_exact(block_size);
+  p.partition_size = partition_size;
+  p.num_partitions = num_partitions_for(max_seq_len, partition_size);
+  p.max_seq_len = max_seq_len;
+  p.scale_log2e = scale * kLog2e;
+  if (p.num_partitions > 65535 || B > 65535) return fail_arg("pa_decode: grid too large (partitions=%d B=%d)", p.num_partitions, B);
+  if (p.num_partitions > 1) {
+    const size_t need = pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size);
+    if (!workspace || workspace_bytes < need)
+      return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
+    p.ws_out = (float*)workspace;
+    p.ws_ml = p.ws_out + (size_t)B * Hq * p.num_partitions * D;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int impl = g_decode_impl.load();
+  bool mfma = decode_mfma_supported(p, q_dtype, kv_dtype);
+  if (impl == 1) mfma = false;
+  if (impl == 2 && !mfma) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
+  if (!mfma && p.num_partitions > 65535) return fail_arg("pa_decode: too many partitions");
+  profile_begin(s);
+  hipError_t e = mfma ? launch_decode_mfma(p, kv_dtype, g_decode_waves.load(), s)
+                      : launch_decode_generic(p, q_dtype, kv_dtype, s);
+  profile_end(s);
+  if (e != hipSuccess) return check_hip(e, "pa_decode launch");
+  if (p.num_partitions > 1) {
+    e = launch_decode_reduce(p, q_dtype, s);
+    if (e != hipSuccess) return check_hip(e, "pa_decode reduce launch");
+  }
+  return 0;
+}
+
+int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
+               const int32_t* block_tables, const int32_t* seq_lens,
+               const int32_t* query_lens, void* out,
+               int B, int T, int Hq, int Hkv, int D, int block_size,
+               int max_blocks_per_seq, int num_blocks,
+               float scale, int dtype, void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_prefill: bad sizes");
+  if (Hq % Hkv) return fail_arg("pa_prefill: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  if (dtype != PA_BF16) return fail_arg("pa_prefill: only bf16 is supported (dtype=%d)", dtype);
+  if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_prefill: bad paging sizes");
+  if (B == 0 || T == 0) return 0;
+  if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens || !out)
+    return fail_arg("pa_prefill: null pointer argument");
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return fail_arg("pa_prefill: q, k_cache, v_cache and out must be 16-byte aligned");
+  PrefillParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q; p.k = k_cache; p.v = v_cache; p.block_tables = block_tables; p.seq_lens = seq_lens;
+  p.query_lens = query_lens; p.out = out;
+  p.B = B; p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
+  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
+  p.scale_log2e = scale * kLog2e;
+  if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipError_t e = launch_prefill(p, s);
+  profile_end(s);
+  return check_hip(e, "pa_prefill launch");
+}
+
+int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* out,
+                           int B, int S, int Hq, int Hkv, int D,
+                           int block, int local_blocks, int vert_stride,
+                           float scale, int dtype, void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || S < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_blocksparse_prefill: bad sizes");
+  if (Hq % Hkv) return fail_arg("pa_blocksparse_prefill: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  if (dtype != PA_BF16) return fail_arg("pa_blocksparse_prefill: only bf16 is supported (dtype=%d)", dtype);
+  if (block != 64) return fail_arg("pa_blocksparse_prefill: sparsity block must be 64 (got %d)", block);
+  if (local_blocks < 1 || vert_stride < 1) return fail_arg("pa_blocksparse_prefill: local_blocks and vert_stride must be >= 1");
+  if (B == 0 || S == 0) return 0;
+  if (!q || !k || !v || !out) return fail_arg("pa_blocksparse_prefill: null pointer argument");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
+    return fail_arg("pa_blocksparse_prefill: q, k, v and out must be 16-byte aligned");
+  PrefillParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q; p.k = k; p.v = v; p.out = out;
+  p.B = B; p.T = S; p.S = S; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
+  p.sparse_local = local_blocks; p.sparse_stride = vert_stride;
+  p.scale_log2e = scale * kLog2e;
+  if (!prefill_supported(p)) return fail_arg("pa_blocksparse_prefill: unsupported shape (D=%d)", D);
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipError_t e = launch_prefill(p, s);
+  profile_end(s);
+  return check_hip(e, "pa_blocksparse_prefill launch");
+}
+
+int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,
+                 void* out, int B, int Hkv, int D, int block_size,
+                 int max_blocks_per_seq, int num_blocks, int max_seq_len,
+                 int elem_bytes, void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || Hkv <= 0 || D <= 0 || block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0 ||
+      max_seq_len < 0 || elem_bytes <= 0)
+    return fail_arg("pa_gather_kv: bad sizes");
+  if ((long)max_seq_len > (long)max_blocks_per_seq * block_size)
+    return fail_arg("pa_gather_kv: max_seq_len=%d exceeds table capacity %ld", max_seq_len,
+                    (long)max_blocks_per_seq * block_size);
+  if (B == 0 || max_seq_len == 0) return 0;
+  if (!cache || !block_tables || !seq_lens || !out) return fail_arg("pa_gather_kv: null pointer argument");
+  if (B > 65535) return fail_arg("pa_gather_kv: B too large");
+  hipError_t e = launch_gather(cache, block_tables, seq_lens, out, B, Hkv * D * elem_bytes, block_size,
+                               max_blocks_per_seq, num_blocks, max_seq_len, (hipStream_t)stream);
+  return check_hip(e, "pa_gather_kv launch");
+}
+
+}  // extern "C"

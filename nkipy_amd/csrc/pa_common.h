@@ -1,0 +1,119 @@
+// Shared device helpers and launch parameter blocks for the paged attention
+// kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/paged_attn.h"
+
+namespace pa {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// ---- host-side error text (thread local) -----------------------------------
+void set_error(const char* fmt, ...);
+int fail_arg(const char* fmt, ...);     // records the text, returns -1
+int check_hip(hipError_t e, const char* what);
+
+// ---- profiling hooks ----------------------------------------------------------
+void profile_begin(hipStream_t s);
+void profile_end(hipStream_t s);
+
+// ---- storage helpers ------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// two floats -> packed bf16 pair (lo = a, hi = b), round-to-nearest-even
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  bf16x2_t v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// four OCP e4m3fn bytes of one dword -> four floats (exact)
+__device__ __forceinline__ void fp8x4_to_float(uint32_t w, float* f) {
+  f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+  f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+  f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
+}
+
+// high halves of two floats packed as a bf16 pair (exact when both values are
+// representable in bf16, as every e4m3 value is): lo = a, hi = b
+__device__ __forceinline__ uint32_t pack_hi16(float a, float b) {
+  return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+
+template <typename T> struct Store;
+template <> struct Store<float> {
+  static __device__ __forceinline__ void put(void* base, long idx, float v) { ((float*)base)[idx] = v; }
+};
+template <> struct Store<uint16_t> {
+  static __device__ __forceinline__ void put(void* base, long idx, float v) {
+    ((uint16_t*)base)[idx] = float_to_bf16_bits(v);
+  }
+};
+
+// ---- decode ------------------------------------------------------------------------
+struct DecodeParams {
+  const void* q;            // [B, Hq, D]
+  const void* k_cache;      // [num_blocks, block_size, Hkv, D]
+  const void* v_cache;
+  const float* k_scale;     // [num_blocks, Hkv] or null
+  const float* v_scale;
+  const int32_t* block_tables;  // [B, max_blocks]
+  const int32_t* seq_lens;      // [B]
+  void* out;                // [B, Hq, D]
+  float* ws_out;            // [B, Hq, P, D]
+  float* ws_ml;             // [B, Hq, P, 2]
+  int B, Hq, Hkv, D;
+  int block_size, max_blocks, num_blocks;
+  int block_shift;          // log2(block_size), or -1 when not a power of two
+  int partition_size, num_partitions, max_seq_len;
+  float scale_log2e;
+};
+
+hipError_t launch_decode_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
+hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hipStream_t s);
+bool decode_mfma_supported(const DecodeParams& p, int q_dtype, int kv_dtype);
+hipError_t launch_decode_reduce(const DecodeParams& p, int q_dtype, hipStream_t s);
+
+// ---- prefill -----------------------------------------------------------------------
+struct PrefillParams {
+  const void* q;            // [B, T, Hq, D] bf16
+  const void* k;            // paged: pool [num_blocks, block_size, Hkv, D]; dense: [B, S, Hkv, D]
+  const void* v;
+  const int32_t* block_tables;  // null for the dense (blocksparse) form
+  const int32_t* seq_lens;      // null for the dense form (then every sequence has S keys)
+  const int32_t* query_lens;    // null for the dense form (then T queries)
+  void* out;
+  int B, T, Hq, Hkv, D;
+  int block_size, max_blocks, num_blocks;
+  int S;                    // dense form: keys per sequence
+  int sparse_local, sparse_stride;  // blocksparse pattern; sparse_stride == 0 -> plain causal
+  float scale_log2e;
+};
+
+hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);
+bool prefill_supported(const PrefillParams& p);
+
+// ---- gather ------------------------------------------------------------------------
+hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,
+                         int B, int row_bytes, int block_size, int max_blocks, int num_blocks,
+                         int max_seq_len, hipStream_t s);
+
+}  // namespace pa

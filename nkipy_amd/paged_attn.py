@@ -1,0 +1,273 @@
+"""Paged flash attention ops on MI355X: NumPy-style signatures over device tensors.
+
+Each op keeps the calling convention of the reference's kernels — positional
+arrays in, array out, static options as keywords (README.md:118-152 of the
+reference) — with the argument order `(q, k_cache, v_cache, block_tables,
+seq_lens, scale) -> out`.  They are hand-kernel ops in the sense of the
+reference's `nki_custom_op` (nkipy/src/nkipy/core/nki_op.py:800-884): there is
+no CPU implementation behind them, and like that hook on the CPU backend
+(nki_op.py:480,557,719-722) they raise NotImplementedError for host arrays.
+
+Ownership follows nkipy/src/nkipy/runtime/device_tensor.py:51-74 and
+spike/src/spike/spike_model.py:248-288: the caller may pass `out=` (written in
+place, returned); otherwise a new tensor is allocated.  Validation errors are
+ValueError (bad shape / dtype / contiguity / device), launch failures are
+RuntimeError, mirroring spike_model.py:198-246.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from . import _lib
+
+F32, BF16, FP8 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float8_e4m3fn: FP8}
+
+_workspaces = {}
+
+
+def _need_device(name, t):
+    if isinstance(t, np.ndarray):
+        raise NotImplementedError(
+            f"{name} is a NumPy array: the paged attention ops run hand-written HIP kernels and have "
+            "no CPU path; pass torch tensors on a ROCm device")
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{name} must be a torch.Tensor on a ROCm device, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise NotImplementedError(f"{name} lives on {t.device}: the paged attention ops have no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _check(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _same_device(ref, **others):
+    for n, t in others.items():
+        if t is not None:
+            _check(t.device == ref.device, f"{n} is on {t.device}, expected {ref.device}")
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _raise_on(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed ({rc}): {_lib.last_error()}")
+
+
+def _kv_code(cache, scale_given):
+    if cache.dtype == torch.uint8:
+        _check(scale_given, "uint8 KV caches are fp8-e4m3fn codes and need k_scale/v_scale")
+        return FP8
+    _check(cache.dtype in _DTYPE_CODE, f"unsupported KV cache dtype {cache.dtype}")
+    return _DTYPE_CODE[cache.dtype]
+
+
+def _check_paging(k_cache, v_cache, block_tables, seq_lens, B):
+    _check(k_cache.dim() == 4, "k_cache must be [num_blocks, block_size, Hkv, D]")
+    _check(v_cache.shape == k_cache.shape and v_cache.dtype == k_cache.dtype,
+           "v_cache must match k_cache in shape and dtype")
+    _check(block_tables.dim() == 2 and block_tables.shape[0] == B and block_tables.dtype == torch.int32,
+           "block_tables must be int32 [B, max_blocks_per_seq]")
+    _check(block_tables.shape[1] > 0, "block_tables needs at least one column")
+    _check(seq_lens.shape == (B,) and seq_lens.dtype == torch.int32, "seq_lens must be int32 [B]")
+
+
+def check_block_tables(block_tables, seq_lens, num_blocks, block_size):
+    """Debug helper (synchronises): every table entry a sequence uses is a valid block id."""
+    bt = block_tables.detach().cpu().numpy()
+    sl = seq_lens.detach().cpu().numpy()
+    for b in range(bt.shape[0]):
+        n = (int(sl[b]) + block_size - 1) // block_size
+        _check(n <= bt.shape[1], f"sequence {b}: seq_len {int(sl[b])} needs {n} blocks, table has {bt.shape[1]}")
+        used = bt[b, :n]
+        _check(used.size == 0 or (used.min() >= 0 and used.max() < num_blocks),
+               f"sequence {b}: block table entry outside [0, {num_blocks})")
+
+
+def decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size) -> int:
+    return int(_lib.load().pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size))
+
+
+def _workspace(device, nbytes):
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, v_scale=None,
+           partition_size=512, max_seq_len=None, out=None, workspace=None, validate_tables=False):
+    """out[b, h] = softmax(q[b, h] . K_b^T * scale) V_b over the paged context.
+
+    q [B, Hq, D] (float32 or bfloat16); k_cache/v_cache [num_blocks, block_size, Hkv, D]
+    in q's dtype, or float8_e4m3fn / uint8 codes with k_scale/v_scale [num_blocks, Hkv]
+    float32; block_tables int32 [B, max_blocks]; seq_lens int32 [B].
+    max_seq_len: host-known upper bound of seq_lens (sizes the split-K grid
+    without a device sync; default = table capacity).
+    """
+    lib = _lib.load()
+    for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache),
+                 ("block_tables", block_tables), ("seq_lens", seq_lens)):
+        _need_device(n, t)
+    _check(q.dim() == 3, "q must be [B, Hq, D]")
+    B, Hq, D = q.shape
+    _check(q.dtype in (torch.float32, torch.bfloat16), f"unsupported q dtype {q.dtype}")
+    _check_paging(k_cache, v_cache, block_tables, seq_lens, B)
+    num_blocks, block_size, Hkv, Dk = k_cache.shape
+    _check(Dk == D, f"head_dim mismatch: q has {D}, cache has {Dk}")
+    _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    _check(D in (32, 64, 128, 256), f"head_dim {D} not in (32, 64, 128, 256)")
+    scaled = k_scale is not None or v_scale is not None
+    kv_code = _kv_code(k_cache, scaled)
+    q_code = _DTYPE_CODE[q.dtype]
+    if kv_code == FP8:
+        _check(q_code == BF16, "fp8 KV needs bfloat16 q")
+        _check(k_scale is not None and v_scale is not None, "fp8 KV needs both k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _need_device(n, t)
+            _check(t.dtype == torch.float32 and t.shape == (num_blocks, Hkv),
+                   f"{n} must be float32 [num_blocks, Hkv]")
+    else:
+        _check(kv_code == q_code, f"KV dtype {k_cache.dtype} does not match q dtype {q.dtype}")
+        _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
+    _check(isinstance(partition_size, int) and partition_size > 0, "partition_size must be a positive int")
+    cap = block_tables.shape[1] * block_size
+    msl = cap if max_seq_len is None else int(max_seq_len)
+    _check(0 < msl <= cap, f"max_seq_len {msl} outside (0, {cap}]")
+    _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
+                 k_scale=k_scale, v_scale=v_scale, out=out)
+    if validate_tables:
+        check_block_tables(block_tables, seq_lens, num_blocks, block_size)
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _need_device("out", out)
+        _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
+    need = int(lib.pa_decode_workspace_bytes(B, Hq, D, msl, partition_size))
+    if workspace is None:
+        workspace = _workspace(q.device, need) if need else None
+    else:
+        _need_device("workspace", workspace)
+        _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    with torch.cuda.device(q.device):
+        rc = lib.pa_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+                           _ptr(block_tables), _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes,
+                           B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
+                           float(scale), partition_size, q_code, kv_code, _stream_ptr(q.device))
+    _raise_on(rc, "pa_decode")
+    return out
+
+
+def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, out=None,
+            validate_tables=False):
+    """Chunked prefill against a cached prefix (causal).
+
+    q [B, T, Hq, D] bfloat16 holds the last query_lens[b] tokens of each sequence
+    (rows t >= query_lens[b] are padding; their output is zero); token i sees keys
+    j <= seq_lens[b] - query_lens[b] + i of the paged context, which already
+    contains the new tokens' K/V.
+    """
+    lib = _lib.load()
+    for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
+                 ("seq_lens", seq_lens), ("query_lens", query_lens)):
+        _need_device(n, t)
+    _check(q.dim() == 4, "q must be [B, T, Hq, D]")
+    B, T, Hq, D = q.shape
+    _check(q.dtype == torch.bfloat16, "prefill supports bfloat16 only")
+    _check_paging(k_cache, v_cache, block_tables, seq_lens, B)
+    _check(k_cache.dtype == torch.bfloat16, "prefill needs a bfloat16 KV cache")
+    _check(query_lens.shape == (B,) and query_lens.dtype == torch.int32, "query_lens must be int32 [B]")
+    num_blocks, block_size, Hkv, Dk = k_cache.shape
+    _check(Dk == D, f"head_dim mismatch: q has {D}, cache has {Dk}")
+    _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
+                 query_lens=query_lens, out=out)
+    if validate_tables:
+        check_block_tables(block_tables, seq_lens, num_blocks, block_size)
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _need_device("out", out)
+        _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
+    with torch.cuda.device(q.device):
+        rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_lens),
+                            _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
+                            block_tables.shape[1], num_blocks, float(scale), BF16, _stream_ptr(q.device))
+    _raise_on(rc, "pa_prefill")
+    return out
+
+
+def blocksparse_prefill(q, k, v, scale, *, block=64, local_blocks=4, vert_stride=8, out=None):
+    """Block-sparse causal prefill over dense q [B, S, Hq, D], k/v [B, S, Hkv, D] (bfloat16).
+
+    q block i attends k block j iff j <= i and (i - j < local_blocks or
+    (j + h % vert_stride) % vert_stride == 0); token-causal inside a block.
+    """
+    lib = _lib.load()
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _need_device(n, t)
+    _check(q.dim() == 4 and k.dim() == 4, "q must be [B, S, Hq, D], k/v [B, S, Hkv, D]")
+    B, S, Hq, D = q.shape
+    _check(q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16,
+           "blocksparse_prefill supports bfloat16 only")
+    _check(v.shape == k.shape and k.shape[0] == B and k.shape[1] == S and k.shape[3] == D,
+           "k/v must be [B, S, Hkv, D] matching q")
+    Hkv = k.shape[2]
+    _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    _check(block == 64, "sparsity block must be 64")
+    _check(local_blocks >= 1 and vert_stride >= 1, "local_blocks and vert_stride must be >= 1")
+    _same_device(q, k=k, v=v, out=out)
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _need_device("out", out)
+        _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
+    with torch.cuda.device(q.device):
+        rc = lib.pa_blocksparse_prefill(_ptr(q), _ptr(k), _ptr(v), _ptr(out), B, S, Hq, Hkv, D, block,
+                                        int(local_blocks), int(vert_stride), float(scale), BF16,
+                                        _stream_ptr(q.device))
+    _raise_on(rc, "pa_blocksparse_prefill")
+    return out
+
+
+def gather_kv(cache, block_tables, seq_lens, max_seq_len=None):
+    """Materialise the block-table gather: [B, max_seq_len, Hkv, D], zero past seq_lens[b]."""
+    lib = _lib.load()
+    for n, t in (("cache", cache), ("block_tables", block_tables), ("seq_lens", seq_lens)):
+        _need_device(n, t)
+    _check(cache.dim() == 4, "cache must be [num_blocks, block_size, Hkv, D]")
+    B = block_tables.shape[0]
+    _check(block_tables.dim() == 2 and block_tables.dtype == torch.int32, "block_tables must be int32 [B, max_blocks]")
+    _check(seq_lens.shape == (B,) and seq_lens.dtype == torch.int32, "seq_lens must be int32 [B]")
+    num_blocks, block_size, Hkv, D = cache.shape
+    cap = block_tables.shape[1] * block_size
+    msl = cap if max_seq_len is None else int(max_seq_len)
+    _check(0 <= msl <= cap, f"max_seq_len {msl} outside [0, {cap}]")
+    out = torch.empty((B, msl, Hkv, D), dtype=cache.dtype, device=cache.device)
+    with torch.cuda.device(cache.device):
+        rc = lib.pa_gather_kv(_ptr(cache), _ptr(block_tables), _ptr(seq_lens), _ptr(out), B, Hkv, D,
+                              block_size, block_tables.shape[1], num_blocks, msl, cache.element_size(),
+                              _stream_ptr(cache.device))
+    _raise_on(rc, "pa_gather_kv")
+    return out
+
+
+def default_scale(head_dim: int) -> float:
+    """1 / sqrt(head_dim) in float32, as examples/models/qwen3/kernels/attention.py:119."""
+    return float(np.float32(1.0) / np.float32(math.sqrt(head_dim)))

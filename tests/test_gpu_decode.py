@@ -1,0 +1,312 @@
+"""GPU parity: HIP paged decode (through the C ABI) vs the NumPy oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_attention_oracle as O
+from tests.pa_testlib import (assert_close_abs, assert_close_fp32, bf16_to_dev, dev_bits, dev_to_f32,
+                              make_paged)
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2   # absolute, bf16 configs
+FP8_TOL = 5e-2    # absolute, fp8 KV after dequantisation
+FP32_REL = 1e-5   # relative to the result's scale, fp32 config
+
+
+@pytest.fixture(scope="module")
+def pa():
+    import nkipy_amd
+    from nkipy_amd import _lib
+    _lib.load()
+    return nkipy_amd
+
+
+def _set_impl(v):
+    from nkipy_amd import _lib
+    _lib.load().pa_debug_set(0, v)
+
+
+def _set_waves(v):
+    from nkipy_amd import _lib
+    _lib.load().pa_debug_set(1, v)
+
+
+def _i32(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.int32)).cuda()
+
+
+def _run_bf16(pa, rng, B, Hq, Hkv, D, bs, ctxs, part, scale=None, impl=0):
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    scale = scale if scale is not None else 1.0 / np.sqrt(D)
+    want = O.paged_decode(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                          np.asarray(ctxs, np.int32), scale, q_dtype="bf16")
+    _set_impl(impl)
+    try:
+        got = pa.decode(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs),
+                        scale, partition_size=part, max_seq_len=max(int(max(ctxs)), 1))
+        torch.cuda.synchronize()
+    finally:
+        _set_impl(0)
+    return dev_to_f32(got), want
+
+
+# ----------------------------------------------------------------------------- config 1 (fp32)
+def test_config1_fp32_exact_config(pa):
+    """BASELINE config 1: B=4, 8/8 heads, D=64, bs=16, ctx U[16,256], pool 128, fp32."""
+    rng = np.random.default_rng(1001)
+    B, H, D, bs = 4, 8, 64, 16
+    ctx = rng.integers(16, 257, size=B)
+    perm = rng.permutation(128).astype(np.int32)
+    nblk = (ctx + bs - 1) // bs
+    tables = np.full((B, 16), -1, np.int32)
+    pos = 0
+    for b in range(B):
+        tables[b, :nblk[b]] = perm[pos:pos + nblk[b]]
+        pos += nblk[b]
+    q = rng.standard_normal((B, H, D)).astype(np.float32)
+    k = rng.standard_normal((128, bs, H, D)).astype(np.float32)
+    v = rng.standard_normal((128, bs, H, D)).astype(np.float32)
+    want = O.paged_decode(q, k, v, tables, ctx.astype(np.int32), 0.125)
+    truth = O.paged_decode(q, k, v, tables, ctx.astype(np.int32), 0.125, acc=np.float64)
+    for part in (512, 64, 16):
+        got = pa.decode(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(),
+                        _i32(tables), _i32(ctx), 0.125, partition_size=part)
+        torch.cuda.synchronize()
+        assert_close_fp32(dev_to_f32(got), want, FP32_REL)
+        assert_close_fp32(dev_to_f32(got), truth, FP32_REL)
+
+
+@pytest.mark.parametrize("D", [32, 64, 128, 256])
+@pytest.mark.parametrize("n_rep", [1, 4])
+def test_fp32_shapes(pa, D, n_rep):
+    rng = np.random.default_rng(7 + D + n_rep)
+    B, Hkv, bs = 3, 2, 8
+    ctxs = [1, 37, 100]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, Hkv * n_rep, D)).astype(np.float32)
+    want = O.paged_decode(q, k, v, tables, np.asarray(ctxs, np.int32), 0.2)
+    got = pa.decode(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(),
+                    _i32(tables), _i32(ctxs), 0.2, partition_size=24)
+    torch.cuda.synchronize()
+    assert_close_fp32(dev_to_f32(got), want, FP32_REL)
+
+
+# ----------------------------------------------------------------------------- bf16
+@pytest.mark.parametrize("impl", [2, 1], ids=["mfma", "scalar"])
+@pytest.mark.parametrize("D,Hq,Hkv,bs", [(128, 32, 8, 32), (128, 8, 8, 16), (64, 16, 2, 16),
+                                         (128, 64, 8, 64), (64, 4, 4, 128), (128, 40, 2, 32)])
+def test_bf16_shapes(pa, impl, D, Hq, Hkv, bs):
+    rng = np.random.default_rng(D * 1000 + Hq * 10 + bs)
+    ctxs = [1, 31, 32, 33, 500, 1025, 64, 77]
+    got, want = _run_bf16(pa, rng, len(ctxs), Hq, Hkv, D, bs, ctxs, part=256, impl=impl)
+    assert_close_abs(got, want, BF16_TOL)
+
+
+@pytest.mark.parametrize("waves", [1, 2, 4])
+def test_bf16_waves_per_workgroup(pa, waves):
+    rng = np.random.default_rng(waves)
+    ctxs = [5, 300, 777, 2048]
+    _set_waves(waves)
+    try:
+        got, want = _run_bf16(pa, rng, 4, 32, 8, 128, 32, ctxs, part=512, impl=2)
+    finally:
+        _set_waves(0)
+    assert_close_abs(got, want, BF16_TOL)
+
+
+def test_zero_length_and_ragged(pa):
+    rng = np.random.default_rng(3)
+    for part in (4096, 64):
+        got, want = _run_bf16(pa, rng, 4, 8, 2, 128, 16, [0, 1, 16, 700], part=part)
+        assert np.all(got[0] == 0)
+        assert_close_abs(got, want, BF16_TOL)
+
+
+def test_partition_size_invariance(pa):
+    rng = np.random.default_rng(11)
+    B, Hq, Hkv, D, bs = 3, 16, 4, 128, 32
+    ctxs = [900, 2000, 64]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    dq, dk, dv = bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v)
+    outs = []
+    for part in (2048, 512, 256, 32):
+        o = pa.decode(dq, dk, dv, _i32(tables), _i32(ctxs), 0.09, partition_size=part, max_seq_len=2000)
+        torch.cuda.synchronize()
+        outs.append(dev_to_f32(o))
+    for o in outs[1:]:
+        assert np.max(np.abs(o - outs[0])) <= 2 ** -7 * max(1.0, np.abs(outs[0]).max())  # a bf16 ulp or so
+
+
+def test_identity_table_equals_dense_cache(pa):
+    """A dense (B, S, Hkv, D) cache viewed as a pool with an identity table."""
+    rng = np.random.default_rng(5)
+    B, S, Hq, Hkv, D, bs = 4, 256, 8, 2, 128, 32
+    ck = O.round_to_bf16(rng.standard_normal((B, S, Hkv, D)).astype(np.float32))
+    cv = O.round_to_bf16(rng.standard_normal((B, S, Hkv, D)).astype(np.float32))
+    q = O.round_to_bf16(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    ctx = np.array([256, 1, 130, 77], np.int32)
+    tables = np.arange(B * S // bs, dtype=np.int32).reshape(B, S // bs)
+    got = pa.decode(bf16_to_dev(q), bf16_to_dev(ck.reshape(-1, bs, Hkv, D)), bf16_to_dev(cv.reshape(-1, bs, Hkv, D)),
+                    _i32(tables), _i32(ctx), 0.1, partition_size=128)
+    torch.cuda.synchronize()
+    want = np.stack([O.dense_attention(q[b][None], ck[b, :ctx[b]], cv[b, :ctx[b]], 0.1, prefix=ctx[b] - 1)[0]
+                     for b in range(B)])
+    assert_close_abs(dev_to_f32(got), O.round_to_bf16(want), BF16_TOL)
+
+
+def test_pool_permutation_gives_identical_bits(pa):
+    """Moving blocks around the pool (and the table with them) must not change one output bit."""
+    rng = np.random.default_rng(9)
+    B, Hq, Hkv, D, bs = 3, 8, 2, 128, 32
+    ctxs = [100, 700, 33]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs, pad_value=0)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    nb = k.shape[0]
+    perm = rng.permutation(nb)
+    k2, v2 = np.empty_like(k), np.empty_like(v)
+    k2[perm], v2[perm] = k, v
+    t2 = perm[tables].astype(np.int32)
+    a = pa.decode(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), 0.09, partition_size=256)
+    b = pa.decode(bf16_to_dev(q), bf16_to_dev(k2), bf16_to_dev(v2), _i32(t2), _i32(ctxs), 0.09, partition_size=256)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(a), dev_bits(b))
+
+
+def test_stale_pool_bytes_do_not_leak(pa):
+    """Rows past seq_len in the last block, unused blocks and padding table entries may hold
+    anything (NaN patterns included) without affecting the result."""
+    rng = np.random.default_rng(13)
+    B, Hq, Hkv, D, bs = 2, 8, 2, 128, 32
+    ctxs = [45, 200]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs, pad_value=-7)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    want = O.paged_decode(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                          np.asarray(ctxs, np.int32), 0.09, q_dtype="bf16")
+    kd, vd = bf16_to_dev(k), bf16_to_dev(v)
+    used = np.zeros(k.shape[:2], bool)
+    for b in range(B):
+        for t in range(ctxs[b]):
+            used[tables[b, t // bs], t % bs] = True
+    mask = torch.from_numpy(~used).cuda()
+    kd[mask] = float("nan")
+    vd[mask] = float("nan")
+    for impl in (2, 1):
+        _set_impl(impl)
+        try:
+            got = pa.decode(bf16_to_dev(q), kd, vd, _i32(tables), _i32(ctxs), 0.09, partition_size=64)
+            torch.cuda.synchronize()
+        finally:
+            _set_impl(0)
+        assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+# ----------------------------------------------------------------------------- fp8 KV
+@pytest.mark.parametrize("impl", [2, 1], ids=["mfma", "scalar"])
+@pytest.mark.parametrize("D,Hq,Hkv,bs", [(128, 64, 8, 64), (128, 8, 2, 16), (64, 8, 1, 32)])
+def test_fp8_kv(pa, impl, D, Hq, Hkv, bs):
+    rng = np.random.default_rng(D + Hq + bs)
+    ctxs = [1, 63, 64, 65, 1500, 300]
+    B = len(ctxs)
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    q = O.round_to_bf16(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_decode(q, kq, vq, tables, np.asarray(ctxs, np.int32), scale, k_scale=ks, v_scale=vs, q_dtype="bf16")
+    _set_impl(impl)
+    try:
+        got = pa.decode(bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+                        torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), scale,
+                        k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(),
+                        partition_size=512)
+        torch.cuda.synchronize()
+    finally:
+        _set_impl(0)
+    assert_close_abs(dev_to_f32(got), want, FP8_TOL)
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)  # in fact as tight as bf16: dequantisation is exact
+
+
+def test_fp8_every_code_decodes_exactly(pa):
+    """All 254 finite e4m3fn codes pass through the device's expansion unchanged:
+    one key, V rows holding each code -> out == decode(code) * scale (ctx = 1)."""
+    D, bs = 128, 16
+    codes = np.array([c for c in range(256) if c not in (0x7F, 0xFF)], np.uint8)
+    nb = (len(codes) + D - 1) // D   # one token per sequence, D codes per row
+    pad = np.zeros(nb * D, np.uint8)
+    pad[:len(codes)] = codes
+    v = np.zeros((nb, bs, 1, D), np.uint8)
+    v[:, 0, 0, :] = pad.reshape(nb, D)
+    k = np.zeros_like(v)
+    sc = np.full((nb, 1), 0.5, np.float32)
+    tables = np.arange(nb, dtype=np.int32)[:, None]
+    q = np.zeros((nb, 1, D), np.float32)
+    for impl in (2, 1):
+        _set_impl(impl)
+        try:
+            got = pa.decode(bf16_to_dev(q), torch.from_numpy(k).cuda().view(torch.float8_e4m3fn),
+                            torch.from_numpy(v).cuda().view(torch.float8_e4m3fn), _i32(tables),
+                            _i32(np.ones(nb)), 1.0, k_scale=torch.from_numpy(sc).cuda(),
+                            v_scale=torch.from_numpy(sc).cuda())
+            torch.cuda.synchronize()
+        finally:
+            _set_impl(0)
+        want = O.round_to_bf16(O.fp8_e4m3fn_decode(pad).reshape(nb, 1, D) * np.float32(0.5))
+        assert np.array_equal(dev_to_f32(got), want)
+
+
+# ----------------------------------------------------------------------------- gather (bit exact)
+@pytest.mark.parametrize("dtype", ["bf16", "fp8", "fp32"])
+def test_gather_bit_exact(pa, dtype):
+    rng = np.random.default_rng(21)
+    B, Hkv, D, bs = 4, 2, 64, 16
+    ctxs = [0, 1, 47, 160]
+    nblk = [(c + bs - 1) // bs for c in ctxs]
+    nb = sum(nblk) + 4
+    perm = rng.permutation(nb).astype(np.int32)
+    tables = np.zeros((B, max(nblk) + 1), np.int32)
+    pos = 0
+    for b in range(B):
+        tables[b, :nblk[b]] = perm[pos:pos + nblk[b]]
+        pos += nblk[b]
+    if dtype == "bf16":
+        bits = rng.integers(0, 65536, size=(nb, bs, Hkv, D)).astype(np.uint16)
+        dev = torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+    elif dtype == "fp8":
+        bits = rng.integers(0, 256, size=(nb, bs, Hkv, D)).astype(np.uint8)
+        dev = torch.from_numpy(bits).cuda().view(torch.float8_e4m3fn)
+    else:
+        bits = rng.integers(0, 2 ** 32, size=(nb, bs, Hkv, D), dtype=np.uint64).astype(np.uint32)
+        dev = torch.from_numpy(bits.view(np.int32)).cuda().view(torch.float32)
+    msl = max(ctxs)
+    got = dev_bits(pa.gather_kv(dev, _i32(tables), _i32(ctxs), max_seq_len=msl))
+    for b in range(B):
+        want = O.gather_kv(bits, tables[b], ctxs[b])
+        assert np.array_equal(got[b, :ctxs[b]], want)
+        assert np.all(got[b, ctxs[b]:] == 0)
+
+
+# ----------------------------------------------------------------------------- host-side errors
+def test_argument_errors(pa):
+    q = torch.zeros(2, 8, 128, dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16, device="cuda")
+    bt = torch.zeros(2, 2, dtype=torch.int32, device="cuda")
+    sl = torch.ones(2, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        pa.decode(q, kc, kc[:, :, :, :64].contiguous(), bt, sl, 1.0)
+    with pytest.raises(ValueError):
+        pa.decode(q, kc, kc, bt.long(), sl, 1.0)
+    with pytest.raises(ValueError):
+        pa.decode(q[:, :7].contiguous(), kc, kc, bt, sl, 1.0)          # 7 q heads over 2 kv heads
+    with pytest.raises(ValueError):
+        pa.decode(q.transpose(0, 1), kc, kc, bt, sl, 1.0)              # not contiguous
+    with pytest.raises(ValueError):
+        pa.decode(q, kc, kc, bt, sl, 1.0, max_seq_len=1000)            # beyond table capacity
+    with pytest.raises(ValueError):
+        pa.decode(q, kc, kc, torch.full_like(bt, 99), sl, 1.0, validate_tables=True)
+    with pytest.raises(NotImplementedError):
+        pa.decode(q.cpu(), kc, kc, bt, sl, 1.0)
+    with pytest.raises(ValueError):
+        pa.decode(q.float(), kc, kc, bt, sl, 1.0)                      # fp32 q with bf16 KV

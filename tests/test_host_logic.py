@@ -1,0 +1,106 @@
+"""CPU-side checks: the C-ABI library loads and exports every declared symbol, host
+validation works without a GPU, and the ops refuse host arrays instead of falling back."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from nkipy_amd import _lib, build
+    if not os.path.exists(build.LIB_PATH):
+        build.build()
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = open(os.path.join(ROOT, "include", "paged_attn.h")).read()
+    names = set(re.findall(r"\b(pa_[a-z0-9_]+)\s*\(", header))
+    assert {"pa_decode", "pa_prefill", "pa_blocksparse_prefill", "pa_gather_kv", "pa_version",
+            "pa_last_error", "pa_decode_workspace_bytes"} <= names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    from nkipy_amd._lib import SIGNATURES
+    assert set(SIGNATURES) == names
+
+
+def test_version_and_workspace_formula(lib):
+    assert lib.pa_version() >= 100
+    assert lib.pa_decode_workspace_bytes(64, 32, 128, 512, 512) == 0          # one partition
+    assert lib.pa_decode_workspace_bytes(64, 32, 128, 8192, 512) == 64 * 32 * 16 * (128 + 2) * 4
+    assert lib.pa_decode_workspace_bytes(2, 4, 64, 513, 512) == 2 * 4 * 2 * 66 * 4
+
+
+def test_c_abi_argument_errors_without_gpu(lib):
+    """Argument errors are found on the host before anything touches a device."""
+    z = ctypes.c_void_p(0)
+    def dec(**kw):
+        a = dict(B=2, Hq=8, Hkv=2, D=128, bs=16, mb=4, nb=8, msl=0, scale=1.0, part=512, qd=1, kd=1)
+        a.update(kw)
+        return lib.pa_decode(z, z, z, z, z, z, z, z, z, 0, a["B"], a["Hq"], a["Hkv"], a["D"], a["bs"],
+                             a["mb"], a["nb"], a["msl"], a["scale"], a["part"], a["qd"], a["kd"], z)
+    assert dec(Hq=7) == -1 and b"multiple" in lib.pa_last_error()
+    assert dec(D=96) == -1 and b"head_dim" in lib.pa_last_error()
+    assert dec(qd=0, kd=1) == -1 and b"dtype" in lib.pa_last_error()
+    assert dec(part=0) == -1
+    assert dec(bs=0) == -1
+    assert dec() == -1 and b"null" in lib.pa_last_error()       # sizes fine, pointers null
+    assert dec(B=0) == 0                                        # empty batch is a no-op
+    assert lib.pa_blocksparse_prefill(z, z, z, z, 1, 64, 4, 4, 128, 32, 4, 8, 1.0, 1, z) == -1
+    assert b"block must be 64" in lib.pa_last_error()
+    assert lib.pa_prefill(z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 0, z) == -1
+    assert lib.pa_gather_kv(z, z, z, z, 1, 2, 64, 16, 2, 8, 100, 2, z) == -1  # beyond table capacity
+
+
+def test_ops_refuse_host_arrays():
+    import nkipy_amd
+    a = np.zeros((1, 1, 64), np.float32)
+    with pytest.raises(NotImplementedError):
+        nkipy_amd.decode(a, a, a, a, a, 1.0)
+    t = torch.zeros(1, 1, 64)
+    with pytest.raises(NotImplementedError):
+        nkipy_amd.decode(t, t, t, t, t, 1.0)
+    with pytest.raises(NotImplementedError):
+        nkipy_amd.prefill(a, a, a, a, a, a, 1.0)
+    with pytest.raises(NotImplementedError):
+        nkipy_amd.blocksparse_prefill(a, a, a, 1.0)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from nkipy_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.PagedAttnLibraryError):
+        _lib.load()
+
+
+def test_workload_index_structures_are_seeded_and_consistent():
+    from nkipy_amd import workloads as W
+    a = W.make_decode(2, device="cpu", shrink=16)
+    b = W.make_decode(2, device="cpu", shrink=16)
+    assert torch.equal(a.block_tables, b.block_tables) and torch.equal(a.seq_lens, b.seq_lens)
+    bt = a.block_tables.numpy()
+    used = bt[bt >= 0]
+    assert len(np.unique(used)) == len(used) and used.max() < a.k_cache.shape[0]
+    nblk = (a.ctx + 31) // 32
+    assert (bt >= 0).sum() == nblk.sum()
+    assert a.k_cache.shape[0] == int(np.ceil(1.1 * nblk.sum()))
+    # algorithmic bytes: K+V rows dominate
+    assert a.algorithmic_bytes() > int(a.ctx.sum()) * 2 * 8 * 128 * 2
+    p = W.make_prefill(device="cpu", shrink=32)
+    t = p.block_tables.numpy()
+    sb = int(p.prefix[0]) // 32
+    assert np.all(p.prefix[:4] == p.prefix[0]) and p.prefix[0] % 32 == 0
+    for b_ in (1, 2, 3):
+        assert np.array_equal(t[b_, :sb], t[0, :sb])
+    priv = np.concatenate([t[0][t[0] >= 0]] + [t[b_, sb:][t[b_, sb:] >= 0] for b_ in (1, 2, 3)] +
+                          [t[b_][t[b_] >= 0] for b_ in range(4, 8)])
+    assert len(np.unique(priv)) == len(priv)
+    s = W.make_blocksparse(device="cpu", shrink=64)
+    assert s.flops() > 0
