@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|5|3|4]
+
+A step is one pass of the op over one batch of synthetic input that is already
+resident in HBM.  Default workload: config 2 (Llama-3-8B-shape paged decode, bf16,
+batch 64, context U[512, 8192], block 32, split-K 512).  Prints ONE JSON line.
+
+value      whole-step throughput: algorithmic HBM bytes / step time for the decode
+           configs (GB/s), attention FLOPs / step time for the prefill configs
+           (TFLOP/s); the step includes every kernel the op launches.
+roofline   the dominant kernel alone, timed with HIP events on its launch stream
+           inside the library (pa_profile_*), over the same K steps.
+cpu_baseline  the NumPy oracle on a bounded sample of the same workload, on this
+           box's host cores (reported, not a target).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+
+
+def _collect_kernel_ms(lib, n):
+    buf = (ctypes.c_float * max(n, 1))()
+    got = lib.pa_profile_collect(buf, n)
+    return [buf[i] for i in range(got)]
+
+
+def _time_steps(step, steps, warmup):
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def _host_info():
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count()
+    return cores
+
+
+def _cpu_decode_baseline(w, budget_s=12.0):
+    """Oracle decode on the first n sequences; n sized so that 1 warm-up + 3
+    repetitions stay near the budget."""
+    from oracle import paged_attention_oracle as O
+    from tests.pa_testlib import dev_bits
+    B = w.q.shape[0]
+    kc, vc = dev_bits(w.k_cache), dev_bits(w.v_cache)
+    q = dev_bits(w.q)
+    tables = w.block_tables.cpu().numpy()
+    ks = w.k_scale.cpu().numpy() if w.k_scale is not None else None
+    vs = w.v_scale.cpu().numpy() if w.v_scale is not None else None
+
+    def run(n):
+        t = time.perf_counter()
+        O.paged_decode(q[:n], kc, vc, tables[:n], w.ctx[:n].astype(np.int32), w.scale,
+                       k_scale=ks, v_scale=vs, q_dtype="bf16")
+        return time.perf_counter() - t
+
+    probe = min(B, 4)
+    t_probe = run(probe)
+    per_seq = t_probe / probe
+    n = int(max(probe, min(B, budget_s / 4.0 / max(per_seq, 1e-6))))
+    times = [run(n) for _ in range(3)]
+    t = float(np.median(times))
+    nb, bs, hkv, d = w.k_cache.shape
+    bytes_n = int(w.ctx[:n].sum()) * 2 * hkv * d * w.k_cache.element_size()
+    return {"value": round(bytes_n / t / 1e9, 4), "unit": "GB/s", "cores": _host_info(), "kind": "port",
+            "tok_per_s": round(n / t, 2),
+            "sample": f"NumPy oracle, first {n} of {B} sequences of the same workload, median of 3 runs "
+                      f"({t:.3f} s each), numpy {np.__version__} default BLAS threading"}
+
+
+def _cpu_prefill_baseline(w, flops_fn, run_fn, desc):
+    t = time.perf_counter()
+    fl = run_fn()
+    dt = time.perf_counter() - t
+    return {"value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": _host_info(), "kind": "port",
+            "sample": f"{desc}, one run of {dt:.2f} s, numpy {np.__version__} default BLAS threading"}
+
+
+def bench_decode(cfg, steps, warmup, lib, pa, W):
+    w = W.make_decode(cfg)
+    out = torch.empty_like(w.q)
+
+    def step():
+        pa.decode(w.q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.scale,
+                  k_scale=w.k_scale, v_scale=w.v_scale, partition_size=w.partition_size,
+                  max_seq_len=w.max_seq_len, out=out)
+
+    sec = _time_steps(step, steps, warmup)
+    lib.pa_profile_enable(1)
+    _time_steps(step, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = _collect_kernel_ms(lib, steps)
+    kavg = float(np.mean(kms)) if kms else float("nan")
+    ab = w.algorithmic_bytes()
+    B, Hq, D = w.q.shape
+    nb, bs, hkv, _ = w.k_cache.shape
+    dtype = "fp8-e4m3 KV / bf16 q, fp32 accumulate" if cfg == 5 else "bf16, fp32 accumulate"
+    res = {
+        "metric": "decode attn HBM GB/s (% peak) + tok/s",
+        "value": round(ab / sec / 1e9, 2), "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * ab / sec / 1e9 / HBM_PEAK_GBS, 2),
+        "tok_per_s": round(B / sec, 1),
+        "ms_per_step": round(sec * 1e3, 5),
+        "dtype": dtype,
+        "config": {"workload": f"C{cfg} paged decode: B={B}, Hq={Hq}, Hkv={hkv}, D={D}, block_size={bs}, "
+                               f"ctx sum={int(w.ctx.sum())} (min {int(w.ctx.min())}, max {int(w.ctx.max())}), "
+                               f"pool={nb} blocks, partition={w.partition_size}",
+                   "algorithmic_bytes": ab},
+        "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel": "decode_mfma_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "launches_timed": len(kms)},
+    }
+    res["cpu_baseline"] = _cpu_decode_baseline(w)
+    return res
+
+
+def bench_prefill(steps, warmup, lib, pa, W):
+    from oracle import paged_attention_oracle as O
+    from tests.pa_testlib import dev_bits
+    w = W.make_prefill()
+    out = torch.empty_like(w.q)
+
+    def step():
+        pa.prefill(w.q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens, w.scale, out=out)
+
+    sec = _time_steps(step, steps, warmup)
+    lib.pa_profile_enable(1)
+    _time_steps(step, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = _collect_kernel_ms(lib, steps)
+    kavg = float(np.mean(kms))
+    fl = w.flops()
+    B, T, Hq, D = w.q.shape
+
+    def cpu():
+        heads = [0, 1, 2, 3]
+        O.paged_prefill(dev_bits(w.q), dev_bits(w.k_cache), dev_bits(w.v_cache), w.block_tables.cpu().numpy(),
+                        w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy(), w.scale, seqs=[7], heads=heads)
+        return 4 * D * len(heads) * (T * int(w.prefix[7]) + T * (T + 1) // 2)
+
+    res = {
+        "metric": "prefill attn TFLOP/s (% MFMA peak)",
+        "value": round(fl / sec / 1e12, 2), "unit": "TFLOP/s",
+        "pct_of_bf16_peak": round(100.0 * fl / sec / 1e12 / BF16_PEAK_TFLOPS, 2),
+        "ms_per_step": round(sec * 1e3, 5), "dtype": "bf16, fp32 accumulate",
+        "config": {"workload": f"C3 paged chunked prefill: B={B}, T={T}, Hq={Hq}, Hkv={w.k_cache.shape[2]}, "
+                               f"D={D}, block_size={w.k_cache.shape[1]}, prefix={w.prefix.tolist()}",
+                   "flops": fl},
+        "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "kernel": "prefill_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "launches_timed": len(kms)},
+    }
+    res["cpu_baseline"] = _cpu_prefill_baseline(w, None, cpu, "NumPy oracle, sequence 7, q heads 0-3 of the same workload")
+    return res
+
+
+def bench_blocksparse(steps, warmup, lib, pa, W):
+    from oracle import paged_attention_oracle as O
+    from tests.pa_testlib import dev_bits
+    w = W.make_blocksparse()
+    out = torch.empty_like(w.q)
+
+    def step():
+        pa.blocksparse_prefill(w.q, w.k, w.v, w.scale, block=w.block, local_blocks=w.local_blocks,
+                               vert_stride=w.vert_stride, out=out)
+
+    sec = _time_steps(step, steps, warmup)
+    lib.pa_profile_enable(1)
+    _time_steps(step, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = _collect_kernel_ms(lib, steps)
+    kavg = float(np.mean(kms))
+    fl = w.flops()
+    B, S, H, D = w.q.shape
+
+    def cpu():
+        O.blocksparse_prefill(dev_bits(w.q), dev_bits(w.k), dev_bits(w.v), w.scale, block=w.block,
+                              local_blocks=w.local_blocks, vert_stride=w.vert_stride, items=[(0, 0)])
+        return fl // (B * H)
+
+    res = {
+        "metric": "prefill attn TFLOP/s (% MFMA peak)",
+        "value": round(fl / sec / 1e12, 2), "unit": "TFLOP/s",
+        "pct_of_bf16_peak": round(100.0 * fl / sec / 1e12 / BF16_PEAK_TFLOPS, 2),
+        "ms_per_step": round(sec * 1e3, 5), "dtype": "bf16, fp32 accumulate",
+        "config": {"workload": f"C4 blocksparse prefill: B={B}, S={S}, H={H}, D={D}, block={w.block}, "
+                               f"local={w.local_blocks}, vert_stride={w.vert_stride}", "flops": fl},
+        "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "kernel": "prefill_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "launches_timed": len(kms)},
+    }
+    res["cpu_baseline"] = _cpu_prefill_baseline(
+        w, None, cpu, "NumPy oracle (dense masked scores), batch 0 head 0 of the same workload; FLOPs counted as the sparse ones")
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is measured on ONE GPU (the kernel on one GPU's share at its real "
+              "shape); --gpus N with N > 1 is not supported.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm device visible; this benchmark has no CPU path.", file=sys.stderr)
+        sys.exit(3)
+    import nkipy_amd as pa
+    from nkipy_amd import _lib, workloads as W
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+    if args.no_cpu:
+        global _cpu_decode_baseline, _cpu_prefill_baseline
+        _cpu_decode_baseline = lambda *a, **k: None      # noqa: E731
+        _cpu_prefill_baseline = lambda *a, **k: None     # noqa: E731
+    if args.config in (2, 5):
+        res = bench_decode(args.config, args.steps, args.warmup, lib, pa, W)
+    elif args.config == 3:
+        res = bench_prefill(args.steps, args.warmup, lib, pa, W)
+    else:
+        res = bench_blocksparse(args.steps, args.warmup, lib, pa, W)
+    line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"),
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": res.pop("dtype"), "data": "synthetic (seeded N(0,1), random block tables)",
+            "config": res.pop("config")}
+    line.update(res)
+    line["device"] = torch.cuda.get_device_name(0)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
