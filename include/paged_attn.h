@@ -55,9 +55,10 @@ int pa_version(void);
  * status strings of spike/src/include/error.h:23-43. */
 const char* pa_last_error(void);
 
-/* Bytes of scratch pa_decode needs for split-K partials: per (sequence, q head,
- * partition) D floats of normalised partial output plus (max, sum).  Zero when
- * max_seq_len fits one partition. */
+/* Bytes of scratch that is enough for pa_decode whichever kernel it picks: split-K
+ * partials of D floats of normalised output plus (max, sum) each — one per
+ * (sequence, q head, partition) for the fixed-partition kernels, one per
+ * (q head, sequence + chunk) for the balanced MFMA schedule. */
 size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int partition_size);
 
 /*
@@ -65,8 +66,13 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
  *   out[b, h, :] = softmax(q[b, h, :] . K_b^T * scale) V_b,  K_b/V_b = the first
  *   seq_lens[b] rows gathered through block_tables[b]   (the decode branch of
  *   examples/models/qwen3/kernels/attention.py:103-144, start_pos = seq_len - 1).
- * Contexts longer than partition_size are split into partitions (split-K) whose
- * partial results go through `workspace` and are merged by a second kernel.
+ * Long contexts are split (split-K); partial results go through `workspace` and
+ * are merged by a second kernel.  The scalar-ALU kernel (fp32, odd shapes) and
+ * the fixed-partition MFMA kernel cut every context into partition_size-token
+ * partitions; the default MFMA kernel for bf16 / fp8 KV instead cuts the
+ * flattened stream of all sequences' 32-token tiles into equal chunks, one per
+ * resident wavefront group, so its partition length follows the batch and the
+ * device, not partition_size.  The result does not depend on the split.
  * max_seq_len: upper bound of seq_lens (sizes the grid; 0 = max_blocks_per_seq *
  * block_size).  seq_lens[b] == 0 yields zeros.
  * q_dtype / kv_dtype: (F32, F32), (BF16, BF16) or (BF16, FP8_E4M3FN).
@@ -118,8 +124,10 @@ int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* 
                  int elem_bytes, void* stream);
 
 /* Debug switches (process-wide; tests only).  key 0: decode kernel choice
- * (0 = automatic, 1 = force the scalar-ALU kernel, 2 = force the MFMA kernel);
- * key 1: waves per workgroup of the MFMA decode kernel (0 = default). */
+ * (0 = automatic, 1 = scalar-ALU kernel, 2 = MFMA kernel with fixed partitions,
+ * 3 = MFMA kernel with the balanced schedule); key 1: waves per workgroup of the
+ * fixed-partition MFMA kernel (0 = default); key 2: its grid order (1 = kv head
+ * fastest, the default; 0 = partition fastest). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

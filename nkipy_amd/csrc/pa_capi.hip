@@ -37,6 +37,7 @@ int check_hip(hipError_t e, const char* what) {
 // ---- debug switches ------------------------------------------------------------
 static std::atomic<int> g_decode_impl{0};
 static std::atomic<int> g_decode_waves{0};
+static std::atomic<int> g_head_major{1};
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 static std::atomic<int> g_profile{0};
@@ -64,6 +65,23 @@ void profile_end(hipStream_t s) {
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+// CUs of the current device (256 on MI355X), cached; 256 when no device is visible
+// so that size queries work on a build machine.
+static int current_num_cus() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 256; }
+  int v = cached[dev].load(std::memory_order_relaxed);
+  if (v > 0) return v;
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
 static int ilog2_exact(int v) {
   if (v <= 0 || (v & (v - 1))) return -1;
   int s = 0;
@@ -84,6 +102,7 @@ const char* pa_last_error(void) { return tl_error; }
 int pa_debug_set(int key, int value) {
   if (key == 0) { g_decode_impl = value; return 0; }
   if (key == 1) { g_decode_waves = value; return 0; }
+  if (key == 2) { g_head_major = value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -118,8 +137,11 @@ static int num_partitions_for(int max_seq_len, int partition_size) {
 size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int partition_size) {
   if (B <= 0 || Hq <= 0 || D <= 0 || partition_size <= 0) return 0;
   const int np = num_partitions_for(max_seq_len, partition_size);
-  if (np <= 1) return 0;
-  return (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+  const size_t fixed = np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+  // the balanced schedule keeps one partial per (q head, sequence + chunk); at
+  // most 8 chunks per CU exist whatever the head layout
+  const size_t balanced = decode_balanced_workspace_bytes(B, Hq, D, 8 * current_num_cus());
+  return fixed > balanced ? fixed : balanced;
 }
 
 int pa_decode(const void* q, const void* k_cache, const void* v_cache,
@@ -160,24 +182,40 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   p.num_partitions = num_partitions_for(max_seq_len, partition_size);
   p.max_seq_len = max_seq_len;
   p.scale_log2e = scale * kLog2e;
+  p.head_major = g_head_major.load();
   if (p.num_partitions > 65535 || B > 65535) return fail_arg("pa_decode: grid too large (partitions=%d B=%d)", p.num_partitions, B);
-  if (p.num_partitions > 1) {
-    const size_t need = pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size);
+  hipStream_t s = (hipStream_t)stream;
+  // kernel choice: 0 automatic, 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced
+  const int impl = g_decode_impl.load();
+  const bool mfma_ok = decode_mfma_supported(p, q_dtype, kv_dtype);
+  if ((impl == 2 || impl == 3) && !mfma_ok) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
+  if (impl == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
+  const int kind = !mfma_ok || impl == 1 ? 1 : (impl == 2 ? 2 : 3);
+  if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
+  if (kind == 3) {
+    plan_decode_balanced(p, current_num_cus());
+    const size_t need = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
     if (!workspace || workspace_bytes < need)
       return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
+    p.ws_out = (float*)workspace;
+    p.ws_ml = p.ws_out + (size_t)Hq * ((size_t)B + p.bal_gv) * D;
+    profile_begin(s);
+    hipError_t e = launch_decode_balanced(p, kv_dtype, s);
+    profile_end(s);
+    if (e != hipSuccess) return check_hip(e, "pa_decode launch");
+    e = launch_decode_balanced_reduce(p, s);
+    return check_hip(e, "pa_decode reduce launch");
+  }
+  if (p.num_partitions > 1) {
+    const size_t need = (size_t)B * Hq * p.num_partitions * ((size_t)D + 2) * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+      return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     p.ws_out = (float*)workspace;
     p.ws_ml = p.ws_out + (size_t)B * Hq * p.num_partitions * D;
   }
-  hipStream_t s = (hipStream_t)stream;
-  const int impl = g_decode_impl.load();
-  bool mfma = decode_mfma_supported(p, q_dtype, kv_dtype);
-  if (impl == 1) mfma = false;
-  if (impl == 2 && !mfma) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
-  if (!mfma && p.num_partitions > 65535) return fail_arg("pa_decode: too many partitions");
   profile_begin(s);
-  hipError_t e = mfma ? launch_decode_mfma(p, kv_dtype, g_decode_waves.load(), s)
-                      : launch_decode_generic(p, q_dtype, kv_dtype, s);
+  hipError_t e = kind == 2 ? launch_decode_mfma(p, kv_dtype, g_decode_waves.load(), s)
+                           : launch_decode_generic(p, q_dtype, kv_dtype, s);
   profile_end(s);
   if (e != hipSuccess) return check_hip(e, "pa_decode launch");
   if (p.num_partitions > 1) {

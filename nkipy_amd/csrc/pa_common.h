@@ -85,12 +85,18 @@ struct DecodeParams {
   int block_shift;          // log2(block_size), or -1 when not a power of two
   int partition_size, num_partitions, max_seq_len;
   float scale_log2e;
+  int head_major;           // fixed-partition grid order: kv head fastest (1) or partition fastest (0)
+  int bal_hsw, bal_ns, bal_gv;  // balanced schedule: head slots and chunks per workgroup, total chunks
 };
 
 hipError_t launch_decode_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
 hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hipStream_t s);
 bool decode_mfma_supported(const DecodeParams& p, int q_dtype, int kv_dtype);
 hipError_t launch_decode_reduce(const DecodeParams& p, int q_dtype, hipStream_t s);
+void plan_decode_balanced(DecodeParams& p, int num_cus);
+size_t decode_balanced_workspace_bytes(int B, int Hq, int D, int gv);
+hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream_t s);
+hipError_t launch_decode_balanced_reduce(const DecodeParams& p, hipStream_t s);
 
 // ---- prefill -----------------------------------------------------------------------
 struct PrefillParams {

@@ -62,52 +62,65 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(uint32_t a, uint32_t b, uint32_t c
   return __builtin_bit_cast(bf16x8_t, v);
 }
 
-// One 32-token tile as loaded (raw bits).
+// One 32-token tile as loaded (raw bits), K and V halves separately so that
+// their register lifetimes can interleave (K of tile n dies after the scores,
+// which frees its registers for V of tile n+1).
 template <int D, bool FP8>
-struct Tile {
-  static constexpr int VEC = D / 16;                       // d's per lane for V
+struct KTile {
   static constexpr int KLD = FP8 ? D / 64 : D / 32;        // 16-byte K loads per 16-token sub-tile
-  static constexpr int VW = (VEC * (FP8 ? 1 : 2)) / 4;     // dwords per V load
   uint32_t k[2][KLD][4];
+  float ksc[2];             // fp8 only: scales of the two 16-token halves
+};
+template <int D, bool FP8>
+struct VTile {
+  static constexpr int VEC = D / 16;                       // d's per lane for V
+  static constexpr int VW = (VEC * (FP8 ? 1 : 2)) / 4;     // dwords per V load
   uint32_t v[8][VW];
-  float ksc[2], vsc[2];     // fp8 only: scales of the two 16-token halves
+  float vsc[2];
 };
 
-template <int D, bool FP8, int NW>
-__global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
-  using T = Tile<D, FP8>;
-  constexpr int VEC = T::VEC, KLD = T::KLD, VW = T::VW;
-  constexpr int KSTEPS = D / 32;
-  constexpr int ESZ = FP8 ? 1 : 2;
-  constexpr int OSTRIDE = D + 16;   // LDS row stride (floats) for the merge
+// Per-wavefront streaming state: Q fragments, online-softmax state and output
+// accumulators for up to 16 query heads of one kv head of one sequence.
+template <int D, bool FP8>
+struct DecodeWave {
+  using KT = KTile<D, FP8>;
+  using VT = VTile<D, FP8>;
+  static constexpr int VEC = VT::VEC, KLD = KT::KLD, VW = VT::VW;
+  static constexpr int KSTEPS = D / 32;
+  static constexpr int ESZ = FP8 ? 1 : 2;
 
-  const int part = blockIdx.x, b = blockIdx.z;
-  const int n_rep = p.Hq / p.Hkv;
-  const int gchunks = (n_rep + 15) / 16;
-  const int hk = blockIdx.y / gchunks;
-  const int hbase = hk * n_rep + (blockIdx.y % gchunks) * 16;       // first q head of this chunk
-  const int nheads = min(16, n_rep - (blockIdx.y % gchunks) * 16);  // valid columns
-
-  int ctx = p.seq_lens[b];
-  ctx = min(max(ctx, 0), p.max_seq_len);
-  const int t_begin = part * p.partition_size;
-  const int tid = threadIdx.x;
-  if (t_begin >= ctx) {
-    if (ctx == 0 && part == 0 && p.num_partitions == 1) {
-      for (int i = tid; i < nheads * D; i += NW * 64)
-        ((uint16_t*)p.out)[((long)b * p.Hq + hbase) * D + i] = 0;
-    }
-    return;
-  }
-  const int t_end = min(ctx, t_begin + p.partition_size);
-  const int ntiles = (t_end - t_begin + 31) >> 5;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, g = lane >> 4;
-
-  // ---- Q^T fragments (B operand), zero for padded head columns --------------
+  const DecodeParams& p;
+  int hk, hbase, nheads;     // kv head, first q head, valid q-head columns
+  int r, g, krow;            // lane = 16 g + r; row order of the K sub-tile
+  const int32_t* table;
+  const char* kbase;
+  const char* vbase;
+  long row_stride;           // bytes between consecutive tokens of a block
+  int last;                  // ctx - 1 of the current sequence
   bf16x8_t qf[KSTEPS];
-  {
+  bf16x8_t pf;               // P^T fragment of the current tile
+  f32x4_t oacc[VEC];
+  float m_run, l_run;
+
+  __device__ __forceinline__ DecodeWave(const DecodeParams& p_, int head_slot, int lane) : p(p_) {
+    const int n_rep = p.Hq / p.Hkv;
+    const int gchunks = (n_rep + 15) / 16;
+    hk = head_slot / gchunks;
+    hbase = hk * n_rep + (head_slot % gchunks) * 16;
+    nheads = min(16, n_rep - (head_slot % gchunks) * 16);
+    r = lane & 15;
+    g = lane >> 4;
+    krow = 4 * (r & 3) + (r >> 2);
+    row_stride = (long)p.Hkv * D * ESZ;
+    kbase = (const char*)p.k_cache + (long)hk * D * ESZ;
+    vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
+  }
+
+  // Start on sequence b (context ctx >= 1): load Q^T fragments (B operand, zero
+  // for padded head columns) and reset the softmax state.
+  __device__ __forceinline__ void begin(int b, int ctx) {
+    table = p.block_tables + (long)b * p.max_blocks;
+    last = ctx - 1;
     const uint16_t* qrow = (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -117,62 +130,65 @@ __global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
       if (r < nheads) v = *(const uint4*)(qrow + d0);
       qf[s] = __builtin_bit_cast(bf16x8_t, v);
     }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) oacc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    m_run = -INFINITY;
+    l_run = 0.f;
   }
 
-  const int32_t* table = p.block_tables + (long)b * p.max_blocks;
-  const long row_stride = (long)p.Hkv * D * ESZ;   // bytes between consecutive tokens of a block
-  const char* kbase = (const char*)p.k_cache + (long)hk * D * ESZ;
-  const char* vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
-  const int krow = 4 * (r & 3) + (r >> 2);         // row order of the K sub-tile
-  const int last = ctx - 1;
-
-  // Issue the loads of tile `ti` (tokens t0 .. t0+31).  Rows past the context
-  // are redirected to the last valid token so that no stale pool bytes (which
-  // could be NaN patterns) ever reach the matrix cores.
-  auto load_tile = [&](T& tl, int ti) {
-    const int t0 = t_begin + (ti << 5);
-    // the two 16-token halves each lie inside one block (block_size is a power
-    // of two >= 16 and t0 is a multiple of 32)
+  // Pool rows of tokens t0 and t0+16 (the two 16-token halves of a tile each lie
+  // inside one block: block_size is a power of two >= 16, t0 a multiple of 32).
+  struct TileRows { long row0, row1; int blk0, blk1, lmax; };
+  __device__ __forceinline__ TileRows tile_rows(int t0) const {
+    TileRows tr;
     const int t1 = min(t0 + 16, last);             // wave-uniform
-    int blk0 = table[t0 >> p.block_shift];
-    int blk1 = table[t1 >> p.block_shift];
-    blk0 = min(max(blk0, 0), p.num_blocks - 1);
-    blk1 = min(max(blk1, 0), p.num_blocks - 1);
+    const int blk0 = table[t0 >> p.block_shift];
+    const int blk1 = table[t1 >> p.block_shift];
+    tr.blk0 = min(max(blk0, 0), p.num_blocks - 1);
+    tr.blk1 = min(max(blk1, 0), p.num_blocks - 1);
     const int bmask = p.block_size - 1;
-    const long row0 = (long)blk0 * p.block_size + (t0 & bmask);          // pool row of token t0
-    const long row1 = (long)blk1 * p.block_size + ((t0 + 16) & bmask);   // pool row of token t0+16
+    tr.row0 = (long)tr.blk0 * p.block_size + (t0 & bmask);
+    tr.row1 = (long)tr.blk1 * p.block_size + ((t0 + 16) & bmask);
+    tr.lmax = last - t0;                           // largest valid local index (>= 0)
+    return tr;
+  }
+
+  // Loads of the tile starting at token t0.  Rows past the context are
+  // redirected to the last valid token so that no stale pool bytes (which could
+  // be NaN patterns) ever reach the matrix cores.
+  __device__ __forceinline__ void load_k(KT& tl, int t0) const {
+    const TileRows tr = tile_rows(t0);
     if (FP8) {
-      tl.ksc[0] = p.k_scale[(long)blk0 * p.Hkv + hk];
-      tl.ksc[1] = p.k_scale[(long)blk1 * p.Hkv + hk];
-      tl.vsc[0] = p.v_scale[(long)blk0 * p.Hkv + hk];
-      tl.vsc[1] = p.v_scale[(long)blk1 * p.Hkv + hk];
+      tl.ksc[0] = p.k_scale[(long)tr.blk0 * p.Hkv + hk];
+      tl.ksc[1] = p.k_scale[(long)tr.blk1 * p.Hkv + hk];
     }
-    const int lmax = last - t0;                    // largest valid local index (>= 0)
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int tl_ = min(16 * u + krow, lmax);
-      const long row = (tl_ < 16) ? row0 + tl_ : row1 + (tl_ - 16);
+      const int tl_ = min(16 * u + krow, tr.lmax);
+      const long row = (tl_ < 16) ? tr.row0 + tl_ : tr.row1 + (tl_ - 16);
       const char* rowp = kbase + row * row_stride;
 #pragma unroll
       for (int s = 0; s < KLD; ++s) VecLoad<4>::get(rowp + (4 * s + g) * 16, tl.k[u][s]);
     }
+  }
+  __device__ __forceinline__ void load_v(VT& tl, int t0) const {
+    const TileRows tr = tile_rows(t0);
+    if (FP8) {
+      tl.vsc[0] = p.v_scale[(long)tr.blk0 * p.Hkv + hk];
+      tl.vsc[1] = p.v_scale[(long)tr.blk1 * p.Hkv + hk];
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int tl_ = min(4 * j + g, lmax);
-      const long row = (tl_ < 16) ? row0 + tl_ : row1 + (tl_ - 16);
+      const int tl_ = min(4 * j + g, tr.lmax);
+      const long row = (tl_ < 16) ? tr.row0 + tl_ : tr.row1 + (tl_ - 16);
       const char* rowp = vbase + row * row_stride;
       VecLoad<VW>::get(rowp + r * (VEC * ESZ), tl.v[j]);
     }
-  };
+  }
 
-  f32x4_t oacc[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) oacc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
-
-  auto compute_tile = [&](const T& tl, int ti) {
-    const int t0 = t_begin + (ti << 5);
-    // ---- scores ----
+  // Scores of the tile at t0 (tokens >= t_end masked), online softmax update,
+  // rescale of the accumulators, P^T fragment.
+  __device__ __forceinline__ void scores_softmax(const KT& tl, const VT& vt, int t0, int t_end) {
     f32x4_t sacc[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -198,7 +214,6 @@ __global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
         }
       }
     }
-    // ---- online softmax for this lane's head column ----
     float sv[8];
     float tmax = -INFINITY;
 #pragma unroll
@@ -228,11 +243,14 @@ __global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
     for (int e = 0; e < VEC; ++e) oacc[e] *= alpha;
     if (FP8) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { pr[i] *= tl.vsc[0]; pr[4 + i] *= tl.vsc[1]; }
+      for (int i = 0; i < 4; ++i) { pr[i] *= vt.vsc[0]; pr[4 + i] *= vt.vsc[1]; }
     }
-    const bf16x8_t pf = as_bf16x8(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]),
-                                  pack_bf16x2(pr[4], pr[5]), pack_bf16x2(pr[6], pr[7]));
-    // ---- V^T fragments: in-register transpose, then O^T += V^T P^T ----
+    pf = as_bf16x8(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]),
+                   pack_bf16x2(pr[4], pr[5]), pack_bf16x2(pr[6], pr[7]));
+  }
+
+  // V^T fragments by in-register transpose, then O^T += V^T P^T.
+  __device__ __forceinline__ void accumulate_pv(const VT& tl) {
     if (!FP8) {
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
@@ -259,38 +277,132 @@ __global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
         }
       }
     }
-  };
+  }
 
-  // ---- stream this wave's tiles, next tile's loads in flight during compute ----
-  {
-    T ta, tb;
-    int ti = wave;
-    if (ti < ntiles) {
-      load_tile(ta, ti);
-      while (true) {
-        if (ti + NW < ntiles) load_tile(tb, ti + NW);
-        compute_tile(ta, ti);
-        ti += NW;
-        if (ti >= ntiles) break;
-        if (ti + NW < ntiles) load_tile(ta, ti + NW);
-        compute_tile(tb, ti);
-        ti += NW;
-        if (ti >= ntiles) break;
-      }
+  // Stream n tiles starting at tokens t_first, t_first + t_step, ...; the next
+  // tile's K is requested before the scores of the current one, its V before the
+  // current P.V.  Loads inside the loop are unconditional (the remainder is
+  // peeled) so that the wait counters stay exact and a wait for tile i never
+  // includes the loads of tile i+1.
+  __device__ __forceinline__ void stream(int t_first, int t_step, int n, int t_end) {
+    if (n <= 0) return;
+    KT ka, kb;
+    VT va, vb;
+    int t = t_first;
+    load_k(ka, t);
+    load_v(va, t);
+    int i = 0;
+    while (i + 2 < n) {
+      load_k(kb, t + t_step);
+      scores_softmax(ka, va, t, t_end);
+      load_v(vb, t + t_step);
+      accumulate_pv(va);
+      load_k(ka, t + 2 * t_step);
+      scores_softmax(kb, vb, t + t_step, t_end);
+      load_v(va, t + 2 * t_step);
+      accumulate_pv(vb);
+      i += 2;
+      t += 2 * t_step;
+    }
+    if (i + 1 < n) {
+      load_k(kb, t + t_step);
+      scores_softmax(ka, va, t, t_end);
+      load_v(vb, t + t_step);
+      accumulate_pv(va);
+      scores_softmax(kb, vb, t + t_step, t_end);
+      accumulate_pv(vb);
+    } else {
+      scores_softmax(ka, va, t, t_end);
+      accumulate_pv(va);
     }
   }
+
+  // Sum of exponentials over the whole tile stream (all lanes of a head column).
+  __device__ __forceinline__ float total_l() const {
+    float l = l_run;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    return l;
+  }
+
+  // Write this wave's normalised result for its head columns: lane (g, r) holds,
+  // for i = 0..3, the VEC consecutive d's starting at VEC * (4g + i).
+  __device__ __forceinline__ void store_final(int b, float l) const {
+    if (r >= nheads) return;
+    const float inv = 1.f / l;
+    uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hbase + r) * D;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t w[VEC / 2];
+#pragma unroll
+      for (int e = 0; e < VEC; e += 2)
+        w[e / 2] = (uint32_t)float_to_bf16_bits(oacc[e][i] * inv) |
+                   ((uint32_t)float_to_bf16_bits(oacc[e + 1][i] * inv) << 16);
+      uint32_t* o = (uint32_t*)(dst + VEC * (4 * g + i));
+      if (VEC == 8) *(uint4*)o = make_uint4(w[0], w[1], w[2], w[3]);
+      else *(uint2*)o = make_uint2(w[0], w[1 % (VEC / 2)]);
+    }
+  }
+  __device__ __forceinline__ void store_partial(long slot, float l) const {
+    if (r >= nheads) return;
+    const float inv = 1.f / l;
+    float* dst = p.ws_out + slot * D;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int e = 0; e < VEC; e += 4)
+        *(float4*)(dst + VEC * (4 * g + i) + e) =
+            make_float4(oacc[e][i] * inv, oacc[e + 1][i] * inv, oacc[e + 2][i] * inv, oacc[e + 3][i] * inv);
+    }
+    if (g == 0) { p.ws_ml[slot * 2] = m_run; p.ws_ml[slot * 2 + 1] = l; }
+  }
+};
+
+__device__ __forceinline__ int clamp_ctx(const DecodeParams& p, int b) {
+  return min(max(p.seq_lens[b], 0), p.max_seq_len);
+}
+
+// ---------------------------------------------------------------------------
+// Fixed partitions: one workgroup per (partition, head slot, sequence), NW waves
+// interleave the partition's tiles and merge through LDS.
+// ---------------------------------------------------------------------------
+template <int D, bool FP8, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void decode_mfma_kernel(DecodeParams p) {
+  using W = DecodeWave<D, FP8>;
+  constexpr int VEC = W::VEC;
+  constexpr int OSTRIDE = D + 16;   // LDS row stride (floats) for the merge
+
+  const int part = p.head_major ? blockIdx.y : blockIdx.x, b = blockIdx.z;
+  const int hidx = p.head_major ? blockIdx.x : blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  W w(p, hidx, lane);
+  const int ctx = clamp_ctx(p, b);
+  const int t_begin = part * p.partition_size;
+  if (t_begin >= ctx) {
+    if (ctx == 0 && part == 0 && p.num_partitions == 1) {
+      for (int i = tid; i < w.nheads * D; i += NW * 64)
+        ((uint16_t*)p.out)[((long)b * p.Hq + w.hbase) * D + i] = 0;
+    }
+    return;
+  }
+  const int t_end = min(ctx, t_begin + p.partition_size);
+  const int ntiles = (t_end - t_begin + 31) >> 5;
+  w.begin(b, ctx);
+  w.stream(t_begin + 32 * wave, 32 * NW, (ntiles - wave + NW - 1) / NW, t_end);
 
   // ---- merge the NW wave states through LDS ----
   __shared__ float sm_m[NW][16];
   __shared__ float sm_l[NW][16];
   __shared__ __attribute__((aligned(16))) float sm_o[NW][16][OSTRIDE];
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-  if (g == 0) { sm_m[wave][r] = m_run; sm_l[wave][r] = l_run; }
+  const float l_tot = w.total_l();
+  const int r = w.r, g = w.g, nheads = w.nheads;
+  if (g == 0) { sm_m[wave][r] = w.m_run; sm_l[wave][r] = l_tot; }
   if (r < nheads) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e)   // value for d = VEC*(4g+i) + e stored at e*16 + 4g + i
-      *(f32x4_t*)&sm_o[wave][r][e * 16 + 4 * g] = oacc[e];
+      *(f32x4_t*)&sm_o[wave][r][e * 16 + 4 * g] = w.oacc[e];
   }
   __syncthreads();
   for (int idx = tid; idx < nheads * D; idx += NW * 64) {
@@ -298,16 +410,16 @@ __global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
     const int pos = (d % VEC) * 16 + d / VEC;
     float mt = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) mt = fmaxf(mt, sm_m[w][h]);
+    for (int x = 0; x < NW; ++x) mt = fmaxf(mt, sm_m[x][h]);
     float lt = 0.f, ot = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      const float wt = __builtin_amdgcn_exp2f(sm_m[w][h] - mt);   // idle waves: 2^-inf = 0
-      lt += sm_l[w][h] * wt;
-      ot += sm_o[w][h][pos] * wt;
+    for (int x = 0; x < NW; ++x) {
+      const float wt = __builtin_amdgcn_exp2f(sm_m[x][h] - mt);   // idle waves: 2^-inf = 0
+      lt += sm_l[x][h] * wt;
+      ot += sm_o[x][h][pos] * wt;
     }
     const float o = ot / lt;
-    const int hq = hbase + h;
+    const int hq = w.hbase + h;
     if (p.num_partitions == 1) {
       ((uint16_t*)p.out)[((long)b * p.Hq + hq) * D + d] = float_to_bf16_bits(o);
     } else {
@@ -318,15 +430,162 @@ __global__ __launch_bounds__(NW * 64) void decode_mfma_kernel(DecodeParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Balanced schedule.  The 32-token tiles of all sequences form one flattened
+// stream of N tiles; it is cut into gv equal chunks of L = ceil(N / gv) tiles,
+// one per resident group of wavefronts, so every group streams the same number
+// of bytes whatever the mix of context lengths.  A workgroup holds `hsw` head
+// slots x `ns` chunks: the waves of one chunk read the same token rows for
+// different kv heads at the same time, which makes each 64 KB block of the pool
+// one contiguous DRAM stream.  Waves never synchronise.
+// A chunk may cover the tail of one sequence, whole sequences, and the head of
+// another; each (sequence, chunk) piece yields either the final output (when
+// the sequence lies inside one chunk) or a split-K partial in slot
+// [q head][b + chunk], merged by decode_balanced_reduce_kernel.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int tiles_of(int ctx) { return (ctx + 31) >> 5; }
+
+// Wave-wide: total number of tiles, and (if f >= 0) the sequence holding
+// flattened tile f with the number of tiles before it.
+__device__ __forceinline__ int scan_tiles(const DecodeParams& p, int lane, int f, int* b_out, int* start_out) {
+  int base = 0;
+  bool found = false;
+  for (int bb = 0; bb < p.B; bb += 64) {
+    const int t = (bb + lane < p.B) ? tiles_of(clamp_ctx(p, bb + lane)) : 0;
+    int incl = t;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += v;
+    }
+    const int total = __shfl(incl, 63, 64);
+    if (!found && f >= 0 && f < base + total) {
+      const unsigned long long m = __ballot(base + incl > f);
+      const int idx = __ffsll((long long)m) - 1;
+      *b_out = bb + idx;
+      *start_out = base + __shfl(incl - t, idx, 64);
+      found = true;
+    }
+    base += total;
+  }
+  return base;
+}
+
+template <int D, bool FP8>
+__global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p) {
+  using W = DecodeWave<D, FP8>;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n_rep = p.Hq / p.Hkv;
+  const int head_slots = p.Hkv * ((n_rep + 15) / 16);
+  const int hs = blockIdx.y * p.bal_hsw + wave % p.bal_hsw;
+  if (hs >= head_slots) return;
+  const int cv = blockIdx.x * p.bal_ns + wave / p.bal_hsw;   // chunk of this wave
+  const int gv = p.bal_gv;
+
+  int dummy_b = 0, dummy_s = 0;
+  const int N = scan_tiles(p, lane, -1, &dummy_b, &dummy_s);
+  if (N == 0) return;
+  const int L = (N + gv - 1) / gv;
+  int f = cv * L;
+  if (f >= N) return;
+  const int f_end = min(N, f + L);
+  int b = 0, start = 0;
+  scan_tiles(p, lane, f, &b, &start);
+  b = __builtin_amdgcn_readfirstlane(b);
+  start = __builtin_amdgcn_readfirstlane(start);
+
+  W w(p, hs, lane);
+  while (f < f_end) {
+    const int ctx = clamp_ctx(p, b);
+    const int T = tiles_of(ctx);
+    if (T == 0) { ++b; continue; }
+    const int ti = f - start;
+    const int n = min(T - ti, f_end - f);
+    w.begin(b, ctx);
+    w.stream(ti << 5, 32, n, ctx);
+    const float l = w.total_l();
+    const int c_first = start / L, c_last = (start + T - 1) / L;
+    if (c_first == c_last) {
+      w.store_final(b, l);
+    } else if (w.r < w.nheads) {
+      w.store_partial((long)(w.hbase + w.r) * (p.B + gv) + b + cv, l);
+    }
+    f += n;
+    start += T;
+    ++b;
+  }
+}
+
+// Merge of the balanced schedule's partials for one (q head, sequence).
+template <int D>
+__global__ __launch_bounds__(64) void decode_balanced_reduce_kernel(DecodeParams p) {
+  const int hq = blockIdx.x, b = blockIdx.y;
+  const int lane = threadIdx.x;
+  int bb = 0, start = 0;
+  const int N = scan_tiles(p, lane, -1, &bb, &start);
+  const int T = tiles_of(clamp_ctx(p, b));
+  uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hq) * D;
+  constexpr int PER = D / 64;   // d's per lane
+  if (T == 0) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) dst[lane * PER + i] = 0;
+    return;
+  }
+  const int gv = p.bal_gv;
+  const int L = (N + gv - 1) / gv;
+  // tiles before sequence b: flattened index of its first tile
+  {
+    int base = 0;
+    for (int x = 0; x < p.B; x += 64) {
+      const int t = (x + lane < p.B && x + lane < b) ? tiles_of(clamp_ctx(p, x + lane)) : 0;
+      int sum = t;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+      base += sum;
+      if (x + 64 > b) break;
+    }
+    start = base;
+  }
+  const int c_first = start / L, c_last = (start + T - 1) / L;
+  if (c_first == c_last) return;   // written by the streaming kernel
+  const long base_slot = (long)hq * (p.B + gv) + b;
+  float mt = -INFINITY;
+  for (int c = c_first; c <= c_last; ++c) mt = fmaxf(mt, p.ws_ml[(base_slot + c) * 2]);
+  float lt = 0.f, acc[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) acc[i] = 0.f;
+  for (int c = c_first; c <= c_last; ++c) {
+    const float wt = p.ws_ml[(base_slot + c) * 2 + 1] * exp2f(p.ws_ml[(base_slot + c) * 2] - mt);
+    lt += wt;
+    const float* src = p.ws_out + (base_slot + c) * D + lane * PER;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) acc[i] += wt * src[i];
+  }
+  const float inv = 1.f / lt;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) dst[lane * PER + i] = float_to_bf16_bits(acc[i] * inv);
+}
+
 template <int D, bool FP8>
 hipError_t launch_typed(const DecodeParams& p, int waves, hipStream_t s) {
   const int n_rep = p.Hq / p.Hkv;
   dim3 grid(p.num_partitions, p.Hkv * ((n_rep + 15) / 16), p.B);
+  if (p.head_major) grid = dim3(p.Hkv * ((n_rep + 15) / 16), p.num_partitions, p.B);
   switch (waves) {
     case 1: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 1>), grid, dim3(64), 0, s, p); break;
     case 2: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 2>), grid, dim3(128), 0, s, p); break;
     default: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 4>), grid, dim3(256), 0, s, p); break;
   }
+  return hipGetLastError();
+}
+
+template <int D, bool FP8>
+hipError_t launch_balanced_typed(const DecodeParams& p, hipStream_t s) {
+  const int n_rep = p.Hq / p.Hkv;
+  const int head_slots = p.Hkv * ((n_rep + 15) / 16);
+  dim3 grid(p.bal_gv / p.bal_ns, (head_slots + p.bal_hsw - 1) / p.bal_hsw);
+  hipLaunchKernelGGL((decode_balanced_kernel<D, FP8>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
   return hipGetLastError();
 }
 
@@ -337,7 +596,6 @@ bool decode_mfma_supported(const DecodeParams& p, int q_dtype, int kv_dtype) {
   if (kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN) return false;
   if (p.D != 64 && p.D != 128) return false;
   if (p.block_shift < 4) return false;   // power-of-two block size >= 16
-  if (p.partition_size % 32 != 0) return false;
   return true;
 }
 
@@ -346,6 +604,36 @@ hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hi
   if (p.D == 128) return fp8 ? launch_typed<128, true>(p, waves, s) : launch_typed<128, false>(p, waves, s);
   if (p.D == 64) return fp8 ? launch_typed<64, true>(p, waves, s) : launch_typed<64, false>(p, waves, s);
   return hipErrorInvalidValue;
+}
+
+void plan_decode_balanced(DecodeParams& p, int num_cus) {
+  const int n_rep = p.Hq / p.Hkv;
+  const int head_slots = p.Hkv * ((n_rep + 15) / 16);
+  constexpr int kWavesPerCu = 8;                       // two per SIMD at this register footprint
+  p.bal_hsw = head_slots < kWavesPerCu ? head_slots : kWavesPerCu;
+  p.bal_ns = kWavesPerCu / p.bal_hsw;
+  const int head_groups = (head_slots + p.bal_hsw - 1) / p.bal_hsw;
+  int wgs = num_cus / head_groups;                     // workgroups per head group: one per CU in total
+  if (wgs < 1) wgs = 1;
+  p.bal_gv = wgs * p.bal_ns;
+}
+
+size_t decode_balanced_workspace_bytes(int B, int Hq, int D, int gv) {
+  return (size_t)Hq * ((size_t)B + gv) * ((size_t)D + 2) * sizeof(float);
+}
+
+hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream_t s) {
+  const bool fp8 = kv_dtype == PA_FP8_E4M3FN;
+  if (p.D == 128) return fp8 ? launch_balanced_typed<128, true>(p, s) : launch_balanced_typed<128, false>(p, s);
+  if (p.D == 64) return fp8 ? launch_balanced_typed<64, true>(p, s) : launch_balanced_typed<64, false>(p, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_decode_balanced_reduce(const DecodeParams& p, hipStream_t s) {
+  dim3 grid(p.Hq, p.B);
+  if (p.D == 128) hipLaunchKernelGGL(decode_balanced_reduce_kernel<128>, grid, dim3(64), 0, s, p);
+  else hipLaunchKernelGGL(decode_balanced_reduce_kernel<64>, grid, dim3(64), 0, s, p);
+  return hipGetLastError();
 }
 
 }  // namespace pa

@@ -94,7 +94,7 @@ def test_fp32_shapes(pa, D, n_rep):
 
 
 # ----------------------------------------------------------------------------- bf16
-@pytest.mark.parametrize("impl", [2, 1], ids=["mfma", "scalar"])
+@pytest.mark.parametrize("impl", [3, 2, 1], ids=["balanced", "mfma", "scalar"])
 @pytest.mark.parametrize("D,Hq,Hkv,bs", [(128, 32, 8, 32), (128, 8, 8, 16), (64, 16, 2, 16),
                                          (128, 64, 8, 64), (64, 4, 4, 128), (128, 40, 2, 32)])
 def test_bf16_shapes(pa, impl, D, Hq, Hkv, bs):
@@ -113,6 +113,24 @@ def test_bf16_waves_per_workgroup(pa, waves):
         got, want = _run_bf16(pa, rng, 4, 32, 8, 128, 32, ctxs, part=512, impl=2)
     finally:
         _set_waves(0)
+    assert_close_abs(got, want, BF16_TOL)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,lo,hi", [
+    (150, 8, 2, 0, 200),      # more sequences than lanes: multi-pass scan, many empty ones
+    (3, 32, 8, 3000, 9000),   # few long sequences: every sequence split over many chunks
+    (1, 8, 1, 20000, 20001),  # one kv head: eight chunks per workgroup
+    (40, 48, 3, 1, 700),      # head slots do not divide the workgroup evenly
+    (9, 32, 16, 100, 1200),   # more head slots than a workgroup holds: two head groups
+    (5, 40, 2, 50, 900),      # 20 q heads per kv head: two 16-column chunks per kv head
+])
+def test_balanced_schedule_shapes(pa, B, Hq, Hkv, lo, hi):
+    rng = np.random.default_rng(B * 7 + Hq)
+    ctxs = rng.integers(lo, hi, size=B).tolist()
+    if B > 10:
+        ctxs[3] = 0
+        ctxs[-1] = 0
+    got, want = _run_bf16(pa, rng, B, Hq, Hkv, 128, 32, ctxs, part=512, impl=3)
     assert_close_abs(got, want, BF16_TOL)
 
 
@@ -193,7 +211,7 @@ def test_stale_pool_bytes_do_not_leak(pa):
     mask = torch.from_numpy(~used).cuda()
     kd[mask] = float("nan")
     vd[mask] = float("nan")
-    for impl in (2, 1):
+    for impl in (3, 2, 1):
         _set_impl(impl)
         try:
             got = pa.decode(bf16_to_dev(q), kd, vd, _i32(tables), _i32(ctxs), 0.09, partition_size=64)
@@ -204,7 +222,7 @@ def test_stale_pool_bytes_do_not_leak(pa):
 
 
 # ----------------------------------------------------------------------------- fp8 KV
-@pytest.mark.parametrize("impl", [2, 1], ids=["mfma", "scalar"])
+@pytest.mark.parametrize("impl", [3, 2, 1], ids=["balanced", "mfma", "scalar"])
 @pytest.mark.parametrize("D,Hq,Hkv,bs", [(128, 64, 8, 64), (128, 8, 2, 16), (64, 8, 1, 32)])
 def test_fp8_kv(pa, impl, D, Hq, Hkv, bs):
     rng = np.random.default_rng(D + Hq + bs)
@@ -243,7 +261,7 @@ def test_fp8_every_code_decodes_exactly(pa):
     sc = np.full((nb, 1), 0.5, np.float32)
     tables = np.arange(nb, dtype=np.int32)[:, None]
     q = np.zeros((nb, 1, D), np.float32)
-    for impl in (2, 1):
+    for impl in (3, 2, 1):
         _set_impl(impl)
         try:
             got = pa.decode(bf16_to_dev(q), torch.from_numpy(k).cuda().view(torch.float8_e4m3fn),
