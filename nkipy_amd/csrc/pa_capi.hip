@@ -247,6 +247,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.query_lens = query_lens; p.out = out;
   p.B = B; p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
+  p.block_shift = ilog2_exact(block_size);
   p.scale_log2e = scale * kLog2e;
   if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
   hipStream_t s = (hipStream_t)stream;
@@ -275,6 +276,7 @@ int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* ou
   p.q = q; p.k = k; p.v = v; p.out = out;
   p.B = B; p.T = S; p.S = S; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
   p.sparse_local = local_blocks; p.sparse_stride = vert_stride;
+  p.block_shift = -1;
   p.scale_log2e = scale * kLog2e;
   if (!prefill_supported(p)) return fail_arg("pa_blocksparse_prefill: unsupported shape (D=%d)", D);
   hipStream_t s = (hipStream_t)stream;

@@ -109,6 +109,7 @@ struct PrefillParams {
   void* out;
   int B, T, Hq, Hkv, D;
   int block_size, max_blocks, num_blocks;
+  int block_shift;          // log2(block_size), or -1 when not a power of two
   int S;                    // dense form: keys per sequence
   int sparse_local, sparse_stride;  // blocksparse pattern; sparse_stride == 0 -> plain causal
   float scale_log2e;

@@ -1,0 +1,198 @@
+"""GPU parity: HIP chunked prefill and blocksparse prefill (through the C ABI) vs the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_attention_oracle as O
+from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_bits, dev_to_f32, make_paged
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def pa():
+    import nkipy_amd
+    from nkipy_amd import _lib
+    _lib.load()
+    return nkipy_amd
+
+
+def _i32(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.int32)).cuda()
+
+
+def _prefill_case(pa, rng, T, qlens, prefixes, Hq, Hkv, bs, D=128, scale=None):
+    B = len(qlens)
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, [max(c, 1) for c in ctxs])
+    q = rng.standard_normal((B, T, Hq, D)).astype(np.float32)
+    scale = scale if scale is not None else 1.0 / np.sqrt(D)
+    want = O.paged_prefill(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                           np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale, q_dtype="bf16")
+    got = pa.prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), scale)
+    torch.cuda.synchronize()
+    return dev_to_f32(got), want
+
+
+@pytest.mark.parametrize("bs", [16, 32, 64])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (4, 4)])
+def test_prefill_with_prefix_ragged(pa, bs, Hq, Hkv):
+    rng = np.random.default_rng(bs + Hq)
+    got, want = _prefill_case(pa, rng, T=200, qlens=[200, 77, 1, 130], prefixes=[0, 300, 65, 1000],
+                              Hq=Hq, Hkv=Hkv, bs=bs)
+    assert_close_abs(got, want, BF16_TOL)
+    assert np.all(got[1, 77:] == 0) and np.all(got[2, 1:] == 0)   # padding rows
+
+
+def test_prefill_many_tiles_and_exact_multiples(pa):
+    rng = np.random.default_rng(5)
+    got, want = _prefill_case(pa, rng, T=384, qlens=[384, 256, 128], prefixes=[640, 64, 0], Hq=4, Hkv=1, bs=32)
+    assert_close_abs(got, want, BF16_TOL)
+
+
+def test_prefill_zero_query_sequence(pa):
+    rng = np.random.default_rng(6)
+    got, want = _prefill_case(pa, rng, T=64, qlens=[0, 64], prefixes=[10, 3], Hq=2, Hkv=2, bs=16)
+    assert np.all(got[0] == 0)
+    assert_close_abs(got, want, BF16_TOL)
+
+
+def test_prefill_T1_equals_decode(pa):
+    rng = np.random.default_rng(7)
+    B, Hq, Hkv, D, bs = 3, 8, 2, 128, 32
+    ctxs = [1, 200, 777]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, 1, Hq, D)).astype(np.float32)
+    dk, dv = bf16_to_dev(k), bf16_to_dev(v)
+    a = pa.prefill(bf16_to_dev(q), dk, dv, _i32(tables), _i32(ctxs), _i32([1, 1, 1]), 0.09)
+    b = pa.decode(bf16_to_dev(q[:, 0]), dk, dv, _i32(tables), _i32(ctxs), 0.09)
+    torch.cuda.synchronize()
+    assert np.max(np.abs(dev_to_f32(a)[:, 0] - dev_to_f32(b))) <= 2 ** -6
+
+
+def test_prefill_shared_prefix_blocks(pa):
+    """Sequences whose tables alias the same physical prefix blocks (and have the same new
+    tokens) produce bit-identical outputs."""
+    rng = np.random.default_rng(8)
+    Hq, Hkv, D, bs, T, P = 4, 2, 128, 32, 96, 128
+    nb = 20
+    k = rng.standard_normal((nb, bs, Hkv, D)).astype(np.float32)
+    v = rng.standard_normal((nb, bs, Hkv, D)).astype(np.float32)
+    shared = [3, 9, 1, 14]
+    t0 = shared + [5, 6, 7]
+    t1 = shared + [10, 11, 12]
+    for a_, b_ in zip(t0[4:], t1[4:]):
+        k[b_], v[b_] = k[a_], v[a_]
+    tables = np.array([t0, t1], np.int32)
+    q1 = rng.standard_normal((1, T, Hq, D)).astype(np.float32)
+    q = np.concatenate([q1, q1])
+    got = pa.prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32([P + T] * 2),
+                     _i32([T, T]), 0.09)
+    torch.cuda.synchronize()
+    bits = dev_bits(got)
+    assert np.array_equal(bits[0], bits[1])
+    want = O.paged_prefill(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                           np.array([P + T] * 2, np.int32), np.array([T, T], np.int32), 0.09)
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_prefill_stale_pool_bytes_do_not_leak(pa):
+    rng = np.random.default_rng(9)
+    B, Hq, Hkv, D, bs, T = 2, 4, 2, 128, 32, 70
+    prefixes, qlens = [45, 3], [70, 50]
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs, pad_value=-3)
+    q = rng.standard_normal((B, T, Hq, D)).astype(np.float32)
+    want = O.paged_prefill(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                           np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), 0.09)
+    kd, vd = bf16_to_dev(k), bf16_to_dev(v)
+    used = np.zeros(k.shape[:2], bool)
+    for b in range(B):
+        for t in range(ctxs[b]):
+            used[tables[b, t // bs], t % bs] = True
+    mask = torch.from_numpy(~used).cuda()
+    kd[mask] = float("nan")
+    vd[mask] = float("nan")
+    qd = bf16_to_dev(q)
+    qd[1, 50:] = float("nan")      # padding query rows may hold anything as well
+    got = pa.prefill(qd, kd, vd, _i32(tables), _i32(ctxs), _i32(qlens), 0.09)
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_config3_shape_shrunk(pa):
+    """BASELINE config 3 at 1/8 length (T=256, prefix U[0,512]) with aliased prefix blocks."""
+    from nkipy_amd import workloads as W
+    w = W.make_prefill(shrink=8)
+    got = pa.prefill(w.q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens, w.scale,
+                     validate_tables=True)
+    torch.cuda.synchronize()
+    want = O.paged_prefill(dev_bits(w.q), dev_bits(w.k_cache), dev_bits(w.v_cache), w.block_tables.cpu().numpy(),
+                           w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy(), w.scale)
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+# ----------------------------------------------------------------------------- blocksparse
+@pytest.mark.parametrize("Hq,Hkv,S,local,stride", [(4, 4, 512, 2, 3), (8, 2, 448, 4, 8), (2, 2, 100, 1, 2),
+                                                  (9, 9, 704, 3, 4)])
+def test_blocksparse_vs_oracle(pa, Hq, Hkv, S, local, stride):
+    rng = np.random.default_rng(S + Hq)
+    B, D = 2, 128
+    q = rng.standard_normal((B, S, Hq, D)).astype(np.float32)
+    k = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
+    v = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
+    scale = 1.0 / np.sqrt(D)
+    want = O.blocksparse_prefill(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), scale, block=64,
+                                 local_blocks=local, vert_stride=stride)
+    got = pa.blocksparse_prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), scale, block=64,
+                                 local_blocks=local, vert_stride=stride)
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_blocksparse_all_active_equals_dense_causal(pa):
+    """local_blocks >= number of blocks: the sparse op is plain causal attention, which the
+    paged prefill op computes too (identity block table, no prefix)."""
+    rng = np.random.default_rng(33)
+    B, S, H, D, bs = 2, 320, 4, 128, 32
+    q = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    k = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    v = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    dq, dk, dv = bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v)
+    a = pa.blocksparse_prefill(dq, dk, dv, 0.09, local_blocks=1000, vert_stride=8)
+    tables = np.arange(B * S // bs, dtype=np.int32).reshape(B, S // bs)
+    b = pa.prefill(dq, dk.view(-1, bs, H, D), dv.view(-1, bs, H, D), _i32(tables), _i32([S] * B), _i32([S] * B), 0.09)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(a), dev_bits(b))
+    want = np.stack([O.dense_attention(O.round_to_bf16(q[i]), O.round_to_bf16(k[i]), O.round_to_bf16(v[i]), 0.09, prefix=0)
+                     for i in range(B)])
+    assert_close_abs(dev_to_f32(a), O.round_to_bf16(want), BF16_TOL)
+
+
+def test_config4_shape_shrunk(pa):
+    """BASELINE config 4 at 1/8 length (S=1024): 32 heads MHA, local 4 + every 8th, per-head phase."""
+    from nkipy_amd import workloads as W
+    w = W.make_blocksparse(shrink=8)
+    got = pa.blocksparse_prefill(w.q, w.k, w.v, w.scale, block=w.block, local_blocks=w.local_blocks,
+                                 vert_stride=w.vert_stride)
+    torch.cuda.synchronize()
+    want = O.blocksparse_prefill(dev_bits(w.q), dev_bits(w.k), dev_bits(w.v), w.scale, block=w.block,
+                                 local_blocks=w.local_blocks, vert_stride=w.vert_stride)
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_prefill_argument_errors(pa):
+    q = torch.zeros(1, 8, 4, 128, dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16, device="cuda")
+    bt = torch.zeros(1, 2, dtype=torch.int32, device="cuda")
+    one = torch.ones(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        pa.prefill(q.float(), kc, kc, bt, one, one, 1.0)
+    with pytest.raises(ValueError):
+        pa.prefill(q[:, :, :3].contiguous(), kc, kc, bt, one, one, 1.0)
+    with pytest.raises(ValueError):
+        pa.blocksparse_prefill(q, q, q, 1.0, block=32)
+    with pytest.raises(RuntimeError):
+        pa.prefill(q[..., :64].contiguous(), kc[..., :64].contiguous(), kc[..., :64].contiguous(), bt, one, one, 1.0)
