@@ -129,7 +129,7 @@ def bench_decode(cfg, steps, warmup, lib, pa, W):
                    "algorithmic_bytes": ab},
         "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "decode_mfma_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "traffic": None, "kernel": "decode_balanced_kernel", "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms)},
     }
     res["cpu_baseline"] = _cpu_decode_baseline(w)
