@@ -26,6 +26,8 @@
 // -100000 there; an exact zero weight here, which is the same number in fp32).
 // The block-sparse form adds the block predicate to the same loop: inactive key
 // tiles are never loaded.
+#include <atomic>
+
 #include "pa_common.h"
 
 namespace pa {
@@ -49,10 +51,14 @@ __device__ __forceinline__ bool block_active(int i, int j, int head, int local, 
   return j <= i && ((i - j) < local || ((j + head % stride) % stride) == 0);
 }
 
-template <bool SPARSE>
+// MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16
+// (one table entry per 16-key group, looked up once per wave on the scalar unit);
+// 2 = paged, any block size (every staged key resolves its own table entry).
+template <bool SPARSE, int MODE>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
-  __shared__ __attribute__((aligned(16))) char ks[BN * K_ROW_BYTES];
-  __shared__ __attribute__((aligned(16))) char vts[VT_BYTES];
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  // two stages, each: K tile [64][272 B] then V^T tile
+  constexpr int STAGE_BYTES = BN * K_ROW_BYTES + VT_BYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -66,7 +72,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   int tq = p.query_lens ? p.query_lens[b] : p.T;
   int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
   tq = min(max(tq, 0), p.T);
-  if (p.block_tables) ctx = min(ctx, p.max_blocks * p.block_size);
+  if (MODE != 0) ctx = min(ctx, p.max_blocks * p.block_size);
   ctx = max(ctx, tq);
   const int prefix = ctx - tq;
   const int q0 = qt * BM;
@@ -107,37 +113,61 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   const int kchunk = tid & 15, kkey = tid >> 4;
   const int vg = tid >> 4;                                       // slot group: slots 4vg .. 4vg+3
   const int vkey0 = 32 * (vg >> 3) + 16 * ((vg >> 2) & 1) + 8 * (vg & 1) + 4 * ((vg >> 1) & 1);
-  const int32_t* table = p.block_tables ? p.block_tables + (long)b * p.max_blocks : nullptr;
+  const int32_t* table = MODE != 0 ? p.block_tables + (long)b * p.max_blocks : nullptr;
   const long kv_row_stride = (long)p.Hkv * HD;                   // elements between consecutive tokens
   const uint16_t* kbase = (const uint16_t*)p.k + (long)hk * HD;
   const uint16_t* vbase = (const uint16_t*)p.v + (long)hk * HD;
 
-  auto pool_row = [&](int key) __attribute__((always_inline)) -> long {                        // row of key `key` (clamped into the context)
+  // generic: row of key `key` (clamped into the context), one table lookup per lane
+  auto pool_row = [&](int key) __attribute__((always_inline)) -> long {
     key = min(key, ctx - 1);
-    if (!table) return (long)b * p.S + key;
-    int blk;
-    int off;
+    if (MODE == 0) return (long)b * p.S + key;
+    int blk, off;
     if (p.block_shift >= 0) { blk = table[key >> p.block_shift]; off = key & (p.block_size - 1); }
     else { blk = table[key / p.block_size]; off = key % p.block_size; }
     blk = min(max(blk, 0), p.num_blocks - 1);
     return (long)blk * p.block_size + off;
   };
+  // fast: first pool row of the 16-key group that starts at the wave-uniform key kb
+  // (the group lies inside one block and inside the context)
+  auto group_row = [&](int kb) __attribute__((always_inline)) -> long {
+    if (MODE == 0) return (long)b * p.S + kb;
+    int blk = table[kb >> p.block_shift];
+    blk = min(max(blk, 0), p.num_blocks - 1);
+    return (long)blk * p.block_size + (kb & (p.block_size - 1));
+  };
+  // per-lane element offsets inside a 16-key group (constant over the whole loop)
+  const int k_lane_off = (int)((kkey & 3) * kv_row_stride) + kchunk * 8;
+  const int v_lane_off = (int)((vkey0 & 15) * kv_row_stride) + kchunk * 8;
 
   typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
   u32x4_t kreg[4], vreg[4];
   auto load_tile = [&](int kt) __attribute__((always_inline)) {
+    const int key0 = kt * BN;
+    if (MODE != 2 && key0 + BN <= ctx) {         // whole tile inside the context: uniform addressing
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const long row = pool_row(kt * BN + 16 * i + kkey);
-      kreg[i] = *(const u32x4_t*)(kbase + row * kv_row_stride + kchunk * 8);
-    }
+      for (int i = 0; i < 4; ++i) {
+        const uint16_t* g = kbase + group_row(key0 + 16 * i + 4 * wave) * kv_row_stride;
+        kreg[i] = *(const u32x4_t*)(g + k_lane_off);
+      }
+      const uint16_t* g = vbase + group_row(key0 + 32 * (wave >> 1) + 16 * (wave & 1)) * kv_row_stride;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const long row = pool_row(kt * BN + vkey0 + i);
-      vreg[i] = *(const u32x4_t*)(vbase + row * kv_row_stride + kchunk * 8);
+      for (int i = 0; i < 4; ++i) vreg[i] = *(const u32x4_t*)(g + v_lane_off + i * kv_row_stride);
+    } else {                                      // last tile of a context, or odd block sizes
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        kreg[i] = *(const u32x4_t*)(kbase + pool_row(key0 + 16 * i + kkey) * kv_row_stride + kchunk * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + vkey0 + i;
+        vreg[i] = *(const u32x4_t*)(vbase + pool_row(key) * kv_row_stride + kchunk * 8);
+        // rows past the context may hold anything (NaN patterns too); their weight is an
+        // exact zero, which only helps if the value is finite
+        if (key >= ctx) vreg[i] = u32x4_t{0u, 0u, 0u, 0u};
+      }
     }
   };
-  auto store_tile = [&]() __attribute__((always_inline)) {
+  auto store_tile = [&](char* ks, char* vts) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) *(u32x4_t*)(ks + (16 * i + kkey) * K_ROW_BYTES + kchunk * 16) = kreg[i];
 #pragma unroll
@@ -158,28 +188,46 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   float m_run = -INFINITY, l_run = 0.f;
   const float sc = p.scale_log2e;
 
-  // first active tile
   const int qblk = wq_lo / BN;                    // sparse: q block of this wave
   const int wg_blk_lo = q0 / BN, wg_blk_hi = (min(q0 + BM, tq) - 1) / BN;
-  auto tile_needed = [&](int kt) __attribute__((always_inline)) -> bool {        // does any wave of the workgroup need key tile kt?
+  auto tile_needed = [&](int kt) __attribute__((always_inline)) -> bool {   // does any wave need key tile kt?
     if (!SPARSE) return true;
     for (int i = wg_blk_lo; i <= wg_blk_hi; ++i)
       if (block_active(i, kt, hq, p.sparse_local, p.sparse_stride)) return true;
     return false;
   };
-  auto next_tile = [&](int kt) __attribute__((always_inline)) -> int {           // first needed tile >= kt (ntiles if none)
+  auto next_tile = [&](int kt) __attribute__((always_inline)) -> int {      // first needed tile >= kt
     while (kt < ntiles && !tile_needed(kt)) ++kt;
     return kt;
   };
 
+  // lane-constant LDS read offsets
+  const int k_rd_off = n * K_ROW_BYTES + 16 * h;
+  const int v_rd_off = vt_row_offset(n) + 16 * h;   // + vt_row_offset(32 c) - vt_row_offset(0) per d chunk
+
+  // Software pipeline over the needed tiles, one barrier per tile: tile j is computed from
+  // LDS stage j%2; tile j+1, loaded into registers during tile j-1, is parked in the other
+  // stage first, and tile j+2's global loads are in flight during the math.
   int kt = next_tile(0);
-  if (kt < ntiles) load_tile(kt);
+  int stage = 0;
+  if (kt < ntiles) {
+    load_tile(kt);
+    store_tile(smem, smem + BN * K_ROW_BYTES);
+  }
+  int kt_next = kt < ntiles ? next_tile(kt + 1) : ntiles;
+  if (kt_next < ntiles) load_tile(kt_next);
+  __syncthreads();
   while (kt < ntiles) {
-    __syncthreads();                               // everyone is done reading the previous tile
-    store_tile();
-    __syncthreads();
-    const int kt_next = next_tile(kt + 1);
-    if (kt_next < ntiles) load_tile(kt_next);      // in flight during the math below
+    char* ks = smem + stage * STAGE_BYTES;
+    char* vts = ks + BN * K_ROW_BYTES;
+    // registers hold tile kt_next: park it in the other stage (last read two tiles ago,
+    // every wave has passed the barrier since), then request the tile after it
+    const int kt_next2 = kt_next < ntiles ? next_tile(kt_next + 1) : ntiles;
+    if (kt_next < ntiles) {
+      char* ks2 = smem + (stage ^ 1) * STAGE_BYTES;
+      store_tile(ks2, ks2 + BN * K_ROW_BYTES);
+      if (kt_next2 < ntiles) load_tile(kt_next2);
+    }
 
     const int key0 = kt * BN;
     bool active = wave_has_rows && key0 <= prefix + wq_hi;
@@ -193,26 +241,27 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
         for (int i = 0; i < 16; ++i) sacc[tt][i] = 0.f;
 #pragma unroll
         for (int s = 0; s < HD / 16; ++s) {
-          const bf16x8_t kf = *(const bf16x8_t*)(ks + (32 * tt + n) * K_ROW_BYTES + 32 * s + 16 * h);
+          const bf16x8_t kf = *(const bf16x8_t*)(ks + k_rd_off + 32 * tt * K_ROW_BYTES + 32 * s);
           sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[tt], 0, 0, 0);
         }
       }
       // ---- online softmax on this lane's column ----
       const bool need_mask = key0 + BN - 1 > prefix + wq_lo;    // tile reaches past the first row's diagonal
       float tmax = -INFINITY;
+      if (need_mask) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
+            sacc[tt][i] = key <= qlim ? sacc[tt][i] : -INFINITY;
+          }
+      }
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float x = sacc[tt][i] * sc;
-          if (need_mask) {
-            const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
-            x = key <= qlim ? x : -INFINITY;
-          }
-          sacc[tt][i] = x;
-          tmax = fmaxf(tmax, x);
-        }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sacc[tt][i]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * sc;        // sc > 0: max commutes with the scale
       // a row whose visible keys all lie in later tiles keeps m = -inf for now
       const float m_new = fmaxf(m_run, tmax);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -223,8 +272,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(sacc[tt][i] - m_use);
-          const float p1 = __builtin_amdgcn_exp2f(sacc[tt][i + 1] - m_use);
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[tt][i], sc, -m_use));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[tt][i + 1], sc, -m_use));
           psum += p0 + p1;
           pw[tt][i >> 1] = pack_bf16x2(p0, p1);
         }
@@ -242,12 +291,15 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
           const bf16x8_t pf = as_bf16x8_prefill(pw[tt][4 * kk], pw[tt][4 * kk + 1], pw[tt][4 * kk + 2], pw[tt][4 * kk + 3]);
 #pragma unroll
           for (int c = 0; c < HD / 32; ++c) {
-            const bf16x8_t vf = *(const bf16x8_t*)(vts + vt_row_offset(32 * c + n) + 16 * (4 * tt + 2 * kk + h));
+            const bf16x8_t vf = *(const bf16x8_t*)(vts + v_rd_off + c * (32 * VT_ROW_BYTES + 4 * 16) + 16 * (4 * tt + 2 * kk));
             oacc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, oacc[c], 0, 0, 0);
           }
         }
     }
+    __syncthreads();       // stage^1 is complete, stage is free
     kt = kt_next;
+    kt_next = kt_next2;
+    stage ^= 1;
   }
 
   // ---- normalise and write this lane's query row ---------------------------------
@@ -267,6 +319,21 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   }
 }
 
+constexpr int kPrefillLdsBytes = 2 * (BN * K_ROW_BYTES + VT_BYTES);
+
+template <bool SPARSE, int MODE>
+hipError_t launch_prefill_typed(const PrefillParams& p, dim3 grid, hipStream_t s) {
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_kernel<SPARSE, MODE>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLdsBytes);
+    if (e != hipSuccess) return e;
+    configured.store(1, std::memory_order_release);
+  }
+  hipLaunchKernelGGL((prefill_kernel<SPARSE, MODE>), grid, dim3(256), kPrefillLdsBytes, s, p);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 bool prefill_supported(const PrefillParams& p) {
@@ -279,9 +346,10 @@ hipError_t launch_prefill(const PrefillParams& p, hipStream_t s) {
   const int nqt = (p.T + BM - 1) / BM;
   if (nqt > 65535 * 32 || p.Hq > 65535 || p.B > 65535) return hipErrorInvalidValue;
   dim3 grid(nqt, p.Hq, p.B);
-  if (p.sparse_stride > 0) hipLaunchKernelGGL(prefill_kernel<true>, grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL(prefill_kernel<false>, grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+  if (p.sparse_stride > 0) return launch_prefill_typed<true, 0>(p, grid, s);
+  if (!p.block_tables) return launch_prefill_typed<false, 0>(p, grid, s);
+  if (p.block_shift >= 4) return launch_prefill_typed<false, 1>(p, grid, s);
+  return launch_prefill_typed<false, 2>(p, grid, s);
 }
 
 }  // namespace pa
