@@ -127,7 +127,9 @@ int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* 
  * (0 = automatic, 1 = scalar-ALU kernel, 2 = MFMA kernel with fixed partitions,
  * 3 = MFMA kernel with the balanced schedule); key 1: waves per workgroup of the
  * fixed-partition MFMA kernel (0 = default); key 2: its grid order (1 = kv head
- * fastest, the default; 0 = partition fastest). */
+ * fastest, the default; 0 = partition fastest); key 3: prefill kernel choice (0 =
+ * automatic, 1 = register-staged kernel, 4 / 8 = asynchronous-copy kernel with that
+ * many wavefronts per workgroup). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

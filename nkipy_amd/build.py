@@ -15,14 +15,14 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpaged_attn.so")
 
-SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip"]
+SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip", "pa_prefill_async.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # hipcc must not form packed-fp32 instructions from float code on these machines
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
 
 

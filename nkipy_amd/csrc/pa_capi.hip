@@ -38,6 +38,7 @@ int check_hip(hipError_t e, const char* what) {
 static std::atomic<int> g_decode_impl{0};
 static std::atomic<int> g_decode_waves{0};
 static std::atomic<int> g_head_major{1};
+static std::atomic<int> g_prefill_impl{0};
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 static std::atomic<int> g_profile{0};
@@ -103,6 +104,7 @@ int pa_debug_set(int key, int value) {
   if (key == 0) { g_decode_impl = value; return 0; }
   if (key == 1) { g_decode_waves = value; return 0; }
   if (key == 2) { g_head_major = value; return 0; }
+  if (key == 3) { g_prefill_impl = value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -249,6 +251,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.scale_log2e = scale * kLog2e;
+  p.impl = g_prefill_impl.load();
   if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
   hipStream_t s = (hipStream_t)stream;
   profile_begin(s);
@@ -277,6 +280,7 @@ int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* ou
   p.B = B; p.T = S; p.S = S; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
   p.sparse_local = local_blocks; p.sparse_stride = vert_stride;
   p.block_shift = -1;
+  p.impl = g_prefill_impl.load();
   p.scale_log2e = scale * kLog2e;
   if (!prefill_supported(p)) return fail_arg("pa_blocksparse_prefill: unsupported shape (D=%d)", D);
   hipStream_t s = (hipStream_t)stream;

@@ -113,10 +113,13 @@ struct PrefillParams {
   int S;                    // dense form: keys per sequence
   int sparse_local, sparse_stride;  // blocksparse pattern; sparse_stride == 0 -> plain causal
   float scale_log2e;
+  int impl;                 // 0 automatic, 1 register-staged kernel, 4 / 8 asynchronous kernel with that many waves
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);
 bool prefill_supported(const PrefillParams& p);
+hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s);
+bool prefill_async_supported(const PrefillParams& p);
 
 // ---- gather ------------------------------------------------------------------------
 hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,

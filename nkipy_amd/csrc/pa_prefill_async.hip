@@ -1,0 +1,394 @@
+// Causal flash-attention prefill on the gfx950 matrix cores, asynchronous form:
+// K and V tiles travel HBM/L2 -> LDS with global_load_lds_dwordx4 (no registers,
+// several tiles in flight in a ring of LDS stages) and V^T fragments are read with
+// the transposing LDS load ds_read_b64_tr_b16, so nothing is transposed by hand.
+//
+// One workgroup of NW wavefronts owns 32*NW query rows of one (sequence, q head);
+// each wavefront owns 32 of them.  Keys are walked in tiles of 64.
+//
+// v_mfma_f32_32x32x16_bf16 operand layout (lane = 32*h + n, h = 0..1, n = 0..31):
+//   A[32 x 16]: lane holds row n, k-slots 8h .. 8h+7
+//   B[16 x 32]: lane holds column n, k-slots 8h .. 8h+7
+//   C/D[32x32]: lane holds column n, rows 8*(i/4) + 4h + (i%4) for i = 0..15
+// Scores are computed transposed, S^T[key, q] = K[key, :] . Q^T[:, q]: a lane's
+// column is one query row, so the online-softmax state is per-lane scalars and
+// the probabilities are already the B operand of O^T[d, q] += V^T[d, key] P^T[key, q]
+// (MFMA kk of a 32-key sub-tile takes accumulator registers 8kk .. 8kk+7, i.e.
+// k-slot 8h+j <-> key 16kk + 8(j/4) + 4h + (j%4)).
+//
+// LDS stage = K tile [64 keys][256 B] + V tile [64 keys][256 B], both row-major
+// exactly as in the pool; the 16-byte chunk index of a row is XORed with
+// (row & 7) so that the b128 reads of K (32 rows, same chunk) and the transposing
+// reads of V (8 rows, 64 B each) spread over all banks.  The swizzle costs
+// nothing: a DMA lane may fetch any global chunk into its fixed LDS slot.
+//
+// ds_read_b64_tr_b16, per group of 16 lanes: lane i receives, for j = 0..3, the
+// (i%4)-th 16-bit element of the 8 bytes addressed by lane (i/4) + 4j.  Source
+// lane s therefore points at key row (s/4) and d columns 4*(s%4) .. +3 of the
+// group's 16-column window; lane i ends up with 4 keys at one d.
+//
+// Masking follows examples/models/gpt_oss/kernels/attention.py:85,127-135: query
+// i of a chunk that starts at `prefix` sees keys j <= prefix + i.
+#include <atomic>
+
+#include "pa_common.h"
+
+namespace pa {
+namespace {
+
+constexpr int BN = 64;                 // keys per tile
+constexpr int HD = 128;                // head dim
+constexpr int ROW_B = HD * 2;          // bytes per K/V row
+constexpr int TILE_B = BN * ROW_B;     // 16 KB
+constexpr int STAGE_B = 2 * TILE_B;    // K then V
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) char lds_char;
+
+__device__ __forceinline__ bool block_active(int i, int j, int head_phase, int local, int stride) {
+  return j <= i && ((i - j) < local || ((j + head_phase) % stride) == 0);
+}
+
+__device__ __forceinline__ bf16x8_t make_frag(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  u32x4_t v = {a, b, c, d};
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// 16-byte-per-lane copy HBM/L2 -> LDS without registers: lane i's bytes land at
+// lds_base + 16 i.  Issued as inline assembly so that the compiler's wait-count
+// insertion does not treat every later LDS read as dependent on every copy still in
+// flight (it would drain the whole ring with vmcnt(0)); the waits are placed by hand.
+__device__ __forceinline__ void dma16_uniform(const char* base, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_lane(const char* addr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(addr), "s"(lds_base) : "memory", "m0");
+}
+
+// Block-table reads go through the constant address space: wave-uniform indices then
+// become scalar loads (their own counter), not vector loads that would have to be
+// waited for in order with the copies above.
+typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+
+// MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16.
+template <bool SPARSE, int MODE, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void prefill_async_kernel(PrefillParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int BMW = 32 * NW;               // query rows per workgroup
+  constexpr int NST = NW == 8 ? 4 : 2;       // LDS stages
+  constexpr int UPW = 32 / NW;               // 1 KB DMA units per wave per tile (16 K + 16 V in all)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+
+  // ---- which (sequence, head, query tile): kv-head groups are spread over the 8 XCDs
+  // (consecutive workgroup ids go to consecutive XCDs), and all query tiles and q heads
+  // that share one kv head run on one XCD, back to back, heavy tiles first: their K/V
+  // stays in that XCD's L2.
+  const int n_rep = p.Hq / p.Hkv;
+  const int nqt = (p.T + BMW - 1) / BMW;
+  const int per_group = nqt * n_rep;
+  const int groups = p.B * p.Hkv;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int grp = xcd + 8 * (slot / per_group);
+  if (grp >= groups) return;
+  const int rr_ = slot % per_group;
+  const int b = grp / p.Hkv, hk = grp % p.Hkv;
+  const int qt = nqt - 1 - rr_ / n_rep;
+  const int hq = hk * n_rep + rr_ % n_rep;
+
+  int tq = p.query_lens ? p.query_lens[b] : p.T;
+  int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
+  tq = min(max(tq, 0), p.T);
+  if (MODE != 0) ctx = min(ctx, p.max_blocks * p.block_size);
+  ctx = max(ctx, tq);
+  const int prefix = ctx - tq;
+  const int q0 = qt * BMW;
+  uint16_t* out = (uint16_t*)p.out;
+  const long q_row_stride = (long)p.Hq * HD;
+
+  if (q0 >= tq) {   // only padding rows here: zeros
+    for (int i = tid; i < BMW * (HD / 8); i += NW * 64) {
+      const int row = q0 + i / (HD / 8);
+      if (row < p.T) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)hq * HD + (i % (HD / 8)) * 8) = make_uint4(0, 0, 0, 0);
+    }
+    return;
+  }
+
+  // ---- this lane's query row and its Q^T fragments --------------------------
+  const int qrow = q0 + wave * 32 + n;
+  const bool qvalid = qrow < tq;
+  const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
+  bf16x8_t qf[HD / 16];
+  {
+    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
+#pragma unroll
+    for (int s = 0; s < HD / 16; ++s) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (qvalid) v = *(const uint4*)(qp + 16 * s + 8 * h);
+      qf[s] = __builtin_bit_cast(bf16x8_t, v);
+    }
+    // the Q loads must be complete (and known to be) before the copy ring starts, or the
+    // first use of a fragment inside the loop would drain the ring with a full wait
+#pragma unroll
+    for (int s = 0; s < HD / 16; ++s) asm volatile("" ::"v"(qf[s]));
+  }
+  const int wq_lo = q0 + wave * 32;                               // first row of this wave
+  const int wq_hi = min(wq_lo + 31, tq - 1);                      // last valid row (may be < wq_lo)
+  const bool wave_has_rows = wq_lo < tq;
+  const int k_end = prefix + min(q0 + BMW, tq);                   // keys the workgroup needs: [0, k_end)
+  const int ntiles = (k_end + BN - 1) / BN;
+
+  // ---- DMA maps ---------------------------------------------------------------------
+  // A tile is 32 units of 1 KB (4 rows): units 0..15 are K, 16..31 are V.  Wave w issues
+  // units w, w + NW, ...  In a unit lane i fills LDS slot (row 4u + i/16, position i%16)
+  // with the global chunk  position ^ (row & 7).
+  const const_i32_ptr table = MODE != 0 ? (const_i32_ptr)(uintptr_t)(p.block_tables + (long)b * p.max_blocks) : nullptr;
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
+  const long kv_row_bytes = (long)p.Hkv * ROW_B;
+  const char* kbase = (const char*)p.k + (long)hk * ROW_B;
+  const char* vbase = (const char*)p.v + (long)hk * ROW_B;
+  const int dma_rr = lane >> 4, dma_pos = lane & 15;
+  // every unit of a wave has the same parity (NW is even), hence the same swizzle
+  const int dma_chunk = dma_pos ^ ((4 * (wave & 1) + dma_rr) & 7);
+  const int dma_lane_off = (int)(dma_rr * kv_row_bytes) + dma_chunk * 16;
+
+  auto group_row = [&](int kb) __attribute__((always_inline)) -> long {   // pool row of wave-uniform key kb
+    if (MODE == 0) return (long)b * p.S + kb;
+    int blk = table[kb >> p.block_shift];
+    blk = min(max(blk, 0), p.num_blocks - 1);
+    return (long)blk * p.block_size + (kb & (p.block_size - 1));
+  };
+  auto lane_row = [&](int key) __attribute__((always_inline)) -> long {   // same, per lane, clamped
+    key = min(key, ctx - 1);
+    if (MODE == 0) return (long)b * p.S + key;
+    int blk = table[key >> p.block_shift];
+    blk = min(max(blk, 0), p.num_blocks - 1);
+    return (long)blk * p.block_size + (key & (p.block_size - 1));
+  };
+  auto issue_tile = [&](int kt, int stage) __attribute__((always_inline)) {
+    const int key0 = kt * BN;
+    const uint32_t sbase = smem_base + stage * STAGE_B;
+    if (key0 + BN <= ctx) {                       // whole tile inside the context: uniform row bases
+#pragma unroll
+      for (int i = 0; i < UPW; ++i) {
+        const int u = wave + NW * i;              // compile-time K/V split: u < 16 <=> i < UPW/2
+        const int r0 = 4 * (u & 15);
+        const char* src = (i < UPW / 2 ? kbase : vbase) + group_row(key0 + r0) * kv_row_bytes;
+        dma16_uniform(src, dma_lane_off, sbase + (i < UPW / 2 ? 0 : TILE_B) + (u & 15) * 1024);
+      }
+    } else {                                      // last tile of a context: rows past it re-read its last row
+#pragma unroll
+      for (int i = 0; i < UPW; ++i) {
+        const int u = wave + NW * i;
+        const int r0 = 4 * (u & 15);
+        const char* src = (i < UPW / 2 ? kbase : vbase) + lane_row(key0 + r0 + dma_rr) * kv_row_bytes + dma_chunk * 16;
+        dma16_lane(src, sbase + (i < UPW / 2 ? 0 : TILE_B) + (u & 15) * 1024);
+      }
+    }
+  };
+
+  // ---- LDS read maps (lane constants) -------------------------------------------------
+  int k_off[HD / 16];                 // K fragment of k-step s: row n, chunk 2s + h
+#pragma unroll
+  for (int s = 0; s < HD / 16; ++s) k_off[s] = n * ROW_B + (((2 * s + h) ^ (n & 7)) << 4);
+  int v_off[HD / 32];                 // V^T fragment source of d-chunk c
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int row = 4 * h + (sl >> 2);                       // key row inside a 16-key window (also row & 7)
+    const int y = 2 * (g & 1) + ((sl & 3) >> 1);             // 16-byte chunk inside the 64-byte d window
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c) v_off[c] = row * ROW_B + (((4 * c + y) ^ row) << 4) + (sl & 1) * 8;
+  }
+
+  // ---- accumulators ------------------------------------------------------------
+  f32x16_t oacc[HD / 32];
+#pragma unroll
+  for (int c = 0; c < HD / 32; ++c)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[c][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float sc = p.scale_log2e;
+
+  const int head_phase = SPARSE ? hq % p.sparse_stride : 0;
+  const int qblk = wq_lo / BN;                    // sparse: q block of this wave
+  const int wg_blk_lo = q0 / BN, wg_blk_hi = (min(q0 + BMW, tq) - 1) / BN;
+  auto next_tile = [&](int kt) __attribute__((always_inline)) -> int {      // first needed tile >= kt
+    if (!SPARSE) return kt;
+    while (kt < ntiles) {
+      // needed by some q block of the workgroup: vertical-stride column, or inside a local window
+      if (((kt + head_phase) % p.sparse_stride) == 0 || kt > wg_blk_lo - p.sparse_local) break;
+      ++kt;
+    }
+    return kt;
+  };
+
+  // ---- ring of NST stages: tiles are requested NST-1 ahead; requests past the end are
+  // repeated on the first tile so that the wait counter stays exact ------------------------
+  const int kt_first = next_tile(0);
+  int kt_c = kt_first;                // tile to compute
+  int kt_i = kt_first;                // tile to request
+#pragma unroll
+  for (int s = 0; s < NST - 1; ++s) {
+    issue_tile(kt_i < ntiles ? kt_i : kt_first, s);
+    if (kt_i < ntiles) kt_i = next_tile(kt_i + 1);
+  }
+  int stage_c = 0, stage_i = NST - 1;
+  while (kt_c < ntiles) {
+    wait_vmcnt<(NST - 2) * UPW>();               // this wave's part of tile kt_c has landed
+    __builtin_amdgcn_s_barrier();                // ... and everyone's; all waves are done with the previous tile
+    issue_tile(kt_i < ntiles ? kt_i : kt_first, stage_i);
+    if (kt_i < ntiles) kt_i = next_tile(kt_i + 1);
+
+    const char* ks = smem + stage_c * STAGE_B;
+    const char* vs = ks + TILE_B;
+    const int key0 = kt_c * BN;
+    bool active = wave_has_rows && key0 <= prefix + wq_hi;
+    if (SPARSE) active = active && block_active(qblk, kt_c, head_phase, p.sparse_local, p.sparse_stride);
+    if (active) {
+      // ---- S^T = K Q^T ----
+      f32x16_t sacc[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sacc[tt][i] = 0.f;
+        bf16x8_t kf[HD / 16];
+#pragma unroll
+        for (int s = 0; s < HD / 16; ++s) kf[s] = *(const bf16x8_t*)(ks + 32 * tt * ROW_B + k_off[s]);
+#pragma unroll
+        for (int s = 0; s < HD / 16; ++s)
+          sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[s], sacc[tt], 0, 0, 0);
+      }
+      // ---- online softmax on this lane's column ----
+      const bool need_mask = key0 + BN - 1 > prefix + wq_lo;    // tile reaches past the first row's diagonal
+      if (need_mask) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
+            sacc[tt][i] = key <= qlim ? sacc[tt][i] : -INFINITY;
+          }
+      }
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sacc[tt][i]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * sc;        // sc > 0: max commutes with the scale
+      // a row whose visible keys all lie in later tiles keeps m = -inf for now
+      const float m_new = fmaxf(m_run, tmax);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+      float psum = 0.f;
+      uint32_t pw[2][8];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[tt][i], sc, -m_use));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[tt][i + 1], sc, -m_use));
+          psum += p0 + p1;
+          pw[tt][i >> 1] = pack_bf16x2(p0, p1);
+        }
+      l_run = l_run * alpha + psum;
+      if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {   // rescale only when some row's max moved
+#pragma unroll
+        for (int c = 0; c < HD / 32; ++c) oacc[c] *= alpha;
+      }
+      m_run = m_new;
+      // ---- O^T += V^T P^T ----
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const bf16x8_t pf = make_frag(pw[tt][4 * kk], pw[tt][4 * kk + 1], pw[tt][4 * kk + 2], pw[tt][4 * kk + 3]);
+          bf16x8_t vf[HD / 32];
+#pragma unroll
+          for (int c = 0; c < HD / 32; ++c) {
+            const lds_char* src = (const lds_char*)(vs + (32 * tt + 16 * kk) * ROW_B + v_off[c]);
+            const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
+            const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 8 * ROW_B));
+            struct { s16x4_t a, b; } pair = {lo, hi};
+            vf[c] = __builtin_bit_cast(bf16x8_t, pair);
+          }
+#pragma unroll
+          for (int c = 0; c < HD / 32; ++c)
+            oacc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[c], pf, oacc[c], 0, 0, 0);
+        }
+    }
+    kt_c = next_tile(kt_c + 1);
+    stage_c = stage_c + 1 == NST ? 0 : stage_c + 1;
+    stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
+  }
+  wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
+
+  // ---- normalise and write this lane's query row ---------------------------------
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (qrow < p.T && wq_lo < p.T) {
+    uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
+    const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d = 32 * c + 8 * i4 + 4 * h;
+        const uint32_t w0 = qvalid ? pack_bf16x2(oacc[c][4 * i4] * inv, oacc[c][4 * i4 + 1] * inv) : 0u;
+        const uint32_t w1 = qvalid ? pack_bf16x2(oacc[c][4 * i4 + 2] * inv, oacc[c][4 * i4 + 3] * inv) : 0u;
+        *(uint2*)(op + d) = make_uint2(w0, w1);
+      }
+  }
+}
+
+template <bool SPARSE, int MODE, int NW>
+hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
+  constexpr int lds = (NW == 8 ? 4 : 2) * STAGE_B;
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    configured.store(1, std::memory_order_release);
+  }
+  const int n_rep = p.Hq / p.Hkv;
+  const int nqt = (p.T + 32 * NW - 1) / (32 * NW);
+  const long per_group = (long)nqt * n_rep;
+  const long groups = (long)p.B * p.Hkv;
+  const long total = 8 * ((groups + 7) / 8) * per_group;
+  if (total > 0x7fffffffL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool prefill_async_supported(const PrefillParams& p) {
+  if (p.D != HD) return false;
+  if (p.block_tables && p.block_shift < 4) return false;   // paged: power-of-two block size >= 16
+  return true;
+}
+
+hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s) {
+  const bool sparse = p.sparse_stride > 0;
+  const bool paged = p.block_tables != nullptr;
+  if (waves == 0) waves = (sparse || p.T <= 128) ? 4 : 8;
+  if (waves == 8) {
+    if (sparse) return launch_typed<true, 0, 8>(p, s);
+    return paged ? launch_typed<false, 1, 8>(p, s) : launch_typed<false, 0, 8>(p, s);
+  }
+  if (sparse) return launch_typed<true, 0, 4>(p, s);
+  return paged ? launch_typed<false, 1, 4>(p, s) : launch_typed<false, 0, 4>(p, s);
+}
+
+}  // namespace pa
