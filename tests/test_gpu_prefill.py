@@ -183,6 +183,40 @@ def test_config4_shape_shrunk(pa):
     assert_close_abs(dev_to_f32(got), want, BF16_TOL)
 
 
+@pytest.mark.parametrize("impl", [1, 4, 8, 16], ids=["staged", "async4", "async8", "async8-two-group"])
+def test_prefill_kernel_variants_agree(pa, impl):
+    """Every prefill kernel variant (register-staged, asynchronous ring with 4 or 8 waves, the
+    two-group schedule) against the oracle on the dense-causal and the sparse form."""
+    from nkipy_amd import _lib
+    rng = np.random.default_rng(77)
+    lib = _lib.load()
+    lib.pa_debug_set(3, impl)
+    try:
+        got, want = _prefill_case(pa, rng, T=300, qlens=[300, 129, 257], prefixes=[70, 515, 0], Hq=8, Hkv=2, bs=32)
+        assert_close_abs(got, want, BF16_TOL)
+        B, S, H, D = 1, 640, 3, 128
+        q = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        k = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        v = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        want = O.blocksparse_prefill(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), 0.09,
+                                     block=64, local_blocks=2, vert_stride=4)
+        got = pa.blocksparse_prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), 0.09, block=64,
+                                     local_blocks=2, vert_stride=4)
+        torch.cuda.synchronize()
+        assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+    finally:
+        lib.pa_debug_set(3, 0)
+
+
+def test_prefill_generic_block_size(pa):
+    """Block sizes that are not a power of two >= 16 take the register-staged kernel."""
+    rng = np.random.default_rng(78)
+    got, want = _prefill_case(pa, rng, T=100, qlens=[100, 33], prefixes=[50, 7], Hq=4, Hkv=2, bs=8)
+    assert_close_abs(got, want, BF16_TOL)
+    got, want = _prefill_case(pa, rng, T=100, qlens=[100, 33], prefixes=[50, 7], Hq=4, Hkv=2, bs=24)
+    assert_close_abs(got, want, BF16_TOL)
+
+
 def test_prefill_argument_errors(pa):
     q = torch.zeros(1, 8, 4, 128, dtype=torch.bfloat16, device="cuda")
     kc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16, device="cuda")
