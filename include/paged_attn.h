@@ -129,7 +129,9 @@ int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* 
  * fixed-partition MFMA kernel (0 = default); key 2: its grid order (1 = kv head
  * fastest, the default; 0 = partition fastest); key 3: prefill kernel choice (0 =
  * automatic, 1 = register-staged kernel, 4 / 8 = asynchronous-copy kernel with that
- * many wavefronts per workgroup). */
+ * many wavefronts per workgroup, 16 = 8 wavefronts in two alternating groups); key 4:
+ * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
+ * the same tile (1 = on, the default). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

@@ -39,6 +39,7 @@ static std::atomic<int> g_decode_impl{0};
 static std::atomic<int> g_decode_waves{0};
 static std::atomic<int> g_head_major{1};
 static std::atomic<int> g_prefill_impl{0};
+static std::atomic<int> g_lockstep{1};
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 static std::atomic<int> g_profile{0};
@@ -105,6 +106,7 @@ int pa_debug_set(int key, int value) {
   if (key == 1) { g_decode_waves = value; return 0; }
   if (key == 2) { g_head_major = value; return 0; }
   if (key == 3) { g_prefill_impl = value; return 0; }
+  if (key == 4) { g_lockstep = value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -196,6 +198,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
   if (kind == 3) {
     plan_decode_balanced(p, current_num_cus());
+    p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
     const size_t need = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
     if (!workspace || workspace_bytes < need)
       return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);

@@ -87,6 +87,7 @@ struct DecodeParams {
   float scale_log2e;
   int head_major;           // fixed-partition grid order: kv head fastest (1) or partition fastest (0)
   int bal_hsw, bal_ns, bal_gv;  // balanced schedule: head slots and chunks per workgroup, total chunks
+  int bal_lockstep;         // keep the head waves of a workgroup on the same tile with a barrier
 };
 
 hipError_t launch_decode_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
