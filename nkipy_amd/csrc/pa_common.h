@@ -114,7 +114,7 @@ struct PrefillParams {
   int S;                    // dense form: keys per sequence
   int sparse_local, sparse_stride;  // blocksparse pattern; sparse_stride == 0 -> plain causal
   float scale_log2e;
-  int impl;                 // 0 automatic, 1 register-staged kernel, 4 / 8 asynchronous kernel with that many waves
+  int impl;                 // 0 automatic, 1 register-staged, 4 / 8 / 16 asynchronous (waves; 16 = two groups)
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);

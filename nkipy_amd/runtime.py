@@ -1,0 +1,129 @@
+"""Name-keyed call convention of the reference's runtime, over the HIP ops.
+
+The reference runs a kernel as
+    k = DeviceKernel.compile_and_load(fn, name=..., **example_args)
+    k(inputs={param_name: DeviceTensor}, outputs={"output0": DeviceTensor})
+(nkipy/src/nkipy/runtime/device_kernel.py:52-193, spike/src/spike/spike_model.py:248-288):
+the caller allocates inputs and outputs, tensors are addressed by parameter name,
+unknown names raise ValueError and shape / dtype mismatches AssertionError
+(spike_model.py:198-246).  This module keeps that convention for the paged attention
+ops; there is nothing to trace or compile, so "compile_and_load" only loads the native
+library and records the I/O signature from the example arguments.
+"""
+from __future__ import annotations
+
+import inspect
+
+import numpy as np
+import torch
+
+from . import _lib, paged_attn
+
+_TENSOR_PARAMS = {"q", "k_cache", "v_cache", "block_tables", "seq_lens", "query_lens", "k", "v",
+                  "k_scale", "v_scale"}
+
+
+class DeviceTensor:
+    """A named-dtype view of device memory (nkipy/src/nkipy/runtime/device_tensor.py:51-74)."""
+
+    def __init__(self, tensor: torch.Tensor):
+        self.tensor = tensor
+
+    @classmethod
+    def from_torch(cls, t: torch.Tensor, device="cuda") -> "DeviceTensor":
+        return cls(t.to(device).contiguous())
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray, dtype: str | None = None, device="cuda") -> "DeviceTensor":
+        """uint16 arrays tagged "bf16" are bf16 bit patterns, uint8 arrays tagged "fp8" e4m3fn codes."""
+        t = torch.from_numpy(np.ascontiguousarray(a))
+        if dtype == "bf16":
+            assert a.dtype == np.uint16, "bf16 host data is passed as uint16 bit patterns"
+            t = torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).view(torch.bfloat16)
+        elif dtype == "fp8":
+            assert a.dtype == np.uint8, "fp8 host data is passed as uint8 codes"
+            t = t.view(torch.float8_e4m3fn)
+        return cls(t.to(device))
+
+    @property
+    def shape(self):
+        return tuple(self.tensor.shape)
+
+    @property
+    def dtype(self):
+        return self.tensor.dtype
+
+    def torch(self) -> torch.Tensor:
+        return self.tensor
+
+    def numpy(self) -> np.ndarray:
+        t = self.tensor.detach().cpu()
+        if t.dtype == torch.bfloat16:
+            return t.view(torch.int16).numpy().view(np.uint16)
+        if t.dtype == torch.float8_e4m3fn:
+            return t.view(torch.uint8).numpy()
+        return t.numpy()
+
+
+class DeviceKernel:
+    """A loaded paged attention op with a fixed I/O signature."""
+
+    _OPS = {"decode": paged_attn.decode, "prefill": paged_attn.prefill,
+            "blocksparse_prefill": paged_attn.blocksparse_prefill}
+
+    def __init__(self, fn, name, signature, static_kwargs):
+        self.fn, self.name = fn, name
+        self.signature = signature          # param name -> (shape, dtype)
+        self.static_kwargs = static_kwargs
+        self.output_names = ["output0"]
+
+    @classmethod
+    def compile_and_load(cls, fn, name: str | None = None, **example_args) -> "DeviceKernel":
+        """fn: one of nkipy_amd.decode / prefill / blocksparse_prefill (or its name).  Tensor
+        arguments (DeviceTensor or torch tensor) fix the expected shapes and dtypes; every
+        other keyword (scale, partition_size, ...) becomes a static argument of the kernel."""
+        if isinstance(fn, str):
+            fn = cls._OPS[fn]
+        if fn not in cls._OPS.values():
+            raise ValueError(f"{getattr(fn, '__name__', fn)!r} is not a paged attention op")
+        _lib.load()
+        params = inspect.signature(fn).parameters
+        signature, static = {}, {}
+        for k, v in example_args.items():
+            if k not in params:
+                raise ValueError(f"{fn.__name__} has no parameter {k!r}")
+            if k in _TENSOR_PARAMS and v is not None:
+                t = v.tensor if isinstance(v, DeviceTensor) else v
+                signature[k] = (tuple(t.shape), t.dtype)
+            else:
+                static[k] = v
+        return cls(fn, name or fn.__name__, signature, static)
+
+    def __call__(self, inputs: dict, outputs: dict | None = None):
+        unknown = [k for k in inputs if k not in self.signature]
+        if unknown:
+            raise ValueError(f"kernel {self.name!r}: unknown input name(s) {unknown}; expected {sorted(self.signature)}")
+        missing = [k for k in self.signature if k not in inputs]
+        if missing:
+            raise ValueError(f"kernel {self.name!r}: missing input(s) {missing}")
+        if outputs is not None:
+            bad = [k for k in outputs if k not in self.output_names]
+            if bad:
+                raise ValueError(f"kernel {self.name!r}: unknown output name(s) {bad}; expected {self.output_names}")
+        args = {}
+        for k, v in inputs.items():
+            t = v.tensor if isinstance(v, DeviceTensor) else v
+            shape, dtype = self.signature[k]
+            assert tuple(t.shape) == shape, f"input {k!r}: shape {tuple(t.shape)} != {shape}"
+            assert t.dtype == dtype, f"input {k!r}: dtype {t.dtype} != {dtype}"
+            args[k] = t
+        out = None
+        if outputs is not None and "output0" in outputs:
+            o = outputs["output0"]
+            out = o.tensor if isinstance(o, DeviceTensor) else o
+            qshape, qdtype = self.signature["q"]
+            assert tuple(out.shape) == qshape and out.dtype == qdtype, "output0 must match q in shape and dtype"
+        res = self.fn(**args, **self.static_kwargs, out=out)
+        if outputs is None:
+            return DeviceTensor(res)
+        return None

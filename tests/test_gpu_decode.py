@@ -328,3 +328,28 @@ def test_argument_errors(pa):
         pa.decode(q.cpu(), kc, kc, bt, sl, 1.0)
     with pytest.raises(ValueError):
         pa.decode(q.float(), kc, kc, bt, sl, 1.0)                      # fp32 q with bf16 KV
+
+
+def test_device_kernel_convention(pa):
+    """compile_and_load + name-keyed call with caller-allocated output, as the reference's
+    DeviceKernel (device_kernel.py:52-193): same result as the direct op."""
+    from nkipy_amd.runtime import DeviceKernel, DeviceTensor
+    rng = np.random.default_rng(4)
+    B, Hq, Hkv, D, bs = 3, 8, 2, 128, 32
+    ctxs = [70, 300, 1]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    ins = dict(q=DeviceTensor.from_numpy(O.f32_to_bf16_bits(q), "bf16"),
+               k_cache=DeviceTensor.from_numpy(O.f32_to_bf16_bits(k), "bf16"),
+               v_cache=DeviceTensor.from_numpy(O.f32_to_bf16_bits(v), "bf16"),
+               block_tables=DeviceTensor.from_numpy(tables), seq_lens=DeviceTensor.from_numpy(np.asarray(ctxs, np.int32)))
+    kern = DeviceKernel.compile_and_load(pa.decode, name="paged_decode", scale=0.09, **ins)
+    out = DeviceTensor(torch.empty_like(ins["q"].torch()))
+    assert kern(inputs=ins, outputs={"output0": out}) is None
+    torch.cuda.synchronize()
+    want = O.paged_decode(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                          np.asarray(ctxs, np.int32), 0.09, q_dtype="bf16")
+    assert_close_abs(O.bf16_bits_to_f32(out.numpy()), want, BF16_TOL)
+    ret = kern(inputs=ins)                      # outputs=None: result returned by value
+    torch.cuda.synchronize()
+    assert np.array_equal(ret.numpy(), out.numpy())

@@ -107,3 +107,33 @@ def test_workload_index_structures_are_seeded_and_consistent():
     assert len(np.unique(priv)) == len(priv)
     s = W.make_blocksparse(device="cpu", shrink=64)
     assert s.flops() > 0
+
+
+def test_device_kernel_name_validation_without_gpu(lib):
+    """The name-keyed call convention rejects unknown tensors before touching a device."""
+    import nkipy_amd
+    from nkipy_amd.runtime import DeviceKernel
+    q = torch.zeros(2, 8, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 2, dtype=torch.int32)
+    sl = torch.ones(2, dtype=torch.int32)
+    k = DeviceKernel.compile_and_load(nkipy_amd.decode, name="dec", q=q, k_cache=kc, v_cache=kc,
+                                      block_tables=bt, seq_lens=sl, scale=0.1, partition_size=256)
+    assert k.static_kwargs == {"scale": 0.1, "partition_size": 256}
+    good = dict(q=q, k_cache=kc, v_cache=kc, block_tables=bt, seq_lens=sl)
+    with pytest.raises(ValueError):
+        k(inputs=dict(good, bogus=q))
+    with pytest.raises(ValueError):
+        k(inputs={n: t for n, t in good.items() if n != "seq_lens"})
+    with pytest.raises(ValueError):
+        k(inputs=good, outputs={"output1": q})
+    with pytest.raises(AssertionError):
+        k(inputs=dict(good, q=q[:1]))
+    with pytest.raises(AssertionError):
+        k(inputs=dict(good, q=q.float()))
+    with pytest.raises(ValueError):
+        DeviceKernel.compile_and_load(nkipy_amd.decode, q=q, nonsense=1)
+    with pytest.raises(ValueError):
+        DeviceKernel.compile_and_load(print)
+    with pytest.raises(NotImplementedError):      # host tensors: no CPU path behind the op
+        k(inputs=good)
