@@ -242,6 +242,8 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   if (dtype != PA_BF16) return fail_arg("pa_prefill: only bf16 is supported (dtype=%d)", dtype);
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_prefill: bad paging sizes");
   if (B == 0 || T == 0) return 0;
+  if ((long)num_blocks * block_size > 0x7fffffffL || (long)Hkv * D * 2 > 0x7fffffffL)
+    return fail_arg("pa_prefill: pool of %d blocks x %d rows exceeds 2^31 rows", num_blocks, block_size);
   if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens || !out)
     return fail_arg("pa_prefill: null pointer argument");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
@@ -274,6 +276,8 @@ int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* ou
   if (block != 64) return fail_arg("pa_blocksparse_prefill: sparsity block must be 64 (got %d)", block);
   if (local_blocks < 1 || vert_stride < 1) return fail_arg("pa_blocksparse_prefill: local_blocks and vert_stride must be >= 1");
   if (B == 0 || S == 0) return 0;
+  if ((long)B * S > 0x7fffffffL || (long)Hkv * D * 2 > 0x7fffffffL)
+    return fail_arg("pa_blocksparse_prefill: B*S=%ld rows exceed 2^31", (long)B * S);
   if (!q || !k || !v || !out) return fail_arg("pa_blocksparse_prefill: null pointer argument");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
     return fail_arg("pa_blocksparse_prefill: q, k, v and out must be 16-byte aligned");

@@ -18,10 +18,11 @@
 //
 // LDS stage = K tile [64 keys][256 B] + V tile [64 keys][256 B], both row-major
 // exactly as in the pool; the 16-byte chunk index of a row is XORed with
-// (row & 7) for K and 2 * (row & 3) for V so that the b128 reads of K (32 rows,
-// same chunk) and the transposing reads of V (8 rows, 64 B each) spread over all
-// banks.  The swizzle costs nothing: a DMA lane may fetch any global chunk into
-// its fixed LDS slot.
+// (row & 15) for K and 4 * (row & 3) for V so that the b128 reads of K (32 rows,
+// same chunk: 16 consecutive lanes must hit 16 different chunk positions) and the
+// transposing reads of V (8 rows, a 64-byte window each: 4 rows must hit 4 different
+// windows) run at the full LDS rate; narrower swizzles measured 65 % of it.  The
+// swizzle costs nothing: a DMA lane may fetch any global chunk into its fixed LDS slot.
 //
 // ds_read_b64_tr_b16, per group of 16 lanes: lane i receives, for j = 0..3, the
 // (i%4)-th 16-bit element of the 8 bytes addressed by lane (i/4) + 4j.  Source
@@ -34,14 +35,12 @@
 
 #include "pa_common.h"
 
+
 namespace pa {
 namespace {
 
-constexpr int BN = 64;                 // keys per tile
 constexpr int HD = 128;                // head dim
 constexpr int ROW_B = HD * 2;          // bytes per K/V row
-constexpr int TILE_B = BN * ROW_B;     // 16 KB
-constexpr int STAGE_B = 2 * TILE_B;    // K then V
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -80,13 +79,19 @@ __device__ __forceinline__ void dma16_lane(const char* addr, uint32_t lds_base) 
 typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
 // MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16.
-template <bool SPARSE, int MODE, int NW, bool PINGPONG>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// TT: 32-key sub-tiles per key tile (2: 64-key tiles, two workgroups of 4 waves per CU;
+// 1: 32-key tiles with a smaller register and LDS footprint, three workgroups per CU).
+template <bool SPARSE, int MODE, int NW, bool PINGPONG, int TT>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(TT == 1 ? 3 : 2, TT == 1 ? 3 : 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int BN = 32 * TT;                // keys per tile
+  constexpr int TILE_B = BN * ROW_B;         // one tensor's tile in LDS
+  constexpr int STAGE_B = 2 * TILE_B;        // K then V
+  constexpr int UK = BN / 4;                 // 1 KB copy units per tensor tile
   constexpr int BMW = 32 * NW;               // query rows per workgroup
-  constexpr int NST = NW == 8 ? 4 : 2;       // LDS stages
-  constexpr int UPW = 32 / NW;               // 1 KB DMA units per wave per tile (16 K + 16 V in all)
+  constexpr int NST = TT == 1 ? 3 : (NW == 8 ? 4 : 2);   // LDS stages
+  constexpr int UPW = 2 * UK / NW;           // copy units per wave per tile
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -131,6 +136,7 @@ void prefill_async_kernel(PrefillParams p) {
   const int qrow = q0 + wave * 32 + n;
   const bool qvalid = qrow < tq;
   const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
+  const float sc = p.scale_log2e;
   bf16x8_t qf[HD / 16];
   {
     const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
@@ -138,7 +144,15 @@ void prefill_async_kernel(PrefillParams p) {
     for (int s = 0; s < HD / 16; ++s) {
       uint4 v = make_uint4(0, 0, 0, 0);
       if (qvalid) v = *(const uint4*)(qp + 16 * s + 8 * h);
-      qf[s] = __builtin_bit_cast(bf16x8_t, v);
+      // scale * log2(e) goes into Q once (rounded to bf16 again: a relative 2^-9 per element,
+      // below the rounding of the probabilities), so that the scores leave the matrix cores
+      // ready for exp2
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      uint32_t r[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        r[j] = pack_bf16x2(bf16_bits_to_float(w[j] & 0xffffu) * sc, bf16_bits_to_float(w[j] >> 16) * sc);
+      qf[s] = make_frag(r[0], r[1], r[2], r[3]);
     }
     // the Q loads must be complete (and known to be) before the copy ring starts, or the
     // first use of a fragment inside the loop would drain the ring with a full wait
@@ -152,7 +166,7 @@ void prefill_async_kernel(PrefillParams p) {
   const int ntiles = (k_end + BN - 1) / BN;
 
   // ---- DMA maps ---------------------------------------------------------------------
-  // A tile is 32 units of 1 KB (4 rows): units 0..15 are K, 16..31 are V.  Wave w issues
+  // A tile is 2 UK units of 1 KB (4 rows): the first UK are K, the rest V.  Wave w issues
   // units w, w + NW, ...  In a unit lane i fills LDS slot (row 4u + i/16, position i%16)
   // with the global chunk  position ^ (row & 7).
   const const_i32_ptr table = MODE != 0 ? (const_i32_ptr)(uintptr_t)(p.block_tables + (long)b * p.max_blocks) : nullptr;
@@ -161,19 +175,13 @@ void prefill_async_kernel(PrefillParams p) {
   const char* kbase = (const char*)p.k + (long)hk * ROW_B;
   const char* vbase = (const char*)p.v + (long)hk * ROW_B;
   const int dma_rr = lane >> 4, dma_pos = lane & 15;
-  // every unit of a wave has the same parity (NW is even), hence the same swizzle:
-  // K rows use row & 7, V rows 2 * (row & 3) (what their two read patterns want)
-  const int dma_chunk_k = dma_pos ^ ((4 * (wave & 1) + dma_rr) & 7);
-  const int dma_chunk_v = dma_pos ^ (2 * dma_rr);
+  // every unit of a wave starts at the same row modulo 16 (NW is a multiple of 4), hence the
+  // same swizzle: K rows use row & 15, V rows 4 * (row & 3) (what their read patterns want)
+  const int dma_chunk_k = dma_pos ^ ((4 * (wave & 3) + dma_rr) & 15);
+  const int dma_chunk_v = dma_pos ^ (4 * dma_rr);
   const int dma_lane_off_k = (int)(dma_rr * kv_row_bytes) + dma_chunk_k * 16;
   const int dma_lane_off_v = (int)(dma_rr * kv_row_bytes) + dma_chunk_v * 16;
 
-  auto group_row = [&](int kb) __attribute__((always_inline)) -> long {   // pool row of wave-uniform key kb
-    if (MODE == 0) return (long)b * p.S + kb;
-    int blk = table[kb >> p.block_shift];
-    blk = min(max(blk, 0), p.num_blocks - 1);
-    return (long)blk * p.block_size + (kb & (p.block_size - 1));
-  };
   auto lane_row = [&](int key) __attribute__((always_inline)) -> long {   // same, per lane, clamped
     key = min(key, ctx - 1);
     if (MODE == 0) return (long)b * p.S + key;
@@ -181,24 +189,45 @@ void prefill_async_kernel(PrefillParams p) {
     blk = min(max(blk, 0), p.num_blocks - 1);
     return (long)blk * p.block_size + (key & (p.block_size - 1));
   };
+  // Block-table entries of the tile that will be requested next, fetched one request early:
+  // the scalar loads then complete under a whole tile of compute instead of in front of the
+  // copies that need them.  K and V units of a wave share their rows, hence UPW/2 entries.
+  int blk_pf[UPW / 2];
+  auto prefetch_table = [&](int kt) __attribute__((always_inline)) {
+    if (MODE == 0) return;
+#pragma unroll
+    for (int i = 0; i < UPW / 2; ++i) {
+      const int r0 = 4 * ((wave + NW * i) & (UK - 1));
+      blk_pf[i] = table[min((kt * BN + r0) >> p.block_shift, p.max_blocks - 1)];
+    }
+  };
+  // The UPW copy units of this wave for tile kt, K first: unit j covers rows 4u .. 4u+3 of
+  // the K (j < UPW/2) or V tile, u = (wave + NW j) mod UK.
   auto issue_tile = [&](int kt, int stage) __attribute__((always_inline)) {
     const int key0 = kt * BN;
     const uint32_t sbase = smem_base + stage * STAGE_B;
-    if (key0 + BN <= ctx) {                       // whole tile inside the context: uniform row bases
+    if (key0 + BN <= ctx) {                       // whole tile inside the context: one row base per unit
 #pragma unroll
-      for (int i = 0; i < UPW; ++i) {
-        const int u = wave + NW * i;              // compile-time K/V split: u < 16 <=> i < UPW/2
-        const int r0 = 4 * (u & 15);
-        const char* src = (i < UPW / 2 ? kbase : vbase) + group_row(key0 + r0) * kv_row_bytes;
-        dma16_uniform(src, i < UPW / 2 ? dma_lane_off_k : dma_lane_off_v, sbase + (i < UPW / 2 ? 0 : TILE_B) + (u & 15) * 1024);
+      for (int j = 0; j < UPW; ++j) {
+        const bool is_k = j < UPW / 2;
+        const int u = (wave + NW * j) & (UK - 1);
+        long row;
+        if (MODE == 0) {
+          row = (long)b * p.S + key0 + 4 * u;
+        } else {
+          const int blk = min(max(blk_pf[j % (UPW / 2)], 0), p.num_blocks - 1);
+          row = (long)blk * p.block_size + ((key0 + 4 * u) & (p.block_size - 1));
+        }
+        dma16_uniform((is_k ? kbase : vbase) + row * kv_row_bytes, is_k ? dma_lane_off_k : dma_lane_off_v,
+                      sbase + (is_k ? 0 : TILE_B) + u * 1024);
       }
     } else {                                      // last tile of a context: rows past it re-read its last row
 #pragma unroll
-      for (int i = 0; i < UPW; ++i) {
-        const int u = wave + NW * i;
-        const int r0 = 4 * (u & 15);
-        const char* src = (i < UPW / 2 ? kbase : vbase) + lane_row(key0 + r0 + dma_rr) * kv_row_bytes + (i < UPW / 2 ? dma_chunk_k : dma_chunk_v) * 16;
-        dma16_lane(src, sbase + (i < UPW / 2 ? 0 : TILE_B) + (u & 15) * 1024);
+      for (int j = 0; j < UPW; ++j) {
+        const bool is_k = j < UPW / 2;
+        const int u = (wave + NW * j) & (UK - 1);
+        const char* src = (is_k ? kbase : vbase) + lane_row(key0 + 4 * u + dma_rr) * kv_row_bytes + (is_k ? dma_chunk_k : dma_chunk_v) * 16;
+        dma16_lane(src, sbase + (is_k ? 0 : TILE_B) + u * 1024);
       }
     }
   };
@@ -206,14 +235,14 @@ void prefill_async_kernel(PrefillParams p) {
   // ---- LDS read maps (lane constants) -------------------------------------------------
   int k_off[HD / 16];                 // K fragment of k-step s: row n, chunk 2s + h
 #pragma unroll
-  for (int s = 0; s < HD / 16; ++s) k_off[s] = n * ROW_B + (((2 * s + h) ^ (n & 7)) << 4);
+  for (int s = 0; s < HD / 16; ++s) k_off[s] = n * ROW_B + (((2 * s + h) ^ (n & 15)) << 4);
   int v_off[HD / 32];                 // V^T fragment source of d-chunk c
   {
     const int g = lane >> 4, sl = lane & 15;
     const int row = 4 * h + (sl >> 2);                       // key row inside a 16-key window (also row & 7)
     const int y = 2 * (g & 1) + ((sl & 3) >> 1);             // 16-byte chunk inside the 64-byte d window
 #pragma unroll
-    for (int c = 0; c < HD / 32; ++c) v_off[c] = row * ROW_B + (((4 * c + y) ^ (2 * (row & 3))) << 4) + (sl & 1) * 8;
+    for (int c = 0; c < HD / 32; ++c) v_off[c] = row * ROW_B + (((4 * c + y) ^ (4 * (row & 3))) << 4) + (sl & 1) * 8;
   }
 
   // ---- accumulators ------------------------------------------------------------
@@ -222,17 +251,27 @@ void prefill_async_kernel(PrefillParams p) {
   for (int c = 0; c < HD / 32; ++c)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[c][i] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  const float sc = p.scale_log2e;
+  // Softmax state of this lane's query row.  Scores come out of the matrix cores already
+  // relative to a reference m_ref (the accumulator starts at -m_ref), in log2 units.  The
+  // reference only follows the running maximum when a tile exceeds it by more than
+  // REF_SLACK, so in the steady state there is no per-element subtraction and no
+  // rescaling of the output accumulators; probabilities stay below 2^REF_SLACK.
+  constexpr float REF_SLACK = 8.f;
+  float m_ref = 0.f, l_run = 0.f;
+  float slack = -INFINITY;            // -inf until the row has seen a finite score (m_ref is arbitrary till then)
+  f32x16_t cinit;                     // -m_ref in every accumulator slot
+#pragma unroll
+  for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
 
   const int head_phase = SPARSE ? hq % p.sparse_stride : 0;
-  const int qblk = wq_lo / BN;                    // sparse: q block of this wave
-  const int wg_blk_lo = q0 / BN, wg_blk_hi = (min(q0 + BMW, tq) - 1) / BN;
+  const int qblk = wq_lo / 64;                    // sparse: q block of this wave
+  const int wg_blk_lo = q0 / 64;
   auto next_tile = [&](int kt) __attribute__((always_inline)) -> int {      // first needed tile >= kt
     if (!SPARSE) return kt;
     while (kt < ntiles) {
       // needed by some q block of the workgroup: vertical-stride column, or inside a local window
-      if (((kt + head_phase) % p.sparse_stride) == 0 || kt > wg_blk_lo - p.sparse_local) break;
+      const int kb = kt / (64 / BN);   // sparsity block of this key tile
+      if (((kb + head_phase) % p.sparse_stride) == 0 || kb > wg_blk_lo - p.sparse_local) break;
       ++kt;
     }
     return kt;
@@ -241,31 +280,103 @@ void prefill_async_kernel(PrefillParams p) {
   // ---- the three steps of one key tile ----------------------------------------------
   auto tile_active = [&](int kt) __attribute__((always_inline)) -> bool {
     bool act = wave_has_rows && kt * BN <= prefix + wq_hi;
-    if (SPARSE) act = act && block_active(qblk, kt, head_phase, p.sparse_local, p.sparse_stride);
+    if (SPARSE) act = act && block_active(qblk, kt / (64 / BN), head_phase, p.sparse_local, p.sparse_stride);
     return act;
   };
-  // S^T = K Q^T for the tile in `stage`
-  auto scores = [&](f32x16_t (&sacc)[2], int stage) __attribute__((always_inline)) {
-    const char* ks = smem + stage * STAGE_B;
+  // ---- ring of NST stages: tiles are requested NST-1 ahead; requests past the end are
+  // repeated on the first tile so that the wait counter stays exact ------------------------
+  const int kt_first = next_tile(0);
+  int kt_i = kt_first;                // next tile to request
+  int stage_i = 0;                    // ... and the stage it goes to
+  // The entries for the following request are fetched in the middle of a tile's work, after
+  // its last wait on K fragments and before the softmax, where no LDS read is pending: a
+  // scalar load in flight turns every LDS wait into a wait for everything.
+  auto prefetch_next = [&]() __attribute__((always_inline)) { prefetch_table(kt_i < ntiles ? kt_i : kt_first); };
+  prefetch_table(kt_first);
+  auto request_next = [&]() __attribute__((always_inline)) {
+    issue_tile(kt_i < ntiles ? kt_i : kt_first, stage_i);
+    if (kt_i < ntiles) kt_i = next_tile(kt_i + 1);
+    stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
+  };
+
+  // ---- fragment loads and matrix steps, one "group" at a time -------------------------
+  // A group is the 8 K fragments of a 32-key sub-tile (8 MFMAs) or the 4 V^T fragments of
+  // a 16-key slice (4 MFMAs).  The loads of group g+1 are issued before the MFMAs of group
+  // g, with scheduling fences in between, so that the LDS reads run under the matrix work
+  // instead of in front of it.
+  auto fence = []() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
+  auto load_k = [&](bf16x8_t (&kf)[HD / 16], int stage, int tt) __attribute__((always_inline)) {
+    const char* ks = smem + stage * STAGE_B + 32 * tt * ROW_B;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
+    for (int s = 0; s < HD / 16; ++s) kf[s] = *(const bf16x8_t*)(ks + k_off[s]);
+  };
+  auto load_v = [&](bf16x8_t (&vf)[HD / 32], int stage, int g) __attribute__((always_inline)) {   // g = 2 tt + kk
+    const char* vs = smem + stage * STAGE_B + TILE_B + 16 * g * ROW_B;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[tt][i] = 0.f;
-      bf16x8_t kf[HD / 16];
-#pragma unroll
-      for (int s = 0; s < HD / 16; ++s) kf[s] = *(const bf16x8_t*)(ks + 32 * tt * ROW_B + k_off[s]);
-#pragma unroll
-      for (int s = 0; s < HD / 16; ++s)
-        sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[s], sacc[tt], 0, 0, 0);
+    for (int c = 0; c < HD / 32; ++c) {
+      const lds_char* src = (const lds_char*)(vs + v_off[c]);
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 8 * ROW_B));
+      struct { s16x4_t a, b; } pair = {lo, hi};
+      vf[c] = __builtin_bit_cast(bf16x8_t, pair);
     }
   };
+  auto mma_qk = [&](f32x16_t& sacc, const bf16x8_t (&kf)[HD / 16]) __attribute__((always_inline)) {
+    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[0], cinit, 0, 0, 0);
+#pragma unroll
+    for (int s = 1; s < HD / 16; ++s)
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[s], sacc, 0, 0, 0);
+  };
+  auto mma_pv = [&](const bf16x8_t (&vf)[HD / 32], const uint32_t (&pw)[TT][8], int g) __attribute__((always_inline)) {
+    const int tt = g >> 1, kk = g & 1;
+    const bf16x8_t pf = make_frag(pw[tt][4 * kk], pw[tt][4 * kk + 1], pw[tt][4 * kk + 2], pw[tt][4 * kk + 3]);
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c)
+      oacc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[c], pf, oacc[c], 0, 0, 0);
+  };
+  // S^T = K Q^T for the tile in `stage`; leaves the first V^T group of `vstage` in flight
+  auto scores = [&](f32x16_t (&sacc)[TT], int stage, bf16x8_t (&v0)[HD / 32], int vstage) __attribute__((always_inline)) {
+    bf16x8_t ka[HD / 16], kb[HD / 16];
+    load_k(ka, stage, 0);
+    fence();
+    if (TT == 2) {
+      load_k(kb, stage, 1);
+      fence();
+      mma_qk(sacc[0], ka);
+      fence();
+      load_v(v0, vstage, 0);
+      fence();
+      mma_qk(sacc[TT - 1], kb);
+    } else {
+      load_v(v0, vstage, 0);
+      fence();
+      mma_qk(sacc[0], ka);
+    }
+    fence();
+  };
+  // O^T += V^T P^T for the tile in `stage`; group 0's fragments were loaded by scores()
+  auto accumulate = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[HD / 32]) __attribute__((always_inline)) {
+    bf16x8_t v1[HD / 32];
+#pragma unroll
+    for (int g = 0; g < 2 * TT; g += 2) {
+      load_v(v1, stage, g + 1);
+      fence();
+      mma_pv(v0, pw, g);
+      fence();
+      if (g + 2 < 2 * TT) load_v(v0, stage, g + 2);
+      fence();
+      mma_pv(v1, pw, g + 1);
+      fence();
+    }
+  };
+
   // online softmax on this lane's column: scores -> packed bf16 probabilities, state update
-  auto softmax = [&](f32x16_t (&sacc)[2], uint32_t (&pw)[2][8], int kt) __attribute__((always_inline)) {
+  auto softmax = [&](f32x16_t (&sacc)[TT], uint32_t (&pw)[TT][8], int kt) __attribute__((always_inline)) {
     const int key0 = kt * BN;
     const bool need_mask = key0 + BN - 1 > prefix + wq_lo;    // tile reaches past the first row's diagonal
     if (need_mask) {
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
+      for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
@@ -274,66 +385,47 @@ void prefill_async_kernel(PrefillParams p) {
     }
     float tmax = -INFINITY;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+    for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sacc[tt][i]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * sc;        // sc > 0: max commutes with the scale
-    // a row whose visible keys all lie in later tiles keeps m = -inf for now
-    const float m_new = fmaxf(m_run, tmax);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    {   // the other half-wave holds the remaining keys of this query row: swap halves in registers
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(tmax), __float_as_uint(tmax), false, false);
+      tmax = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+    // move the reference only for the first finite tile of a row or a jump beyond the slack
+    const bool move = tmax > slack;
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float shift = move ? tmax : 0.f;
+      const float alpha = (move && slack != -INFINITY) ? __builtin_amdgcn_exp2f(-shift) : 1.f;   // a fresh row has nothing to rescale
+      m_ref += shift;
+      slack = move ? REF_SLACK : slack;
+      l_run *= alpha;
+#pragma unroll
+      for (int c = 0; c < HD / 32; ++c) oacc[c] *= alpha;
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sacc[tt][i] -= shift;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) cinit[i] = -m_ref;
+    }
     float psum = 0.f;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+    for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[tt][i], sc, -m_use));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[tt][i + 1], sc, -m_use));
+        const float p0 = __builtin_amdgcn_exp2f(sacc[tt][i]);
+        const float p1 = __builtin_amdgcn_exp2f(sacc[tt][i + 1]);
         psum += p0 + p1;
         pw[tt][i >> 1] = pack_bf16x2(p0, p1);
       }
-    l_run = l_run * alpha + psum;
-    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {   // rescale only when some row's max moved
-#pragma unroll
-      for (int c = 0; c < HD / 32; ++c) oacc[c] *= alpha;
-    }
-    m_run = m_new;
-  };
-  // O^T += V^T P^T for the tile in `stage`
-  auto accumulate = [&](const uint32_t (&pw)[2][8], int stage) __attribute__((always_inline)) {
-    const char* vs = smem + stage * STAGE_B + TILE_B;
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const bf16x8_t pf = make_frag(pw[tt][4 * kk], pw[tt][4 * kk + 1], pw[tt][4 * kk + 2], pw[tt][4 * kk + 3]);
-        bf16x8_t vf[HD / 32];
-#pragma unroll
-        for (int c = 0; c < HD / 32; ++c) {
-          const lds_char* src = (const lds_char*)(vs + (32 * tt + 16 * kk) * ROW_B + v_off[c]);
-          const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
-          const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 8 * ROW_B));
-          struct { s16x4_t a, b; } pair = {lo, hi};
-          vf[c] = __builtin_bit_cast(bf16x8_t, pair);
-        }
-#pragma unroll
-        for (int c = 0; c < HD / 32; ++c)
-          oacc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[c], pf, oacc[c], 0, 0, 0);
-      }
-  };
-
-  // ---- ring of NST stages: tiles are requested NST-1 ahead; requests past the end are
-  // repeated on the first tile so that the wait counter stays exact ------------------------
-  const int kt_first = next_tile(0);
-  int kt_i = kt_first;                // next tile to request
-  int stage_i = 0;                    // ... and the stage it goes to
-  auto request_next = [&]() __attribute__((always_inline)) {
-    issue_tile(kt_i < ntiles ? kt_i : kt_first, stage_i);
-    if (kt_i < ntiles) kt_i = next_tile(kt_i + 1);
-    stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
+    l_run += psum;
   };
 #pragma unroll
-  for (int s = 0; s < NST - 1; ++s) request_next();
+  for (int s = 0; s < NST - 1; ++s) {
+    request_next();
+    prefetch_next();
+  }
 
   if (!PINGPONG) {
     int kt_c = kt_first, stage_c = 0;
@@ -342,11 +434,15 @@ void prefill_async_kernel(PrefillParams p) {
       __builtin_amdgcn_s_barrier();                // ... and everyone's; all waves are done with the previous tile
       request_next();
       if (tile_active(kt_c)) {
-        f32x16_t sacc[2];
-        uint32_t pw[2][8];
-        scores(sacc, stage_c);
+        f32x16_t sacc[TT];
+        uint32_t pw[TT][8];
+        bf16x8_t v0[HD / 32];
+        scores(sacc, stage_c, v0, stage_c);
+        prefetch_next();
         softmax(sacc, pw, kt_c);
-        accumulate(pw, stage_c);
+        accumulate(pw, stage_c, v0);
+      } else {
+        prefetch_next();
       }
       kt_c = next_tile(kt_c + 1);
       stage_c = stage_c + 1 == NST ? 0 : stage_c + 1;
@@ -357,15 +453,16 @@ void prefill_async_kernel(PrefillParams p) {
     // the other is in its vector step (softmax of its tile), and a barrier flips them.
     // Step order per wave: [softmax j | barrier | scores j+1, P.V j | barrier]; the second
     // group starts one barrier later and the first group ends one barrier later.
-    static_assert(!PINGPONG || NST == 4, "ping-pong needs the 4-stage ring");
+    static_assert(!PINGPONG || NST == 4, "the two-group schedule needs the 4-stage ring");
     const bool second = wave >= NW / 2;
     int kt_c = kt_first, stage_c = 0;
-    f32x16_t s_cur[2], s_nxt[2];
-    uint32_t pw[2][8];
+    f32x16_t s_cur[TT], s_nxt[TT];
+    uint32_t pw[TT][8];
+    bf16x8_t v0[HD / 32];
     wait_vmcnt<2 * UPW>();                         // tile 0 (own part)
     __builtin_amdgcn_s_barrier();
     bool act_cur = tile_active(kt_c);
-    if (act_cur) scores(s_cur, stage_c);
+    if (act_cur) scores(s_cur, stage_c, v0, stage_c);
     if (second) {
       wait_vmcnt<UPW>();                           // tile 1 (own part): the first group reads it next
       __builtin_amdgcn_s_barrier();
@@ -381,13 +478,14 @@ void prefill_async_kernel(PrefillParams p) {
       const int kt_n = next_tile(kt_c + 1);
       const int stage_n = stage_c + 1 == NST ? 0 : stage_c + 1;
       const bool act_nxt = kt_n < ntiles && tile_active(kt_n);
-      if (act_nxt) scores(s_nxt, stage_n);
-      if (act_cur) accumulate(pw, stage_c);
+      if (act_cur) accumulate(pw, stage_c, v0);
+      if (act_nxt) scores(s_nxt, stage_n, v0, stage_n);
       __builtin_amdgcn_s_setprio(0);
+      prefetch_next();
       wait_vmcnt<UPW>();                           // own part of the tile after next
       __builtin_amdgcn_s_barrier();
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) s_cur[tt] = s_nxt[tt];
+      for (int tt = 0; tt < TT; ++tt) s_cur[tt] = s_nxt[tt];
       act_cur = act_nxt;
       kt_c = kt_n;
       stage_c = stage_n;
@@ -397,7 +495,10 @@ void prefill_async_kernel(PrefillParams p) {
   wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
 
   // ---- normalise and write this lane's query row ---------------------------------
-  l_run += __shfl_xor(l_run, 32, 64);
+  {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+    l_run = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  }
   if (qrow < p.T && wq_lo < p.T) {
     uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
     const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
@@ -413,12 +514,12 @@ void prefill_async_kernel(PrefillParams p) {
   }
 }
 
-template <bool SPARSE, int MODE, int NW, bool PINGPONG>
+template <bool SPARSE, int MODE, int NW, bool PINGPONG, int TT = 2>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
-  constexpr int lds = (NW == 8 ? 4 : 2) * STAGE_B;
+  constexpr int lds = (TT == 1 ? 3 : (NW == 8 ? 4 : 2)) * 2 * 32 * TT * ROW_B;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, PINGPONG>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, PINGPONG, TT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
@@ -429,7 +530,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   const long groups = (long)p.B * p.Hkv;
   const long total = 8 * ((groups + 7) / 8) * per_group;
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, PINGPONG>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, PINGPONG, TT>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   return hipGetLastError();
 }
 
