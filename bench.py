@@ -136,6 +136,26 @@ def bench_decode(cfg, steps, warmup, lib, pa, W):
     return res
 
 
+def _mfma_ceiling(lib, sample):
+    """Matrix-core rate of a registers-only MFMA loop fed with operands drawn from `sample`
+    (a bf16 device tensor of the benchmark's own inputs): what the power-limited chip
+    sustains on this data distribution, to read the nominal-peak fraction against."""
+    import ctypes
+    blocks, iters = 256, 4000
+    need = blocks * 65536 // 2
+    flat = sample.reshape(-1)
+    ops = flat[:need].contiguous() if flat.numel() >= need else flat.repeat((need + flat.numel() - 1) // flat.numel())[:need].contiguous()
+    sink = torch.empty(blocks * 512, dtype=torch.float32, device=ops.device)
+    ms = ctypes.c_float(0.0)
+    best = 0.0
+    for _ in range(3):
+        rc = lib.pa_probe_mfma(ops.data_ptr(), sink.data_ptr(), blocks, iters, ctypes.byref(ms), torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(lib.pa_last_error().decode())
+        best = max(best, blocks * 8 * iters * 16 * 32768.0 / (ms.value * 1e-3) / 1e12)
+    return round(best, 1)
+
+
 def bench_prefill(steps, warmup, lib, pa, W):
     from oracle import paged_attention_oracle as O
     from tests.pa_testlib import dev_bits
@@ -170,8 +190,9 @@ def bench_prefill(steps, warmup, lib, pa, W):
                    "flops": fl},
         "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel": "prefill_kernel", "kernel_avg_ms": round(kavg, 5),
-                     "launches_timed": len(kms)},
+                     "traffic": None, "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "launches_timed": len(kms),
+                     "mfma_only_loop_same_data": _mfma_ceiling(lib, w.k_cache)},
     }
     res["cpu_baseline"] = _cpu_prefill_baseline(w, None, cpu, "NumPy oracle, sequence 7, q heads 0-3 of the same workload")
     return res
@@ -210,8 +231,9 @@ def bench_blocksparse(steps, warmup, lib, pa, W):
                                f"local={w.local_blocks}, vert_stride={w.vert_stride}", "flops": fl},
         "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel": "prefill_kernel", "kernel_avg_ms": round(kavg, 5),
-                     "launches_timed": len(kms)},
+                     "traffic": None, "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "launches_timed": len(kms),
+                     "mfma_only_loop_same_data": _mfma_ceiling(lib, w.k)},
     }
     res["cpu_baseline"] = _cpu_prefill_baseline(
         w, None, cpu, "NumPy oracle (dense masked scores), batch 0 head 0 of the same workload; FLOPs counted as the sparse ones")

@@ -129,7 +129,7 @@ int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* 
  * fixed-partition MFMA kernel (0 = default); key 2: its grid order (1 = kv head
  * fastest, the default; 0 = partition fastest); key 3: prefill kernel choice (0 =
  * automatic, 1 = register-staged kernel, 4 / 8 = asynchronous-copy kernel with that
- * many wavefronts per workgroup, 16 = 8 wavefronts in two alternating groups); key 4:
+ * many wavefronts per workgroup); key 4:
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
  * the same tile (1 = on, the default). */
 int pa_debug_set(int key, int value);
@@ -142,6 +142,16 @@ int pa_debug_set(int key, int value);
  * spike/src/spike/spike_model.py:290-363. */
 int pa_profile_enable(int on);
 int pa_profile_collect(float* ms, int cap);
+
+/* Matrix-core ceiling probe for benchmarks (no counterpart in the reference): runs
+ * `iters` x 16 back-to-back v_mfma_f32_32x32x16_bf16 per wavefront on `blocks`
+ * workgroups of 8 wavefronts, operands taken once from `operands` (blocks * 65536
+ * bytes of bf16 values, device memory), nothing else in the loop; `sink` receives
+ * blocks * 512 floats.  Synchronous; *ms is the kernel time.  FLOP = blocks * 8 *
+ * iters * 16 * 32768.  The rate depends on the operand data (the chip is power
+ * limited): benchmarks quote it for their own data distribution beside the nominal
+ * peak. */
+int pa_probe_mfma(const void* operands, void* sink, int blocks, int iters, float* ms, void* stream);
 
 #ifdef __cplusplus
 }

@@ -133,6 +133,23 @@ int pa_profile_collect(float* ms, int cap) {
   return n;
 }
 
+int pa_probe_mfma(const void* operands, void* sink, int blocks, int iters, float* ms, void* stream) {
+  tl_error[0] = 0;
+  if (!operands || !sink || !ms || blocks <= 0 || iters <= 0) return fail_arg("pa_probe_mfma: bad arguments");
+  if (!aligned16(operands)) return fail_arg("pa_probe_mfma: operands must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return check_hip(hipGetLastError(), "pa_probe_mfma events");
+  (void)hipEventRecord(e0, s);
+  hipError_t e = launch_mfma_probe(operands, sink, blocks, iters, s);
+  (void)hipEventRecord(e1, s);
+  if (e == hipSuccess) e = hipEventSynchronize(e1);
+  if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return check_hip(e, "pa_probe_mfma");
+}
+
 static int num_partitions_for(int max_seq_len, int partition_size) {
   if (max_seq_len <= 0) return 1;
   return (max_seq_len + partition_size - 1) / partition_size;

@@ -123,6 +123,8 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
 bool prefill_async_supported(const PrefillParams& p);
 
 // ---- gather ------------------------------------------------------------------------
+// matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats
+hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s);
 hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,
                          int B, int row_bytes, int block_size, int max_blocks, int num_blocks,
                          int max_seq_len, hipStream_t s);

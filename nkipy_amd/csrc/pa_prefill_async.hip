@@ -36,6 +36,7 @@
 #include "pa_common.h"
 
 
+
 namespace pa {
 namespace {
 
@@ -79,10 +80,9 @@ __device__ __forceinline__ void dma16_lane(const char* addr, uint32_t lds_base) 
 typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
 // MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16.
-// TT: 32-key sub-tiles per key tile (2: 64-key tiles, two workgroups of 4 waves per CU;
-// 1: 32-key tiles with a smaller register and LDS footprint, three workgroups per CU).
-template <bool SPARSE, int MODE, int NW, bool PINGPONG, int TT>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(TT == 1 ? 3 : 2, TT == 1 ? 3 : 2)))
+// TT: 32-key sub-tiles per key tile (2: 64-key tiles).
+template <bool SPARSE, int MODE, int NW, int TT>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int BN = 32 * TT;                // keys per tile
@@ -90,7 +90,7 @@ void prefill_async_kernel(PrefillParams p) {
   constexpr int STAGE_B = 2 * TILE_B;        // K then V
   constexpr int UK = BN / 4;                 // 1 KB copy units per tensor tile
   constexpr int BMW = 32 * NW;               // query rows per workgroup
-  constexpr int NST = TT == 1 ? 3 : (NW == 8 ? 4 : 2);   // LDS stages
+  constexpr int NST = NW == 8 ? 4 : 2;   // LDS stages
   constexpr int UPW = 2 * UK / NW;           // copy units per wave per tile
 
   const int tid = threadIdx.x;
@@ -301,10 +301,9 @@ void prefill_async_kernel(PrefillParams p) {
 
   // ---- fragment loads and matrix steps, one "group" at a time -------------------------
   // A group is the 8 K fragments of a 32-key sub-tile (8 MFMAs) or the 4 V^T fragments of
-  // a 16-key slice (4 MFMAs).  The loads of group g+1 are issued before the MFMAs of group
-  // g, with scheduling fences in between, so that the LDS reads run under the matrix work
-  // instead of in front of it.
-  auto fence = []() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
+  // a 16-key slice (4 MFMAs).  The loads of group g+1 are written before the MFMAs of group
+  // g; where exactly they issue is left to the compiler's scheduler (pinning the order with
+  // scheduling barriers measured 3 % slower).
   auto load_k = [&](bf16x8_t (&kf)[HD / 16], int stage, int tt) __attribute__((always_inline)) {
     const char* ks = smem + stage * STAGE_B + 32 * tt * ROW_B;
 #pragma unroll
@@ -338,21 +337,15 @@ void prefill_async_kernel(PrefillParams p) {
   auto scores = [&](f32x16_t (&sacc)[TT], int stage, bf16x8_t (&v0)[HD / 32], int vstage) __attribute__((always_inline)) {
     bf16x8_t ka[HD / 16], kb[HD / 16];
     load_k(ka, stage, 0);
-    fence();
     if (TT == 2) {
       load_k(kb, stage, 1);
-      fence();
       mma_qk(sacc[0], ka);
-      fence();
       load_v(v0, vstage, 0);
-      fence();
       mma_qk(sacc[TT - 1], kb);
     } else {
       load_v(v0, vstage, 0);
-      fence();
       mma_qk(sacc[0], ka);
     }
-    fence();
   };
   // O^T += V^T P^T for the tile in `stage`; group 0's fragments were loaded by scores()
   auto accumulate = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[HD / 32]) __attribute__((always_inline)) {
@@ -360,13 +353,9 @@ void prefill_async_kernel(PrefillParams p) {
 #pragma unroll
     for (int g = 0; g < 2 * TT; g += 2) {
       load_v(v1, stage, g + 1);
-      fence();
       mma_pv(v0, pw, g);
-      fence();
       if (g + 2 < 2 * TT) load_v(v0, stage, g + 2);
-      fence();
       mma_pv(v1, pw, g + 1);
-      fence();
     }
   };
 
@@ -427,7 +416,7 @@ void prefill_async_kernel(PrefillParams p) {
     prefetch_next();
   }
 
-  if (!PINGPONG) {
+  {
     int kt_c = kt_first, stage_c = 0;
     while (kt_c < ntiles) {
       wait_vmcnt<(NST - 2) * UPW>();               // this wave's part of tile kt_c has landed
@@ -447,50 +436,6 @@ void prefill_async_kernel(PrefillParams p) {
       kt_c = next_tile(kt_c + 1);
       stage_c = stage_c + 1 == NST ? 0 : stage_c + 1;
     }
-  } else {
-    // Two groups of four waves (one wave of each group per SIMD) run half a tile apart:
-    // while one group is in its matrix-core step (scores of tile j+1, then P.V of tile j)
-    // the other is in its vector step (softmax of its tile), and a barrier flips them.
-    // Step order per wave: [softmax j | barrier | scores j+1, P.V j | barrier]; the second
-    // group starts one barrier later and the first group ends one barrier later.
-    static_assert(!PINGPONG || NST == 4, "the two-group schedule needs the 4-stage ring");
-    const bool second = wave >= NW / 2;
-    int kt_c = kt_first, stage_c = 0;
-    f32x16_t s_cur[TT], s_nxt[TT];
-    uint32_t pw[TT][8];
-    bf16x8_t v0[HD / 32];
-    wait_vmcnt<2 * UPW>();                         // tile 0 (own part)
-    __builtin_amdgcn_s_barrier();
-    bool act_cur = tile_active(kt_c);
-    if (act_cur) scores(s_cur, stage_c, v0, stage_c);
-    if (second) {
-      wait_vmcnt<UPW>();                           // tile 1 (own part): the first group reads it next
-      __builtin_amdgcn_s_barrier();
-    }
-    while (kt_c < ntiles) {
-      // ---- vector step ----
-      if (act_cur) softmax(s_cur, pw, kt_c);
-      wait_vmcnt<UPW>();                           // own part of the next tile
-      __builtin_amdgcn_s_barrier();
-      request_next();                              // into the stage every wave left one step ago
-      // ---- matrix step ----
-      __builtin_amdgcn_s_setprio(1);
-      const int kt_n = next_tile(kt_c + 1);
-      const int stage_n = stage_c + 1 == NST ? 0 : stage_c + 1;
-      const bool act_nxt = kt_n < ntiles && tile_active(kt_n);
-      if (act_cur) accumulate(pw, stage_c, v0);
-      if (act_nxt) scores(s_nxt, stage_n, v0, stage_n);
-      __builtin_amdgcn_s_setprio(0);
-      prefetch_next();
-      wait_vmcnt<UPW>();                           // own part of the tile after next
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt) s_cur[tt] = s_nxt[tt];
-      act_cur = act_nxt;
-      kt_c = kt_n;
-      stage_c = stage_n;
-    }
-    if (!second) __builtin_amdgcn_s_barrier();
   }
   wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
 
@@ -514,12 +459,12 @@ void prefill_async_kernel(PrefillParams p) {
   }
 }
 
-template <bool SPARSE, int MODE, int NW, bool PINGPONG, int TT = 2>
+template <bool SPARSE, int MODE, int NW, int TT = 2>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
-  constexpr int lds = (TT == 1 ? 3 : (NW == 8 ? 4 : 2)) * 2 * 32 * TT * ROW_B;
+  constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, PINGPONG, TT>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
@@ -530,7 +475,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   const long groups = (long)p.B * p.Hkv;
   const long total = 8 * ((groups + 7) / 8) * per_group;
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, PINGPONG, TT>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   return hipGetLastError();
 }
 
@@ -545,18 +490,15 @@ bool prefill_async_supported(const PrefillParams& p) {
 hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s) {
   const bool sparse = p.sparse_stride > 0;
   const bool paged = p.block_tables != nullptr;
-  // waves: 4 or 8 = plain ring with that many waves; 16 = 8 waves with the two-group schedule
-  if (waves == 0) waves = 4;   // measured: 4 waves (two workgroups per CU) beat 8 on both the dense and the sparse form
-  if (waves == 16) {
-    if (sparse) return launch_typed<true, 0, 8, true>(p, s);
-    return paged ? launch_typed<false, 1, 8, true>(p, s) : launch_typed<false, 0, 8, true>(p, s);
-  }
+  // waves: 4 (two workgroups of 128 query rows per CU, 2-stage ring) or 8 (one workgroup of
+  // 256 rows, 4-stage ring).  Measured within a few per cent of each other on the dense form;
+  // 4 is the default: it wins on the sparse form and on short query chunks.
   if (waves == 8) {
-    if (sparse) return launch_typed<true, 0, 8, false>(p, s);
-    return paged ? launch_typed<false, 1, 8, false>(p, s) : launch_typed<false, 0, 8, false>(p, s);
+    if (sparse) return launch_typed<true, 0, 8>(p, s);
+    return paged ? launch_typed<false, 1, 8>(p, s) : launch_typed<false, 0, 8>(p, s);
   }
-  if (sparse) return launch_typed<true, 0, 4, false>(p, s);
-  return paged ? launch_typed<false, 1, 4, false>(p, s) : launch_typed<false, 0, 4, false>(p, s);
+  if (sparse) return launch_typed<true, 0, 4>(p, s);
+  return paged ? launch_typed<false, 1, 4>(p, s) : launch_typed<false, 0, 4>(p, s);
 }
 
 }  // namespace pa
