@@ -97,6 +97,21 @@ def _cpu_prefill_baseline(w, flops_fn, run_fn, desc):
             "sample": f"{desc}, one run of {dt:.2f} s, numpy {np.__version__} default BLAS threading"}
 
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this file on the seeded workloads (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00: the factors a plain copy
+# of known size shows); the summaries with the commands are under profiles/.  Not re-measured at run time.
+MEASURED_TRAFFIC_BYTES = {
+    2: {"bytes": 1_098_900_000, "source": "profiles/decode_balanced_kernel_C2.md"},
+    3: {"bytes": 394_700_000, "source": "profiles/prefill_async_kernel_C3.md"},
+    4: {"bytes": 692_400_000, "source": "profiles/prefill_async_kernel_C4.md"},
+}
+
+
+def _traffic(cfg):
+    t = MEASURED_TRAFFIC_BYTES.get(cfg)
+    return (t["bytes"], t["source"]) if t else (None, None)
+
+
 def bench_decode(cfg, steps, warmup, lib, pa, W):
     w = W.make_decode(cfg)
     out = torch.empty_like(w.q)
@@ -129,7 +144,8 @@ def bench_decode(cfg, steps, warmup, lib, pa, W):
                    "algorithmic_bytes": ab},
         "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "decode_balanced_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "traffic": _traffic(cfg)[0], "traffic_source": _traffic(cfg)[1],
+                     "kernel": "decode_balanced_kernel", "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms)},
     }
     res["cpu_baseline"] = _cpu_decode_baseline(w)
@@ -190,7 +206,8 @@ def bench_prefill(steps, warmup, lib, pa, W):
                    "flops": fl},
         "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "traffic": _traffic(3)[0], "traffic_source": _traffic(3)[1],
+                     "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms),
                      "mfma_only_loop_same_data": _mfma_ceiling(lib, w.k_cache)},
     }
@@ -231,7 +248,8 @@ def bench_blocksparse(steps, warmup, lib, pa, W):
                                f"local={w.local_blocks}, vert_stride={w.vert_stride}", "flops": fl},
         "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "traffic": _traffic(4)[0], "traffic_source": _traffic(4)[1],
+                     "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms),
                      "mfma_only_loop_same_data": _mfma_ceiling(lib, w.k)},
     }
