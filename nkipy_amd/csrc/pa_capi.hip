@@ -259,8 +259,8 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   if (dtype != PA_BF16) return fail_arg("pa_prefill: only bf16 is supported (dtype=%d)", dtype);
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_prefill: bad paging sizes");
   if (B == 0 || T == 0) return 0;
-  if ((long)num_blocks * block_size > 0x7fffffffL || (long)Hkv * D * 2 > 0x7fffffffL)
-    return fail_arg("pa_prefill: pool of %d blocks x %d rows exceeds 2^31 rows", num_blocks, block_size);
+  if ((long)num_blocks * block_size > 0x7fffffffL || (long)block_size * Hkv * D * 2 > 0xffffffffL)
+    return fail_arg("pa_prefill: pool of %d blocks x %d rows exceeds 2^31 rows (or a block 4 GiB)", num_blocks, block_size);
   if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens || !out)
     return fail_arg("pa_prefill: null pointer argument");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))

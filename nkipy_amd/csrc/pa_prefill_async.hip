@@ -137,28 +137,7 @@ void prefill_async_kernel(PrefillParams p) {
   const bool qvalid = qrow < tq;
   const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
   const float sc = p.scale_log2e;
-  bf16x8_t qf[HD / 16];
-  {
-    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
-#pragma unroll
-    for (int s = 0; s < HD / 16; ++s) {
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (qvalid) v = *(const uint4*)(qp + 16 * s + 8 * h);
-      // scale * log2(e) goes into Q once (rounded to bf16 again: a relative 2^-9 per element,
-      // below the rounding of the probabilities), so that the scores leave the matrix cores
-      // ready for exp2
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-      uint32_t r[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        r[j] = pack_bf16x2(bf16_bits_to_float(w[j] & 0xffffu) * sc, bf16_bits_to_float(w[j] >> 16) * sc);
-      qf[s] = make_frag(r[0], r[1], r[2], r[3]);
-    }
-    // the Q loads must be complete (and known to be) before the copy ring starts, or the
-    // first use of a fragment inside the loop would drain the ring with a full wait
-#pragma unroll
-    for (int s = 0; s < HD / 16; ++s) asm volatile("" ::"v"(qf[s]));
-  }
+  bf16x8_t qf[HD / 16];           // loaded below, between the first copy requests
   const int wq_lo = q0 + wave * 32;                               // first row of this wave
   const int wq_hi = min(wq_lo + 31, tq - 1);                      // last valid row (may be < wq_lo)
   const bool wave_has_rows = wq_lo < tq;
@@ -179,6 +158,8 @@ void prefill_async_kernel(PrefillParams p) {
   // same swizzle: K rows use row & 15, V rows 4 * (row & 3) (what their read patterns want)
   const int dma_chunk_k = dma_pos ^ ((4 * (wave & 3) + dma_rr) & 15);
   const int dma_chunk_v = dma_pos ^ (4 * dma_rr);
+  const uint32_t kv_row_bytes_u = (uint32_t)kv_row_bytes;
+  const uint32_t block_bytes_u = MODE != 0 ? (uint32_t)p.block_size * kv_row_bytes_u : 0u;
   const int dma_lane_off_k = (int)(dma_rr * kv_row_bytes) + dma_chunk_k * 16;
   const int dma_lane_off_v = (int)(dma_rr * kv_row_bytes) + dma_chunk_v * 16;
 
@@ -207,19 +188,21 @@ void prefill_async_kernel(PrefillParams p) {
     const int key0 = kt * BN;
     const uint32_t sbase = smem_base + stage * STAGE_B;
     if (key0 + BN <= ctx) {                       // whole tile inside the context: one row base per unit
+      // byte offset of a unit's first row = block * (block bytes) + in-block row * (row bytes):
+      // one 32x32->64 multiply and one 32-bit multiply on the scalar ALU (both factors fit 32
+      // bits, checked on the host); K and V units of a wave share it
 #pragma unroll
-      for (int j = 0; j < UPW; ++j) {
-        const bool is_k = j < UPW / 2;
+      for (int j = 0; j < UPW / 2; ++j) {
         const int u = (wave + NW * j) & (UK - 1);
-        long row;
+        uint64_t off;
         if (MODE == 0) {
-          row = (long)b * p.S + key0 + 4 * u;
+          off = (uint64_t)(uint32_t)(b * p.S + key0 + 4 * u) * kv_row_bytes_u;
         } else {
-          const int blk = min(max(blk_pf[j % (UPW / 2)], 0), p.num_blocks - 1);
-          row = (long)blk * p.block_size + ((key0 + 4 * u) & (p.block_size - 1));
+          const uint32_t blk = (uint32_t)min(max(blk_pf[j], 0), p.num_blocks - 1);
+          off = (uint64_t)blk * block_bytes_u + (uint32_t)((key0 + 4 * u) & (p.block_size - 1)) * kv_row_bytes_u;
         }
-        dma16_uniform((is_k ? kbase : vbase) + row * kv_row_bytes, is_k ? dma_lane_off_k : dma_lane_off_v,
-                      sbase + (is_k ? 0 : TILE_B) + u * 1024);
+        dma16_uniform(kbase + off, dma_lane_off_k, sbase + u * 1024);
+        dma16_uniform(vbase + off, dma_lane_off_v, sbase + TILE_B + u * 1024);
       }
     } else {                                      // last tile of a context: rows past it re-read its last row
 #pragma unroll
@@ -410,8 +393,33 @@ void prefill_async_kernel(PrefillParams p) {
       }
     l_run += psum;
   };
+  // ---- prologue: the first tile's copies, then Q, then the rest of the ring: the Q loads and
+  // the first tile travel together instead of one memory latency after the other
+  request_next();
+  prefetch_next();
+  {
+    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
 #pragma unroll
-  for (int s = 0; s < NST - 1; ++s) {
+    for (int s = 0; s < HD / 16; ++s) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (qvalid) v = *(const uint4*)(qp + 16 * s + 8 * h);
+      // scale * log2(e) goes into Q once (rounded to bf16 again: a relative 2^-9 per element,
+      // below the rounding of the probabilities), so that the scores leave the matrix cores
+      // ready for exp2
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      uint32_t r[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        r[j] = pack_bf16x2(bf16_bits_to_float(w[j] & 0xffffu) * sc, bf16_bits_to_float(w[j] >> 16) * sc);
+      qf[s] = make_frag(r[0], r[1], r[2], r[3]);
+    }
+    // the Q loads must be complete (and known to the compiler to be) before the loop, or the
+    // first use of a fragment inside it would drain the ring with a full wait
+#pragma unroll
+    for (int s = 0; s < HD / 16; ++s) asm volatile("" ::"v"(qf[s]));
+  }
+#pragma unroll
+  for (int s = 1; s < NST - 1; ++s) {
     request_next();
     prefetch_next();
   }
@@ -491,8 +499,10 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   const bool sparse = p.sparse_stride > 0;
   const bool paged = p.block_tables != nullptr;
   // waves: 4 (two workgroups of 128 query rows per CU, 2-stage ring) or 8 (one workgroup of
-  // 256 rows, 4-stage ring).  Measured within a few per cent of each other on the dense form;
-  // 4 is the default: it wins on the sparse form and on short query chunks.
+  // 256 rows, 4-stage ring: half the copy requests per FLOP).  Measured within a few per cent of
+  // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
+  // and for the sparse form.
+  if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
   if (waves == 8) {
     if (sparse) return launch_typed<true, 0, 8>(p, s);
     return paged ? launch_typed<false, 1, 8>(p, s) : launch_typed<false, 0, 8>(p, s);
