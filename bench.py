@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the paged attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|5|3|4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|5|3|4|6]
 
 A step is one pass of the op over one batch of synthetic input that is already
 resident in HBM.  Default workload: config 2 (Llama-3-8B-shape paged decode, bf16,
@@ -28,6 +28,7 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+_NO_CPU = False
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
@@ -258,12 +259,63 @@ def bench_blocksparse(steps, warmup, lib, pa, W):
     return res
 
 
+def bench_kv_write(steps, warmup, lib, pa, W):
+    """Paged KV write with fp8 quantise-on-write (the step in front of the attention call).
+    The kernel mutates the pool; every step rewrites the same rows with the same values, so the
+    steady state (scales already at their maximum: no re-encode of earlier rows) is what is timed."""
+    from oracle import paged_attention_oracle as O
+    from tests.pa_testlib import dev_bits
+    w = W.make_kv_write()
+
+    def step():
+        pa.kv_write(w.k_new, w.v_new, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens,
+                    k_scale=w.k_scale, v_scale=w.v_scale)
+
+    sec = _time_steps(step, steps, warmup)
+    lib.pa_profile_enable(1)
+    _time_steps(step, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = _collect_kernel_ms(lib, steps)
+    kavg = float(np.mean(kms))
+    ab = w.algorithmic_bytes()
+    B, T, Hkv, D = w.k_new.shape
+    res = {
+        "metric": "paged KV write HBM GB/s (% peak)",
+        "value": round(ab / sec / 1e9, 2), "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * ab / sec / 1e9 / HBM_PEAK_GBS, 2),
+        "tok_per_s": round(B * T / sec, 1),
+        "ms_per_step": round(sec * 1e3, 5), "dtype": "bf16 rows -> fp8-e4m3 pool, fp32 scales",
+        "config": {"workload": f"C6 paged KV write: B={B}, T={T} new tokens, Hkv={Hkv}, D={D}, block_size={w.k_cache.shape[1]}, "
+                               f"prefix={w.prefix.tolist()}, pool={w.k_cache.shape[0]} blocks",
+                   "algorithmic_bytes": ab},
+        "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel": "kv_write_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "launches_timed": len(kms)},
+    }
+
+    def cpu():
+        n = 2
+        kn, vn = dev_bits(w.k_new[:n]), dev_bits(w.v_new[:n])
+        kc, vc = dev_bits(w.k_cache), dev_bits(w.v_cache)
+        ks, vs = w.k_scale.cpu().numpy(), w.v_scale.cpu().numpy()
+        t = time.perf_counter()
+        O.kv_write(kn, vn, kc, vc, w.block_tables[:n].cpu().numpy(), w.seq_lens[:n].cpu().numpy(),
+                   w.query_lens[:n].cpu().numpy(), k_scale=ks, v_scale=vs)
+        dt = time.perf_counter() - t
+        return {"value": round(ab * n / B / dt / 1e9, 4), "unit": "GB/s", "cores": _host_info(), "kind": "port",
+                "sample": f"NumPy oracle, first {n} of {B} sequences of the same workload, one run of {dt:.2f} s"}
+
+    res["cpu_baseline"] = None if _NO_CPU else cpu()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -278,13 +330,16 @@ def main():
     lib = _lib.load()
     torch.cuda.set_device(0)
     if args.no_cpu:
-        global _cpu_decode_baseline, _cpu_prefill_baseline
+        global _cpu_decode_baseline, _cpu_prefill_baseline, _NO_CPU
+        _NO_CPU = True
         _cpu_decode_baseline = lambda *a, **k: None      # noqa: E731
         _cpu_prefill_baseline = lambda *a, **k: None     # noqa: E731
     if args.config in (2, 5):
         res = bench_decode(args.config, args.steps, args.warmup, lib, pa, W)
     elif args.config == 3:
         res = bench_prefill(args.steps, args.warmup, lib, pa, W)
+    elif args.config == 6:
+        res = bench_kv_write(args.steps, args.warmup, lib, pa, W)
     else:
         res = bench_blocksparse(args.steps, args.warmup, lib, pa, W)
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"),

@@ -123,6 +123,28 @@ int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* 
                  int max_blocks_per_seq, int num_blocks, int max_seq_len,
                  int elem_bytes, void* stream);
 
+/* Paged KV-cache write, to be run before the attention call of the same step: token
+ * t < query_lens[b] of sequence b sits at position seq_lens[b] - query_lens[b] + t and its
+ * K/V rows go to pool row (block_tables[b, pos / block_size], pos % block_size).  Replaces
+ * the reference's dense cache update `cache_k[:, query_pos] = xk` with query_pos =
+ * start_pos + arange(seq_len) (examples/models/gpt_oss/kernels/attention.py:85,92-100;
+ * examples/models/qwen3/kernels/attention.py:100-106); the pool is updated in place like the
+ * reference's aliased cache tensors (examples/models/qwen3/qwen3.py:289-301).
+ *   k_new, v_new  [B, T, Hkv, D], bf16 (float32 when kv_dtype is PA_F32); rows t >= query_lens[b] are padding
+ *   k/v_cache     [num_blocks, block_size, Hkv, D] of kv_dtype
+ *   k/v_scale     [num_blocks, Hkv] float32, PA_FP8_E4M3FN only (NULL otherwise): kept as the running
+ *                 maximum of absmax / 448 over the tokens a block holds; when a write raises it the
+ *                 block's earlier rows are re-encoded; a block whose first row is written is fresh.
+ *                 The fp8 part has no counterpart in the reference.
+ * Blocks being written must belong to one sequence only (shared prefix blocks are read-only).
+ * Sequences with query_lens[b] <= 0 or seq_lens[b] < query_lens[b], and table entries outside
+ * the pool, write nothing. */
+int pa_kv_write(const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                float* k_scale, float* v_scale,
+                const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+                int B, int T, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks,
+                int kv_dtype, void* stream);
+
 /* Debug switches (process-wide; tests only).  key 0: decode kernel choice
  * (0 = automatic, 1 = scalar-ALU kernel, 2 = MFMA kernel with fixed partitions,
  * 3 = MFMA kernel with the balanced schedule); key 1: waves per workgroup of the

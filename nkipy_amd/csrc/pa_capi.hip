@@ -314,6 +314,41 @@ int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* ou
   return check_hip(e, "pa_blocksparse_prefill launch");
 }
 
+int pa_kv_write(const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                float* k_scale, float* v_scale,
+                const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+                int B, int T, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks,
+                int kv_dtype, void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || T < 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_kv_write: bad sizes");
+  if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_kv_write: bad paging sizes");
+  if (kv_dtype != PA_F32 && kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN)
+    return fail_arg("pa_kv_write: unknown kv_dtype %d", kv_dtype);
+  const int src_esz = kv_dtype == PA_F32 ? 4 : 2;
+  if ((D * src_esz) % 16 != 0 || (kv_dtype == PA_FP8_E4M3FN && D % 8 != 0))
+    return fail_arg("pa_kv_write: D=%d rows must be a multiple of 16 bytes", D);
+  if ((long)max_blocks_per_seq * block_size > 0x7fffffffL) return fail_arg("pa_kv_write: table capacity exceeds 2^31 tokens");
+  if (B == 0 || T == 0) return 0;
+  if (B > 65535 || Hkv > 65535) return fail_arg("pa_kv_write: B and Hkv are limited to 65535 (grid dimensions)");
+  if (!k_new || !v_new || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens)
+    return fail_arg("pa_kv_write: null pointer argument");
+  if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_kv_write: fp8 pools need k_scale and v_scale");
+  if (!aligned16(k_new) || !aligned16(v_new) || !aligned16(k_cache) || !aligned16(v_cache))
+    return fail_arg("pa_kv_write: k_new, v_new, k_cache and v_cache must be 16-byte aligned");
+  KvWriteParams p;
+  memset(&p, 0, sizeof(p));
+  p.k_new = k_new; p.v_new = v_new; p.k_cache = k_cache; p.v_cache = v_cache;
+  p.k_scale = k_scale; p.v_scale = v_scale;
+  p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens;
+  p.B = B; p.T = T; p.Hkv = Hkv; p.D = D; p.block_size = block_size; p.max_blocks = max_blocks_per_seq;
+  p.num_blocks = num_blocks; p.kv_dtype = kv_dtype;
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipError_t e = launch_kv_write(p, s);
+  profile_end(s);
+  return check_hip(e, "pa_kv_write launch");
+}
+
 int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,
                  void* out, int B, int Hkv, int D, int block_size,
                  int max_blocks_per_seq, int num_blocks, int max_seq_len,

@@ -123,6 +123,21 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
 bool prefill_async_supported(const PrefillParams& p);
 
 // ---- gather ------------------------------------------------------------------------
+// ---- paged KV write --------------------------------------------------------------
+struct KvWriteParams {
+  const void* k_new;        // [B, T, Hkv, D] bf16 (fp32 for an fp32 pool)
+  const void* v_new;
+  void* k_cache;            // [num_blocks, block_size, Hkv, D]
+  void* v_cache;
+  float* k_scale;           // [num_blocks, Hkv] (fp8 pools) or null
+  float* v_scale;
+  const int32_t* block_tables;
+  const int32_t* seq_lens;
+  const int32_t* query_lens;
+  int B, T, Hkv, D, block_size, max_blocks, num_blocks, kv_dtype;
+};
+hipError_t launch_kv_write(const KvWriteParams& p, hipStream_t s);
+
 // matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats
 hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s);
 hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,

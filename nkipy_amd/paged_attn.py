@@ -268,6 +268,57 @@ def gather_kv(cache, block_tables, seq_lens, max_seq_len=None):
     return out
 
 
+def kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens, *, k_scale=None, v_scale=None):
+    """Write the new tokens' K/V into the paged pool, in place, before the attention call.
+
+    The reference's `cache_k[:, query_pos] = xk` with query_pos = start_pos + arange(seq_len)
+    (examples/models/gpt_oss/kernels/attention.py:85,92-100): token t < query_lens[b] of sequence
+    b lands at position seq_lens[b] - query_lens[b] + t, i.e. in pool row
+    (block_tables[b, pos // block_size], pos % block_size).  k_new/v_new [B, T, Hkv, D] are
+    bfloat16 (float32 for a float32 pool).  float8_e4m3fn pools are quantised on the way in and
+    k_scale/v_scale [num_blocks, Hkv] float32 are maintained (running absmax / 448 per block and
+    kv head; earlier rows of a block are re-encoded when its scale grows).  Returns None: the
+    pool tensors are the outputs, aliased to the inputs as the reference's cache tensors are
+    (examples/models/qwen3/qwen3.py:289-301).
+    """
+    lib = _lib.load()
+    for n, t in (("k_new", k_new), ("v_new", v_new), ("k_cache", k_cache), ("v_cache", v_cache),
+                 ("block_tables", block_tables), ("seq_lens", seq_lens), ("query_lens", query_lens)):
+        _need_device(n, t)
+    _check(k_new.dim() == 4, "k_new must be [B, T, Hkv, D]")
+    _check(v_new.shape == k_new.shape and v_new.dtype == k_new.dtype, "v_new must match k_new")
+    _check(k_cache.dim() == 4, "k_cache must be [num_blocks, block_size, Hkv, D]")
+    _check(v_cache.shape == k_cache.shape and v_cache.dtype == k_cache.dtype, "v_cache must match k_cache")
+    _check(k_cache.dtype in _DTYPE_CODE, f"unsupported pool dtype {k_cache.dtype}")
+    B, T, Hkv, D = k_new.shape
+    num_blocks, block_size = k_cache.shape[:2]
+    _check(tuple(k_cache.shape[2:]) == (Hkv, D), f"pool rows are {tuple(k_cache.shape[2:])}, new rows {(Hkv, D)}")
+    kv_dtype = _DTYPE_CODE[k_cache.dtype]
+    want = torch.float32 if kv_dtype == F32 else torch.bfloat16
+    _check(k_new.dtype == want, f"k_new must be {want} for a {k_cache.dtype} pool, got {k_new.dtype}")
+    _check(block_tables.dim() == 2 and block_tables.shape[0] == B and block_tables.dtype == torch.int32,
+           "block_tables must be int32 [B, max_blocks]")
+    _check(seq_lens.shape == (B,) and seq_lens.dtype == torch.int32, "seq_lens must be int32 [B]")
+    _check(query_lens.shape == (B,) and query_lens.dtype == torch.int32, "query_lens must be int32 [B]")
+    if kv_dtype == FP8:
+        _check(k_scale is not None and v_scale is not None, "float8 pools need k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _need_device(n, t)
+            _check(t.dtype == torch.float32 and tuple(t.shape) == (num_blocks, Hkv), f"{n} must be float32 [num_blocks, Hkv]")
+    else:
+        _check(k_scale is None and v_scale is None, "k_scale / v_scale are for float8 pools only")
+    _same_device(k_new, v_new=v_new, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables,
+                 seq_lens=seq_lens, query_lens=query_lens, k_scale=k_scale, v_scale=v_scale)
+    with torch.cuda.device(k_new.device):
+        rc = lib.pa_kv_write(_ptr(k_new), _ptr(v_new), _ptr(k_cache), _ptr(v_cache),
+                             _ptr(k_scale) if k_scale is not None else None,
+                             _ptr(v_scale) if v_scale is not None else None,
+                             _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens),
+                             B, T, Hkv, D, block_size, block_tables.shape[1], num_blocks, kv_dtype,
+                             _stream_ptr(k_new.device))
+    _raise_on(rc, "pa_kv_write")
+
+
 def default_scale(head_dim: int) -> float:
     """1 / sqrt(head_dim) in float32, as examples/models/qwen3/kernels/attention.py:119."""
     return float(np.float32(1.0) / np.float32(math.sqrt(head_dim)))

@@ -99,6 +99,33 @@ class BlocksparseWorkload:
         return 4 * d * B * pairs
 
 
+@dataclass
+class KvWriteWorkload:
+    name: str
+    k_new: torch.Tensor
+    v_new: torch.Tensor
+    k_cache: torch.Tensor
+    v_cache: torch.Tensor
+    k_scale: Optional[torch.Tensor]
+    v_scale: Optional[torch.Tensor]
+    block_tables: torch.Tensor
+    seq_lens: torch.Tensor
+    query_lens: torch.Tensor
+    prefix: np.ndarray = field(default=None, repr=False)
+
+    def algorithmic_bytes(self) -> int:
+        """Every new K and V row read once and stored once in the pool's element size, one scale per
+        touched (block, kv head) and tensor, the used table entries and the two length vectors."""
+        B, T, hkv, d = self.k_new.shape
+        bs = self.k_cache.shape[1]
+        tq = self.query_lens.cpu().numpy().astype(np.int64)
+        seq = self.seq_lens.cpu().numpy().astype(np.int64)
+        rows = int(tq.sum())
+        touched = int(((seq - 1) // bs - (seq - tq) // bs + 1)[tq > 0].sum())
+        scales = 2 * touched * hkv * 4 if self.k_scale is not None else 0
+        return 2 * rows * hkv * d * (self.k_new.element_size() + self.k_cache.element_size()) + scales + 4 * touched + 8 * B
+
+
 def _randn(shape, dtype, gen, device, chunk=1 << 27):
     """N(0,1) drawn in float32 and rounded to `dtype`, in bounded chunks."""
     out = torch.empty(shape, dtype=dtype, device=device)
@@ -231,3 +258,35 @@ def make_blocksparse(device="cuda", shrink: int = 1) -> BlocksparseWorkload:
     return BlocksparseWorkload(name="C4" + (f"/shrink{shrink}" if shrink > 1 else ""), q=q, k=k, v=v,
                                scale=float(np.float32(1.0) / np.float32(math.sqrt(D))),
                                block=64, local_blocks=4, vert_stride=8)
+
+
+def make_kv_write(device="cuda", shrink: int = 1, fp8: bool = True) -> KvWriteWorkload:
+    """config 6 (the step in front of config 3's attention): the 2048 new tokens of each of 8
+    sequences are written behind prefixes U[0,4096] into a block-64 pool, 8 kv heads, D=128;
+    fp8-e4m3 pool with per-(block, kv head) scales by default (bf16 new rows quantised on the
+    way in), or a bf16 pool (plain scatter)."""
+    rng = np.random.default_rng(1006)
+    gen = _gen(1006, device)
+    B, Hkv, D, bs = 8, 8, 128, 64
+    T = max(2048 // shrink, 1)
+    prefix = rng.integers(0, 4096 // shrink + 1, size=B).astype(np.int64)
+    seq = prefix + T
+    nblk = (seq + bs - 1) // bs
+    pool_blocks = int(math.ceil(1.1 * int(nblk.sum())))
+    tables = _tables(rng, nblk, pool_blocks)
+    k_new = _randn((B, T, Hkv, D), torch.bfloat16, gen, device)
+    v_new = _randn((B, T, Hkv, D), torch.bfloat16, gen, device)
+    if fp8:
+        # earlier context already in the pool (the blocks the chunk starts inside carry a scale)
+        k_cache, k_scale = quantize_pool_fp8(_randn((pool_blocks, bs, Hkv, D), torch.bfloat16, gen, device))
+        v_cache, v_scale = quantize_pool_fp8(_randn((pool_blocks, bs, Hkv, D), torch.bfloat16, gen, device))
+    else:
+        k_cache = _randn((pool_blocks, bs, Hkv, D), torch.bfloat16, gen, device)
+        v_cache = _randn((pool_blocks, bs, Hkv, D), torch.bfloat16, gen, device)
+        k_scale = v_scale = None
+    return KvWriteWorkload(
+        name="C6" + ("" if fp8 else "/bf16") + (f"/shrink{shrink}" if shrink > 1 else ""),
+        k_new=k_new, v_new=v_new, k_cache=k_cache, v_cache=v_cache, k_scale=k_scale, v_scale=v_scale,
+        block_tables=torch.from_numpy(tables).to(device),
+        seq_lens=torch.from_numpy(seq.astype(np.int32)).to(device),
+        query_lens=torch.full((B,), T, dtype=torch.int32, device=device), prefix=prefix)

@@ -21,6 +21,9 @@ in the one-dynamic-index `np.take` form the reference's tracer supports:
                         examples/models/qwen3/kernels/attention.py:100-106
 * gather primitive      nkipy/src/nkipy/core/tensor.py:575-640 (np.take, one
                         dynamic index per expression)
+* cache update          examples/models/gpt_oss/kernels/attention.py:92-100
+                        (`cache_k[:, query_pos] = xk`, query_pos = start_pos +
+                        arange(seq_len)), examples/models/qwen3/kernels/attention.py:100-106
 
 Dtype policy: inputs are values already rounded to their storage type (bf16 /
 fp8-e4m3fn with a per-(block, kv-head) scale / fp32); every product and sum is
@@ -43,6 +46,13 @@ paged_decode/prefill   identity table over a reshaped dense cache == dense
 merge_partitions       split-K merge == single pass in float64 for any split
 blocksparse_prefill    == dense attention under the expanded boolean mask;
                        all-active pattern == dense causal
+kv_write               bf16/fp32 pools: identity table == the reference's dense
+                       `cache[:, query_pos] = x`; untouched pool bytes keep their
+                       bits.  fp8 pools (no reference counterpart): a whole fresh
+                       block == quantize_kv_fp8 of that block; scales never
+                       shrink; codes of earlier tokens keep their bits when the
+                       scale stays; token-by-token append dequantises within the
+                       e4m3 rounding bound of the final scale
 No reference test or fixture exists for the paged / split-K / blocksparse /
 fp8-KV forms, so against the reference itself their parity is unpinned; they
 are pinned by the mathematics above.
@@ -210,6 +220,67 @@ def gather_kv(pool, table_row, seq_len: int, block_scale=None) -> np.ndarray:
 # ---------------------------------------------------------------------------
 # dense attention core (the reference's math on one sequence)
 # ---------------------------------------------------------------------------
+
+
+def kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens, *,
+             k_scale=None, v_scale=None) -> None:
+    """Write the new tokens' K/V into the paged pool, in place, before attention.
+
+    The reference updates a dense cache with `cache_k[:, query_pos] = xk`,
+    query_pos = start_pos + arange(seq_len) (gpt_oss/kernels/attention.py:85,92-100;
+    qwen3/kernels/attention.py:100-106).  Paged form: token t < query_lens[b] of
+    sequence b sits at position pos = seq_lens[b] - query_lens[b] + t and goes to
+    pool row (block_tables[b, pos // bs], pos % bs).
+
+    k_new/v_new [B, T, Hkv, D]: uint16 bf16 bit patterns or float32 values.
+    k/v_cache [num_blocks, bs, Hkv, D]: uint16 / float32 pools receive the rows bit
+    for bit.  uint8 pools hold e4m3fn codes with k_scale/v_scale [num_blocks, Hkv]
+    float32, maintained per (block, kv head) -- this part has no counterpart in the
+    reference:
+      s_old = scale of the block if it already holds earlier tokens of the sequence
+              (pos of the first written token is not the block's first row), else 0
+      s_new = max(s_old, absmax(new rows of the block) / 448)   (1.0 if that is 0)
+      earlier rows are re-encoded as encode(decode(code) * s_old / s_new) when the
+      scale grew; new rows are encode(x / s_new).  All arithmetic float32.
+    """
+    kn, vn = np.asarray(k_new), np.asarray(v_new)
+    B, T = kn.shape[:2]
+    bs = k_cache.shape[1]
+    fp8 = k_cache.dtype == np.uint8
+    if fp8 and (k_scale is None or v_scale is None):
+        raise ValueError("fp8 pools need k_scale and v_scale")
+    for b in range(B):
+        seq, tq = int(seq_lens[b]), int(query_lens[b])
+        tq = min(max(tq, 0), T)
+        if tq == 0:
+            continue
+        start = seq - tq
+        if start < 0:
+            raise ValueError("seq_lens must count the new tokens")
+        for jb in range(start // bs, (seq - 1) // bs + 1):
+            blk = int(block_tables[b, jb])
+            if not 0 <= blk < k_cache.shape[0]:
+                raise IndexError(f"block table entry {blk} out of range")
+            lo = max(start, jb * bs) - jb * bs
+            hi = min(seq, (jb + 1) * bs) - jb * bs
+            t0 = jb * bs + lo - start
+            for new, cache, scale in ((kn, k_cache, k_scale), (vn, v_cache, v_scale)):
+                rows = new[b, t0:t0 + (hi - lo)]                      # [n, Hkv, D]
+                if not fp8:
+                    cache[blk, lo:hi] = rows if cache.dtype == rows.dtype else to_f32(rows).astype(cache.dtype)
+                    continue
+                x = to_f32(rows)
+                amax = np.max(np.abs(x), axis=(0, 2)).astype(np.float32)          # [Hkv]
+                s_old = scale[blk].astype(np.float32) if lo > 0 else np.zeros_like(amax)
+                s_new = np.maximum(s_old, (amax / np.float32(FP8_E4M3_MAX)).astype(np.float32))
+                s_new = np.where(s_new == 0, np.float32(1.0), s_new).astype(np.float32)
+                if lo > 0:
+                    grew = s_new != s_old
+                    old = (fp8_e4m3fn_decode(cache[blk, :lo]) * s_old[None, :, None]).astype(np.float32)
+                    recoded = fp8_e4m3fn_encode((old / s_new[None, :, None]).astype(np.float32))
+                    cache[blk, :lo] = np.where(grew[None, :, None], recoded, cache[blk, :lo])
+                cache[blk, lo:hi] = fp8_e4m3fn_encode((x / s_new[None, :, None]).astype(np.float32))
+                scale[blk] = s_new
 
 
 def repeat_kv(x, n_rep: int) -> np.ndarray:

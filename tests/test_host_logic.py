@@ -59,6 +59,15 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert b"block must be 64" in lib.pa_last_error()
     assert lib.pa_prefill(z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 0, z) == -1
     assert lib.pa_gather_kv(z, z, z, z, 1, 2, 64, 16, 2, 8, 100, 2, z) == -1  # beyond table capacity
+    def kvw(**kw):
+        a = dict(B=2, T=4, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1)
+        a.update(kw)
+        return lib.pa_kv_write(z, z, z, z, z, z, z, z, z, a["B"], a["T"], a["Hkv"], a["D"], a["bs"], a["mb"], a["nb"], a["kd"], z)
+    assert kvw(kd=3) == -1 and b"kv_dtype" in lib.pa_last_error()
+    assert kvw(D=100) == -1 and b"16 bytes" in lib.pa_last_error()
+    assert kvw(bs=0) == -1
+    assert kvw() == -1 and b"null" in lib.pa_last_error()
+    assert kvw(T=0) == 0
 
 
 def test_ops_refuse_host_arrays():
