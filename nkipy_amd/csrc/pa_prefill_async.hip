@@ -47,10 +47,6 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) char lds_char;
 
-__device__ __forceinline__ bool block_active(int i, int j, int head_phase, int local, int stride) {
-  return j <= i && ((i - j) < local || ((j + head_phase) % stride) == 0);
-}
-
 __device__ __forceinline__ bf16x8_t make_frag(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   u32x4_t v = {a, b, c, d};
   return __builtin_bit_cast(bf16x8_t, v);
@@ -249,36 +245,55 @@ void prefill_async_kernel(PrefillParams p) {
   const int head_phase = SPARSE ? hq % p.sparse_stride : 0;
   const int qblk = wq_lo / 64;                    // sparse: q block of this wave
   const int wg_blk_lo = q0 / 64;
-  auto next_tile = [&](int kt) __attribute__((always_inline)) -> int {      // first needed tile >= kt
-    if (!SPARSE) return kt;
-    while (kt < ntiles) {
-      // needed by some q block of the workgroup: vertical-stride column, or inside a local window
-      const int kb = kt / (64 / BN);   // sparsity block of this key tile
-      if (((kb + head_phase) % p.sparse_stride) == 0 || kb > wg_blk_lo - p.sparse_local) break;
-      ++kt;
+  // Walk over the key tiles the workgroup needs.  Dense: every tile.  Sparse: a tile (= one
+  // 64-key sparsity block) is needed if it is a vertical-stride column, (kt + head_phase) %
+  // stride == 0, or lies in the local window of some q block of the workgroup, kt >=
+  // first_local.  The phase is carried along, so a step costs a few scalar instructions and no
+  // integer division however many tiles it skips.
+  struct Walk { int kt, ph; };
+  const int first_local = wg_blk_lo - p.sparse_local + 1;
+  auto walk_settle = [&](Walk& w) __attribute__((always_inline)) {      // to the first needed tile >= w.kt
+    if (!SPARSE) return;
+    if (w.kt >= first_local || w.ph == 0) return;
+    const int jump = p.sparse_stride - w.ph;                             // to the next vertical column
+    if (w.kt + jump >= first_local) {
+      w.ph += first_local - w.kt;
+      if (w.ph == p.sparse_stride) w.ph = 0;
+      w.kt = first_local;
+    } else {
+      w.kt += jump;
+      w.ph = 0;
     }
-    return kt;
+  };
+  auto walk_step = [&](Walk& w) __attribute__((always_inline)) {
+    ++w.kt;
+    if (SPARSE) {
+      if (++w.ph == p.sparse_stride) w.ph = 0;
+      walk_settle(w);
+    }
   };
 
-  // ---- the three steps of one key tile ----------------------------------------------
-  auto tile_active = [&](int kt) __attribute__((always_inline)) -> bool {
-    bool act = wave_has_rows && kt * BN <= prefix + wq_hi;
-    if (SPARSE) act = act && block_active(qblk, kt / (64 / BN), head_phase, p.sparse_local, p.sparse_stride);
+  // does this wave compute on tile w.kt?
+  auto tile_active = [&](const Walk& w) __attribute__((always_inline)) -> bool {
+    bool act = wave_has_rows && w.kt * BN <= prefix + wq_hi;
+    if (SPARSE) act = act && w.kt <= qblk && (qblk - w.kt < p.sparse_local || w.ph == 0);
     return act;
   };
   // ---- ring of NST stages: tiles are requested NST-1 ahead; requests past the end are
   // repeated on the first tile so that the wait counter stays exact ------------------------
-  const int kt_first = next_tile(0);
-  int kt_i = kt_first;                // next tile to request
+  Walk w_first = {0, head_phase};
+  walk_settle(w_first);
+  const int kt_first = w_first.kt;
+  Walk w_i = w_first;                 // next tile to request
   int stage_i = 0;                    // ... and the stage it goes to
   // The entries for the following request are fetched in the middle of a tile's work, after
   // its last wait on K fragments and before the softmax, where no LDS read is pending: a
   // scalar load in flight turns every LDS wait into a wait for everything.
-  auto prefetch_next = [&]() __attribute__((always_inline)) { prefetch_table(kt_i < ntiles ? kt_i : kt_first); };
+  auto prefetch_next = [&]() __attribute__((always_inline)) { prefetch_table(w_i.kt < ntiles ? w_i.kt : kt_first); };
   prefetch_table(kt_first);
   auto request_next = [&]() __attribute__((always_inline)) {
-    issue_tile(kt_i < ntiles ? kt_i : kt_first, stage_i);
-    if (kt_i < ntiles) kt_i = next_tile(kt_i + 1);
+    issue_tile(w_i.kt < ntiles ? w_i.kt : kt_first, stage_i);
+    if (w_i.kt < ntiles) walk_step(w_i);
     stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
   };
 
@@ -425,23 +440,24 @@ void prefill_async_kernel(PrefillParams p) {
   }
 
   {
-    int kt_c = kt_first, stage_c = 0;
-    while (kt_c < ntiles) {
-      wait_vmcnt<(NST - 2) * UPW>();               // this wave's part of tile kt_c has landed
+    Walk w_c = w_first;
+    int stage_c = 0;
+    while (w_c.kt < ntiles) {
+      wait_vmcnt<(NST - 2) * UPW>();               // this wave's part of the current tile has landed
       __builtin_amdgcn_s_barrier();                // ... and everyone's; all waves are done with the previous tile
       request_next();
-      if (tile_active(kt_c)) {
+      if (tile_active(w_c)) {
         f32x16_t sacc[TT];
         uint32_t pw[TT][8];
         bf16x8_t v0[HD / 32];
         scores(sacc, stage_c, v0, stage_c);
         prefetch_next();
-        softmax(sacc, pw, kt_c);
+        softmax(sacc, pw, w_c.kt);
         accumulate(pw, stage_c, v0);
       } else {
         prefetch_next();
       }
-      kt_c = next_tile(kt_c + 1);
+      walk_step(w_c);
       stage_c = stage_c + 1 == NST ? 0 : stage_c + 1;
     }
   }
