@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the paged attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|5|3|4|6]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|5|3|4|6|7]
 
 A step is one pass of the op over one batch of synthetic input that is already
 resident in HBM.  Default workload: config 2 (Llama-3-8B-shape paged decode, bf16,
@@ -310,12 +310,51 @@ def bench_kv_write(steps, warmup, lib, pa, W):
     return res
 
 
+def bench_pre_attention(steps, warmup, lib, pa, W):
+    """QK RMSNorm + RoPE on q and k fused with the fp8 KV write (config 6's write plus the q tensor)."""
+    w = W.make_kv_write()
+    B, T, Hkv, D = w.k_new.shape
+    Hq = 4 * Hkv
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1007)
+    xq = torch.randn((B, T, Hq, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    wq = (1.0 + 0.1 * torch.randn(D, generator=gen, device="cuda")).to(torch.bfloat16)
+    wk = (1.0 + 0.1 * torch.randn(D, generator=gen, device="cuda")).to(torch.bfloat16)
+    max_pos = int(w.seq_lens.max().item())
+    cos, sin = pa.rope_tables(D, max_pos, 1000000.0)
+    q_out = torch.empty_like(xq)
+
+    def step():
+        pa.qk_norm_rope_kv_write(xq, w.k_new, w.v_new, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens,
+                                 cos, sin, q_norm_weight=wq, k_norm_weight=wk, eps=1e-6,
+                                 k_scale=w.k_scale, v_scale=w.v_scale, out=q_out)
+
+    sec = _time_steps(step, steps, warmup)
+    ab = w.algorithmic_bytes() + 2 * xq.numel() * 2 + 2 * cos.numel() * 2
+    res = {
+        "metric": "fused QK-norm + RoPE + paged KV write HBM GB/s (% peak)",
+        "value": round(ab / sec / 1e9, 2), "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * ab / sec / 1e9 / HBM_PEAK_GBS, 2),
+        "tok_per_s": round(B * T / sec, 1),
+        "ms_per_step": round(sec * 1e3, 5), "dtype": "bf16 rows, float32 norm, bf16 rotation -> fp8-e4m3 pool",
+        "config": {"workload": f"C7 pre-attention: B={B}, T={T} new tokens, Hq={Hq}, Hkv={Hkv}, D={D}, "
+                               f"block_size={w.k_cache.shape[1]}, prefix={w.prefix.tolist()}",
+                   "algorithmic_bytes": ab},
+        "roofline": {"bound": "hbm", "achieved": round(ab / sec / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "q_norm_rope_kernel + kv_write_kernel (two launches, step time)",
+                     "kernel_avg_ms": round(sec * 1e3, 5), "launches_timed": steps},
+        "cpu_baseline": None,
+    }
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -340,6 +379,8 @@ def main():
         res = bench_prefill(args.steps, args.warmup, lib, pa, W)
     elif args.config == 6:
         res = bench_kv_write(args.steps, args.warmup, lib, pa, W)
+    elif args.config == 7:
+        res = bench_pre_attention(args.steps, args.warmup, lib, pa, W)
     else:
         res = bench_blocksparse(args.steps, args.warmup, lib, pa, W)
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"),

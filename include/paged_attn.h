@@ -145,6 +145,27 @@ int pa_kv_write(const void* k_new, const void* v_new, void* k_cache, void* v_cac
                 int B, int T, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks,
                 int kv_dtype, void* stream);
 
+/* The reference's pre-attention step fused with the KV write: QK RMSNorm
+ * (examples/models/qwen3/kernels/rmsnorm.py:4-21, applied at qwen3/kernels/attention.py:78-80),
+ * RoPE at the tokens' absolute positions start_pos + t, start_pos = seq_lens[b] -
+ * query_lens[b] (rope.py:23-48; attention.py:83-97; gpt_oss/kernels/attention.py:85-90), then
+ * pa_kv_write of the rotated K and of V.  Two launches: Q rows, then the K/V scatter.
+ *   xq [B, T, Hq, D], xk, xv [B, T, Hkv, D]  bf16; q_out [B, T, Hq, D] bf16 (may be xq); rows
+ *                 t >= query_lens[b] of q_out are zero
+ *   q_norm_weight, k_norm_weight [D] bf16, or NULL for no norm on that tensor
+ *   rope_cos, rope_sin [rope_max_pos, D/2] bf16 (rope.py:4-20 cast to bf16); positions past the
+ *                 table are clamped to its last row
+ * Arithmetic as the reference's bf16 tensors give it: the norm in float32 rounded once to bf16,
+ * every product and sum of the rotation rounded to bf16.  D in {64, 128, 256};
+ * kv_dtype PA_BF16 or PA_FP8_E4M3FN (then scales as in pa_kv_write). */
+int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, void* q_out,
+                             const void* q_norm_weight, const void* k_norm_weight, float norm_eps,
+                             const void* rope_cos, const void* rope_sin, int rope_max_pos,
+                             void* k_cache, void* v_cache, float* k_scale, float* v_scale,
+                             const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+                             int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq,
+                             int num_blocks, int kv_dtype, void* stream);
+
 /* Debug switches (process-wide; tests only).  key 0: decode kernel choice
  * (0 = automatic, 1 = scalar-ALU kernel, 2 = MFMA kernel with fixed partitions,
  * 3 = MFMA kernel with the balanced schedule); key 1: waves per workgroup of the

@@ -349,6 +349,46 @@ int pa_kv_write(const void* k_new, const void* v_new, void* k_cache, void* v_cac
   return check_hip(e, "pa_kv_write launch");
 }
 
+int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, void* q_out,
+                             const void* q_norm_weight, const void* k_norm_weight, float norm_eps,
+                             const void* rope_cos, const void* rope_sin, int rope_max_pos,
+                             void* k_cache, void* v_cache, float* k_scale, float* v_scale,
+                             const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+                             int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq,
+                             int num_blocks, int kv_dtype, void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_qk_norm_rope_kv_write: bad sizes");
+  if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0 || rope_max_pos <= 0)
+    return fail_arg("pa_qk_norm_rope_kv_write: bad paging or table sizes");
+  if (kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN)
+    return fail_arg("pa_qk_norm_rope_kv_write: kv_dtype must be bf16 or fp8-e4m3fn (got %d)", kv_dtype);
+  if (!kv_write_xform_supported(D)) return fail_arg("pa_qk_norm_rope_kv_write: head_dim %d must be 64, 128 or 256", D);
+  if ((long)max_blocks_per_seq * block_size > 0x7fffffffL) return fail_arg("pa_qk_norm_rope_kv_write: table capacity exceeds 2^31 tokens");
+  if (B == 0 || T == 0) return 0;
+  if (B > 65535 || Hkv > 65535) return fail_arg("pa_qk_norm_rope_kv_write: B and Hkv are limited to 65535 (grid dimensions)");
+  if (!xq || !xk || !xv || !q_out || !rope_cos || !rope_sin || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens)
+    return fail_arg("pa_qk_norm_rope_kv_write: null pointer argument");
+  if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_qk_norm_rope_kv_write: fp8 pools need k_scale and v_scale");
+  if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache))
+    return fail_arg("pa_qk_norm_rope_kv_write: xq, xk, xv, q_out, k_cache and v_cache must be 16-byte aligned");
+  KvWriteParams p;
+  memset(&p, 0, sizeof(p));
+  p.k_new = xk; p.v_new = xv; p.k_cache = k_cache; p.v_cache = v_cache;
+  p.k_scale = k_scale; p.v_scale = v_scale;
+  p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens;
+  p.B = B; p.T = T; p.Hkv = Hkv; p.D = D; p.block_size = block_size; p.max_blocks = max_blocks_per_seq;
+  p.num_blocks = num_blocks; p.kv_dtype = kv_dtype;
+  p.q_in = xq; p.q_out = q_out; p.Hq = Hq;
+  p.q_norm_weight = (const uint16_t*)q_norm_weight; p.k_norm_weight = (const uint16_t*)k_norm_weight;
+  p.rope_cos = (const uint16_t*)rope_cos; p.rope_sin = (const uint16_t*)rope_sin;
+  p.norm_eps = norm_eps; p.rope_max_pos = rope_max_pos;
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipError_t e = launch_kv_write(p, s);
+  profile_end(s);
+  return check_hip(e, "pa_qk_norm_rope_kv_write launch");
+}
+
 int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,
                  void* out, int B, int Hkv, int D, int block_size,
                  int max_blocks_per_seq, int num_blocks, int max_seq_len,

@@ -135,8 +135,19 @@ struct KvWriteParams {
   const int32_t* seq_lens;
   const int32_t* query_lens;
   int B, T, Hkv, D, block_size, max_blocks, num_blocks, kv_dtype;
+  // pre-attention transform (all null / zero for a plain write): RMSNorm weights [D] bf16 (null: no
+  // norm), RoPE tables [rope_max_pos, D/2] bf16, Q rows [B, T, Hq, D] bf16 transformed into q_out
+  const void* q_in;
+  void* q_out;
+  const uint16_t* q_norm_weight;
+  const uint16_t* k_norm_weight;
+  const uint16_t* rope_cos;
+  const uint16_t* rope_sin;
+  float norm_eps;
+  int Hq, rope_max_pos;
 };
 hipError_t launch_kv_write(const KvWriteParams& p, hipStream_t s);
+bool kv_write_xform_supported(int D);   // head dims the fused RMSNorm + RoPE write is built for
 
 // matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats
 hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s);

@@ -319,6 +319,81 @@ def kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens,
     _raise_on(rc, "pa_kv_write")
 
 
+def rope_tables(head_dim: int, max_seq_len: int, base: float = 10000.0, device="cuda"):
+    """cos / sin tables [max_seq_len, head_dim // 2] in bfloat16 on `device`, computed as
+    examples/models/qwen3/kernels/rope.py:4-20 does (float64 frequencies, float32 angles and
+    cos / sin, cast to bf16 at the call site attention.py:84-86)."""
+    freqs = 1.0 / (base ** (np.arange(0, head_dim, 2)[: (head_dim // 2)] / head_dim))
+    ang = np.outer(np.arange(max_seq_len, dtype=np.float32), freqs)
+    cos, sin = np.cos(ang, dtype=np.float32), np.sin(ang, dtype=np.float32)
+    return (torch.from_numpy(cos).to(device).to(torch.bfloat16), torch.from_numpy(sin).to(device).to(torch.bfloat16))
+
+
+def qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, rope_cos, rope_sin, *,
+                          q_norm_weight=None, k_norm_weight=None, eps=1e-6, k_scale=None, v_scale=None, out=None):
+    """The reference's pre-attention step fused with the paged KV write.
+
+    QK RMSNorm (examples/models/qwen3/kernels/rmsnorm.py:4-21; skipped for a tensor whose weight
+    is None), RoPE at absolute positions seq_lens[b] - query_lens[b] + t (rope.py:23-48;
+    qwen3/kernels/attention.py:78-97), then `kv_write` of the rotated K and of V.  xq [B, T, Hq, D],
+    xk / xv [B, T, Hkv, D] bfloat16; rope_cos / rope_sin [max_pos, D/2] bfloat16 (`rope_tables`).
+    Returns the transformed q (`out`, which may be xq itself; padding rows are zero); the pool
+    (and its scales for float8) is updated in place.
+    """
+    lib = _lib.load()
+    for n, t in (("xq", xq), ("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
+                 ("block_tables", block_tables), ("seq_lens", seq_lens), ("query_lens", query_lens),
+                 ("rope_cos", rope_cos), ("rope_sin", rope_sin)):
+        _need_device(n, t)
+    _check(xq.dim() == 4 and xq.dtype == torch.bfloat16, "xq must be bfloat16 [B, T, Hq, D]")
+    B, T, Hq, D = xq.shape
+    _check(xk.dim() == 4 and xk.dtype == torch.bfloat16 and xk.shape[:2] == (B, T) and xk.shape[3] == D,
+           "xk must be bfloat16 [B, T, Hkv, D]")
+    Hkv = xk.shape[2]
+    _check(xv.shape == xk.shape and xv.dtype == torch.bfloat16, "xv must match xk")
+    _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    _check(D in (64, 128, 256), f"head_dim {D} must be 64, 128 or 256")
+    _check(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (Hkv, D), "k_cache must be [num_blocks, block_size, Hkv, D]")
+    _check(v_cache.shape == k_cache.shape and v_cache.dtype == k_cache.dtype, "v_cache must match k_cache")
+    _check(k_cache.dtype in (torch.bfloat16, torch.float8_e4m3fn), f"unsupported pool dtype {k_cache.dtype}")
+    num_blocks, block_size = k_cache.shape[:2]
+    kv_dtype = _DTYPE_CODE[k_cache.dtype]
+    for n, t in (("rope_cos", rope_cos), ("rope_sin", rope_sin)):
+        _check(t.dim() == 2 and t.shape[1] == D // 2 and t.dtype == torch.bfloat16, f"{n} must be bfloat16 [max_pos, D/2]")
+    _check(rope_sin.shape == rope_cos.shape, "rope_sin must match rope_cos")
+    for n, t in (("q_norm_weight", q_norm_weight), ("k_norm_weight", k_norm_weight)):
+        if t is not None:
+            _need_device(n, t)
+            _check(tuple(t.shape) == (D,) and t.dtype == torch.bfloat16, f"{n} must be bfloat16 [D]")
+    _check(block_tables.dim() == 2 and block_tables.shape[0] == B and block_tables.dtype == torch.int32,
+           "block_tables must be int32 [B, max_blocks]")
+    _check(seq_lens.shape == (B,) and seq_lens.dtype == torch.int32, "seq_lens must be int32 [B]")
+    _check(query_lens.shape == (B,) and query_lens.dtype == torch.int32, "query_lens must be int32 [B]")
+    if kv_dtype == FP8:
+        _check(k_scale is not None and v_scale is not None, "float8 pools need k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _need_device(n, t)
+            _check(t.dtype == torch.float32 and tuple(t.shape) == (num_blocks, Hkv), f"{n} must be float32 [num_blocks, Hkv]")
+    else:
+        _check(k_scale is None and v_scale is None, "k_scale / v_scale are for float8 pools only")
+    if out is None:
+        out = torch.empty_like(xq)
+    else:
+        _need_device("out", out)
+        _check(out.shape == xq.shape and out.dtype == xq.dtype, "out must match xq")
+    _same_device(xq, xk=xk, xv=xv, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
+                 query_lens=query_lens, rope_cos=rope_cos, rope_sin=rope_sin, q_norm_weight=q_norm_weight,
+                 k_norm_weight=k_norm_weight, k_scale=k_scale, v_scale=v_scale, out=out)
+    with torch.cuda.device(xq.device):
+        rc = lib.pa_qk_norm_rope_kv_write(
+            _ptr(xq), _ptr(xk), _ptr(xv), _ptr(out), _ptr(q_norm_weight), _ptr(k_norm_weight), ctypes.c_float(eps),
+            _ptr(rope_cos), _ptr(rope_sin), rope_cos.shape[0], _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+            _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), B, T, Hq, Hkv, D, block_size, block_tables.shape[1],
+            num_blocks, kv_dtype, _stream_ptr(xq.device))
+    _raise_on(rc, "pa_qk_norm_rope_kv_write")
+    return out
+
+
 def default_scale(head_dim: int) -> float:
     """1 / sqrt(head_dim) in float32, as examples/models/qwen3/kernels/attention.py:119."""
     return float(np.float32(1.0) / np.float32(math.sqrt(head_dim)))

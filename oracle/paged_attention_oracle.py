@@ -21,6 +21,9 @@ in the one-dynamic-index `np.take` form the reference's tracer supports:
                         examples/models/qwen3/kernels/attention.py:100-106
 * gather primitive      nkipy/src/nkipy/core/tensor.py:575-640 (np.take, one
                         dynamic index per expression)
+* QK RMSNorm + RoPE     examples/models/qwen3/kernels/rmsnorm.py:4-21, rope.py:4-48 and
+                        their call sites attention.py:78-97 (bf16 tensors: every
+                        RoPE product and sum is rounded to bf16, the norm is float32)
 * cache update          examples/models/gpt_oss/kernels/attention.py:92-100
                         (`cache_k[:, query_pos] = xk`, query_pos = start_pos +
                         arange(seq_len)), examples/models/qwen3/kernels/attention.py:100-106
@@ -46,6 +49,9 @@ paged_decode/prefill   identity table over a reshaped dense cache == dense
 merge_partitions       split-K merge == single pass in float64 for any split
 blocksparse_prefill    == dense attention under the expanded boolean mask;
                        all-active pattern == dense causal
+rope_tables / rmsnorm / apply_rope   closed forms (position 0 is the identity,
+                       rotation preserves the pair norm, angle addition), float64
+                       restatement, torch.nn.functional.rms_norm on CPU
 kv_write               bf16/fp32 pools: identity table == the reference's dense
                        `cache[:, query_pos] = x`; untouched pool bytes keep their
                        bits.  fp8 pools (no reference counterpart): a whole fresh
@@ -220,6 +226,69 @@ def gather_kv(pool, table_row, seq_len: int, block_scale=None) -> np.ndarray:
 # ---------------------------------------------------------------------------
 # dense attention core (the reference's math on one sequence)
 # ---------------------------------------------------------------------------
+
+
+def rope_tables(head_dim: int, max_seq_len: int, base: float = 10000.0):
+    """cos / sin tables [max_seq_len, head_dim // 2] as bf16-rounded float32 values.
+
+    examples/models/qwen3/kernels/rope.py:4-20: freqs = 1 / base ** (arange(0, D, 2) / D)
+    (float64), t = arange(max_seq_len) float32, outer product, cos / sin evaluated in float32,
+    then cast to the tensor dtype (bf16 at the call site, attention.py:84-86).
+    """
+    freqs = 1.0 / (base ** (np.arange(0, head_dim, 2)[: (head_dim // 2)] / head_dim))
+    t = np.arange(max_seq_len, dtype=np.float32)
+    ang = np.outer(t, freqs)
+    return round_to_bf16(np.cos(ang, dtype=np.float32)), round_to_bf16(np.sin(ang, dtype=np.float32))
+
+
+def rmsnorm(x, weight, eps: float) -> np.ndarray:
+    """examples/models/qwen3/kernels/rmsnorm.py:4-21 on bf16 storage: float32 compute,
+    x / sqrt(mean(x^2) + eps) * weight, result rounded to bf16 (returned as float32)."""
+    x = to_f32(x)
+    w = to_f32(weight)
+    z = np.mean(np.square(x), axis=-1, keepdims=True, dtype=np.float32)
+    z = (z + np.float32(eps)).astype(np.float32)
+    return round_to_bf16((x / np.sqrt(z)) * w)
+
+
+def apply_rope(x, cos, sin) -> np.ndarray:
+    """examples/models/qwen3/kernels/rope.py:23-48 for one tensor x [..., T, H, D] with
+    cos / sin [T, D/2]: halves (x0, x1) -> (x0 c - x1 s, x0 s + x1 c).  All operands are bf16
+    there, so each product and each sum is rounded to bf16."""
+    x = to_f32(x)
+    c = np.expand_dims(np.asarray(cos, np.float32), axis=-2)      # [T, 1, D/2]
+    s_ = np.expand_dims(np.asarray(sin, np.float32), axis=-2)
+    half = x.shape[-1] // 2
+    x0, x1 = x[..., :half], x[..., half:]
+    r = round_to_bf16
+    o0 = r(r(x0 * c) - r(x1 * s_))
+    o1 = r(r(x0 * s_) + r(x1 * c))
+    return np.concatenate([o0, o1], axis=-1)
+
+
+def qk_norm_rope(xq, xk, seq_lens, query_lens, cos, sin, *, q_norm_weight=None, k_norm_weight=None, eps=1e-6):
+    """The reference's pre-attention step on q and k (qwen3/kernels/attention.py:78-97): optional
+    QK RMSNorm, then RoPE at the tokens' absolute positions start_pos + t with start_pos =
+    seq_lens[b] - query_lens[b] (gpt_oss/kernels/attention.py:85-90).  xq [B, T, Hq, D],
+    xk [B, T, Hkv, D] bf16 bits or values; rows t >= query_lens[b] come back as zeros.
+    Returns (q_out, k_out) as bf16-rounded float32."""
+    q, k = to_f32(xq), to_f32(xk)
+    B, T = q.shape[:2]
+    qo, ko = np.zeros_like(q), np.zeros_like(k)
+    for b in range(B):
+        tq = min(max(int(query_lens[b]), 0), T)
+        if tq == 0:
+            continue
+        start = int(seq_lens[b]) - tq
+        pos = start + np.arange(tq)
+        qb, kb = q[b, :tq], k[b, :tq]
+        if q_norm_weight is not None:
+            qb = rmsnorm(qb, q_norm_weight, eps)
+        if k_norm_weight is not None:
+            kb = rmsnorm(kb, k_norm_weight, eps)
+        qo[b, :tq] = apply_rope(qb, cos[pos], sin[pos])
+        ko[b, :tq] = apply_rope(kb, cos[pos], sin[pos])
+    return qo, ko
 
 
 def kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens, *,

@@ -68,6 +68,16 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert kvw(bs=0) == -1
     assert kvw() == -1 and b"null" in lib.pa_last_error()
     assert kvw(T=0) == 0
+    def pre(**kw):
+        a = dict(B=2, T=4, Hq=4, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1, mp=64)
+        a.update(kw)
+        return lib.pa_qk_norm_rope_kv_write(z, z, z, z, z, z, 1e-6, z, z, a["mp"], z, z, z, z, z, z, z, a["B"], a["T"],
+                                            a["Hq"], a["Hkv"], a["D"], a["bs"], a["mb"], a["nb"], a["kd"], z)
+    assert pre(D=96) == -1 and b"64, 128 or 256" in lib.pa_last_error()
+    assert pre(kd=0) == -1 and b"kv_dtype" in lib.pa_last_error()
+    assert pre(mp=0) == -1
+    assert pre() == -1 and b"null" in lib.pa_last_error()
+    assert pre(B=0) == 0
 
 
 def test_ops_refuse_host_arrays():
