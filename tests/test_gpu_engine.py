@@ -1,0 +1,113 @@
+"""GPU end-to-end: a serving loop in miniature (ragged prompts, decode steps, a forked prefix,
+slot reuse) through the engine glue, every step checked against the oracle's dense attention
+over the tokens each sequence has seen."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_attention_oracle as O
+from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+class _Mirror:
+    """Dense per-sequence history kept by the oracle: rotated K, V as the reference's cache holds them."""
+
+    def __init__(self, n_slots, cos, sin, wq, wk, eps):
+        self.k = [None] * n_slots
+        self.v = [None] * n_slots
+        self.cos, self.sin, self.wq, self.wk, self.eps = cos, sin, wq, wk, eps
+
+    def step(self, xq, xk, xv, qlens, scale):
+        B, T, Hq, D = xq.shape
+        out = np.zeros((B, T, Hq, D), np.float32)
+        for b in range(B):
+            n = qlens[b]
+            if n == 0:
+                continue
+            start = 0 if self.k[b] is None else self.k[b].shape[0]
+            seq = np.array([start + n], np.int32)
+            if self.cos is not None:
+                q, k = O.qk_norm_rope(xq[b:b + 1, :n], xk[b:b + 1, :n], seq, np.array([n], np.int32), self.cos, self.sin,
+                                      q_norm_weight=self.wq, k_norm_weight=self.wk, eps=self.eps)
+                q, k = q[0], k[0]
+            else:
+                q, k = xq[b, :n], xk[b, :n]
+            self.k[b] = k if self.k[b] is None else np.concatenate([self.k[b], k])
+            self.v[b] = xv[b, :n] if self.v[b] is None else np.concatenate([self.v[b], xv[b, :n]])
+            n_rep = Hq // k.shape[1]
+            o = O.dense_attention(q, O.repeat_kv(self.k[b], n_rep), O.repeat_kv(self.v[b], n_rep), scale, prefix=start)
+            out[b, :n] = O.round_output(o, "bf16")
+        return out
+
+
+def _rand(rng, shape, amp=1.0):
+    return O.round_to_bf16(rng.standard_normal(shape).astype(np.float32) * amp)
+
+
+@pytest.mark.parametrize("rope", [False, True])
+def test_serving_loop_bf16_pool(rng, rope):
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    S, Hq, Hkv, D, bs = 4, 8, 2, 128, 16
+    cache = PagedKVCache(num_blocks=40, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=12)
+    wq = wk = cos = sin = None
+    kw = {}
+    if rope:
+        wq, wk = _rand(rng, D) * 0.1 + 1.0, _rand(rng, D) * 0.1 + 1.0
+        wq, wk = O.round_to_bf16(wq), O.round_to_bf16(wk)
+        cos, sin = O.rope_tables(D, 256, 1000000.0)
+        kw = dict(rope_base=1000000.0, max_positions=256, q_norm_weight=bf16_to_dev(wq), k_norm_weight=bf16_to_dev(wk), norm_eps=1e-6)
+    layer = PagedAttention(cache, Hq, **kw)
+    mirror = _Mirror(S, cos, sin, wq, wk, 1e-6)
+    tol = 2e-2 if not rope else 3e-2        # with the norm q/k differ from the oracle's by a bf16 step here and there
+
+    def run(T, qlens):
+        xq, xk, xv = _rand(rng, (S, T, Hq, D)), _rand(rng, (S, T, Hkv, D)), _rand(rng, (S, T, Hkv, D))
+        got = dev_to_f32(layer.step(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv), qlens))
+        want = mirror.step(xq, xk, xv, qlens, layer.scale)
+        for b in range(S):
+            if qlens[b]:
+                assert_close_abs(got[b, :qlens[b]], want[b, :qlens[b]], tol)
+
+    run(37, [37, 20, 0, 5])                      # ragged prompts, slot 2 idle
+    for _ in range(3):
+        run(1, [1, 1, 0, 1])                     # decode
+    run(9, [0, 9, 0, 0])                         # a second chunk for slot 1 (chunked prefill against its cached prefix)
+    # fork slot 0 into slot 2: shared full blocks, private tail; both continue independently
+    cache.fork(0, 2)
+    mirror.k[2], mirror.v[2] = mirror.k[0].copy(), mirror.v[0].copy()
+    shared = cache.blocks[0][:cache.lens[0] // bs]
+    assert shared and all(cache.allocator.refcount(b) == 2 for b in shared)
+    for _ in range(bs + 2):                      # long enough to fill the tail and open new blocks on both sides
+        run(1, [1, 1, 1, 1])
+    assert cache.blocks[0][len(shared):] != cache.blocks[2][len(shared):]
+    # release a slot and reuse it for a new prompt: its blocks go back and stale contents do not leak
+    free_before = cache.allocator.num_free
+    cache.release(1)
+    mirror.k[1] = mirror.v[1] = None
+    assert cache.allocator.num_free > free_before
+    run(21, [0, 21, 0, 0])
+    run(1, [1, 1, 1, 1])
+
+
+def test_serving_loop_fp8_pool_token_by_token(rng):
+    """fp8 pool: the write kernel maintains the scales; attention follows the oracle run on the
+    dequantised pool within the fp8 bar."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    S, Hq, Hkv, D, bs = 2, 8, 2, 128, 16
+    cache = PagedKVCache(num_blocks=12, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=4,
+                         dtype=torch.float8_e4m3fn)
+    layer = PagedAttention(cache, Hq)
+    for step in range(40):
+        xq, xk, xv = _rand(rng, (S, 1, Hq, D)), _rand(rng, (S, 1, Hkv, D), 1.0 + 0.05 * step), _rand(rng, (S, 1, Hkv, D))
+        got = dev_to_f32(layer.step(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv), [1, 1]))[:, 0]
+        codes_k = cache.k_cache.view(torch.uint8).cpu().numpy()
+        codes_v = cache.v_cache.view(torch.uint8).cpu().numpy()
+        want = O.paged_decode(xq[:, 0], codes_k, codes_v, cache.block_tables.cpu().numpy(), cache.seq_lens.cpu().numpy(),
+                              layer.scale, k_scale=cache.k_scale.cpu().numpy(), v_scale=cache.v_scale.cpu().numpy(), q_dtype="bf16")
+        assert_close_abs(got, want, 5e-2)
+    assert cache.lens == [40, 40] and len(cache.blocks[0]) == 3
+    with pytest.raises(NotImplementedError):
+        layer.step(bf16_to_dev(_rand(rng, (S, 2, Hq, D))), bf16_to_dev(_rand(rng, (S, 2, Hkv, D))),
+                   bf16_to_dev(_rand(rng, (S, 2, Hkv, D))), [2, 2])
