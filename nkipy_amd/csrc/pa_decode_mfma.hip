@@ -524,7 +524,10 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 // sequence, a single pass with online rescaling so that the loads of all chunks can be in
 // flight together.  Sequences that were written as final output are skipped, empty ones
 // are zero-filled.
-template <int D>
+// G consecutive lanes share one item and take every G-th piece of the sequence; their partial
+// merges are combined with a butterfly.  G = 1 when there are many sequences (each spans a few
+// chunks), 8 when there are few (one long sequence spans every chunk).
+template <int D, int G>
 __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParams p) {
   const int b = blockIdx.x;
   const int lane = threadIdx.x & 63;
@@ -533,10 +536,11 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int T = tiles_of(clamp_ctx(p, b));
   uint16_t* dst = (uint16_t*)p.out + (long)b * p.Hq * D;
   constexpr int QUADS = D / 4;
-  const int item = blockIdx.y * 256 + threadIdx.x;
+  const int item = blockIdx.y * (256 / G) + threadIdx.x / G;
+  const int g = threadIdx.x % G;
   const bool mine = item < p.Hq * QUADS;
   if (T == 0) {
-    if (mine) *(uint2*)(dst + 4 * item) = make_uint2(0u, 0u);
+    if (mine && g == 0) *(uint2*)(dst + 4 * item) = make_uint2(0u, 0u);
     return;
   }
   const int gv = p.bal_gv;
@@ -558,7 +562,7 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   float m = -INFINITY, l = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
-  for (int c = c_first; c <= c_last; ++c) {
+  for (int c = c_first + g; c <= c_last; c += G) {
     const float2 ml = *(const float2*)(p.ws_ml + (base_slot + c) * 2);
     const float4 o = *(const float4*)(p.ws_out + (base_slot + c) * D + 4 * q4);
     const float m_new = fmaxf(m, ml.x);
@@ -569,6 +573,19 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
     acc.z = acc.z * a + wt * o.z; acc.w = acc.w * a + wt * o.w;
     m = m_new;
   }
+#pragma unroll
+  for (int off = 1; off < G; off <<= 1) {      // lanes without a piece carry m = -inf, l = 0
+    const float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
+    const float4 a2 = make_float4(__shfl_xor(acc.x, off, 64), __shfl_xor(acc.y, off, 64),
+                                  __shfl_xor(acc.z, off, 64), __shfl_xor(acc.w, off, 64));
+    const float m_new = fmaxf(m, m2);
+    const float a = m == -INFINITY ? 0.f : exp2f(m - m_new), b2 = m2 == -INFINITY ? 0.f : exp2f(m2 - m_new);
+    l = l * a + l2 * b2;
+    acc.x = acc.x * a + a2.x * b2; acc.y = acc.y * a + a2.y * b2;
+    acc.z = acc.z * a + a2.z * b2; acc.w = acc.w * a + a2.w * b2;
+    m = m_new;
+  }
+  if (g != 0) return;
   const float inv = 1.f / l;
   *(uint2*)(dst + (long)hq * D + 4 * q4) =
       make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
@@ -637,9 +654,16 @@ hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream
 }
 
 hipError_t launch_decode_balanced_reduce(const DecodeParams& p, hipStream_t s) {
-  dim3 grid(p.B, (p.Hq * (p.D / 4) + 255) / 256);
-  if (p.D == 128) hipLaunchKernelGGL(decode_balanced_reduce_kernel<128>, grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL(decode_balanced_reduce_kernel<64>, grid, dim3(256), 0, s, p);
+  const int items = p.Hq * (p.D / 4);
+  if (p.B <= 8) {     // few sequences: each spans many chunks
+    dim3 grid(p.B, (items + 31) / 32);
+    if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, 8>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, 8>), grid, dim3(256), 0, s, p);
+  } else {
+    dim3 grid(p.B, (items + 255) / 256);
+    if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, 1>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, 1>), grid, dim3(256), 0, s, p);
+  }
   return hipGetLastError();
 }
 
