@@ -87,6 +87,30 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               void* stream);
 
 /*
+ * Speculative verify: a few query tokens per sequence against the paged context, causal among
+ * themselves -- the non-prefill branch of examples/models/gpt_oss/kernels/attention.py:80-100,
+ * 127-135 with seq_len = K+1 ("query at start_pos+i attends to keys <= start_pos+i"), driven by
+ * examples/models/gpt_oss/peagle/speculate.py:137-202.  Same result as pa_prefill on the same
+ * arguments, and fp8 pools are accepted; built for small T: the (token, head) pairs of a kv group
+ * ride along as extra rows of the decode kernel's 16-row query operand, so the context is streamed
+ * from HBM once per kv head however many tokens are verified, at decode's bandwidth.
+ *   q, out       [B, T, Hq, D] bf16; rows t >= query_lens[b] are padding, zero in out
+ *   seq_lens[b]  context length including the query tokens, whose K/V are already in the pool
+ *   kv_dtype     PA_BF16 or PA_FP8_E4M3FN (then k_scale / v_scale [num_blocks, Hkv] f32)
+ *   workspace    pa_verify_workspace_bytes(B, T, Hq, D) bytes, 16-byte aligned
+ * D in {64, 128}; block_size a power of two >= 16; T <= PA_VERIFY_MAX_TOKENS.
+ */
+#define PA_VERIFY_MAX_TOKENS 64
+size_t pa_verify_workspace_bytes(int B, int T, int Hq, int D);
+int pa_verify(const void* q, const void* k_cache, const void* v_cache,
+              const float* k_scale, const float* v_scale,
+              const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+              void* out, void* workspace, size_t workspace_bytes,
+              int B, int T, int Hq, int Hkv, int D, int block_size,
+              int max_blocks_per_seq, int num_blocks,
+              float scale, int kv_dtype, void* stream);
+
+/*
  * Paged chunked prefill with a cached prefix, causal: query token i of sequence
  * b (i < query_lens[b]) sees keys j <= seq_lens[b] - query_lens[b] + i
  * (examples/models/gpt_oss/kernels/attention.py:85,127-135: "query at

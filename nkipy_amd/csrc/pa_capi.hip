@@ -196,7 +196,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   memset(&p, 0, sizeof(p));
   p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
   p.block_tables = block_tables; p.seq_lens = seq_lens; p.out = out;
-  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = 1;
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.partition_size = partition_size;
@@ -245,6 +245,63 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
     if (e != hipSuccess) return check_hip(e, "pa_decode reduce launch");
   }
   return 0;
+}
+
+size_t pa_verify_workspace_bytes(int B, int T, int Hq, int D) {
+  if (B <= 0 || T <= 0 || Hq <= 0 || D <= 0 || (long)Hq * T > 0x7fffffffL) return 0;
+  return decode_balanced_workspace_bytes(B, Hq * T, D, 8 * current_num_cus());
+}
+
+int pa_verify(const void* q, const void* k_cache, const void* v_cache,
+              const float* k_scale, const float* v_scale,
+              const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+              void* out, void* workspace, size_t workspace_bytes,
+              int B, int T, int Hq, int Hkv, int D, int block_size,
+              int max_blocks_per_seq, int num_blocks,
+              float scale, int kv_dtype, void* stream) {
+  tl_error[0] = 0;
+  if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_verify: bad sizes B=%d T=%d Hq=%d Hkv=%d D=%d", B, T, Hq, Hkv, D);
+  if (Hq % Hkv) return fail_arg("pa_verify: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_verify: bad paging sizes");
+  if (kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN)
+    return fail_arg("pa_verify: kv_dtype must be bf16 or fp8-e4m3fn (got %d)", kv_dtype);
+  if (T > PA_VERIFY_MAX_TOKENS) return fail_arg("pa_verify: T=%d exceeds %d query tokens per sequence; use pa_prefill", T, PA_VERIFY_MAX_TOKENS);
+  if (B == 0 || T == 0) return 0;
+  if (B > 65535) return fail_arg("pa_verify: B=%d exceeds 65535", B);
+  if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens || !out)
+    return fail_arg("pa_verify: null pointer argument");
+  if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_verify: fp8 KV needs k_scale and v_scale");
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out) || !aligned16(workspace))
+    return fail_arg("pa_verify: q, k_cache, v_cache, out and workspace must be 16-byte aligned");
+  const long cap = (long)max_blocks_per_seq * block_size;
+
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
+  p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens; p.out = out;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = T;
+  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
+  p.block_shift = ilog2_exact(block_size);
+  p.max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
+  p.partition_size = p.max_seq_len;
+  p.num_partitions = 1;
+  p.scale_log2e = scale * kLog2e;
+  if (!decode_mfma_supported(p, PA_BF16, kv_dtype))
+    return fail_arg("pa_verify: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", D, block_size);
+  plan_decode_balanced(p, current_num_cus());
+  p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
+  const size_t need = decode_balanced_workspace_bytes(B, Hq * T, D, p.bal_gv);
+  if (!workspace || workspace_bytes < need)
+    return fail_arg("pa_verify: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  p.ws_out = (float*)workspace;
+  p.ws_ml = p.ws_out + (size_t)Hq * T * ((size_t)B + p.bal_gv) * D;
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipError_t e = launch_decode_balanced(p, kv_dtype, s);
+  profile_end(s);
+  if (e != hipSuccess) return check_hip(e, "pa_verify launch");
+  e = launch_decode_balanced_reduce(p, s);
+  return check_hip(e, "pa_verify reduce launch");
 }
 
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,

@@ -70,17 +70,19 @@ template <> struct Store<uint16_t> {
 
 // ---- decode ------------------------------------------------------------------------
 struct DecodeParams {
-  const void* q;            // [B, Hq, D]
+  const void* q;            // [B, Hq, D]; [B, T, Hq, D] for a multi-token call
   const void* k_cache;      // [num_blocks, block_size, Hkv, D]
   const void* v_cache;
   const float* k_scale;     // [num_blocks, Hkv] or null
   const float* v_scale;
   const int32_t* block_tables;  // [B, max_blocks]
   const int32_t* seq_lens;      // [B]
-  void* out;                // [B, Hq, D]
+  const int32_t* query_lens;    // [B] for a multi-token call (balanced schedule only), else null
+  void* out;                // shaped like q
   float* ws_out;            // [B, Hq, P, D]
   float* ws_ml;             // [B, Hq, P, 2]
   int B, Hq, Hkv, D;
+  int T;                    // query tokens per sequence (1: decode)
   int block_size, max_blocks, num_blocks;
   int block_shift;          // log2(block_size), or -1 when not a power of two
   int partition_size, num_partitions, max_seq_len;

@@ -80,8 +80,17 @@ struct VTile {
 };
 
 // Per-wavefront streaming state: Q fragments, online-softmax state and output
-// accumulators for up to 16 query heads of one kv head of one sequence.
-template <int D, bool FP8>
+// accumulators for up to 16 query rows of one kv head of one sequence.
+//
+// MULTI = false: one query token per sequence; the rows are the q heads of the
+// kv group.  MULTI = true: p.T query tokens per sequence (the last query_lens[b]
+// tokens of the context, K/V already in the pool); the rows of a kv group are
+// its n_rep * T (token, head) pairs, token-major, numbered as "virtual heads"
+// hk * n_rep * T + t * n_rep + head.  Row (t, .) sees keys
+// < ctx - tq + t + 1, so the causal mask is one more per-lane bound on the token
+// index; a row may then see no key at all in a tile or in a whole chunk, which the
+// softmax update and the stores allow for (state m = -inf, l = 0, o = 0).
+template <int D, bool FP8, bool MULTI = false>
 struct DecodeWave {
   using KT = KTile<D, FP8>;
   using VT = VTile<D, FP8>;
@@ -97,17 +106,21 @@ struct DecodeWave {
   const char* vbase;
   long row_stride;           // bytes between consecutive tokens of a block
   int last;                  // ctx - 1 of the current sequence
+  int jbase;                 // first row of this wave inside its kv group
+  int row_end;               // MULTI: keys [0, row_end) are visible to this lane's row (0: padding row)
+  long row_off;              // MULTI: element offset of this lane's row in q and out
   bf16x8_t qf[KSTEPS];
   bf16x8_t pf;               // P^T fragment of the current tile
   f32x4_t oacc[VEC];
   float m_run, l_run;
 
   __device__ __forceinline__ DecodeWave(const DecodeParams& p_, int head_slot, int lane) : p(p_) {
-    const int n_rep = p.Hq / p.Hkv;
-    const int gchunks = (n_rep + 15) / 16;
+    const int n_rows = (p.Hq / p.Hkv) * (MULTI ? p.T : 1);
+    const int gchunks = (n_rows + 15) / 16;
     hk = head_slot / gchunks;
-    hbase = hk * n_rep + (head_slot % gchunks) * 16;
-    nheads = min(16, n_rep - (head_slot % gchunks) * 16);
+    jbase = (head_slot % gchunks) * 16;
+    hbase = hk * n_rows + jbase;
+    nheads = min(16, n_rows - jbase);
     r = lane & 15;
     g = lane >> 4;
     krow = 4 * (r & 3) + (r >> 2);
@@ -116,18 +129,29 @@ struct DecodeWave {
     vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
   }
 
-  // Start on sequence b (context ctx >= 1): load Q^T fragments (B operand, zero
-  // for padded head columns) and reset the softmax state.
-  __device__ __forceinline__ void begin(int b, int ctx) {
+  // Start on sequence b (context ctx >= 1, of which the last tq tokens are the
+  // queries): load Q^T fragments (B operand, zero for padded columns) and reset
+  // the softmax state.
+  __device__ __forceinline__ void begin(int b, int ctx, int tq = 1) {
     table = p.block_tables + (long)b * p.max_blocks;
     last = ctx - 1;
-    const uint16_t* qrow = (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
+    bool row_valid = r < nheads;
+    if (MULTI) {
+      const int n_rep = p.Hq / p.Hkv;
+      const int j = jbase + r;
+      const int t = j / n_rep;
+      row_off = (((long)b * p.T + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D;
+      row_valid = row_valid && t < tq;
+      row_end = row_valid ? ctx - tq + t + 1 : 0;
+    }
+    const uint16_t* qrow = MULTI ? (const uint16_t*)p.q + row_off
+                                 : (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
       // d range of k-slots 8g..8g+7 in step s (must mirror the K loads below)
       const int d0 = FP8 ? ((4 * (s >> 1) + g) * 16 + (s & 1) * 8) : ((4 * s + g) * 8);
       uint4 v = make_uint4(0, 0, 0, 0);
-      if (r < nheads) v = *(const uint4*)(qrow + d0);
+      if (row_valid) v = *(const uint4*)(qrow + d0);
       qf[s] = __builtin_bit_cast(bf16x8_t, v);
     }
 #pragma unroll
@@ -216,6 +240,7 @@ struct DecodeWave {
     }
     float sv[8];
     float tmax = -INFINITY;
+    if (MULTI) t_end = min(t_end, row_end);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const float sc = FP8 ? p.scale_log2e * tl.ksc[u] : p.scale_log2e;
@@ -230,12 +255,14 @@ struct DecodeWave {
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m_run, tmax);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    // MULTI: a row that has seen no key yet keeps m = -inf; exponents are then taken against 0
+    const float m_ref = (MULTI && m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
     m_run = m_new;
     float pr[8], psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      pr[i] = __builtin_amdgcn_exp2f(sv[i] - m_new);
+      pr[i] = __builtin_amdgcn_exp2f(sv[i] - m_ref);
       psum += pr[i];
     }
     l_run = l_run * alpha + psum;
@@ -331,8 +358,8 @@ struct DecodeWave {
   // for i = 0..3, the VEC consecutive d's starting at VEC * (4g + i).
   __device__ __forceinline__ void store_final(int b, float l) const {
     if (r >= nheads) return;
-    const float inv = 1.f / l;
-    uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hbase + r) * D;
+    const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;    // padding rows: zeros
+    uint16_t* dst = MULTI ? (uint16_t*)p.out + row_off : (uint16_t*)p.out + ((long)b * p.Hq + hbase + r) * D;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       uint32_t w[VEC / 2];
@@ -347,7 +374,7 @@ struct DecodeWave {
   }
   __device__ __forceinline__ void store_partial(long slot, float l) const {
     if (r >= nheads) return;
-    const float inv = 1.f / l;
+    const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;
     float* dst = p.ws_out + slot * D;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -362,6 +389,11 @@ struct DecodeWave {
 
 __device__ __forceinline__ int clamp_ctx(const DecodeParams& p, int b) {
   return min(max(p.seq_lens[b], 0), p.max_seq_len);
+}
+
+// 16-row groups over all kv heads: rows of a kv head = its q heads x query tokens
+__host__ __device__ __forceinline__ int head_slots_of(const DecodeParams& p) {
+  return p.Hkv * (((p.Hq / p.Hkv) * p.T + 15) / 16);
 }
 
 // ---------------------------------------------------------------------------
@@ -474,13 +506,12 @@ __device__ __forceinline__ int scan_tiles(const DecodeParams& p, int lane, int f
   return base;
 }
 
-template <int D, bool FP8>
+template <int D, bool FP8, bool MULTI>
 __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p) {
-  using W = DecodeWave<D, FP8>;
+  using W = DecodeWave<D, FP8, MULTI>;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n_rep = p.Hq / p.Hkv;
-  const int head_slots = p.Hkv * ((n_rep + 15) / 16);
+  const int head_slots = head_slots_of(p);
   const int hs = blockIdx.y * p.bal_hsw + wave % p.bal_hsw;
   if (hs >= head_slots) return;
   const int cv = blockIdx.x * p.bal_ns + wave / p.bal_hsw;   // chunk of this wave
@@ -505,7 +536,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
     if (T == 0) { ++b; continue; }
     const int ti = f - start;
     const int n = min(T - ti, f_end - f);
-    w.begin(b, ctx);
+    w.begin(b, ctx, MULTI ? min(min(max(p.query_lens[b], 0), p.T), ctx) : 1);
     w.stream(ti << 5, 32, n, ctx, p.bal_lockstep != 0);
     const float l = w.total_l();
     const int c_first = start / L, c_last = (start + T - 1) / L;
@@ -534,13 +565,19 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   int bb = 0, start = 0;
   const int N = scan_tiles(p, lane, -1, &bb, &start);
   const int T = tiles_of(clamp_ctx(p, b));
-  uint16_t* dst = (uint16_t*)p.out + (long)b * p.Hq * D;
   constexpr int QUADS = D / 4;
   const int item = blockIdx.y * (256 / G) + threadIdx.x / G;
   const int g = threadIdx.x % G;
-  const bool mine = item < p.Hq * QUADS;
+  const bool mine = item < p.Hq * p.T * QUADS;
+  const int hq = item / QUADS, q4 = item % QUADS;     // hq: virtual head when p.T > 1
+  uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hq) * D + 4 * q4;
+  if (p.T > 1) {
+    const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
+    const int hk = hq / n_rows, j = hq % n_rows, t = j / n_rep;
+    dst = (uint16_t*)p.out + (((long)b * p.T + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D + 4 * q4;
+  }
   if (T == 0) {
-    if (mine && g == 0) *(uint2*)(dst + 4 * item) = make_uint2(0u, 0u);
+    if (mine && g == 0) *(uint2*)dst = make_uint2(0u, 0u);
     return;
   }
   const int gv = p.bal_gv;
@@ -557,7 +594,6 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   }
   const int c_first = start / L, c_last = (start + T - 1) / L;
   if (c_first == c_last || !mine) return;   // single piece: written by the streaming kernel
-  const int hq = item / QUADS, q4 = item % QUADS;
   const long base_slot = (long)hq * (p.B + gv) + b;
   float m = -INFINITY, l = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -566,8 +602,9 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
     const float2 ml = *(const float2*)(p.ws_ml + (base_slot + c) * 2);
     const float4 o = *(const float4*)(p.ws_out + (base_slot + c) * D + 4 * q4);
     const float m_new = fmaxf(m, ml.x);
-    const float a = exp2f(m - m_new);
-    const float wt = ml.y * exp2f(ml.x - m_new);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;   // pieces in which a row saw no key carry m = -inf, l = 0
+    const float a = exp2f(m - m_ref);
+    const float wt = ml.y * exp2f(ml.x - m_ref);
     l = l * a + wt;
     acc.x = acc.x * a + wt * o.x; acc.y = acc.y * a + wt * o.y;
     acc.z = acc.z * a + wt * o.z; acc.w = acc.w * a + wt * o.w;
@@ -586,8 +623,8 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
     m = m_new;
   }
   if (g != 0) return;
-  const float inv = 1.f / l;
-  *(uint2*)(dst + (long)hq * D + 4 * q4) =
+  const float inv = l == 0.f ? 0.f : 1.f / l;     // padding rows of a multi-token call: zeros
+  *(uint2*)dst =
       make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
 }
 
@@ -606,10 +643,12 @@ hipError_t launch_typed(const DecodeParams& p, int waves, hipStream_t s) {
 
 template <int D, bool FP8>
 hipError_t launch_balanced_typed(const DecodeParams& p, hipStream_t s) {
-  const int n_rep = p.Hq / p.Hkv;
-  const int head_slots = p.Hkv * ((n_rep + 15) / 16);
+  const int head_slots = head_slots_of(p);
   dim3 grid(p.bal_gv / p.bal_ns, (head_slots + p.bal_hsw - 1) / p.bal_hsw);
-  hipLaunchKernelGGL((decode_balanced_kernel<D, FP8>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
+  if (p.query_lens)
+    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
+  else
+    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, false>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
   return hipGetLastError();
 }
 
@@ -631,8 +670,7 @@ hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hi
 }
 
 void plan_decode_balanced(DecodeParams& p, int num_cus) {
-  const int n_rep = p.Hq / p.Hkv;
-  const int head_slots = p.Hkv * ((n_rep + 15) / 16);
+  const int head_slots = head_slots_of(p);
   constexpr int kWavesPerCu = 8;                       // two per SIMD at this register footprint
   p.bal_hsw = head_slots < kWavesPerCu ? head_slots : kWavesPerCu;
   p.bal_ns = kWavesPerCu / p.bal_hsw;
@@ -654,7 +692,7 @@ hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream
 }
 
 hipError_t launch_decode_balanced_reduce(const DecodeParams& p, hipStream_t s) {
-  const int items = p.Hq * (p.D / 4);
+  const int items = p.Hq * p.T * (p.D / 4);
   if (p.B <= 8) {     // few sequences: each spans many chunks
     dim3 grid(p.B, (items + 31) / 32);
     if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, 8>), grid, dim3(256), 0, s, p);

@@ -174,14 +174,27 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
     return out
 
 
-def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, out=None,
-            validate_tables=False):
+VERIFY_MAX_ROWS = 64    # (query token, q head) pairs per kv head up to which prefill takes the verify kernel
+
+
+def _verify_supported(T, D, block_size):
+    return T <= 64 and D in (64, 128) and block_size >= 16 and block_size & (block_size - 1) == 0
+
+
+def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
+            out=None, workspace=None, route=None, validate_tables=False):
     """Chunked prefill against a cached prefix (causal).
 
     q [B, T, Hq, D] bfloat16 holds the last query_lens[b] tokens of each sequence
     (rows t >= query_lens[b] are padding; their output is zero); token i sees keys
     j <= seq_lens[b] - query_lens[b] + i of the paged context, which already
     contains the new tokens' K/V.
+
+    Two kernels stand behind it.  Short query runs -- speculative verify, T * (Hq / Hkv) <=
+    VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query
+    rows (HBM-bound: the context is read once per kv head); longer ones through the tiled
+    matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
+    (float8_e4m3fn / uint8 codes with k_scale, v_scale) are read by the verify kernel only.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -191,13 +204,32 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, o
     B, T, Hq, D = q.shape
     _check(q.dtype == torch.bfloat16, "prefill supports bfloat16 only")
     _check_paging(k_cache, v_cache, block_tables, seq_lens, B)
-    _check(k_cache.dtype == torch.bfloat16, "prefill needs a bfloat16 KV cache")
+    scaled = k_scale is not None or v_scale is not None
+    kv_code = _kv_code(k_cache, scaled)
+    _check(kv_code in (BF16, FP8), "prefill needs a bfloat16 or fp8 KV cache")
     _check(query_lens.shape == (B,) and query_lens.dtype == torch.int32, "query_lens must be int32 [B]")
     num_blocks, block_size, Hkv, Dk = k_cache.shape
     _check(Dk == D, f"head_dim mismatch: q has {D}, cache has {Dk}")
     _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    if kv_code == FP8:
+        _check(k_scale is not None and v_scale is not None, "fp8 KV needs both k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _need_device(n, t)
+            _check(t.dtype == torch.float32 and t.shape == (num_blocks, Hkv),
+                   f"{n} must be float32 [num_blocks, Hkv]")
+    else:
+        _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
+    _check(route in (None, "verify", "tiled"), "route must be None, 'verify' or 'tiled'")
+    can_verify = _verify_supported(T, D, block_size)
+    if route is None:
+        route = "verify" if can_verify and (kv_code == FP8 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
+    if route == "verify":
+        _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
+                           f"(T={T}, D={D}, block_size={block_size})")
+    else:
+        _check(kv_code == BF16, "fp8 KV caches are read by the verify kernel only (T <= 64, head_dim 64 or 128)")
     _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
-                 query_lens=query_lens, out=out)
+                 query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out)
     if validate_tables:
         check_block_tables(block_tables, seq_lens, num_blocks, block_size)
     if out is None:
@@ -205,12 +237,33 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, o
     else:
         _need_device("out", out)
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
+    if route == "verify":
+        need = int(lib.pa_verify_workspace_bytes(B, T, Hq, D))
+        if workspace is None:
+            workspace = _workspace(q.device, need)
+        else:
+            _need_device("workspace", workspace)
+            _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
+        ws_bytes = workspace.numel() * workspace.element_size()
+        with torch.cuda.device(q.device):
+            rc = lib.pa_verify(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+                               _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), _ptr(out),
+                               _ptr(workspace), ws_bytes, B, T, Hq, Hkv, D, block_size,
+                               block_tables.shape[1], num_blocks, float(scale), kv_code, _stream_ptr(q.device))
+        _raise_on(rc, "pa_verify")
+        return out
     with torch.cuda.device(q.device):
         rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
                             block_tables.shape[1], num_blocks, float(scale), BF16, _stream_ptr(q.device))
     _raise_on(rc, "pa_prefill")
     return out
+
+
+def verify(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, **kw):
+    """Speculative verify (gpt_oss/kernels/attention.py:80-100 with seq_len = K+1): prefill through
+    the decode-shaped kernel whatever T * (Hq / Hkv) is."""
+    return prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, route="verify", **kw)
 
 
 def blocksparse_prefill(q, k, v, scale, *, block=64, local_blocks=4, vert_stride=8, out=None):

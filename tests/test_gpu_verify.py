@@ -1,0 +1,150 @@
+"""GPU parity: speculative verify (a few query tokens per sequence, through pa_verify) vs the oracle
+and vs the tiled prefill kernel on the same arguments."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_attention_oracle as O
+from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_bits, dev_to_f32, make_paged
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2
+FP8_TOL = 5e-2
+
+
+@pytest.fixture(scope="module")
+def pa():
+    import nkipy_amd
+    from nkipy_amd import _lib
+    _lib.load()
+    return nkipy_amd
+
+
+def _i32(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.int32)).cuda()
+
+
+def _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D):
+    B = len(qlens)
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, [max(c, 1) for c in ctxs])
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    return q, O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32)
+
+
+@pytest.mark.parametrize("T,Hq,Hkv", [(4, 32, 8), (2, 8, 2), (5, 6, 2), (8, 32, 8), (16, 16, 4), (3, 40, 2),
+                                      (64, 4, 4), (7, 1, 1)])
+@pytest.mark.parametrize("D,bs", [(128, 32), (64, 16)])
+def test_verify_matches_oracle(pa, T, Hq, Hkv, D, bs):
+    """Rows per kv head from 7 to 64: less than, exactly, and several times the 16-row operand."""
+    rng = np.random.default_rng(1000 * T + Hq + D)
+    qlens = [T, max(T - 1, 1), 1, T, 0, T]
+    prefixes = [0, 300, 65, 1533, 40, 31]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_prefill(q, k, v, tables, ctxs, ql, scale, q_dtype="bf16")
+    got = pa.verify(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), scale)
+    torch.cuda.synchronize()
+    got = dev_to_f32(got)
+    assert_close_abs(got, want, BF16_TOL)
+    for b, n in enumerate(qlens):
+        assert np.all(got[b, n:] == 0)          # padding rows
+
+
+def test_verify_rows_without_keys_in_the_last_chunk(pa):
+    """One long sequence spans every chunk of the schedule; its last 32-token tile holds 3 tokens,
+    which the first 5 of 8 query tokens do not see, so their partial of that chunk is empty."""
+    rng = np.random.default_rng(11)
+    T, Hq, Hkv, D, bs = 8, 8, 2, 128, 32
+    for ctx in (32 * 40 + 3, 32 * 700 + 1, 9):
+        q, k, v, tables, ctxs, ql = _case(rng, T, [T], [ctx - T], Hq, Hkv, bs, D)
+        want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.09, q_dtype="bf16")
+        got = pa.verify(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.09)
+        torch.cuda.synchronize()
+        assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_verify_agrees_with_tiled_prefill_and_decode(pa):
+    rng = np.random.default_rng(12)
+    T, Hq, Hkv, D, bs = 4, 32, 8, 128, 32
+    qlens, prefixes = [4, 4, 2, 4], [700, 0, 129, 4000]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.09)
+    a = dev_to_f32(pa.prefill(*args, route="verify"))
+    b = dev_to_f32(pa.prefill(*args, route="tiled"))
+    c = dev_to_f32(pa.prefill(*args))                   # 16 rows per kv head: the verify kernel by default
+    assert np.max(np.abs(a - b)) <= 2 ** -6
+    assert np.array_equal(a, c)
+    # the last query token of a full-length sequence is a decode step over the whole context
+    full = [i for i, n in enumerate(qlens) if n == T]
+    d = pa.decode(args[0][full, T - 1].contiguous(), args[1], args[2], args[3][full].contiguous(),
+                  args[4][full].contiguous(), 0.09)
+    torch.cuda.synchronize()
+    assert np.max(np.abs(dev_to_f32(d) - a[full, T - 1])) <= 2 ** -6
+
+
+@pytest.mark.parametrize("D,Hq,Hkv,bs,T", [(128, 32, 8, 64, 4), (64, 8, 1, 16, 6)])
+def test_verify_fp8_pool(pa, D, Hq, Hkv, bs, T):
+    rng = np.random.default_rng(D + T)
+    qlens, prefixes = [T, 1, T, T - 1], [0, 63, 1500, 300]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_prefill(q, kq, vq, tables, ctxs, ql, scale, k_scale=ks, v_scale=vs, q_dtype="bf16")
+    got = pa.prefill(bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+                     torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(ql), scale,
+                     k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda())
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, FP8_TOL)
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_verify_stale_pool_bytes_and_padding_rows_do_not_leak(pa):
+    rng = np.random.default_rng(13)
+    T, Hq, Hkv, D, bs = 6, 8, 2, 128, 32
+    qlens, prefixes = [6, 3], [45, 3]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.09)
+    kd, vd = bf16_to_dev(k), bf16_to_dev(v)
+    used = np.zeros(k.shape[:2], bool)
+    for b in range(len(qlens)):
+        for t in range(ctxs[b]):
+            used[tables[b, t // bs], t % bs] = True
+    mask = torch.from_numpy(~used).cuda()
+    kd[mask] = float("nan")
+    vd[mask] = float("nan")
+    qd = bf16_to_dev(q)
+    qd[1, 3:] = float("nan")
+    got = pa.verify(qd, kd, vd, _i32(tables), _i32(ctxs), _i32(ql), 0.09)
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+    assert np.all(dev_to_f32(got)[1, 3:] == 0)
+
+
+def test_verify_is_deterministic_and_keeps_out_argument(pa):
+    rng = np.random.default_rng(14)
+    T, Hq, Hkv, D, bs = 4, 16, 4, 128, 32
+    q, k, v, tables, ctxs, ql = _case(rng, T, [4] * 5, [5000, 17, 900, 2222, 64], Hq, Hkv, bs, D)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.09)
+    out = torch.full_like(args[0], 7.0)
+    r = pa.verify(*args, out=out)
+    assert r is out
+    again = pa.verify(*args)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(out), dev_bits(again))
+
+
+def test_verify_argument_errors(pa):
+    rng = np.random.default_rng(15)
+    q, k, v, tables, ctxs, ql = _case(rng, 4, [4], [10], 4, 2, 32, 128)
+    args = [bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.09]
+    with pytest.raises(ValueError):
+        pa.verify(*args, workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+    big = bf16_to_dev(np.zeros((1, 65, 4, 128), np.float32))
+    with pytest.raises(ValueError):
+        pa.verify(big, *args[1:])
+    with pytest.raises(ValueError):     # fp8 pools need the verify kernel
+        pa.prefill(big, args[1].view(torch.uint8)[..., :128].contiguous(), args[2].view(torch.uint8)[..., :128].contiguous(),
+                   *args[3:], k_scale=torch.ones(k.shape[0], 2, device="cuda"), v_scale=torch.ones(k.shape[0], 2, device="cuda"))

@@ -78,6 +78,17 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert pre(mp=0) == -1
     assert pre() == -1 and b"null" in lib.pa_last_error()
     assert pre(B=0) == 0
+    def ver(**kw):
+        a = dict(B=2, T=4, Hq=8, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1)
+        a.update(kw)
+        return lib.pa_verify(z, z, z, z, z, z, z, z, z, z, 0, a["B"], a["T"], a["Hq"], a["Hkv"], a["D"], a["bs"],
+                             a["mb"], a["nb"], 1.0, a["kd"], z)
+    assert ver(Hq=7) == -1 and b"multiple" in lib.pa_last_error()
+    assert ver(kd=0) == -1 and b"kv_dtype" in lib.pa_last_error()
+    assert ver(T=65) == -1 and b"pa_prefill" in lib.pa_last_error()
+    assert ver() == -1 and b"null" in lib.pa_last_error()
+    assert ver(T=0) == 0
+    assert lib.pa_verify_workspace_bytes(0, 4, 8, 128) == 0
 
 
 def test_ops_refuse_host_arrays():
