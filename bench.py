@@ -153,6 +153,60 @@ def bench_decode(cfg, steps, warmup, lib, pa, W):
     return res
 
 
+def bench_verify(steps, warmup, lib, pa, W, T=4):
+    """Speculative verify on the pool and tables of the C2 decode workload: the last T tokens of every
+    context are the queries (K = T - 1 drafts plus the last accepted token)."""
+    from oracle import paged_attention_oracle as O
+    from tests.pa_testlib import dev_bits
+    w = W.make_decode(2)
+    B, Hq, D = w.q.shape
+    gen = torch.Generator(device=w.q.device)
+    gen.manual_seed(1008)
+    q = torch.randn((B, T, Hq, D), generator=gen, device=w.q.device).to(torch.bfloat16)
+    qlens = torch.full((B,), T, dtype=torch.int32, device=w.q.device)
+    out = torch.empty_like(q)
+
+    def step():
+        pa.verify(q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, qlens, w.scale, out=out)
+
+    sec = _time_steps(step, steps, warmup)
+    lib.pa_profile_enable(1)
+    _time_steps(step, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = _collect_kernel_ms(lib, steps)
+    kavg = float(np.mean(kms)) if kms else float("nan")
+    ab = w.algorithmic_bytes() + 2 * B * (T - 1) * Hq * D * 2 + 4 * B     # more q / out rows, query_lens
+    nb, bs, hkv, _ = w.k_cache.shape
+    res = {
+        "metric": "verify attn HBM GB/s (% peak) + tok/s",
+        "value": round(ab / sec / 1e9, 2), "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * ab / sec / 1e9 / HBM_PEAK_GBS, 2),
+        "tok_per_s": round(B * T / sec, 1),
+        "ms_per_step": round(sec * 1e3, 5),
+        "dtype": "bf16, fp32 accumulate",
+        "config": {"workload": f"speculative verify on the C2 pool: B={B}, T={T} query tokens per sequence, Hq={Hq}, "
+                               f"Hkv={hkv}, D={D}, block_size={bs}, ctx sum={int(w.ctx.sum())}",
+                   "algorithmic_bytes": ab},
+        "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel": "decode_balanced_kernel (multi-token rows)",
+                     "kernel_avg_ms": round(kavg, 5), "launches_timed": len(kms)},
+    }
+    if not _NO_CPU:
+        n = 4
+        kc, vc = dev_bits(w.k_cache), dev_bits(w.v_cache)
+        t0 = time.perf_counter()
+        O.paged_prefill(dev_bits(q)[:n], kc, vc, w.block_tables.cpu().numpy()[:n], w.ctx[:n].astype(np.int32),
+                        np.full(n, T, np.int32), w.scale, q_dtype="bf16")
+        dt = time.perf_counter() - t0
+        bytes_n = int(w.ctx[:n].sum()) * 2 * hkv * D * 2
+        res["cpu_baseline"] = {"value": round(bytes_n / dt / 1e9, 4), "unit": "GB/s", "cores": _host_info(), "kind": "port",
+                               "tok_per_s": round(n * T / dt, 2),
+                               "sample": f"NumPy oracle, first {n} of {B} sequences of the same workload, one run of "
+                                         f"{dt:.2f} s, numpy {np.__version__} default BLAS threading"}
+    return res
+
+
 def _mfma_ceiling(lib, sample):
     """Matrix-core rate of a registers-only MFMA loop fed with operands drawn from `sample`
     (a bf16 device tensor of the benchmark's own inputs): what the power-limited chip
@@ -354,7 +408,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -381,6 +435,8 @@ def main():
         res = bench_kv_write(args.steps, args.warmup, lib, pa, W)
     elif args.config == 7:
         res = bench_pre_attention(args.steps, args.warmup, lib, pa, W)
+    elif args.config == 8:
+        res = bench_verify(args.steps, args.warmup, lib, pa, W)
     else:
         res = bench_blocksparse(args.steps, args.warmup, lib, pa, W)
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"),

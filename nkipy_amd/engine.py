@@ -184,7 +184,7 @@ class PagedAttention:
     `step(xq, xk, xv, query_lens)` takes the projected q/k/v of every slot, [max_seqs, T, H, D]
     bfloat16 (slot b contributes its first query_lens[b] rows; idle slots 0), reserves the
     blocks, applies the optional QK RMSNorm + RoPE, writes K/V into the pool and runs the
-    chunked-prefill kernel (T > 1) or the decode kernel (T == 1).  Returns [max_seqs, T, Hq, D]
+    prefill / verify kernel (T > 1) or the decode kernel (T == 1).  Returns [max_seqs, T, Hq, D]
     (a preallocated buffer, overwritten by the next step of the same T).
     """
 
@@ -212,9 +212,10 @@ class PagedAttention:
             raise ValueError(f"expected one row per slot ({c.max_seqs}), got {B} rows and {len(query_lens)} lengths")
         if any(n < 0 or n > T for n in query_lens):
             raise ValueError("query_lens must lie in [0, T]")
-        if T > 1 and c.k_scale is not None:
-            raise NotImplementedError("chunked prefill reads bf16 pools only; feed an fp8 cache one token per step "
-                                      "or keep the prompt's K/V in a bf16 pool")
+        if T > 1 and c.k_scale is not None and not paged_attn.verify_supported(T, c.head_dim, c.block_size):
+            raise NotImplementedError("only the verify kernel (up to 64 tokens per step, head_dim 64 or 128) reads fp8 "
+                                      "pools with several query tokens; feed an fp8 cache in chunks of at most 64 "
+                                      "tokens or keep the prompt's K/V in a bf16 pool")
         active = [s for s in range(B) if query_lens[s] > 0]
         c.extend(active, [query_lens[s] for s in active])
         self._qlens.copy_(torch.tensor(list(query_lens), dtype=torch.int32))
@@ -236,5 +237,6 @@ class PagedAttention:
                               max_seq_len=max(c.max_seq_len, 1), out=out[:, 0])
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:
-            paged_attn.prefill(q, c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self._qlens, self.scale, out=out)
+            paged_attn.prefill(q, c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self._qlens, self.scale,
+                               k_scale=c.k_scale, v_scale=c.v_scale, out=out)
         return out

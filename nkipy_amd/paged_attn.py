@@ -177,7 +177,8 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
 VERIFY_MAX_ROWS = 64    # (query token, q head) pairs per kv head up to which prefill takes the verify kernel
 
 
-def _verify_supported(T, D, block_size):
+def verify_supported(T, D, block_size) -> bool:
+    """Shapes the verify kernel is built for."""
     return T <= 64 and D in (64, 128) and block_size >= 16 and block_size & (block_size - 1) == 0
 
 
@@ -220,7 +221,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     else:
         _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
     _check(route in (None, "verify", "tiled"), "route must be None, 'verify' or 'tiled'")
-    can_verify = _verify_supported(T, D, block_size)
+    can_verify = verify_supported(T, D, block_size)
     if route is None:
         route = "verify" if can_verify and (kv_code == FP8 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
     if route == "verify":
