@@ -198,7 +198,8 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * automatic, 1 = register-staged kernel, 4 / 8 = asynchronous-copy kernel with that
  * many wavefronts per workgroup); key 4:
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
- * the same tile (1 = on, the default). */
+ * the same tile (1 = on, the default); key 5: query rows per wavefront of pa_verify (0 =
+ * automatic, 16 or 32 = forced). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

@@ -40,6 +40,7 @@ static std::atomic<int> g_decode_waves{0};
 static std::atomic<int> g_head_major{1};
 static std::atomic<int> g_prefill_impl{0};
 static std::atomic<int> g_lockstep{1};
+static std::atomic<int> g_verify_rows{0};
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 static std::atomic<int> g_profile{0};
@@ -107,6 +108,7 @@ int pa_debug_set(int key, int value) {
   if (key == 2) { g_head_major = value; return 0; }
   if (key == 3) { g_prefill_impl = value; return 0; }
   if (key == 4) { g_lockstep = value; return 0; }
+  if (key == 5) { g_verify_rows = value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -196,7 +198,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   memset(&p, 0, sizeof(p));
   p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
   p.block_tables = block_tables; p.seq_lens = seq_lens; p.out = out;
-  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = 1;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = 1; p.rows_per_wave = 16;
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.partition_size = partition_size;
@@ -280,6 +282,14 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
   p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
   p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens; p.out = out;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = T;
+  {
+    // One wave carries 16 query rows of a kv head, or 32 where that measured faster: with more than 16 rows
+    // and a batch large enough to be bandwidth-bound, for D = 64 and for fp8 pools (which fit the registers),
+    // and for bf16 at D = 128 (which spills a little) only from four 16-row groups on.
+    const int n_rows = (Hq / Hkv) * T, forced = g_verify_rows.load();
+    const bool wide = n_rows > 16 && B >= 16 && (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
+    p.rows_per_wave = forced == 16 || forced == 32 ? forced : (wide ? 32 : 16);
+  }
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);

@@ -80,7 +80,7 @@ struct VTile {
 };
 
 // Per-wavefront streaming state: Q fragments, online-softmax state and output
-// accumulators for up to 16 query rows of one kv head of one sequence.
+// accumulators for R groups of up to 16 query rows of one kv head of one sequence.
 //
 // MULTI = false: one query token per sequence; the rows are the q heads of the
 // kv group.  MULTI = true: p.T query tokens per sequence (the last query_lens[b]
@@ -90,7 +90,13 @@ struct VTile {
 // < ctx - tq + t + 1, so the causal mask is one more per-lane bound on the token
 // index; a row may then see no key at all in a tile or in a whole chunk, which the
 // softmax update and the stores allow for (state m = -inf, l = 0, o = 0).
-template <int D, bool FP8, bool MULTI = false>
+// R = 2 (MULTI only): the wave carries two 16-row operands, rows jbase + 16 rg + r,
+// against the same K and V registers, so a kv group of up to 32 rows streams its
+// context once through one wave.  LEAN (for R = 2 at D = 128, which would not fit
+// 256 registers otherwise): the Q fragments live in LDS, each lane reading back
+// the 16-byte pieces it wrote itself (no conflicts, no barrier), and V is single-
+// buffered: the next tile's V is requested right after the current P.V.
+template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false>
 struct DecodeWave {
   using KT = KTile<D, FP8>;
   using VT = VTile<D, FP8>;
@@ -99,7 +105,7 @@ struct DecodeWave {
   static constexpr int ESZ = FP8 ? 1 : 2;
 
   const DecodeParams& p;
-  int hk, hbase, nheads;     // kv head, first q head, valid q-head columns
+  int hk, hbase, nheads;     // kv head, first (virtual) q head, valid rows of this wave
   int r, g, krow;            // lane = 16 g + r; row order of the K sub-tile
   const int32_t* table;
   const char* kbase;
@@ -107,20 +113,22 @@ struct DecodeWave {
   long row_stride;           // bytes between consecutive tokens of a block
   int last;                  // ctx - 1 of the current sequence
   int jbase;                 // first row of this wave inside its kv group
-  int row_end;               // MULTI: keys [0, row_end) are visible to this lane's row (0: padding row)
-  long row_off;              // MULTI: element offset of this lane's row in q and out
-  bf16x8_t qf[KSTEPS];
-  bf16x8_t pf;               // P^T fragment of the current tile
-  f32x4_t oacc[VEC];
-  float m_run, l_run;
+  int row_end[R];            // MULTI: keys [0, row_end) are visible to this lane's row (0: padding row)
+  bf16x8_t qf[LEAN ? 1 : R][LEAN ? 1 : KSTEPS];
+  uint4* qlds;               // LEAN: this wave's [R][KSTEPS][64] fragment store in LDS
+  int qlane;                 // LEAN: lane index into it, re-made opaque per tile so the reads stay in the loop
+  bf16x8_t pf[R];            // P^T fragments of the current tile
+  f32x4_t oacc[R][VEC];
+  float m_run[R], l_run[R];
 
-  __device__ __forceinline__ DecodeWave(const DecodeParams& p_, int head_slot, int lane) : p(p_) {
+  __device__ __forceinline__ DecodeWave(const DecodeParams& p_, int head_slot, int lane, uint4* qlds_ = nullptr)
+      : p(p_), qlds(qlds_), qlane(lane) {
     const int n_rows = (p.Hq / p.Hkv) * (MULTI ? p.T : 1);
-    const int gchunks = (n_rows + 15) / 16;
+    const int gchunks = (n_rows + 16 * R - 1) / (16 * R);
     hk = head_slot / gchunks;
-    jbase = (head_slot % gchunks) * 16;
+    jbase = (head_slot % gchunks) * (16 * R);
     hbase = hk * n_rows + jbase;
-    nheads = min(16, n_rows - jbase);
+    nheads = min(16 * R, n_rows - jbase);
     r = lane & 15;
     g = lane >> 4;
     krow = 4 * (r & 3) + (r >> 2);
@@ -129,35 +137,47 @@ struct DecodeWave {
     vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
   }
 
+  // MULTI: element offset in q / out of row group rg's row of this lane, and its query token
+  __device__ __forceinline__ long row_offset(int b, int rg, int* t_out) const {
+    const int n_rep = p.Hq / p.Hkv;
+    const int j = jbase + 16 * rg + r;
+    const int t = j / n_rep;
+    *t_out = t;
+    return (((long)b * p.T + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D;
+  }
+
   // Start on sequence b (context ctx >= 1, of which the last tq tokens are the
   // queries): load Q^T fragments (B operand, zero for padded columns) and reset
   // the softmax state.
   __device__ __forceinline__ void begin(int b, int ctx, int tq = 1) {
     table = p.block_tables + (long)b * p.max_blocks;
     last = ctx - 1;
-    bool row_valid = r < nheads;
-    if (MULTI) {
-      const int n_rep = p.Hq / p.Hkv;
-      const int j = jbase + r;
-      const int t = j / n_rep;
-      row_off = (((long)b * p.T + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D;
-      row_valid = row_valid && t < tq;
-      row_end = row_valid ? ctx - tq + t + 1 : 0;
-    }
-    const uint16_t* qrow = MULTI ? (const uint16_t*)p.q + row_off
-                                 : (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      // d range of k-slots 8g..8g+7 in step s (must mirror the K loads below)
-      const int d0 = FP8 ? ((4 * (s >> 1) + g) * 16 + (s & 1) * 8) : ((4 * s + g) * 8);
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (row_valid) v = *(const uint4*)(qrow + d0);
-      qf[s] = __builtin_bit_cast(bf16x8_t, v);
-    }
+    for (int rg = 0; rg < R; ++rg) {
+      bool row_valid = 16 * rg + r < nheads;
+      const uint16_t* qrow;
+      if (MULTI) {
+        int t;
+        qrow = (const uint16_t*)p.q + row_offset(b, rg, &t);
+        row_valid = row_valid && t < tq;
+        row_end[rg] = row_valid ? ctx - tq + t + 1 : 0;
+      } else {
+        qrow = (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
+      }
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) oacc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    m_run = -INFINITY;
-    l_run = 0.f;
+      for (int s = 0; s < KSTEPS; ++s) {
+        // d range of k-slots 8g..8g+7 in step s (must mirror the K loads below)
+        const int d0 = FP8 ? ((4 * (s >> 1) + g) * 16 + (s & 1) * 8) : ((4 * s + g) * 8);
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (row_valid) v = *(const uint4*)(qrow + d0);
+        if (LEAN) qlds[(rg * KSTEPS + s) * 64 + qlane] = v;
+        else qf[rg][s] = __builtin_bit_cast(bf16x8_t, v);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) oacc[rg][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      m_run[rg] = -INFINITY;
+      l_run[rg] = 0.f;
+    }
   }
 
   // Pool rows of tokens t0 and t0+16 (the two 16-token halves of a tile each lie
@@ -211,69 +231,94 @@ struct DecodeWave {
   }
 
   // Scores of the tile at t0 (tokens >= t_end masked), online softmax update,
-  // rescale of the accumulators, P^T fragment.
+  // rescale of the accumulators, P^T fragments.
+  __device__ __forceinline__ bf16x8_t q_frag(int rg, int s) const {
+    if (LEAN) return __builtin_bit_cast(bf16x8_t, qlds[(rg * KSTEPS + s) * 64 + qlane]);
+    return qf[LEAN ? 0 : rg][LEAN ? 0 : s];
+  }
+
   __device__ __forceinline__ void scores_softmax(const KT& tl, const VT& vt, int t0, int t_end) {
-    f32x4_t sacc[2];
+    f32x4_t sacc[R][2];
+    if (LEAN) asm volatile("" : "+v"(qlane));
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      sacc[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (!FP8) {
+    for (int rg = 0; rg < R; ++rg) sacc[rg][0] = sacc[rg][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    // each Q fragment is fetched once and used for both 16-token halves
+    if (!FP8) {
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s)
-          sacc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              as_bf16x8(tl.k[u][s][0], tl.k[u][s][1], tl.k[u][s][2], tl.k[u][s][3]), qf[s], sacc[u], 0, 0, 0);
-      } else {
+      for (int s = 0; s < KSTEPS; ++s) {
 #pragma unroll
-        for (int s = 0; s < KLD; ++s) {
-          uint32_t w[8];
+        for (int rg = 0; rg < R; ++rg) {
+          const bf16x8_t q = q_frag(rg, s);
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            sacc[rg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                as_bf16x8(tl.k[u][s][0], tl.k[u][s][1], tl.k[u][s][2], tl.k[u][s][3]), q, sacc[rg][u], 0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < KLD; ++s) {
+        uint32_t w[2][8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             float f[4];
             fp8x4_to_float(tl.k[u][s][d], f);
-            w[2 * d] = pack_hi16(f[0], f[1]);
-            w[2 * d + 1] = pack_hi16(f[2], f[3]);
+            w[u][2 * d] = pack_hi16(f[0], f[1]);
+            w[u][2 * d + 1] = pack_hi16(f[2], f[3]);
           }
-          sacc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), qf[2 * s], sacc[u], 0, 0, 0);
-          sacc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[4], w[5], w[6], w[7]), qf[2 * s + 1], sacc[u], 0, 0, 0);
+        }
+#pragma unroll
+        for (int rg = 0; rg < R; ++rg) {
+          const bf16x8_t q0 = q_frag(rg, 2 * s), q1 = q_frag(rg, 2 * s + 1);
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            sacc[rg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[u][0], w[u][1], w[u][2], w[u][3]), q0, sacc[rg][u], 0, 0, 0);
+            sacc[rg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[u][4], w[u][5], w[u][6], w[u][7]), q1, sacc[rg][u], 0, 0, 0);
+          }
         }
       }
     }
-    float sv[8];
-    float tmax = -INFINITY;
-    if (MULTI) t_end = min(t_end, row_end);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const float sc = FP8 ? p.scale_log2e * tl.ksc[u] : p.scale_log2e;
+    for (int rg = 0; rg < R; ++rg) {
+      float sv[8];
+      float tmax = -INFINITY;
+      const int lim = MULTI ? min(t_end, row_end[rg]) : t_end;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = t0 + 16 * u + 4 * i + g;
-        const float x = sacc[u][i] * sc;
-        sv[4 * u + i] = tok < t_end ? x : -INFINITY;
-        tmax = fmaxf(tmax, sv[4 * u + i]);
+      for (int u = 0; u < 2; ++u) {
+        const float sc = FP8 ? p.scale_log2e * tl.ksc[u] : p.scale_log2e;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = t0 + 16 * u + 4 * i + g;
+          const float x = sacc[rg][u][i] * sc;
+          sv[4 * u + i] = tok < lim ? x : -INFINITY;
+          tmax = fmaxf(tmax, sv[4 * u + i]);
+        }
       }
-    }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);
-    // MULTI: a row that has seen no key yet keeps m = -inf; exponents are then taken against 0
-    const float m_ref = (MULTI && m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-    m_run = m_new;
-    float pr[8], psum = 0.f;
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run[rg], tmax);
+      // MULTI: a row that has seen no key yet keeps m = -inf; exponents are then taken against 0
+      const float m_ref = (MULTI && m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run[rg] - m_ref);
+      m_run[rg] = m_new;
+      float pr[8], psum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      pr[i] = __builtin_amdgcn_exp2f(sv[i] - m_ref);
-      psum += pr[i];
-    }
-    l_run = l_run * alpha + psum;
+      for (int i = 0; i < 8; ++i) {
+        pr[i] = __builtin_amdgcn_exp2f(sv[i] - m_ref);
+        psum += pr[i];
+      }
+      l_run[rg] = l_run[rg] * alpha + psum;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) oacc[e] *= alpha;
-    if (FP8) {
+      for (int e = 0; e < VEC; ++e) oacc[rg][e] *= alpha;
+      if (FP8) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { pr[i] *= vt.vsc[0]; pr[4 + i] *= vt.vsc[1]; }
+        for (int i = 0; i < 4; ++i) { pr[i] *= vt.vsc[0]; pr[4 + i] *= vt.vsc[1]; }
+      }
+      pf[rg] = as_bf16x8(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]),
+                         pack_bf16x2(pr[4], pr[5]), pack_bf16x2(pr[6], pr[7]));
     }
-    pf = as_bf16x8(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]),
-                   pack_bf16x2(pr[4], pr[5]), pack_bf16x2(pr[6], pr[7]));
   }
 
   // V^T fragments by in-register transpose, then O^T += V^T P^T.
@@ -286,7 +331,9 @@ struct DecodeWave {
 #pragma unroll
         for (int jp = 0; jp < 4; ++jp)
           w[jp] = __builtin_amdgcn_perm(tl.v[2 * jp + 1][e >> 1], tl.v[2 * jp][e >> 1], sel);
-        oacc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), pf, oacc[e], 0, 0, 0);
+#pragma unroll
+        for (int rg = 0; rg < R; ++rg)
+          oacc[rg][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), pf[rg], oacc[rg][e], 0, 0, 0);
       }
     } else {
 #pragma unroll
@@ -300,7 +347,9 @@ struct DecodeWave {
           uint32_t w[4];
 #pragma unroll
           for (int jp = 0; jp < 4; ++jp) w[jp] = pack_hi16(f[2 * jp][eb], f[2 * jp + 1][eb]);
-          oacc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), pf, oacc[e], 0, 0, 0);
+#pragma unroll
+          for (int rg = 0; rg < R; ++rg)
+            oacc[rg][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), pf[rg], oacc[rg][e], 0, 0, 0);
         }
       }
     }
@@ -314,11 +363,40 @@ struct DecodeWave {
   __device__ __forceinline__ void stream(int t_first, int t_step, int n, int t_end, bool lockstep = false) {
     if (n <= 0) return;
     KT ka, kb;
-    VT va, vb;
+    VT va;
     int t = t_first;
     load_k(ka, t);
     load_v(va, t);
     int i = 0;
+    if (LEAN) {
+      while (i + 2 < n) {
+        if (lockstep) __builtin_amdgcn_s_barrier();
+        load_k(kb, t + t_step);
+        scores_softmax(ka, va, t, t_end);
+        accumulate_pv(va);
+        load_v(va, t + t_step);
+        if (lockstep) __builtin_amdgcn_s_barrier();
+        load_k(ka, t + 2 * t_step);
+        scores_softmax(kb, va, t + t_step, t_end);
+        accumulate_pv(va);
+        load_v(va, t + 2 * t_step);
+        i += 2;
+        t += 2 * t_step;
+      }
+      if (i + 1 < n) {
+        load_k(kb, t + t_step);
+        scores_softmax(ka, va, t, t_end);
+        accumulate_pv(va);
+        load_v(va, t + t_step);
+        scores_softmax(kb, va, t + t_step, t_end);
+        accumulate_pv(va);
+      } else {
+        scores_softmax(ka, va, t, t_end);
+        accumulate_pv(va);
+      }
+      return;
+    }
+    VT vb;
     while (i + 2 < n) {
       if (lockstep) __builtin_amdgcn_s_barrier();
       load_k(kb, t + t_step);
@@ -346,44 +424,56 @@ struct DecodeWave {
     }
   }
 
-  // Sum of exponentials over the whole tile stream (all lanes of a head column).
-  __device__ __forceinline__ float total_l() const {
-    float l = l_run;
+  // Sum of exponentials over the whole tile stream (all lanes of a row).
+  __device__ __forceinline__ float total_l(int rg = 0) const {
+    float l = l_run[rg];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     return l;
   }
 
-  // Write this wave's normalised result for its head columns: lane (g, r) holds,
-  // for i = 0..3, the VEC consecutive d's starting at VEC * (4g + i).
-  __device__ __forceinline__ void store_final(int b, float l) const {
-    if (r >= nheads) return;
-    const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;    // padding rows: zeros
-    uint16_t* dst = MULTI ? (uint16_t*)p.out + row_off : (uint16_t*)p.out + ((long)b * p.Hq + hbase + r) * D;
+  // Write this wave's normalised result for its rows: lane (g, r) holds, for
+  // i = 0..3, the VEC consecutive d's starting at VEC * (4g + i).
+  __device__ __forceinline__ void store_final(int b) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint32_t w[VEC / 2];
+    for (int rg = 0; rg < R; ++rg) {
+      const float l = total_l(rg);
+      if (16 * rg + r >= nheads) continue;
+      const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;    // padding rows: zeros
+      int t;
+      uint16_t* dst = MULTI ? (uint16_t*)p.out + row_offset(b, rg, &t)
+                            : (uint16_t*)p.out + ((long)b * p.Hq + hbase + r) * D;
 #pragma unroll
-      for (int e = 0; e < VEC; e += 2)
-        w[e / 2] = (uint32_t)float_to_bf16_bits(oacc[e][i] * inv) |
-                   ((uint32_t)float_to_bf16_bits(oacc[e + 1][i] * inv) << 16);
-      uint32_t* o = (uint32_t*)(dst + VEC * (4 * g + i));
-      if (VEC == 8) *(uint4*)o = make_uint4(w[0], w[1], w[2], w[3]);
-      else *(uint2*)o = make_uint2(w[0], w[1 % (VEC / 2)]);
+      for (int i = 0; i < 4; ++i) {
+        uint32_t w[VEC / 2];
+#pragma unroll
+        for (int e = 0; e < VEC; e += 2)
+          w[e / 2] = (uint32_t)float_to_bf16_bits(oacc[rg][e][i] * inv) |
+                     ((uint32_t)float_to_bf16_bits(oacc[rg][e + 1][i] * inv) << 16);
+        uint32_t* o = (uint32_t*)(dst + VEC * (4 * g + i));
+        if (VEC == 8) *(uint4*)o = make_uint4(w[0], w[1], w[2], w[3]);
+        else *(uint2*)o = make_uint2(w[0], w[1 % (VEC / 2)]);
+      }
     }
   }
-  __device__ __forceinline__ void store_partial(long slot, float l) const {
-    if (r >= nheads) return;
-    const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;
-    float* dst = p.ws_out + slot * D;
+  // Split-K partials of this wave's rows: slot(row) = (hbase + row) * slots_per_head + piece
+  __device__ __forceinline__ void store_partial(long slots_per_head, long piece) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int rg = 0; rg < R; ++rg) {
+      const float l = total_l(rg);
+      if (16 * rg + r >= nheads) continue;
+      const long slot = (long)(hbase + 16 * rg + r) * slots_per_head + piece;
+      const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;
+      float* dst = p.ws_out + slot * D;
 #pragma unroll
-      for (int e = 0; e < VEC; e += 4)
-        *(float4*)(dst + VEC * (4 * g + i) + e) =
-            make_float4(oacc[e][i] * inv, oacc[e + 1][i] * inv, oacc[e + 2][i] * inv, oacc[e + 3][i] * inv);
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int e = 0; e < VEC; e += 4)
+          *(float4*)(dst + VEC * (4 * g + i) + e) =
+              make_float4(oacc[rg][e][i] * inv, oacc[rg][e + 1][i] * inv, oacc[rg][e + 2][i] * inv, oacc[rg][e + 3][i] * inv);
+      }
+      if (g == 0) { p.ws_ml[slot * 2] = m_run[rg]; p.ws_ml[slot * 2 + 1] = l; }
     }
-    if (g == 0) { p.ws_ml[slot * 2] = m_run; p.ws_ml[slot * 2 + 1] = l; }
   }
 };
 
@@ -391,9 +481,10 @@ __device__ __forceinline__ int clamp_ctx(const DecodeParams& p, int b) {
   return min(max(p.seq_lens[b], 0), p.max_seq_len);
 }
 
-// 16-row groups over all kv heads: rows of a kv head = its q heads x query tokens
+// Waves' worth of rows over all kv heads: rows of a kv head = its q heads x query tokens,
+// p.rows_per_wave (16 or 32) of them per wave
 __host__ __device__ __forceinline__ int head_slots_of(const DecodeParams& p) {
-  return p.Hkv * (((p.Hq / p.Hkv) * p.T + 15) / 16);
+  return p.Hkv * (((p.Hq / p.Hkv) * p.T + p.rows_per_wave - 1) / p.rows_per_wave);
 }
 
 // ---------------------------------------------------------------------------
@@ -432,11 +523,11 @@ __global__ __launch_bounds__(NW * 64, 2) void decode_mfma_kernel(DecodeParams p)
   __shared__ __attribute__((aligned(16))) float sm_o[NW][16][OSTRIDE];
   const float l_tot = w.total_l();
   const int r = w.r, g = w.g, nheads = w.nheads;
-  if (g == 0) { sm_m[wave][r] = w.m_run; sm_l[wave][r] = l_tot; }
+  if (g == 0) { sm_m[wave][r] = w.m_run[0]; sm_l[wave][r] = l_tot; }
   if (r < nheads) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e)   // value for d = VEC*(4g+i) + e stored at e*16 + 4g + i
-      *(f32x4_t*)&sm_o[wave][r][e * 16 + 4 * g] = w.oacc[e];
+      *(f32x4_t*)&sm_o[wave][r][e * 16 + 4 * g] = w.oacc[0][e];
   }
   __syncthreads();
   for (int idx = tid; idx < nheads * D; idx += NW * 64) {
@@ -506,9 +597,11 @@ __device__ __forceinline__ int scan_tiles(const DecodeParams& p, int lane, int f
   return base;
 }
 
-template <int D, bool FP8, bool MULTI>
+template <int D, bool FP8, bool MULTI, int R>
 __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p) {
-  using W = DecodeWave<D, FP8, MULTI>;
+  constexpr bool LEAN = R == 2 && D == 128;
+  using W = DecodeWave<D, FP8, MULTI, R, LEAN>;
+  __shared__ uint4 q_store[LEAN ? 8 * R * W::KSTEPS * 64 : 1];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int head_slots = head_slots_of(p);
@@ -529,7 +622,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
   b = __builtin_amdgcn_readfirstlane(b);
   start = __builtin_amdgcn_readfirstlane(start);
 
-  W w(p, hs, lane);
+  W w(p, hs, lane, LEAN ? q_store + wave * (R * W::KSTEPS * 64) : nullptr);
   while (f < f_end) {
     const int ctx = clamp_ctx(p, b);
     const int T = tiles_of(ctx);
@@ -538,13 +631,9 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
     const int n = min(T - ti, f_end - f);
     w.begin(b, ctx, MULTI ? min(min(max(p.query_lens[b], 0), p.T), ctx) : 1);
     w.stream(ti << 5, 32, n, ctx, p.bal_lockstep != 0);
-    const float l = w.total_l();
     const int c_first = start / L, c_last = (start + T - 1) / L;
-    if (c_first == c_last) {
-      w.store_final(b, l);
-    } else if (w.r < w.nheads) {
-      w.store_partial((long)(w.hbase + w.r) * (p.B + gv) + b + cv, l);
-    }
+    if (c_first == c_last) w.store_final(b);
+    else w.store_partial(p.B + gv, b + cv);
     f += n;
     start += T;
     ++b;
@@ -645,10 +734,12 @@ template <int D, bool FP8>
 hipError_t launch_balanced_typed(const DecodeParams& p, hipStream_t s) {
   const int head_slots = head_slots_of(p);
   dim3 grid(p.bal_gv / p.bal_ns, (head_slots + p.bal_hsw - 1) / p.bal_hsw);
-  if (p.query_lens)
-    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
+  if (p.query_lens && p.rows_per_wave == 32)
+    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 2>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
+  else if (p.query_lens)
+    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 1>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
   else
-    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, false>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
+    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, false, 1>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
   return hipGetLastError();
 }
 

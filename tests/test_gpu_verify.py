@@ -25,6 +25,16 @@ def _i32(x):
     return torch.from_numpy(np.asarray(x, dtype=np.int32)).cuda()
 
 
+@pytest.fixture(params=[16, 32], ids=["rows16", "rows32"])
+def rows(request):
+    """Force 16 or 32 query rows per wavefront (the library picks by shape otherwise)."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    lib.pa_debug_set(5, request.param)
+    yield request.param
+    lib.pa_debug_set(5, 0)
+
+
 def _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D):
     B = len(qlens)
     ctxs = [p + t for p, t in zip(prefixes, qlens)]
@@ -36,7 +46,7 @@ def _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D):
 @pytest.mark.parametrize("T,Hq,Hkv", [(4, 32, 8), (2, 8, 2), (5, 6, 2), (8, 32, 8), (16, 16, 4), (3, 40, 2),
                                       (64, 4, 4), (7, 1, 1)])
 @pytest.mark.parametrize("D,bs", [(128, 32), (64, 16)])
-def test_verify_matches_oracle(pa, T, Hq, Hkv, D, bs):
+def test_verify_matches_oracle(pa, rows, T, Hq, Hkv, D, bs):
     """Rows per kv head from 7 to 64: less than, exactly, and several times the 16-row operand."""
     rng = np.random.default_rng(1000 * T + Hq + D)
     qlens = [T, max(T - 1, 1), 1, T, 0, T]
@@ -52,7 +62,7 @@ def test_verify_matches_oracle(pa, T, Hq, Hkv, D, bs):
         assert np.all(got[b, n:] == 0)          # padding rows
 
 
-def test_verify_rows_without_keys_in_the_last_chunk(pa):
+def test_verify_rows_without_keys_in_the_last_chunk(pa, rows):
     """One long sequence spans every chunk of the schedule; its last 32-token tile holds 3 tokens,
     which the first 5 of 8 query tokens do not see, so their partial of that chunk is empty."""
     rng = np.random.default_rng(11)
@@ -84,8 +94,8 @@ def test_verify_agrees_with_tiled_prefill_and_decode(pa):
     assert np.max(np.abs(dev_to_f32(d) - a[full, T - 1])) <= 2 ** -6
 
 
-@pytest.mark.parametrize("D,Hq,Hkv,bs,T", [(128, 32, 8, 64, 4), (64, 8, 1, 16, 6)])
-def test_verify_fp8_pool(pa, D, Hq, Hkv, bs, T):
+@pytest.mark.parametrize("D,Hq,Hkv,bs,T", [(128, 32, 8, 64, 4), (64, 8, 1, 16, 6), (128, 16, 2, 32, 5)])
+def test_verify_fp8_pool(pa, rows, D, Hq, Hkv, bs, T):
     rng = np.random.default_rng(D + T)
     qlens, prefixes = [T, 1, T, T - 1], [0, 63, 1500, 300]
     q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
@@ -101,9 +111,9 @@ def test_verify_fp8_pool(pa, D, Hq, Hkv, bs, T):
     assert_close_abs(dev_to_f32(got), want, BF16_TOL)
 
 
-def test_verify_stale_pool_bytes_and_padding_rows_do_not_leak(pa):
+def test_verify_stale_pool_bytes_and_padding_rows_do_not_leak(pa, rows):
     rng = np.random.default_rng(13)
-    T, Hq, Hkv, D, bs = 6, 8, 2, 128, 32
+    T, Hq, Hkv, D, bs = 6, 8, 2, 128, 32      # 24 rows per kv head
     qlens, prefixes = [6, 3], [45, 3]
     q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
     want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.09)
