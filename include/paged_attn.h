@@ -76,6 +76,12 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
  * max_seq_len: upper bound of seq_lens (sizes the grid; 0 = max_blocks_per_seq *
  * block_size).  seq_lens[b] == 0 yields zeros.
  * q_dtype / kv_dtype: (F32, F32), (BF16, BF16) or (BF16, FP8_E4M3FN).
+ * sinks: NULL, or [Hq] float32 per-head logits that join every softmax as one more column and
+ *   are dropped afterwards (examples/models/gpt_oss/kernels/attention.py:137-148): they only
+ *   enlarge the denominator.  sliding_window: 0, or W >= 1: the query at position p sees the W
+ *   keys (p - W, p] (attention.py:118-125).  Both need the MFMA kernel's shapes (bf16 q, bf16 or
+ *   fp8 KV, D in {64, 128}, block_size a power of two >= 16); tiles wholly outside the window are
+ *   not read.
  */
 int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               const float* k_scale, const float* v_scale,
@@ -84,7 +90,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               int B, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks, int max_seq_len,
               float scale, int partition_size, int q_dtype, int kv_dtype,
-              void* stream);
+              const float* sinks, int sliding_window, void* stream);
 
 /*
  * Speculative verify: a few query tokens per sequence against the paged context, causal among
@@ -98,6 +104,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
  *   seq_lens[b]  context length including the query tokens, whose K/V are already in the pool
  *   kv_dtype     PA_BF16 or PA_FP8_E4M3FN (then k_scale / v_scale [num_blocks, Hkv] f32)
  *   workspace    pa_verify_workspace_bytes(B, T, Hq, D) bytes, 16-byte aligned
+ *   sinks, sliding_window   as for pa_decode (the window counts back from each query token's own position)
  * D in {64, 128}; block_size a power of two >= 16; T <= PA_VERIFY_MAX_TOKENS.
  */
 #define PA_VERIFY_MAX_TOKENS 64
@@ -108,7 +115,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
               void* out, void* workspace, size_t workspace_bytes,
               int B, int T, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks,
-              float scale, int kv_dtype, void* stream);
+              float scale, int kv_dtype, const float* sinks, int sliding_window, void* stream);
 
 /*
  * Paged chunked prefill with a cached prefix, causal: query token i of sequence

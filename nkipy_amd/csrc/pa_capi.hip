@@ -174,8 +174,9 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               int B, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks, int max_seq_len,
               float scale, int partition_size, int q_dtype, int kv_dtype,
-              void* stream) {
+              const float* sinks, int sliding_window, void* stream) {
   tl_error[0] = 0;
+  if (sliding_window < 0) return fail_arg("pa_decode: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
   if (B < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_decode: bad sizes B=%d Hq=%d Hkv=%d D=%d", B, Hq, Hkv, D);
   if (Hq % Hkv) return fail_arg("pa_decode: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0)
@@ -214,6 +215,10 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   if ((impl == 2 || impl == 3) && !mfma_ok) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
   if (impl == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
   const int kind = !mfma_ok || impl == 1 ? 1 : (impl == 2 ? 2 : 3);
+  if ((sinks || sliding_window > 0) && kind != 3)
+    return fail_arg("pa_decode: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
+                    "head_dim 64 or 128, block_size a power of two >= 16)");
+  p.sinks = sinks; p.window = sliding_window;
   if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
   if (kind == 3) {
     plan_decode_balanced(p, current_num_cus());
@@ -260,8 +265,9 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
               void* out, void* workspace, size_t workspace_bytes,
               int B, int T, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks,
-              float scale, int kv_dtype, void* stream) {
+              float scale, int kv_dtype, const float* sinks, int sliding_window, void* stream) {
   tl_error[0] = 0;
+  if (sliding_window < 0) return fail_arg("pa_verify: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
   if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_verify: bad sizes B=%d T=%d Hq=%d Hkv=%d D=%d", B, T, Hq, Hkv, D);
   if (Hq % Hkv) return fail_arg("pa_verify: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_verify: bad paging sizes");
@@ -293,6 +299,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
+  p.sinks = sinks; p.window = sliding_window;
   p.partition_size = p.max_seq_len;
   p.num_partitions = 1;
   p.scale_log2e = scale * kLog2e;

@@ -83,6 +83,8 @@ struct DecodeParams {
   float* ws_ml;             // [B, Hq, P, 2]
   int B, Hq, Hkv, D;
   int T;                    // query tokens per sequence (1: decode)
+  int window;               // sliding window in tokens (balanced schedule only), 0 = none
+  const float* sinks;       // [Hq] per-head sink logits (balanced schedule only) or null
   int rows_per_wave;        // query rows of a kv head carried by one wavefront: 16, or 32 (multi-token calls only)
   int block_size, max_blocks, num_blocks;
   int block_shift;          // log2(block_size), or -1 when not a power of two

@@ -137,13 +137,14 @@ struct DecodeWave {
     vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
   }
 
-  // MULTI: element offset in q / out of row group rg's row of this lane, and its query token
-  __device__ __forceinline__ long row_offset(int b, int rg, int* t_out) const {
+  // MULTI: element offset in q / out of row group rg's row of this lane, its query token and q head
+  __device__ __forceinline__ long row_offset(int b, int rg, int* t_out, int* head_out) const {
     const int n_rep = p.Hq / p.Hkv;
     const int j = jbase + 16 * rg + r;
     const int t = j / n_rep;
     *t_out = t;
-    return (((long)b * p.T + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D;
+    *head_out = hk * n_rep + (j - t * n_rep);
+    return (((long)b * p.T + t) * p.Hq + *head_out) * D;
   }
 
   // Start on sequence b (context ctx >= 1, of which the last tq tokens are the
@@ -157,8 +158,8 @@ struct DecodeWave {
       bool row_valid = 16 * rg + r < nheads;
       const uint16_t* qrow;
       if (MULTI) {
-        int t;
-        qrow = (const uint16_t*)p.q + row_offset(b, rg, &t);
+        int t, head;
+        qrow = (const uint16_t*)p.q + row_offset(b, rg, &t, &head);
         row_valid = row_valid && t < tq;
         row_end[rg] = row_valid ? ctx - tq + t + 1 : 0;
       } else {
@@ -293,9 +294,18 @@ struct DecodeWave {
           const int tok = t0 + 16 * u + 4 * i + g;
           const float x = sacc[rg][u][i] * sc;
           sv[4 * u + i] = tok < lim ? x : -INFINITY;
-          tmax = fmaxf(tmax, sv[4 * u + i]);
         }
       }
+      // sliding window: keys more than window - 1 tokens behind the row's own position are
+      // hidden; only the first tiles of a sequence's span reach below the newest row's bound
+      if (p.window > 0 && t0 < last + 1 - p.window) {
+        const int lo = (MULTI ? row_end[rg] : last + 1) - p.window;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (t0 + 16 * (i >> 2) + 4 * (i & 3) + g < lo) sv[i] = -INFINITY;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tmax = fmaxf(tmax, sv[i]);
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
       const float m_new = fmaxf(m_run[rg], tmax);
@@ -437,12 +447,14 @@ struct DecodeWave {
   __device__ __forceinline__ void store_final(int b) const {
 #pragma unroll
     for (int rg = 0; rg < R; ++rg) {
-      const float l = total_l(rg);
+      float l = total_l(rg);
       if (16 * rg + r >= nheads) continue;
-      const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;    // padding rows: zeros
-      int t;
-      uint16_t* dst = MULTI ? (uint16_t*)p.out + row_offset(b, rg, &t)
+      int t, head = hbase + r;
+      uint16_t* dst = MULTI ? (uint16_t*)p.out + row_offset(b, rg, &t, &head)
                             : (uint16_t*)p.out + ((long)b * p.Hq + hbase + r) * D;
+      // attention sink: one more term of the denominator, no value
+      if (p.sinks && l > 0.f) l += __builtin_amdgcn_exp2f(p.sinks[head] * kLog2e - m_run[rg]);
+      const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;    // padding rows: zeros
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         uint32_t w[VEC / 2];
@@ -479,6 +491,16 @@ struct DecodeWave {
 
 __device__ __forceinline__ int clamp_ctx(const DecodeParams& p, int b) {
   return min(max(p.seq_lens[b], 0), p.max_seq_len);
+}
+
+// Query tokens of sequence b (decode: 1)
+__device__ __forceinline__ int query_len(const DecodeParams& p, int b, int ctx) {
+  return p.query_lens ? min(min(max(p.query_lens[b], 0), p.T), ctx) : 1;
+}
+// First 32-token tile that any query row of sequence b sees (0 without a sliding window)
+__device__ __forceinline__ int first_tile(const DecodeParams& p, int b, int ctx) {
+  if (p.window <= 0) return 0;
+  return max(ctx - query_len(p, b, ctx) + 1 - p.window, 0) >> 5;
 }
 
 // Waves' worth of rows over all kv heads: rows of a kv head = its q heads x query tokens,
@@ -570,6 +592,11 @@ __global__ __launch_bounds__(NW * 64, 2) void decode_mfma_kernel(DecodeParams p)
 // [q head][b + chunk], merged by decode_balanced_reduce_kernel.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ int tiles_of(int ctx) { return (ctx + 31) >> 5; }
+// Tiles of sequence b that the schedule streams: all of them, or those the window reaches
+__device__ __forceinline__ int span_tiles(const DecodeParams& p, int b) {
+  const int ctx = clamp_ctx(p, b);
+  return tiles_of(ctx) - first_tile(p, b, ctx);
+}
 
 // Wave-wide: total number of tiles, and (if f >= 0) the sequence holding
 // flattened tile f with the number of tiles before it.
@@ -577,7 +604,7 @@ __device__ __forceinline__ int scan_tiles(const DecodeParams& p, int lane, int f
   int base = 0;
   bool found = false;
   for (int bb = 0; bb < p.B; bb += 64) {
-    const int t = (bb + lane < p.B) ? tiles_of(clamp_ctx(p, bb + lane)) : 0;
+    const int t = (bb + lane < p.B) ? span_tiles(p, bb + lane) : 0;
     int incl = t;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -625,10 +652,10 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
   W w(p, hs, lane, LEAN ? q_store + wave * (R * W::KSTEPS * 64) : nullptr);
   while (f < f_end) {
     const int ctx = clamp_ctx(p, b);
-    const int T = tiles_of(ctx);
+    const int T = span_tiles(p, b);
     if (T == 0) { ++b; continue; }
-    const int ti = f - start;
-    const int n = min(T - ti, f_end - f);
+    const int ti = f - start + first_tile(p, b, ctx);
+    const int n = min(T - (f - start), f_end - f);
     w.begin(b, ctx, MULTI ? min(min(max(p.query_lens[b], 0), p.T), ctx) : 1);
     w.stream(ti << 5, 32, n, ctx, p.bal_lockstep != 0);
     const int c_first = start / L, c_last = (start + T - 1) / L;
@@ -653,17 +680,19 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int lane = threadIdx.x & 63;
   int bb = 0, start = 0;
   const int N = scan_tiles(p, lane, -1, &bb, &start);
-  const int T = tiles_of(clamp_ctx(p, b));
+  const int T = span_tiles(p, b);
   constexpr int QUADS = D / 4;
   const int item = blockIdx.y * (256 / G) + threadIdx.x / G;
   const int g = threadIdx.x % G;
   const bool mine = item < p.Hq * p.T * QUADS;
   const int hq = item / QUADS, q4 = item % QUADS;     // hq: virtual head when p.T > 1
   uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hq) * D + 4 * q4;
+  int head = hq;                                      // the real q head of this item
   if (p.T > 1) {
     const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
     const int hk = hq / n_rows, j = hq % n_rows, t = j / n_rep;
-    dst = (uint16_t*)p.out + (((long)b * p.T + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D + 4 * q4;
+    head = hk * n_rep + (j - t * n_rep);
+    dst = (uint16_t*)p.out + (((long)b * p.T + t) * p.Hq + head) * D + 4 * q4;
   }
   if (T == 0) {
     if (mine && g == 0) *(uint2*)dst = make_uint2(0u, 0u);
@@ -674,7 +703,7 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   {   // tiles before sequence b = flattened index of its first tile
     int base = 0;
     for (int x = 0; x < b; x += 64) {
-      int t = (x + lane < b) ? tiles_of(clamp_ctx(p, x + lane)) : 0;
+      int t = (x + lane < b) ? span_tiles(p, x + lane) : 0;
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
       base += t;
@@ -712,6 +741,7 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
     m = m_new;
   }
   if (g != 0) return;
+  if (p.sinks && l > 0.f) l += exp2f(p.sinks[head] * kLog2e - m);    // attention sink: denominator only
   const float inv = l == 0.f ? 0.f : 1.f / l;     // padding rows of a multi-token call: zeros
   *(uint2*)dst =
       make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));

@@ -97,6 +97,20 @@ def check_block_tables(block_tables, seq_lens, num_blocks, block_size):
                f"sequence {b}: block table entry outside [0, {num_blocks})")
 
 
+def _check_variant(sinks, sliding_window, Hq, ref):
+    """sinks [Hq] (any float dtype; passed on as float32) and the window size of the gpt-oss attention
+    variant (examples/models/gpt_oss/kernels/attention.py:117-148).  Returns (sinks_f32 or None, window int)."""
+    win = 0 if sliding_window is None else int(sliding_window)
+    _check(win >= 0 and (sliding_window is None or win >= 1), "sliding_window must be None or >= 1")
+    if sinks is not None:
+        _need_device("sinks", sinks)
+        _check(sinks.shape == (Hq,), f"sinks must have one logit per q head ([{Hq}])")
+        _check(sinks.is_floating_point(), "sinks must be floating point")
+        _check(sinks.device == ref.device, f"sinks is on {sinks.device}, expected {ref.device}")
+        sinks = sinks.to(torch.float32).contiguous()
+    return sinks, win
+
+
 def decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size) -> int:
     return int(_lib.load().pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size))
 
@@ -111,7 +125,8 @@ def _workspace(device, nbytes):
 
 
 def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, v_scale=None,
-           partition_size=512, max_seq_len=None, out=None, workspace=None, validate_tables=False):
+           partition_size=512, max_seq_len=None, out=None, workspace=None, validate_tables=False,
+           sinks=None, sliding_window=None):
     """out[b, h] = softmax(q[b, h] . K_b^T * scale) V_b over the paged context.
 
     q [B, Hq, D] (float32 or bfloat16); k_cache/v_cache [num_blocks, block_size, Hkv, D]
@@ -119,6 +134,8 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
     float32; block_tables int32 [B, max_blocks]; seq_lens int32 [B].
     max_seq_len: host-known upper bound of seq_lens (sizes the split-K grid
     without a device sync; default = table capacity).
+    sinks [Hq]: per-head logits that join the softmax as one more column and carry no value;
+    sliding_window W: only the last W keys are visible (bf16 / fp8 pools, head_dim 64 or 128).
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache),
@@ -145,6 +162,7 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
     else:
         _check(kv_code == q_code, f"KV dtype {k_cache.dtype} does not match q dtype {q.dtype}")
         _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
+    sinks, win = _check_variant(sinks, sliding_window, Hq, q)
     _check(isinstance(partition_size, int) and partition_size > 0, "partition_size must be a positive int")
     cap = block_tables.shape[1] * block_size
     msl = cap if max_seq_len is None else int(max_seq_len)
@@ -169,7 +187,7 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
         rc = lib.pa_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                            _ptr(block_tables), _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes,
                            B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
-                           float(scale), partition_size, q_code, kv_code, _stream_ptr(q.device))
+                           float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, _stream_ptr(q.device))
     _raise_on(rc, "pa_decode")
     return out
 
@@ -183,7 +201,7 @@ def verify_supported(T, D, block_size) -> bool:
 
 
 def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
-            out=None, workspace=None, route=None, validate_tables=False):
+            out=None, workspace=None, route=None, validate_tables=False, sinks=None, sliding_window=None):
     """Chunked prefill against a cached prefix (causal).
 
     q [B, T, Hq, D] bfloat16 holds the last query_lens[b] tokens of each sequence
@@ -195,7 +213,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query
     rows (HBM-bound: the context is read once per kv head); longer ones through the tiled
     matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
-    (float8_e4m3fn / uint8 codes with k_scale, v_scale) are read by the verify kernel only.
+    (float8_e4m3fn / uint8 codes with k_scale, v_scale), sinks and sliding_window (as in
+    `decode`, the window counted back from each query token) are the verify kernel's only.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -221,14 +240,17 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     else:
         _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
     _check(route in (None, "verify", "tiled"), "route must be None, 'verify' or 'tiled'")
+    sinks, win = _check_variant(sinks, sliding_window, Hq, q)
+    variant = sinks is not None or win > 0
     can_verify = verify_supported(T, D, block_size)
     if route is None:
-        route = "verify" if can_verify and (kv_code == FP8 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
+        route = "verify" if can_verify and (kv_code == FP8 or variant or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")
     else:
         _check(kv_code == BF16, "fp8 KV caches are read by the verify kernel only (T <= 64, head_dim 64 or 128)")
+        _check(not variant, "sinks and sliding_window are the verify kernel's only (T <= 64, head_dim 64 or 128)")
     _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
                  query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out)
     if validate_tables:
@@ -250,7 +272,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
             rc = lib.pa_verify(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                                _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), _ptr(out),
                                _ptr(workspace), ws_bytes, B, T, Hq, Hkv, D, block_size,
-                               block_tables.shape[1], num_blocks, float(scale), kv_code, _stream_ptr(q.device))
+                               block_tables.shape[1], num_blocks, float(scale), kv_code, _ptr(sinks), win,
+                               _stream_ptr(q.device))
         _raise_on(rc, "pa_verify")
         return out
     with torch.cuda.device(q.device):

@@ -15,6 +15,9 @@ in the one-dynamic-index `np.take` form the reference's tracer supports:
 * additive causal mask  examples/models/qwen3/kernels/attention.py:124-134
 * multi-token-at-offset examples/models/gpt_oss/kernels/attention.py:85,117-135
   ("query at start_pos+i attends to keys <= start_pos+i")
+* sliding window, sinks examples/models/gpt_oss/kernels/attention.py:118-125 (keys
+                        further back than W tokens masked), 137-148 (per-head logit
+                        as one more softmax column, dropped afterwards)
 * softmax               examples/models/qwen3/kernels/softmax.py:4-6
 * weights @ values      examples/models/qwen3/kernels/attention.py:139-144
 * cache layout/write-before-attend   examples/models/qwen3/qwen3.py:54-71,
@@ -46,6 +49,9 @@ dense_attention        float64 triple-loop brute force on tiny inputs; torch
 paged_decode/prefill   identity table over a reshaped dense cache == dense
                        attention; GQA == MHA on np.repeat'ed KV; T=1 prefill ==
                        decode; P=0 prefill == plain causal
+sliding window, sinks  float64 brute force; W >= context == no window; W = 1 ==
+                       the query's own V row; sink = -inf == no sink; a sink is a
+                       key with a zero value row; a huge sink drives the output to 0
 merge_partitions       split-K merge == single pass in float64 for any split
 blocksparse_prefill    == dense attention under the expanded boolean mask;
                        all-active pattern == dense causal
@@ -368,13 +374,20 @@ def softmax_lastaxis(x) -> np.ndarray:
     return e / np.sum(e, axis=-1, keepdims=True)
 
 
-def dense_attention(q, k, v, scale, *, prefix=None, mask=None, acc=np.float32) -> np.ndarray:
+def dense_attention(q, k, v, scale, *, prefix=None, mask=None, window=None, sinks=None,
+                    acc=np.float32) -> np.ndarray:
     """softmax(q k^T * scale + mask) v for ONE sequence.
 
     q [T, Hq, D], k/v [S, Hkv, D] (float), Hq % Hkv == 0.
     prefix: if not None, query i sees keys j <= prefix + i (additive -100000
             mask as in attention.py:124-134; decode is T == 1, prefix == S-1).
     mask:   optional boolean [Hq or 1, T, S], True = visible (ANDed with causal).
+    window: sliding window W (needs prefix): query at position p = prefix + i does not
+            see keys j <= p - W, i.e. it sees the W keys (p - W, p]
+            (examples/models/gpt_oss/kernels/attention.py:118-125, np.tril(..., k=-W)).
+    sinks:  [Hq] per-head logits appended to every score row as one more column
+            before the softmax and dropped after it (gpt_oss attention.py:137-148):
+            they take probability mass and contribute no value.
     Returns [T, Hq, D] in `acc` precision (no output rounding here).
     """
     q = np.asarray(q, dtype=acc)
@@ -393,17 +406,27 @@ def dense_attention(q, k, v, scale, *, prefix=None, mask=None, acc=np.float32) -
         jj = np.arange(S)[None, :]
         ii = np.arange(T)[:, None]
         visible = visible & (jj <= (int(prefix) + ii))[None]
+    if window is not None:
+        assert prefix is not None and int(window) >= 1
+        jj = np.arange(S)[None, :]
+        ii = np.arange(T)[:, None]
+        visible = visible & ((int(prefix) + ii) - jj < int(window))[None]
     if mask is not None:
         visible = visible & np.asarray(mask, dtype=bool)
     scores = scores + np.where(visible, acc(0), acc(NEG_MASK))
-    weights = softmax_lastaxis(scores)
+    if sinks is not None:
+        sink_col = np.broadcast_to(np.asarray(sinks, dtype=acc).reshape(Hq, 1, 1), (Hq, T, 1))
+        weights = softmax_lastaxis(np.concatenate([scores, sink_col], axis=-1))[:, :, :S]
+    else:
+        weights = softmax_lastaxis(scores)
     out = np.matmul(weights, vals)  # [Hq, T, D]
     return out.transpose(1, 0, 2)
 
 
-def attention_bruteforce_f64(q, k, v, scale, *, prefix=None, mask=None) -> np.ndarray:
+def attention_bruteforce_f64(q, k, v, scale, *, prefix=None, mask=None, window=None, sinks=None) -> np.ndarray:
     """Same contract as dense_attention, written as explicit float64 loops with
-    hard masking (masked keys are skipped, not offset).  Tiny inputs only."""
+    hard masking (masked keys are skipped, not offset; a sink is one more term of
+    the denominator).  Tiny inputs only."""
     q = np.asarray(q, dtype=np.float64)
     k = np.asarray(k, dtype=np.float64)
     v = np.asarray(v, dtype=np.float64)
@@ -418,15 +441,17 @@ def attention_bruteforce_f64(q, k, v, scale, *, prefix=None, mask=None) -> np.nd
             for j in range(S):
                 if prefix is not None and j > prefix + t:
                     continue
+                if window is not None and j <= prefix + t - window:
+                    continue
                 if mask is not None:
                     mh = h if np.asarray(mask).shape[0] > 1 else 0
                     if not mask[mh][t][j]:
                         continue
                 js.append(j)
             s = [float(scale) * sum(q[t, h, d] * k[j, hk, d] for d in range(D)) for j in js]
-            mx = max(s)
+            mx = max(s) if sinks is None else max(s + [float(sinks[h])])
             w = [np.exp(x - mx) for x in s]
-            z = sum(w)
+            z = sum(w) + (0.0 if sinks is None else np.exp(float(sinks[h]) - mx))
             for d in range(D):
                 out[t, h, d] = sum(wi * v[j, hk, d] for wi, j in zip(w, js)) / z
     return out
@@ -444,7 +469,8 @@ def _pool_f32_rows(cache, scale_tbl, table_row, ctx):
 
 
 def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *,
-                 k_scale=None, v_scale=None, q_dtype="fp32", acc=np.float32) -> np.ndarray:
+                 k_scale=None, v_scale=None, q_dtype="fp32", acc=np.float32,
+                 sliding_window=None, sinks=None) -> np.ndarray:
     """One new query token per sequence against its paged context.
 
     q            [B, Hq, D]       float32 values (or uint16 bf16 bits)
@@ -454,6 +480,7 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *,
                  the current token's K/V already written: attention.py:100-106)
     Returns      [B, Hq, D] float32 holding values rounded to `q_dtype`.
     A sequence with seq_len == 0 yields zeros.
+    sliding_window / sinks [Hq]: as in dense_attention (gpt_oss attention.py:117-148).
     """
     qf = to_f32(q)
     B, Hq, D = qf.shape
@@ -464,14 +491,14 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *,
             continue
         k = _pool_f32_rows(k_cache, k_scale, block_tables[b], ctx)
         v = _pool_f32_rows(v_cache, v_scale, block_tables[b], ctx)
-        o = dense_attention(qf[b][None], k, v, scale, prefix=ctx - 1, acc=acc)
+        o = dense_attention(qf[b][None], k, v, scale, prefix=ctx - 1, window=sliding_window, sinks=sinks, acc=acc)
         out[b] = o[0]
     return round_output(out, q_dtype)
 
 
 def paged_prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *,
                   k_scale=None, v_scale=None, q_dtype="bf16", acc=np.float32,
-                  seqs=None, heads=None) -> np.ndarray:
+                  seqs=None, heads=None, sliding_window=None, sinks=None) -> np.ndarray:
     """Chunked prefill: the last query_lens[b] tokens of each sequence attend to
     the whole paged context causally (query i sees keys <= prefix_b + i, with
     prefix_b = seq_lens[b] - query_lens[b]); the new tokens' K/V are already in
@@ -499,7 +526,8 @@ def paged_prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale
             if not hs:
                 continue
             o = dense_attention(qf[b, :tq][:, hs], k[:, hk:hk + 1], v[:, hk:hk + 1],
-                                scale, prefix=prefix, acc=acc)
+                                scale, prefix=prefix, window=sliding_window,
+                                sinks=None if sinks is None else np.asarray(sinks)[hs], acc=acc)
             out[b, :tq][:, hs] = o
     return round_output(out, q_dtype)
 

@@ -1,0 +1,139 @@
+"""GPU parity: sliding window and attention sinks (the gpt-oss attention variant,
+examples/models/gpt_oss/kernels/attention.py:117-148) in decode and speculative verify vs the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_attention_oracle as O
+from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_bits, dev_to_f32, make_paged
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2
+FP8_TOL = 5e-2
+
+
+@pytest.fixture(scope="module")
+def pa():
+    import nkipy_amd
+    from nkipy_amd import _lib
+    _lib.load()
+    return nkipy_amd
+
+
+def _i32(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.int32)).cuda()
+
+
+def _f32(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.float32)).cuda()
+
+
+CTXS = [1, 31, 32, 33, 64, 65, 200, 1500, 4097]
+
+
+@pytest.mark.parametrize("window", [None, 1, 2, 31, 32, 33, 128, 5000])
+@pytest.mark.parametrize("with_sinks", [False, True])
+@pytest.mark.parametrize("D,Hq,Hkv,bs", [(64, 8, 1, 16), (128, 32, 8, 32)])
+def test_decode_window_and_sinks(pa, window, with_sinks, D, Hq, Hkv, bs):
+    if window is None and not with_sinks:
+        pytest.skip("plain decode is covered elsewhere")
+    rng = np.random.default_rng(7 + (window or 0) + D)
+    B = len(CTXS)
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, CTXS)
+    k, v = O.round_to_bf16(k), O.round_to_bf16(v)
+    q = O.round_to_bf16(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32) * 2) if with_sinks else None
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_decode(q, k, v, tables, np.asarray(CTXS, np.int32), scale, q_dtype="bf16",
+                          sliding_window=window, sinks=sinks)
+    got = pa.decode(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(CTXS), scale,
+                    sliding_window=window, sinks=None if sinks is None else bf16_to_dev(sinks))
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_decode_window_fp8_long_single_sequence(pa):
+    """One 20 000-token sequence cut into every chunk of the schedule; with a 128-token window only the
+    last five tiles are streamed."""
+    rng = np.random.default_rng(21)
+    D, Hq, Hkv, bs, ctx = 128, 16, 2, 64, 20000
+    k, v, tables = make_paged(rng, 1, Hkv, D, bs, [ctx])
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    q = O.round_to_bf16(rng.standard_normal((1, Hq, D)).astype(np.float32))
+    sinks = rng.standard_normal(Hq).astype(np.float32)
+    for window in (128, 3000, None):
+        want = O.paged_decode(q, kq, vq, tables, np.asarray([ctx], np.int32), 0.09, k_scale=ks, v_scale=vs,
+                              q_dtype="bf16", sliding_window=window, sinks=sinks)
+        got = pa.decode(bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+                        torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32([ctx]), 0.09,
+                        k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(),
+                        sliding_window=window, sinks=_f32(sinks))
+        torch.cuda.synchronize()
+        assert_close_abs(dev_to_f32(got), want, FP8_TOL)
+
+
+def test_neutral_options_change_nothing(pa):
+    """A window at least as long as every context and sinks of -inf give the plain result bit for bit."""
+    rng = np.random.default_rng(22)
+    D, Hq, Hkv, bs = 128, 8, 2, 32
+    ctxs = [5, 700, 2049]
+    k, v, tables = make_paged(rng, len(ctxs), Hkv, D, bs, ctxs)
+    q = rng.standard_normal((len(ctxs), Hq, D)).astype(np.float32)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), 0.09)
+    plain = dev_bits(pa.decode(*args))
+    assert np.array_equal(dev_bits(pa.decode(*args, sliding_window=2049)), plain)
+    assert np.array_equal(dev_bits(pa.decode(*args, sinks=_f32(np.full(Hq, -np.inf)))), plain)
+    assert not np.array_equal(dev_bits(pa.decode(*args, sliding_window=2048)), plain)
+
+
+@pytest.fixture(params=[16, 32], ids=["rows16", "rows32"])
+def rows(request):
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    lib.pa_debug_set(5, request.param)
+    yield request.param
+    lib.pa_debug_set(5, 0)
+
+
+@pytest.mark.parametrize("window", [1, 3, 30, 33, 64, 128, 4000])
+@pytest.mark.parametrize("T,Hq,Hkv,D,bs", [(4, 16, 2, 64, 16), (4, 32, 8, 128, 32), (40, 2, 1, 128, 32)])
+def test_verify_window_and_sinks(pa, rows, window, T, Hq, Hkv, D, bs):
+    """Query tokens of one sequence have different window starts, up to T - 1 tokens apart: rows that see
+    nothing in the first tiles of the span, and (T = 40) windows shorter than the query run."""
+    rng = np.random.default_rng(100 * T + window)
+    qlens = [T, max(T - 1, 1), 1, T, 0, T]
+    prefixes = [0, 300, 65, 1533, 40, 31]
+    B = len(qlens)
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, [max(c, 1) for c in ctxs])
+    k, v = O.round_to_bf16(k), O.round_to_bf16(v)
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_prefill(q, k, v, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale,
+                           q_dtype="bf16", sliding_window=window, sinks=sinks)
+    got = pa.prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), scale,
+                     sliding_window=window, sinks=bf16_to_dev(sinks))
+    torch.cuda.synchronize()
+    got = dev_to_f32(got)
+    assert_close_abs(got, want, BF16_TOL)
+    for b, n in enumerate(qlens):
+        assert np.all(got[b, n:] == 0)
+
+
+def test_variant_argument_errors(pa):
+    rng = np.random.default_rng(23)
+    k, v, tables = make_paged(rng, 1, 2, 128, 32, [40])
+    q = bf16_to_dev(rng.standard_normal((1, 4, 128)).astype(np.float32))
+    args = (q, bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32([40]), 0.09)
+    with pytest.raises(ValueError):
+        pa.decode(*args, sliding_window=0)
+    with pytest.raises(ValueError):
+        pa.decode(*args, sinks=_f32(np.zeros(3)))
+    with pytest.raises(RuntimeError):      # fp32 decode runs the scalar kernel, which has no window
+        pa.decode(q.float(), args[1].float(), args[2].float(), *args[3:], sliding_window=8)
+    q4 = bf16_to_dev(rng.standard_normal((1, 100, 4, 128)).astype(np.float32))
+    with pytest.raises(ValueError):        # longer than the verify kernel takes
+        pa.prefill(q4, *args[1:5], _i32([40]), 0.09, sliding_window=8)
