@@ -122,14 +122,16 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * b (i < query_lens[b]) sees keys j <= seq_lens[b] - query_lens[b] + i
  * (examples/models/gpt_oss/kernels/attention.py:85,127-135: "query at
  * start_pos+i attends to keys <= start_pos+i").  The new tokens' K/V are
- * already in the pool.  dtype: BF16 for q/k/v/out.
+ * already in the pool.  dtype: BF16 for q/k/v/out.  sinks / sliding_window as for pa_decode, the
+ * window counted back from each query token's own position; key tiles outside every row's
+ * window are skipped.
  */
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
-               float scale, int dtype, void* stream);
+               float scale, int dtype, const float* sinks, int sliding_window, void* stream);
 
 /*
  * Block-sparse causal prefill over dense q [B, S, Hq, D], k/v [B, S, Hkv, D]:

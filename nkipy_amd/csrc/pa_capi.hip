@@ -326,9 +326,10 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
-               float scale, int dtype, void* stream) {
+               float scale, int dtype, const float* sinks, int sliding_window, void* stream) {
   tl_error[0] = 0;
   if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_prefill: bad sizes");
+  if (sliding_window < 0) return fail_arg("pa_prefill: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
   if (Hq % Hkv) return fail_arg("pa_prefill: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   if (dtype != PA_BF16) return fail_arg("pa_prefill: only bf16 is supported (dtype=%d)", dtype);
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_prefill: bad paging sizes");
@@ -349,6 +350,9 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.scale_log2e = scale * kLog2e;
   p.impl = g_prefill_impl.load();
   if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
+  if ((sinks || sliding_window > 0) && (p.impl == 1 || !prefill_async_supported(p)))
+    return fail_arg("pa_prefill: sinks and sliding_window need the asynchronous-copy kernel (block_size a power of two >= 16)");
+  p.sinks = sinks; p.window = sliding_window;
   hipStream_t s = (hipStream_t)stream;
   profile_begin(s);
   hipError_t e = launch_prefill(p, s);

@@ -77,7 +77,7 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
 // MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16.
 // TT: 32-key sub-tiles per key tile (2: 64-key tiles).
-template <bool SPARSE, int MODE, int NW, int TT>
+template <bool SPARSE, int MODE, int NW, int TT, bool WIN>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -139,6 +139,9 @@ void prefill_async_kernel(PrefillParams p) {
   const bool wave_has_rows = wq_lo < tq;
   const int k_end = prefix + min(q0 + BMW, tq);                   // keys the workgroup needs: [0, k_end)
   const int ntiles = (k_end + BN - 1) / BN;
+  // sliding window (its own instantiation, so that the plain form carries none of its scalar
+  // work): the row at position pos sees keys (pos - win, pos]
+  const int win = WIN ? p.window : 0;
 
   // ---- DMA maps ---------------------------------------------------------------------
   // A tile is 2 UK units of 1 KB (4 rows): the first UK are K, the rest V.  Wave w issues
@@ -276,12 +279,13 @@ void prefill_async_kernel(PrefillParams p) {
   // does this wave compute on tile w.kt?
   auto tile_active = [&](const Walk& w) __attribute__((always_inline)) -> bool {
     bool act = wave_has_rows && w.kt * BN <= prefix + wq_hi;
+    if (win > 0) act = act && (w.kt + 1) * BN > prefix + wq_lo - win + 1;   // tile ends inside the first row's window
     if (SPARSE) act = act && w.kt <= qblk && (qblk - w.kt < p.sparse_local || w.ph == 0);
     return act;
   };
   // ---- ring of NST stages: tiles are requested NST-1 ahead; requests past the end are
   // repeated on the first tile so that the wait counter stays exact ------------------------
-  Walk w_first = {0, head_phase};
+  Walk w_first = {win > 0 ? max(prefix + q0 - win + 1, 0) / BN : 0, head_phase};   // first tile the first row sees
   walk_settle(w_first);
   const int kt_first = w_first.kt;
   Walk w_i = w_first;                 // next tile to request
@@ -368,6 +372,16 @@ void prefill_async_kernel(PrefillParams p) {
         for (int i = 0; i < 16; ++i) {
           const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
           sacc[tt][i] = key <= qlim ? sacc[tt][i] : -INFINITY;
+        }
+    }
+    if (win > 0 && key0 < prefix + wq_hi - win + 1) {         // tile starts below the last row's window
+      const int qlo = qlim - win + 1;
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
+          sacc[tt][i] = key >= qlo ? sacc[tt][i] : -INFINITY;
         }
     }
     float tmax = -INFINITY;
@@ -468,6 +482,8 @@ void prefill_async_kernel(PrefillParams p) {
     const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
     l_run = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
   }
+  // attention sink: a per-head logit that joins the softmax as one more column with no value
+  if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq] * kLog2e - m_ref);
   if (qrow < p.T && wq_lo < p.T) {
     uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
     const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
@@ -483,12 +499,12 @@ void prefill_async_kernel(PrefillParams p) {
   }
 }
 
-template <bool SPARSE, int MODE, int NW, int TT = 2>
+template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
@@ -499,7 +515,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   const long groups = (long)p.B * p.Hkv;
   const long total = 8 * ((groups + 7) / 8) * per_group;
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   return hipGetLastError();
 }
 
@@ -519,6 +535,10 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
   // and for the sparse form.
   if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
+  if (p.window > 0) {
+    if (sparse || !paged) return hipErrorInvalidValue;
+    return waves == 8 ? launch_typed<false, 1, 8, 2, true>(p, s) : launch_typed<false, 1, 4, 2, true>(p, s);
+  }
   if (waves == 8) {
     if (sparse) return launch_typed<true, 0, 8>(p, s);
     return paged ? launch_typed<false, 1, 8>(p, s) : launch_typed<false, 0, 8>(p, s);

@@ -213,8 +213,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query
     rows (HBM-bound: the context is read once per kv head); longer ones through the tiled
     matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
-    (float8_e4m3fn / uint8 codes with k_scale, v_scale), sinks and sliding_window (as in
-    `decode`, the window counted back from each query token) are the verify kernel's only.
+    (float8_e4m3fn / uint8 codes with k_scale, v_scale) are the verify kernel's only; sinks and
+    sliding_window (as in `decode`, the window counted back from each query token) work on both.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -241,16 +241,14 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
         _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
     _check(route in (None, "verify", "tiled"), "route must be None, 'verify' or 'tiled'")
     sinks, win = _check_variant(sinks, sliding_window, Hq, q)
-    variant = sinks is not None or win > 0
     can_verify = verify_supported(T, D, block_size)
     if route is None:
-        route = "verify" if can_verify and (kv_code == FP8 or variant or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
+        route = "verify" if can_verify and (kv_code == FP8 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")
     else:
         _check(kv_code == BF16, "fp8 KV caches are read by the verify kernel only (T <= 64, head_dim 64 or 128)")
-        _check(not variant, "sinks and sliding_window are the verify kernel's only (T <= 64, head_dim 64 or 128)")
     _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
                  query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out)
     if validate_tables:
@@ -279,7 +277,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     with torch.cuda.device(q.device):
         rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
-                            block_tables.shape[1], num_blocks, float(scale), BF16, _stream_ptr(q.device))
+                            block_tables.shape[1], num_blocks, float(scale), BF16, _ptr(sinks), win,
+                            _stream_ptr(q.device))
     _raise_on(rc, "pa_prefill")
     return out
 

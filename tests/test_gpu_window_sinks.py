@@ -134,6 +134,51 @@ def test_variant_argument_errors(pa):
         pa.decode(*args, sinks=_f32(np.zeros(3)))
     with pytest.raises(RuntimeError):      # fp32 decode runs the scalar kernel, which has no window
         pa.decode(q.float(), args[1].float(), args[2].float(), *args[3:], sliding_window=8)
+    k8, v8, t8 = make_paged(rng, 1, 2, 128, 24, [140])
     q4 = bf16_to_dev(rng.standard_normal((1, 100, 4, 128)).astype(np.float32))
-    with pytest.raises(ValueError):        # longer than the verify kernel takes
-        pa.prefill(q4, *args[1:5], _i32([40]), 0.09, sliding_window=8)
+    with pytest.raises(RuntimeError):      # a block size of 24 takes the register-staged prefill kernel, which has no window
+        pa.prefill(q4, bf16_to_dev(k8), bf16_to_dev(v8), _i32(t8), _i32([140]), _i32([100]), 0.09, sliding_window=8)
+
+
+@pytest.mark.parametrize("window", [1, 50, 64, 65, 128, 300, 5000])
+@pytest.mark.parametrize("waves", [4, 8])
+def test_tiled_prefill_window_and_sinks(pa, window, waves):
+    """Long query runs through the tiled kernel: windows shorter and longer than a 64-key tile, than a
+    wave's 32 rows and than the whole chunk; first tiles in which a wave's later rows see nothing."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(300 + window)
+    T, Hq, Hkv, D, bs = 200, 4, 2, 128, 32
+    qlens, prefixes = [200, 77, 1, 130], [0, 300, 65, 1000]
+    B = len(qlens)
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    k, v = O.round_to_bf16(k), O.round_to_bf16(v)
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_prefill(q, k, v, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale,
+                           q_dtype="bf16", sliding_window=window, sinks=sinks)
+    lib.pa_debug_set(3, waves)
+    try:
+        got = pa.prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), scale,
+                         sliding_window=window, sinks=bf16_to_dev(sinks), route="tiled")
+        torch.cuda.synchronize()
+    finally:
+        lib.pa_debug_set(3, 0)
+    got = dev_to_f32(got)
+    assert_close_abs(got, want, BF16_TOL)
+    assert np.all(got[1, 77:] == 0) and np.all(got[2, 1:] == 0)
+
+
+def test_tiled_prefill_neutral_options_change_nothing(pa):
+    rng = np.random.default_rng(31)
+    T, Hq, Hkv, D, bs = 300, 4, 2, 128, 32
+    ctxs = [300 + 700, 150 + 0]
+    k, v, tables = make_paged(rng, 2, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((2, T, Hq, D)).astype(np.float32)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32([300, 150]), 0.09)
+    plain = dev_bits(pa.prefill(*args))
+    assert np.array_equal(dev_bits(pa.prefill(*args, sliding_window=1000)), plain)
+    assert np.array_equal(dev_bits(pa.prefill(*args, sinks=_f32(np.full(Hq, -np.inf)))), plain)
+    assert not np.array_equal(dev_bits(pa.prefill(*args, sliding_window=999)), plain)
