@@ -190,11 +190,15 @@ class PagedAttention:
 
     def __init__(self, cache: PagedKVCache, n_heads: int, *, scale: Optional[float] = None, rope_base: Optional[float] = None,
                  max_positions: int = 0, q_norm_weight=None, k_norm_weight=None, norm_eps: float = 1e-6,
-                 partition_size: int = 512):
+                 partition_size: int = 512, sinks=None, sliding_window: Optional[int] = None):
         self.cache, self.n_heads = cache, n_heads
         self.scale = paged_attn.default_scale(cache.head_dim) if scale is None else float(scale)
         self.partition_size = partition_size
         self.q_norm_weight, self.k_norm_weight, self.norm_eps = q_norm_weight, k_norm_weight, norm_eps
+        # the gpt-oss layer variant (examples/models/gpt_oss/kernels/attention.py:117-148): per-head sink
+        # logits [n_heads] and a sliding window, fixed per layer
+        self.sinks = None if sinks is None else sinks.to(torch.float32).contiguous()
+        self.sliding_window = sliding_window
         self.rope = None
         if rope_base is not None:
             if max_positions <= 0:
@@ -234,9 +238,11 @@ class PagedAttention:
         if T == 1:
             paged_attn.decode(q[:, 0], c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self.scale,
                               k_scale=c.k_scale, v_scale=c.v_scale, partition_size=self.partition_size,
-                              max_seq_len=max(c.max_seq_len, 1), out=out[:, 0])
+                              max_seq_len=max(c.max_seq_len, 1), out=out[:, 0],
+                              sinks=self.sinks, sliding_window=self.sliding_window)
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:
             paged_attn.prefill(q, c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self._qlens, self.scale,
-                               k_scale=c.k_scale, v_scale=c.v_scale, out=out)
+                               k_scale=c.k_scale, v_scale=c.v_scale, out=out,
+                               sinks=self.sinks, sliding_window=self.sliding_window)
         return out

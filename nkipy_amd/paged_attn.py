@@ -243,7 +243,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     sinks, win = _check_variant(sinks, sliding_window, Hq, q)
     can_verify = verify_supported(T, D, block_size)
     if route is None:
-        route = "verify" if can_verify and (kv_code == FP8 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
+        # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
+        route = "verify" if can_verify and (kv_code == FP8 or D != 128 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")

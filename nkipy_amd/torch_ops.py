@@ -1,0 +1,113 @@
+"""The paged attention ops as PyTorch custom operators (`torch.ops.nkipy_amd.*`).
+
+A serving engine built on PyTorch-ROCm calls kernels through the dispatcher so that they can sit
+inside traced or compiled graphs; this is the MI355X counterpart of the reference's hook for
+hand-written kernels inside a traced function (`nki_custom_op`,
+nkipy/src/nkipy/core/nki_op.py:800-884): the operator is opaque to the tracer, declares what it
+mutates, and has a shape-only ("fake") implementation for tracing.  There is no CPU kernel behind
+any of them: host tensors raise NotImplementedError, as that hook does on the CPU backend
+(nki_op.py:480,557,719-722).
+
+Every operator writes into buffers the caller passes (`out`, the caches) and returns nothing, so
+the caller-allocates rule of nkipy/src/nkipy/runtime/device_tensor.py:51-74 carries over and a
+captured graph replays without allocations.  Optional tensors may be None; `sliding_window` 0 means
+none.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import paged_attn
+
+_NS = "nkipy_amd"
+
+
+def _win(w: int):
+    return None if w <= 0 else int(w)
+
+
+@torch.library.custom_op(f"{_NS}::paged_decode", mutates_args=("out",), device_types="cuda")
+def paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                 seq_lens: torch.Tensor, scale: float, out: torch.Tensor,
+                 k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                 max_seq_len: int = 0, sinks: Optional[torch.Tensor] = None, sliding_window: int = 0) -> None:
+    paged_attn.decode(q, k_cache, v_cache, block_tables, seq_lens, scale, k_scale=k_scale, v_scale=v_scale,
+                      max_seq_len=max_seq_len or None, out=out, sinks=sinks, sliding_window=_win(sliding_window))
+
+
+@torch.library.custom_op(f"{_NS}::paged_prefill", mutates_args=("out",), device_types="cuda")
+def paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                  seq_lens: torch.Tensor, query_lens: torch.Tensor, scale: float, out: torch.Tensor,
+                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                  sinks: Optional[torch.Tensor] = None, sliding_window: int = 0) -> None:
+    paged_attn.prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, k_scale=k_scale,
+                       v_scale=v_scale, out=out, sinks=sinks, sliding_window=_win(sliding_window))
+
+
+@torch.library.custom_op(f"{_NS}::blocksparse_prefill", mutates_args=("out",), device_types="cuda")
+def blocksparse_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, out: torch.Tensor,
+                        block: int = 64, local_blocks: int = 4, vert_stride: int = 8) -> None:
+    paged_attn.blocksparse_prefill(q, k, v, scale, block=block, local_blocks=local_blocks, vert_stride=vert_stride,
+                                   out=out)
+
+
+# Operators that write scale tables exist in a second form (`*_fp8`): a mutated argument of a custom
+# operator cannot be optional.
+@torch.library.custom_op(f"{_NS}::paged_kv_write", mutates_args=("k_cache", "v_cache"), device_types="cuda")
+def paged_kv_write(k_new: torch.Tensor, v_new: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   block_tables: torch.Tensor, seq_lens: torch.Tensor, query_lens: torch.Tensor) -> None:
+    paged_attn.kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens)
+
+
+@torch.library.custom_op(f"{_NS}::paged_kv_write_fp8", mutates_args=("k_cache", "v_cache", "k_scale", "v_scale"),
+                         device_types="cuda")
+def paged_kv_write_fp8(k_new: torch.Tensor, v_new: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                       k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
+                       seq_lens: torch.Tensor, query_lens: torch.Tensor) -> None:
+    paged_attn.kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens,
+                        k_scale=k_scale, v_scale=v_scale)
+
+
+@torch.library.custom_op(f"{_NS}::qk_norm_rope_kv_write", mutates_args=("q_out", "k_cache", "v_cache"),
+                         device_types="cuda")
+def qk_norm_rope_kv_write(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, q_out: torch.Tensor,
+                          k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                          seq_lens: torch.Tensor, query_lens: torch.Tensor, rope_cos: torch.Tensor,
+                          rope_sin: torch.Tensor, q_norm_weight: Optional[torch.Tensor] = None,
+                          k_norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> None:
+    paged_attn.qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, rope_cos,
+                                     rope_sin, q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight, eps=eps,
+                                     out=q_out)
+
+
+@torch.library.custom_op(f"{_NS}::qk_norm_rope_kv_write_fp8",
+                         mutates_args=("q_out", "k_cache", "v_cache", "k_scale", "v_scale"), device_types="cuda")
+def qk_norm_rope_kv_write_fp8(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, q_out: torch.Tensor,
+                              k_cache: torch.Tensor, v_cache: torch.Tensor, k_scale: torch.Tensor,
+                              v_scale: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                              query_lens: torch.Tensor, rope_cos: torch.Tensor, rope_sin: torch.Tensor,
+                              q_norm_weight: Optional[torch.Tensor] = None,
+                              k_norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> None:
+    paged_attn.qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, rope_cos,
+                                     rope_sin, q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight, eps=eps,
+                                     k_scale=k_scale, v_scale=v_scale, out=q_out)
+
+
+def _no_cpu(name):
+    def impl(*args, **kwargs):
+        raise NotImplementedError(f"{_NS}::{name} runs hand-written HIP kernels and has no CPU path; "
+                                  "pass tensors on a ROCm device")
+    return impl
+
+
+for _op, _name in ((paged_decode, "paged_decode"), (paged_prefill, "paged_prefill"),
+                   (blocksparse_prefill, "blocksparse_prefill"), (paged_kv_write, "paged_kv_write"),
+                   (paged_kv_write_fp8, "paged_kv_write_fp8"), (qk_norm_rope_kv_write, "qk_norm_rope_kv_write"),
+                   (qk_norm_rope_kv_write_fp8, "qk_norm_rope_kv_write_fp8")):
+    _op.register_kernel("cpu")(_no_cpu(_name))
+    _op.register_fake(lambda *args, **kwargs: None)      # outputs are caller-allocated: nothing to infer
+
+OPS = ("paged_decode", "paged_prefill", "blocksparse_prefill", "paged_kv_write", "paged_kv_write_fp8",
+       "qk_norm_rope_kv_write", "qk_norm_rope_kv_write_fp8")

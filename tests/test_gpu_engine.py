@@ -14,10 +14,11 @@ pytestmark = pytest.mark.gpu
 class _Mirror:
     """Dense per-sequence history kept by the oracle: rotated K, V as the reference's cache holds them."""
 
-    def __init__(self, n_slots, cos, sin, wq, wk, eps):
+    def __init__(self, n_slots, cos, sin, wq, wk, eps, window=None, sinks=None):
         self.k = [None] * n_slots
         self.v = [None] * n_slots
         self.cos, self.sin, self.wq, self.wk, self.eps = cos, sin, wq, wk, eps
+        self.window, self.sinks = window, sinks
 
     def step(self, xq, xk, xv, qlens, scale):
         B, T, Hq, D = xq.shape
@@ -37,7 +38,8 @@ class _Mirror:
             self.k[b] = k if self.k[b] is None else np.concatenate([self.k[b], k])
             self.v[b] = xv[b, :n] if self.v[b] is None else np.concatenate([self.v[b], xv[b, :n]])
             n_rep = Hq // k.shape[1]
-            o = O.dense_attention(q, O.repeat_kv(self.k[b], n_rep), O.repeat_kv(self.v[b], n_rep), scale, prefix=start)
+            o = O.dense_attention(q, O.repeat_kv(self.k[b], n_rep), O.repeat_kv(self.v[b], n_rep), scale, prefix=start,
+                                  window=self.window, sinks=self.sinks)
             out[b, :n] = O.round_output(o, "bf16")
         return out
 
@@ -89,6 +91,34 @@ def test_serving_loop_bf16_pool(rng, rope):
     assert cache.allocator.num_free > free_before
     run(21, [0, 21, 0, 0])
     run(1, [1, 1, 1, 1])
+
+
+def test_serving_loop_gpt_oss_variant(rng):
+    """head_dim 64, RoPE, per-head sinks and a 24-token sliding window (shorter than the prompts): prompt
+    chunks, verify-sized steps and decode steps all go through the decode-shaped kernel."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    S, Hq, Hkv, D, bs = 3, 8, 2, 64, 16
+    cache = PagedKVCache(num_blocks=30, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=8)
+    sinks = _rand(rng, Hq)
+    cos, sin = O.rope_tables(D, 128, 150000.0)
+    layer = PagedAttention(cache, Hq, rope_base=150000.0, max_positions=128, sinks=bf16_to_dev(sinks), sliding_window=24)
+    mirror = _Mirror(S, cos, sin, None, None, 1e-6, window=24, sinks=sinks)
+
+    def run(T, qlens):
+        xq, xk, xv = _rand(rng, (S, T, Hq, D)), _rand(rng, (S, T, Hkv, D)), _rand(rng, (S, T, Hkv, D))
+        got = dev_to_f32(layer.step(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv), qlens))
+        want = mirror.step(xq, xk, xv, qlens, layer.scale)
+        for b in range(S):
+            if qlens[b]:
+                assert_close_abs(got[b, :qlens[b]], want[b, :qlens[b]], 2e-2)
+
+    run(40, [40, 13, 0])            # prompts; slot 0's is longer than the window
+    for _ in range(3):
+        run(1, [1, 1, 0])
+    run(4, [4, 4, 0])               # speculative verify: the last accepted token plus three drafts
+    run(30, [0, 0, 30])
+    for _ in range(20):
+        run(1, [1, 1, 1])
 
 
 def test_serving_loop_fp8_pool(rng):

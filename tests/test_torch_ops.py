@@ -1,0 +1,83 @@
+"""The dispatcher-level operators: registration, schemas and the CPU refusal without a GPU; on the
+GPU the same results as the Python ops, through torch.ops and inside a captured HIP graph."""
+import numpy as np
+import pytest
+import torch
+
+from tests.pa_testlib import bf16_to_dev, dev_bits, make_paged
+
+
+def test_ops_are_registered_with_mutation_schemas():
+    import nkipy_amd.torch_ops as T
+    for name in T.OPS:
+        assert hasattr(torch.ops.nkipy_amd, name)
+    s = str(torch.ops.nkipy_amd.paged_decode.default._schema)
+    assert "Tensor(a6!) out" in s and "-> ()" in s
+    assert str(torch.ops.nkipy_amd.paged_kv_write.default._schema).count("!") == 2        # both caches
+    assert str(torch.ops.nkipy_amd.paged_kv_write_fp8.default._schema).count("!") == 4    # ... and both scale tables
+
+
+def test_ops_refuse_cpu_tensors_and_trace_with_fake_tensors():
+    import nkipy_amd.torch_ops  # noqa: F401
+    q = torch.zeros(2, 4, 64, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 16, 2, 64, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 2, dtype=torch.int32)
+    sl = torch.ones(2, dtype=torch.int32)
+    with pytest.raises(NotImplementedError):
+        torch.ops.nkipy_amd.paged_decode(q, kc, kc, bt, sl, 0.1, torch.empty_like(q))
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        fq = torch.zeros(2, 4, 64, dtype=torch.bfloat16, device="cuda")
+        fk = torch.zeros(4, 16, 2, 64, dtype=torch.bfloat16, device="cuda")
+        fb = torch.zeros(2, 2, dtype=torch.int32, device="cuda")
+        fs = torch.ones(2, dtype=torch.int32, device="cuda")
+        assert torch.ops.nkipy_amd.paged_decode(fq, fk, fk, fb, fs, 0.1, torch.empty_like(fq)) is None
+
+
+def _i32(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.int32)).cuda()
+
+
+@pytest.mark.gpu
+def test_ops_match_the_python_ops_and_replay_in_a_graph():
+    import nkipy_amd as pa
+    import nkipy_amd.torch_ops  # noqa: F401
+    rng = np.random.default_rng(5)
+    B, Hq, Hkv, D, bs = 3, 8, 2, 128, 32
+    ctxs = [40, 700, 2100]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    kd, vd, td, sd = bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs)
+    q = bf16_to_dev(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    sinks = torch.randn(Hq, device="cuda")
+    want = pa.decode(q, kd, vd, td, sd, 0.09, sinks=sinks, sliding_window=600)
+    out = torch.empty_like(q)
+    torch.ops.nkipy_amd.paged_decode(q, kd, vd, td, sd, 0.09, out, sinks=sinks, sliding_window=600)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(out), dev_bits(want))
+
+    # verify-sized prefill + the KV write in front of it, as one captured graph replayed on new inputs
+    T = 4
+    qlens = _i32([4, 4, 4])
+    xq = bf16_to_dev(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    xk = bf16_to_dev(rng.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    xv = bf16_to_dev(rng.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    o = torch.empty_like(xq)
+
+    def step():
+        torch.ops.nkipy_amd.paged_kv_write(xk, xv, kd, vd, td, sd, qlens)
+        torch.ops.nkipy_amd.paged_prefill(xq, kd, vd, td, sd, qlens, 0.09, o)
+
+    step()                                   # eager once: loads the library, sizes the cached workspace
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for _ in range(3):
+        for t in (xq, xk, xv):
+            t.copy_(bf16_to_dev(rng.standard_normal(tuple(t.shape)).astype(np.float32)))
+        g.replay()
+        torch.cuda.synchronize()
+        got = dev_bits(o).copy()
+        step()                               # the program's own eager work between replays
+        torch.cuda.synchronize()
+        assert np.array_equal(got, dev_bits(o))
