@@ -103,8 +103,9 @@ def _cpu_prefill_baseline(w, flops_fn, run_fn, desc):
 # of known size shows); the summaries with the commands are under profiles/.  Not re-measured at run time.
 MEASURED_TRAFFIC_BYTES = {
     2: {"bytes": 1_098_900_000, "source": "profiles/decode_balanced_kernel_C2.md"},
-    3: {"bytes": 394_700_000, "source": "profiles/prefill_async_kernel_C3.md"},
-    4: {"bytes": 692_400_000, "source": "profiles/prefill_async_kernel_C4.md"},
+    3: {"bytes": 385_200_000, "source": "profiles/prefill_async_kernel_C3.md"},
+    4: {"bytes": 743_900_000, "source": "profiles/prefill_async_kernel_C4.md"},
+    8: {"bytes": 1_123_600_000, "source": "profiles/decode_balanced_kernel_verify_T4.md"},
 }
 
 
@@ -189,7 +190,8 @@ def bench_verify(steps, warmup, lib, pa, W, T=4):
                    "algorithmic_bytes": ab},
         "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "decode_balanced_kernel (multi-token rows)",
+                     "traffic": _traffic(8)[0], "traffic_source": _traffic(8)[1],
+                     "kernel": "decode_balanced_kernel (multi-token rows)",
                      "kernel_avg_ms": round(kavg, 5), "launches_timed": len(kms)},
     }
     if not _NO_CPU:
