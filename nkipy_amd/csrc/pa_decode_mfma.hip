@@ -673,7 +673,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 // are zero-filled.
 // G consecutive lanes share one item and take every G-th piece of the sequence; their partial
 // merges are combined with a butterfly.  G = 1 when there are many sequences (each spans a few
-// chunks), 8 when there are few (one long sequence spans every chunk).
+// chunks), 8 or 32 when a sequence spans many.
 template <int D, int G>
 __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParams p) {
   const int b = blockIdx.x;
@@ -812,18 +812,22 @@ hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_decode_balanced_reduce(const DecodeParams& p, hipStream_t s) {
+template <int G>
+static hipError_t launch_reduce_g(const DecodeParams& p, hipStream_t s) {
   const int items = p.Hq * p.T * (p.D / 4);
-  if (p.B <= 8) {     // few sequences: each spans many chunks
-    dim3 grid(p.B, (items + 31) / 32);
-    if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, 8>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, 8>), grid, dim3(256), 0, s, p);
-  } else {
-    dim3 grid(p.B, (items + 255) / 256);
-    if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, 1>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, 1>), grid, dim3(256), 0, s, p);
-  }
+  dim3 grid(p.B, (items * G + 255) / 256);
+  if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, G>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, G>), grid, dim3(256), 0, s, p);
   return hipGetLastError();
+}
+
+hipError_t launch_decode_balanced_reduce(const DecodeParams& p, hipStream_t s) {
+  // lanes per item by the number of pieces a sequence is cut into on average: a sequence spans
+  // about gv / B chunks (few sequences, or few kv heads and hence several chunks per workgroup)
+  const int pieces = p.bal_gv / p.B;
+  if (pieces >= 64) return launch_reduce_g<32>(p, s);
+  if (pieces >= 8) return launch_reduce_g<8>(p, s);
+  return launch_reduce_g<1>(p, s);
 }
 
 }  // namespace pa
