@@ -205,7 +205,8 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * fixed-partition MFMA kernel (0 = default); key 2: its grid order (1 = kv head
  * fastest, the default; 0 = partition fastest); key 3: prefill kernel choice (0 =
  * automatic, 1 = register-staged kernel, 4 / 8 = asynchronous-copy kernel with that
- * many wavefronts per workgroup); key 4:
+ * many wavefronts per workgroup and one q head per workgroup, 5 = the same with the rows of a
+ * workgroup packed over the q heads of a kv head, which is what short chunks get by default); key 4:
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
  * the same tile (1 = on, the default); key 5: query rows per wavefront of pa_verify (0 =
  * automatic, 16 or 32 = forced). */

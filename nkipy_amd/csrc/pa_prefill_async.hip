@@ -77,7 +77,11 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
 // MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16.
 // TT: 32-key sub-tiles per key tile (2: 64-key tiles).
-template <bool SPARSE, int MODE, int NW, int TT, bool WIN>
+// PACK (short chunks of a GQA model): the query rows of a workgroup are (token, head) pairs of one
+// kv head, token-major, instead of 32*NW tokens of one q head: a chunk of T < 32*NW tokens then fills
+// the tile with n_rep heads' rows that share every K/V tile, where the plain form would run n_rep
+// workgroups with mostly padding rows.
+template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -99,16 +103,20 @@ void prefill_async_kernel(PrefillParams p) {
   // that share one kv head run on one XCD, back to back, heavy tiles first: their K/V
   // stays in that XCD's L2.
   const int n_rep = p.Hq / p.Hkv;
-  const int nqt = (p.T + BMW - 1) / BMW;
-  const int per_group = nqt * n_rep;
+  const int nqt = PACK ? (p.T * n_rep + BMW - 1) / BMW : (p.T + BMW - 1) / BMW;
+  const int per_group = PACK ? nqt : nqt * n_rep;
   const int groups = p.B * p.Hkv;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int grp = xcd + 8 * (slot / per_group);
   if (grp >= groups) return;
   const int rr_ = slot % per_group;
   const int b = grp / p.Hkv, hk = grp % p.Hkv;
-  const int qt = nqt - 1 - rr_ / n_rep;
-  const int hq = hk * n_rep + rr_ % n_rep;
+  const int qt = PACK ? nqt - 1 - rr_ : nqt - 1 - rr_ / n_rep;
+  const int hq = PACK ? hk * n_rep : hk * n_rep + rr_ % n_rep;     // PACK: first head of the group
+  // row r of the workgroup (0 .. BMW-1) -> query token and q head
+  const int v0 = qt * BMW;
+  auto row_token = [&](int r) __attribute__((always_inline)) { return PACK ? (v0 + r) / n_rep : v0 + r; };
+  auto row_head = [&](int r) __attribute__((always_inline)) { return PACK ? hq + (v0 + r) % n_rep : hq; };
 
   int tq = p.query_lens ? p.query_lens[b] : p.T;
   int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
@@ -116,28 +124,30 @@ void prefill_async_kernel(PrefillParams p) {
   if (MODE != 0) ctx = min(ctx, p.max_blocks * p.block_size);
   ctx = max(ctx, tq);
   const int prefix = ctx - tq;
-  const int q0 = qt * BMW;
+  const int q0 = row_token(0);                                    // first query token of the workgroup
   uint16_t* out = (uint16_t*)p.out;
   const long q_row_stride = (long)p.Hq * HD;
 
   if (q0 >= tq) {   // only padding rows here: zeros
     for (int i = tid; i < BMW * (HD / 8); i += NW * 64) {
-      const int row = q0 + i / (HD / 8);
-      if (row < p.T) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)hq * HD + (i % (HD / 8)) * 8) = make_uint4(0, 0, 0, 0);
+      const int r = i / (HD / 8);
+      const int row = row_token(r);
+      if (row < p.T) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)row_head(r) * HD + (i % (HD / 8)) * 8) = make_uint4(0, 0, 0, 0);
     }
     return;
   }
 
-  // ---- this lane's query row and its Q^T fragments --------------------------
-  const int qrow = q0 + wave * 32 + n;
+  // ---- this lane's query row (token index qrow, head hq_l) and its Q^T fragments ------------
+  const int qrow = row_token(wave * 32 + n);
+  const int hq_l = row_head(wave * 32 + n);
   const bool qvalid = qrow < tq;
   const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
   const float sc = p.scale_log2e;
   bf16x8_t qf[HD / 16];           // loaded below, between the first copy requests
-  const int wq_lo = q0 + wave * 32;                               // first row of this wave
-  const int wq_hi = min(wq_lo + 31, tq - 1);                      // last valid row (may be < wq_lo)
+  const int wq_lo = row_token(wave * 32);                         // first token of this wave
+  const int wq_hi = min(row_token(wave * 32 + 31), tq - 1);       // last valid token (may be < wq_lo)
   const bool wave_has_rows = wq_lo < tq;
-  const int k_end = prefix + min(q0 + BMW, tq);                   // keys the workgroup needs: [0, k_end)
+  const int k_end = prefix + min(row_token(BMW - 1) + 1, tq);     // keys the workgroup needs: [0, k_end)
   const int ntiles = (k_end + BN - 1) / BN;
   // sliding window (its own instantiation, so that the plain form carries none of its scalar
   // work): the row at position pos sees keys (pos - win, pos]
@@ -427,7 +437,7 @@ void prefill_async_kernel(PrefillParams p) {
   request_next();
   prefetch_next();
   {
-    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
+    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * HD;
 #pragma unroll
     for (int s = 0; s < HD / 16; ++s) {
       uint4 v = make_uint4(0, 0, 0, 0);
@@ -483,9 +493,9 @@ void prefill_async_kernel(PrefillParams p) {
     l_run = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
   }
   // attention sink: a per-head logit that joins the softmax as one more column with no value
-  if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq] * kLog2e - m_ref);
+  if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq_l] * kLog2e - m_ref);
   if (qrow < p.T && wq_lo < p.T) {
-    uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
+    uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * HD;
     const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
 #pragma unroll
     for (int c = 0; c < HD / 32; ++c)
@@ -499,23 +509,23 @@ void prefill_async_kernel(PrefillParams p) {
   }
 }
 
-template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false>
+template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
   }
   const int n_rep = p.Hq / p.Hkv;
-  const int nqt = (p.T + 32 * NW - 1) / (32 * NW);
-  const long per_group = (long)nqt * n_rep;
+  const long per_group = PACK ? ((long)p.T * n_rep + 32 * NW - 1) / (32 * NW)
+                              : (long)((p.T + 32 * NW - 1) / (32 * NW)) * n_rep;
   const long groups = (long)p.B * p.Hkv;
   const long total = 8 * ((groups + 7) / 8) * per_group;
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   return hipGetLastError();
 }
 
@@ -535,10 +545,14 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
   // and for the sparse form.
   if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
+  // chunks shorter than a 4-wave tile of a GQA model: rows packed over the heads of a kv group
+  const bool pack = paged && !sparse && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
   if (p.window > 0) {
     if (sparse || !paged) return hipErrorInvalidValue;
+    if (pack) return launch_typed<false, 1, 4, 2, true, true>(p, s);
     return waves == 8 ? launch_typed<false, 1, 8, 2, true>(p, s) : launch_typed<false, 1, 4, 2, true>(p, s);
   }
+  if (pack) return launch_typed<false, 1, 4, 2, false, true>(p, s);
   if (waves == 8) {
     if (sparse) return launch_typed<true, 0, 8>(p, s);
     return paged ? launch_typed<false, 1, 8>(p, s) : launch_typed<false, 0, 8>(p, s);

@@ -233,3 +233,34 @@ def test_prefill_argument_errors(pa):
                    route="tiled")
     with pytest.raises(ValueError):
         pa.prefill(q, kc, kc, bt, one, one, 1.0, route="fast")
+
+
+@pytest.mark.parametrize("impl", [5, 4], ids=["packed", "one_head_per_workgroup"])
+@pytest.mark.parametrize("T,Hq,Hkv", [(20, 8, 2), (64, 32, 8), (100, 10, 2), (127, 4, 2), (33, 16, 1)])
+def test_prefill_short_chunks_packed_rows(pa, impl, T, Hq, Hkv):
+    """Chunks shorter than a 128-row tile: by default the rows of a workgroup are (token, head) pairs of
+    one kv head (ratios 2, 4, 5 and 16: head groups that do and do not divide a wave's 32 rows)."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(T + Hq)
+    qlens = [T, max(T - 7, 1), 1, 0, T]
+    prefixes = [0, 300, 65, 10, 1500]
+    B, D, bs = len(qlens), 128, 32
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, [max(c, 1) for c in ctxs])
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    for window in (None, 40):
+        want = O.paged_prefill(q, O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32),
+                               np.asarray(qlens, np.int32), 0.09, q_dtype="bf16", sliding_window=window, sinks=sinks)
+        lib.pa_debug_set(3, impl)
+        try:
+            got = pa.prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), 0.09,
+                             sliding_window=window, sinks=bf16_to_dev(sinks), route="tiled")
+            torch.cuda.synchronize()
+        finally:
+            lib.pa_debug_set(3, 0)
+        got = dev_to_f32(got)
+        assert_close_abs(got, want, BF16_TOL)
+        for b, n in enumerate(qlens):
+            assert np.all(got[b, n:] == 0)
