@@ -125,13 +125,19 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * already in the pool.  dtype: BF16 for q/k/v/out.  sinks / sliding_window as for pa_decode, the
  * window counted back from each query token's own position; key tiles outside every row's
  * window are skipped.
+ * workspace: NULL, or pa_prefill_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed).  With
+ * it, a call with too few query tiles to fill the device (one long-context request prefilled in
+ * chunks) splits the key tiles of each query tile over up to 16 workgroups and merges their partial
+ * results in a second kernel; the result does not depend on the split.
  */
+size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq);
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
-               float scale, int dtype, const float* sinks, int sliding_window, void* stream);
+               float scale, int dtype, const float* sinks, int sliding_window,
+               void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Block-sparse causal prefill over dense q [B, S, Hq, D], k/v [B, S, Hkv, D]:
@@ -209,7 +215,7 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * workgroup packed over the q heads of a kv head, which is what short chunks get by default); key 4:
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
  * the same tile (1 = on, the default); key 5: query rows per wavefront of pa_verify (0 =
- * automatic, 16 or 32 = forced). */
+ * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

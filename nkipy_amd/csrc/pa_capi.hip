@@ -41,6 +41,7 @@ static std::atomic<int> g_head_major{1};
 static std::atomic<int> g_prefill_impl{0};
 static std::atomic<int> g_lockstep{1};
 static std::atomic<int> g_verify_rows{0};
+static std::atomic<int> g_prefill_split{1};
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 static std::atomic<int> g_profile{0};
@@ -109,6 +110,7 @@ int pa_debug_set(int key, int value) {
   if (key == 3) { g_prefill_impl = value; return 0; }
   if (key == 4) { g_lockstep = value; return 0; }
   if (key == 5) { g_verify_rows = value; return 0; }
+  if (key == 6) { g_prefill_split = value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -321,12 +323,34 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
   return check_hip(e, "pa_verify reduce launch");
 }
 
+static void fill_prefill_shape(PrefillParams& p, int B, int T, int Hq, int Hkv, int D, int block_size,
+                               int max_blocks_per_seq, int num_blocks) {
+  p.B = B; p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
+  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
+  p.block_shift = ilog2_exact(block_size);
+  p.impl = g_prefill_impl.load();
+}
+
+static size_t prefill_split_bytes(const PrefillParams& p, int splits) {
+  return splits > 1 ? (size_t)p.B * p.T * p.Hq * splits * ((size_t)p.D + 2) * sizeof(float) : 0;
+}
+
+size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq) {
+  if (B <= 0 || T <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || block_size <= 0 || max_blocks_per_seq <= 0 || Hq % Hkv) return 0;
+  PrefillParams p;
+  memset(&p, 0, sizeof(p));
+  fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, 1);
+  p.block_tables = (const int32_t*)16;     // paged form (only tested for null)
+  return prefill_split_bytes(p, prefill_async_splits(p, current_num_cus()));
+}
+
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
-               float scale, int dtype, const float* sinks, int sliding_window, void* stream) {
+               float scale, int dtype, const float* sinks, int sliding_window,
+               void* workspace, size_t workspace_bytes, void* stream) {
   tl_error[0] = 0;
   if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_prefill: bad sizes");
   if (sliding_window < 0) return fail_arg("pa_prefill: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
@@ -344,15 +368,24 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   memset(&p, 0, sizeof(p));
   p.q = q; p.k = k_cache; p.v = v_cache; p.block_tables = block_tables; p.seq_lens = seq_lens;
   p.query_lens = query_lens; p.out = out;
-  p.B = B; p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.D = D;
-  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
-  p.block_shift = ilog2_exact(block_size);
+  fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
   p.scale_log2e = scale * kLog2e;
-  p.impl = g_prefill_impl.load();
   if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
   if ((sinks || sliding_window > 0) && (p.impl == 1 || !prefill_async_supported(p)))
     return fail_arg("pa_prefill: sinks and sliding_window need the asynchronous-copy kernel (block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
+  // few workgroups and a long table: split the key tiles of a query tile over several workgroups when the
+  // caller brought the workspace for it (without one the call runs unsplit)
+  p.splits = 1;
+  if (workspace) {
+    if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
+    const int want = g_prefill_split.load() ? prefill_async_splits(p, current_num_cus()) : 1;
+    if (want > 1 && workspace_bytes >= prefill_split_bytes(p, want)) {
+      p.splits = want;
+      p.ws_o = (float*)workspace;
+      p.ws_ml = p.ws_o + (size_t)B * T * Hq * want * D;
+    }
+  }
   hipStream_t s = (hipStream_t)stream;
   profile_begin(s);
   hipError_t e = launch_prefill(p, s);

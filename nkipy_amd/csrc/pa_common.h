@@ -122,9 +122,13 @@ struct PrefillParams {
   int impl;                 // 0 automatic, 1 register-staged, 4 / 8 asynchronous (waves per workgroup), 5 asynchronous with packed rows
   int window;               // paged form, asynchronous kernel only: sliding window in tokens, 0 = none
   const float* sinks;       // same: [Hq] per-head sink logits or null
+  int splits;               // same: workgroups sharing the key tiles of one query tile (1: no split)
+  float* ws_o;              // splits > 1: [B * T * Hq, splits, D] partial outputs
+  float* ws_ml;             // splits > 1: [B * T * Hq, splits, 2] partial (max, sum)
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);
+int prefill_async_splits(const PrefillParams& p, int num_cus);   // split the launcher would like for this call
 bool prefill_supported(const PrefillParams& p);
 hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s);
 bool prefill_async_supported(const PrefillParams& p);

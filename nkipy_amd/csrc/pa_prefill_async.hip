@@ -81,7 +81,10 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 // kv head, token-major, instead of 32*NW tokens of one q head: a chunk of T < 32*NW tokens then fills
 // the tile with n_rep heads' rows that share every K/V tile, where the plain form would run n_rep
 // workgroups with mostly padding rows.
-template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK>
+// SPLIT (few workgroups, long contexts): p.splits workgroups share the key tiles of one query tile
+// and leave unnormalised partial results (m, l, O) in the workspace for prefill_split_reduce_kernel:
+// a lone workgroup walks its tiles at about a microsecond each, whatever the rest of the chip does.
+template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -106,7 +109,9 @@ void prefill_async_kernel(PrefillParams p) {
   const int nqt = PACK ? (p.T * n_rep + BMW - 1) / BMW : (p.T + BMW - 1) / BMW;
   const int per_group = PACK ? nqt : nqt * n_rep;
   const int groups = p.B * p.Hkv;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int xcd = blockIdx.x & 7;
+  const int part = SPLIT ? (int)(blockIdx.x >> 3) % p.splits : 0;      // which share of the key tiles
+  const int slot = SPLIT ? (int)(blockIdx.x >> 3) / p.splits : (int)(blockIdx.x >> 3);
   const int grp = xcd + 8 * (slot / per_group);
   if (grp >= groups) return;
   const int rr_ = slot % per_group;
@@ -128,7 +133,8 @@ void prefill_async_kernel(PrefillParams p) {
   uint16_t* out = (uint16_t*)p.out;
   const long q_row_stride = (long)p.Hq * HD;
 
-  if (q0 >= tq) {   // only padding rows here: zeros
+  if (q0 >= tq) {   // only padding rows here: zeros (written by the reduce kernel when splitting)
+    if (SPLIT) return;
     for (int i = tid; i < BMW * (HD / 8); i += NW * 64) {
       const int r = i / (HD / 8);
       const int row = row_token(r);
@@ -148,10 +154,23 @@ void prefill_async_kernel(PrefillParams p) {
   const int wq_hi = min(row_token(wave * 32 + 31), tq - 1);       // last valid token (may be < wq_lo)
   const bool wave_has_rows = wq_lo < tq;
   const int k_end = prefix + min(row_token(BMW - 1) + 1, tq);     // keys the workgroup needs: [0, k_end)
-  const int ntiles = (k_end + BN - 1) / BN;
   // sliding window (its own instantiation, so that the plain form carries none of its scalar
   // work): the row at position pos sees keys (pos - win, pos]
   const int win = WIN ? p.window : 0;
+  // key tiles of this workgroup: [kt_begin, ntiles)
+  int kt_begin = win > 0 ? max(prefix + q0 - win + 1, 0) / BN : 0;   // first tile the first row sees
+  int ntiles = (k_end + BN - 1) / BN;
+  const long row_g = ((long)b * p.T + qrow) * p.Hq + hq_l;            // this lane's row among all B * T * Hq
+  if (SPLIT) {
+    const int n_all = ntiles - kt_begin;
+    const int lo = kt_begin + (int)((long)part * n_all / p.splits);
+    ntiles = kt_begin + (int)((long)(part + 1) * n_all / p.splits);
+    kt_begin = lo;
+    if (kt_begin >= ntiles) {                  // nothing for this share: an empty partial
+      if (qvalid && h == 0) *(float2*)(p.ws_ml + (row_g * p.splits + part) * 2) = make_float2(-INFINITY, 0.f);
+      return;
+    }
+  }
 
   // ---- DMA maps ---------------------------------------------------------------------
   // A tile is 2 UK units of 1 KB (4 rows): the first UK are K, the rest V.  Wave w issues
@@ -295,7 +314,7 @@ void prefill_async_kernel(PrefillParams p) {
   };
   // ---- ring of NST stages: tiles are requested NST-1 ahead; requests past the end are
   // repeated on the first tile so that the wait counter stays exact ------------------------
-  Walk w_first = {win > 0 ? max(prefix + q0 - win + 1, 0) / BN : 0, head_phase};   // first tile the first row sees
+  Walk w_first = {kt_begin, head_phase};
   walk_settle(w_first);
   const int kt_first = w_first.kt;
   Walk w_i = w_first;                 // next tile to request
@@ -492,6 +511,19 @@ void prefill_async_kernel(PrefillParams p) {
     const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
     l_run = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
   }
+  if (SPLIT) {     // partial result relative to m_ref; the sink and the division belong to the merge
+    if (qvalid) {
+      float* po = p.ws_o + (row_g * p.splits + part) * HD;
+#pragma unroll
+      for (int c = 0; c < HD / 32; ++c)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4)
+          *(float4*)(po + 32 * c + 8 * i4 + 4 * h) =
+              make_float4(oacc[c][4 * i4], oacc[c][4 * i4 + 1], oacc[c][4 * i4 + 2], oacc[c][4 * i4 + 3]);
+      if (h == 0) *(float2*)(p.ws_ml + (row_g * p.splits + part) * 2) = make_float2(slack == -INFINITY ? -INFINITY : m_ref, l_run);
+    }
+    return;
+  }
   // attention sink: a per-head logit that joins the softmax as one more column with no value
   if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq_l] * kLog2e - m_ref);
   if (qrow < p.T && wq_lo < p.T) {
@@ -509,12 +541,42 @@ void prefill_async_kernel(PrefillParams p) {
   }
 }
 
-template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false>
+// Merge of the split form: one thread per (query row, 4 consecutive d); rows past query_lens become zeros.
+__global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams p) {
+  const long item = (long)blockIdx.x * 256 + threadIdx.x;
+  const long row = item / (HD / 4);
+  const int q4 = (int)(item % (HD / 4));
+  if (row >= (long)p.B * p.T * p.Hq) return;
+  const int hq = (int)(row % p.Hq);
+  const long bt = row / p.Hq;
+  const int t = (int)(bt % p.T), b = (int)(bt / p.T);
+  const int tq = min(max(p.query_lens[b], 0), p.T);
+  uint16_t* dst = (uint16_t*)p.out + row * HD + 4 * q4;
+  if (t >= tq) { *(uint2*)dst = make_uint2(0u, 0u); return; }
+  float m = -INFINITY, l = 0.f;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int c = 0; c < p.splits; ++c) {
+    const float2 ml = *(const float2*)(p.ws_ml + (row * p.splits + c) * 2);
+    if (ml.y == 0.f) continue;                 // a share in which the row saw no key (its O may be unwritten)
+    const float4 o = *(const float4*)(p.ws_o + (row * p.splits + c) * HD + 4 * q4);
+    const float m_new = fmaxf(m, ml.x);
+    const float a = exp2f(m - m_new), w = exp2f(ml.x - m_new);
+    l = l * a + ml.y * w;
+    acc.x = acc.x * a + o.x * w; acc.y = acc.y * a + o.y * w;
+    acc.z = acc.z * a + o.z * w; acc.w = acc.w * a + o.w * w;
+    m = m_new;
+  }
+  if (p.sinks && l > 0.f) l += exp2f(p.sinks[hq] * kLog2e - m);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  *(uint2*)dst = make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
+}
+
+template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
@@ -523,10 +585,22 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   const long per_group = PACK ? ((long)p.T * n_rep + 32 * NW - 1) / (32 * NW)
                               : (long)((p.T + 32 * NW - 1) / (32 * NW)) * n_rep;
   const long groups = (long)p.B * p.Hkv;
-  const long total = 8 * ((groups + 7) / 8) * per_group;
+  const long total = 8 * ((groups + 7) / 8) * per_group * (SPLIT ? p.splits : 1);
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  if (SPLIT) {
+    const long items = (long)p.B * p.T * p.Hq * (HD / 4);
+    hipLaunchKernelGGL(prefill_split_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, p);
+  }
   return hipGetLastError();
+}
+
+// workgroups of the paged dense form for a given choice of waves and packing
+long prefill_workgroups(const PrefillParams& p, int waves, bool pack) {
+  const int n_rep = p.Hq / p.Hkv;
+  const long per_group = pack ? ((long)p.T * n_rep + 32 * waves - 1) / (32 * waves)
+                              : (long)((p.T + 32 * waves - 1) / (32 * waves)) * n_rep;
+  return (long)p.B * p.Hkv * per_group;
 }
 
 }  // namespace
@@ -537,16 +611,47 @@ bool prefill_async_supported(const PrefillParams& p) {
   return true;
 }
 
-hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s) {
+static bool prefill_packs(const PrefillParams& p) {
+  const bool sparse = p.sparse_stride > 0, paged = p.block_tables != nullptr;
+  // chunks shorter than a 4-wave tile of a GQA model: rows packed over the heads of a kv group
+  return paged && !sparse && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
+}
+static int prefill_waves(const PrefillParams& p, int waves) {
   const bool sparse = p.sparse_stride > 0;
-  const bool paged = p.block_tables != nullptr;
   // waves: 4 (two workgroups of 128 query rows per CU, 2-stage ring) or 8 (one workgroup of
   // 256 rows, 4-stage ring: half the copy requests per FLOP).  Measured within a few per cent of
   // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
   // and for the sparse form.
+  if (prefill_packs(p)) return 4;
   if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
-  // chunks shorter than a 4-wave tile of a GQA model: rows packed over the heads of a kv group
-  const bool pack = paged && !sparse && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
+  return waves;
+}
+
+int prefill_async_splits(const PrefillParams& p, int num_cus) {
+  if (p.sparse_stride > 0 || !p.block_tables || !prefill_async_supported(p) || p.impl == 1) return 1;
+  const long wgs = prefill_workgroups(p, prefill_waves(p, p.impl == 4 || p.impl == 8 ? p.impl : 0), prefill_packs(p));
+  if (wgs >= num_cus) return 1;                       // enough workgroups to fill the chip
+  const long cap_tiles = ((long)p.max_blocks * p.block_size + 63) / 64;
+  long s = (2L * num_cus + wgs - 1) / wgs;            // aim at two workgroups per CU
+  if (s > cap_tiles / 8) s = cap_tiles / 8;           // ... of at least 8 key tiles each at table capacity
+  if (s > 16) s = 16;
+  return s < 2 ? 1 : (int)s;
+}
+
+hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s) {
+  const bool sparse = p.sparse_stride > 0;
+  const bool paged = p.block_tables != nullptr;
+  const bool pack = prefill_packs(p);
+  waves = prefill_waves(p, waves);
+  if (p.splits > 1) {
+    if (sparse || !paged || !p.ws_o || !p.ws_ml) return hipErrorInvalidValue;
+    if (p.window > 0) {
+      if (pack) return launch_typed<false, 1, 4, 2, true, true, true>(p, s);
+      return waves == 8 ? launch_typed<false, 1, 8, 2, true, false, true>(p, s) : launch_typed<false, 1, 4, 2, true, false, true>(p, s);
+    }
+    if (pack) return launch_typed<false, 1, 4, 2, false, true, true>(p, s);
+    return waves == 8 ? launch_typed<false, 1, 8, 2, false, false, true>(p, s) : launch_typed<false, 1, 4, 2, false, false, true>(p, s);
+  }
   if (p.window > 0) {
     if (sparse || !paged) return hipErrorInvalidValue;
     if (pack) return launch_typed<false, 1, 4, 2, true, true>(p, s);

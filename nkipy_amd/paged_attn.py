@@ -281,10 +281,17 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
         _raise_on(rc, "pa_verify")
         return out
     with torch.cuda.device(q.device):
+        need = int(lib.pa_prefill_workspace_bytes(B, T, Hq, Hkv, D, block_size, block_tables.shape[1]))
+        if workspace is None:
+            workspace = _workspace(q.device, need) if need else None
+        else:
+            _need_device("workspace", workspace)
+            _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
         rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
                             block_tables.shape[1], num_blocks, float(scale), BF16, _ptr(sinks), win,
-                            _stream_ptr(q.device))
+                            _ptr(workspace), ws_bytes, _stream_ptr(q.device))
     _raise_on(rc, "pa_prefill")
     return out
 

@@ -264,3 +264,37 @@ def test_prefill_short_chunks_packed_rows(pa, impl, T, Hq, Hkv):
         assert_close_abs(got, want, BF16_TOL)
         for b, n in enumerate(qlens):
             assert np.all(got[b, n:] == 0)
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,window", [(128, 8, 2, None), (100, 8, 2, None), (300, 4, 4, None), (200, 8, 1, 700),
+                                             (90, 4, 1, 64), (256, 2, 2, 1500)])
+def test_prefill_split_over_key_tiles(pa, T, Hq, Hkv, window):
+    """Few query tiles against long contexts: the key tiles of a query tile are shared by several
+    workgroups (4- and 8-wave, packed rows, windowed); shares that are empty for some rows or for a
+    whole short sequence; same result as the unsplit kernel."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(T + Hq)
+    qlens, prefixes = [T, 5], [5000, 3]
+    B, D, bs = 2, 128, 32
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    need = lib.pa_prefill_workspace_bytes(B, T, Hq, Hkv, D, bs, tables.shape[1])
+    assert need > 0                                   # this shape is one the launcher wants to split
+    want = O.paged_prefill(q, O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32),
+                           np.asarray(qlens, np.int32), 0.09, q_dtype="bf16", sliding_window=window, sinks=sinks)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), 0.09)
+    kw = dict(sliding_window=window, sinks=bf16_to_dev(sinks), route="tiled")
+    got = dev_to_f32(pa.prefill(*args, **kw))
+    lib.pa_debug_set(6, 0)
+    try:
+        unsplit = dev_to_f32(pa.prefill(*args, **kw))
+    finally:
+        lib.pa_debug_set(6, 1)
+    assert_close_abs(got, want, BF16_TOL)
+    assert np.max(np.abs(got - unsplit)) <= 2 ** -6
+    assert np.all(got[1, 5:] == 0)
+    with pytest.raises(ValueError):
+        pa.prefill(*args, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"), **kw)
