@@ -192,10 +192,10 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
     return out
 
 
-# prefill() takes the verify kernel when a kv head has at most 16 (query token, q head) rows, or while
-# rows x sequences x kv heads stays below this (measured crossover against the tiled kernel, which has a
-# fixed cost per call — the serial walk over the longest context — and a lower cost per row)
-VERIFY_MAX_WORK = 12800
+# prefill() takes the verify kernel up to this many (query token, q head) rows per kv head: the measured
+# crossover against the tiled kernel (rows packed over the kv group, key tiles split over workgroups when
+# the grid is small) lies between 16 and 48 rows for batches of 1 to 64 sequences
+VERIFY_MAX_ROWS = 32
 
 
 def verify_supported(T, D, block_size) -> bool:
@@ -212,10 +212,10 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     j <= seq_lens[b] - query_lens[b] + i of the paged context, which already
     contains the new tokens' K/V.
 
-    Two kernels stand behind it.  Short query runs of small batches -- speculative verify: up to 16
-    (token, head) rows per kv head, or rows * B * Hkv <= VERIFY_MAX_WORK -- go through the decode
-    kernel with the (token, head) pairs as its query rows (HBM-bound: the context is read once per
-    kv head); everything else through the tiled matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
+    Two kernels stand behind it.  Short query runs -- speculative verify: T * (Hq / Hkv) <=
+    VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query rows
+    (HBM-bound: the context is read once per kv head); everything else through the tiled
+    matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
     (float8_e4m3fn / uint8 codes with k_scale, v_scale) are the verify kernel's only; sinks and
     sliding_window (as in `decode`, the window counted back from each query token) work on both.
     """
@@ -247,9 +247,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     can_verify = verify_supported(T, D, block_size)
     if route is None:
         # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
-        rows = T * (Hq // Hkv)
-        small = rows <= 16 or rows * B * Hkv <= VERIFY_MAX_WORK
-        route = "verify" if can_verify and (kv_code == FP8 or D != 128 or small) else "tiled"
+        route = "verify" if can_verify and (kv_code == FP8 or D != 128 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")
