@@ -629,8 +629,10 @@ static int prefill_waves(const PrefillParams& p, int waves) {
 
 int prefill_async_splits(const PrefillParams& p, int num_cus) {
   if (p.sparse_stride > 0 || !p.block_tables || !prefill_async_supported(p) || p.impl == 1) return 1;
-  const long wgs = prefill_workgroups(p, prefill_waves(p, p.impl == 4 || p.impl == 8 ? p.impl : 0), prefill_packs(p));
-  if (wgs >= num_cus) return 1;                       // enough workgroups to fill the chip
+  const int waves = prefill_waves(p, p.impl == 4 || p.impl == 8 ? p.impl : 0);
+  const long wgs = prefill_workgroups(p, waves, prefill_packs(p));
+  const long slots = (long)num_cus * (waves == 4 ? 2 : 1);     // workgroups the device holds at once
+  if (wgs >= slots) return 1;                         // enough workgroups to fill the chip
   const long cap_tiles = ((long)p.max_blocks * p.block_size + 63) / 64;
   long s = (2L * num_cus + wgs - 1) / wgs;            // aim at two workgroups per CU
   if (s > cap_tiles / 8) s = cap_tiles / 8;           // ... of at least 8 key tiles each at table capacity
