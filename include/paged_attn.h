@@ -122,7 +122,10 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * b (i < query_lens[b]) sees keys j <= seq_lens[b] - query_lens[b] + i
  * (examples/models/gpt_oss/kernels/attention.py:85,127-135: "query at
  * start_pos+i attends to keys <= start_pos+i").  The new tokens' K/V are
- * already in the pool.  dtype: BF16 for q/k/v/out.  sinks / sliding_window as for pa_decode, the
+ * already in the pool.  dtype: BF16 for q and out; kv_dtype PA_BF16, or PA_FP8_E4M3FN with
+ * k_scale / v_scale [num_blocks, Hkv] (NULL otherwise): fp8 pools go through the register-staged
+ * kernel, which expands the codes times their block's scale to bf16 on the way into LDS, and take no
+ * sliding window.  sinks / sliding_window as for pa_decode, the
  * window counted back from each query token's own position; key tiles outside every row's
  * window are skipped.
  * workspace: NULL, or pa_prefill_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed).  With
@@ -132,11 +135,12 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  */
 size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq);
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
+               const float* k_scale, const float* v_scale,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
-               float scale, int dtype, const float* sinks, int sliding_window,
+               float scale, int dtype, int kv_dtype, const float* sinks, int sliding_window,
                void* workspace, size_t workspace_bytes, void* stream);
 
 /*

@@ -345,23 +345,28 @@ size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int bloc
 }
 
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
+               const float* k_scale, const float* v_scale,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
-               float scale, int dtype, const float* sinks, int sliding_window,
+               float scale, int dtype, int kv_dtype, const float* sinks, int sliding_window,
                void* workspace, size_t workspace_bytes, void* stream) {
   tl_error[0] = 0;
   if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_prefill: bad sizes");
   if (sliding_window < 0) return fail_arg("pa_prefill: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
   if (Hq % Hkv) return fail_arg("pa_prefill: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
-  if (dtype != PA_BF16) return fail_arg("pa_prefill: only bf16 is supported (dtype=%d)", dtype);
+  if (dtype != PA_BF16) return fail_arg("pa_prefill: only bf16 queries are supported (dtype=%d)", dtype);
+  if (kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN)
+    return fail_arg("pa_prefill: kv_dtype must be bf16 or fp8-e4m3fn (got %d)", kv_dtype);
+  const bool fp8 = kv_dtype == PA_FP8_E4M3FN;
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_prefill: bad paging sizes");
   if (B == 0 || T == 0) return 0;
   if ((long)num_blocks * block_size > 0x7fffffffL || (long)block_size * Hkv * D * 2 > 0xffffffffL)
     return fail_arg("pa_prefill: pool of %d blocks x %d rows exceeds 2^31 rows (or a block 4 GiB)", num_blocks, block_size);
   if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens || !out)
     return fail_arg("pa_prefill: null pointer argument");
+  if (fp8 && (!k_scale || !v_scale)) return fail_arg("pa_prefill: fp8 KV needs k_scale and v_scale");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
     return fail_arg("pa_prefill: q, k_cache, v_cache and out must be 16-byte aligned");
   PrefillParams p;
@@ -371,13 +376,14 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
   p.scale_log2e = scale * kLog2e;
   if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
-  if ((sinks || sliding_window > 0) && (p.impl == 1 || !prefill_async_supported(p)))
-    return fail_arg("pa_prefill: sinks and sliding_window need the asynchronous-copy kernel (block_size a power of two >= 16)");
+  if (sliding_window > 0 && (fp8 || p.impl == 1 || !prefill_async_supported(p)))
+    return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (bf16 pool, block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
+  p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
   // few workgroups and a long table: split the key tiles of a query tile over several workgroups when the
   // caller brought the workspace for it (without one the call runs unsplit)
   p.splits = 1;
-  if (workspace) {
+  if (workspace && !fp8) {
     if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
     const int want = g_prefill_split.load() ? prefill_async_splits(p, current_num_cus()) : 1;
     if (want > 1 && workspace_bytes >= prefill_split_bytes(p, want)) {

@@ -122,6 +122,9 @@ struct PrefillParams {
   int impl;                 // 0 automatic, 1 register-staged, 4 / 8 asynchronous (waves per workgroup), 5 asynchronous with packed rows
   int window;               // paged form, asynchronous kernel only: sliding window in tokens, 0 = none
   const float* sinks;       // same: [Hq] per-head sink logits or null
+  int kv_fp8;               // paged form: the pool holds e4m3fn codes (register-staged kernel only)
+  const float* k_scale;     // kv_fp8: [num_blocks, Hkv] scales
+  const float* v_scale;
   int splits;               // same: workgroups sharing the key tiles of one query tile (1: no split)
   float* ws_o;              // splits > 1: [B * T * Hq, splits, D] partial outputs
   float* ws_ml;             // splits > 1: [B * T * Hq, splits, 2] partial (max, sum)

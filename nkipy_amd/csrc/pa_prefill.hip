@@ -54,7 +54,10 @@ __device__ __forceinline__ bool block_active(int i, int j, int head, int local, 
 // MODE: 0 = dense K/V [B, S, Hkv, D]; 1 = paged, block size a power of two >= 16
 // (one table entry per 16-key group, looked up once per wave on the scalar unit);
 // 2 = paged, any block size (every staged key resolves its own table entry).
-template <bool SPARSE, int MODE>
+// FP8 (paged only): the pool holds e4m3fn codes with one float32 scale per (block, kv head); a
+// thread fetches 8 codes where it would fetch 8 bf16 values and expands them, times the scale of
+// their block, to bf16 on the way into LDS, so the dequantised cache exists only there.
+template <bool SPARSE, int MODE, bool FP8>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // two stages, each: K tile [64][272 B] then V^T tile
@@ -114,60 +117,88 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   const int vg = tid >> 4;                                       // slot group: slots 4vg .. 4vg+3
   const int vkey0 = 32 * (vg >> 3) + 16 * ((vg >> 2) & 1) + 8 * (vg & 1) + 4 * ((vg >> 1) & 1);
   const int32_t* table = MODE != 0 ? p.block_tables + (long)b * p.max_blocks : nullptr;
-  const long kv_row_stride = (long)p.Hkv * HD;                   // elements between consecutive tokens
-  const uint16_t* kbase = (const uint16_t*)p.k + (long)hk * HD;
-  const uint16_t* vbase = (const uint16_t*)p.v + (long)hk * HD;
+  constexpr int ESZ = FP8 ? 1 : 2;                               // bytes per pool element
+  const long kv_row_stride = (long)p.Hkv * HD * ESZ;             // bytes between consecutive tokens
+  const char* kbase = (const char*)p.k + (long)hk * HD * ESZ;
+  const char* vbase = (const char*)p.v + (long)hk * HD * ESZ;
 
   // generic: row of key `key` (clamped into the context), one table lookup per lane
-  auto pool_row = [&](int key) __attribute__((always_inline)) -> long {
+  auto pool_row = [&](int key, int* blk_out) __attribute__((always_inline)) -> long {
     key = min(key, ctx - 1);
     if (MODE == 0) return (long)b * p.S + key;
     int blk, off;
     if (p.block_shift >= 0) { blk = table[key >> p.block_shift]; off = key & (p.block_size - 1); }
     else { blk = table[key / p.block_size]; off = key % p.block_size; }
     blk = min(max(blk, 0), p.num_blocks - 1);
+    *blk_out = blk;
     return (long)blk * p.block_size + off;
   };
   // fast: first pool row of the 16-key group that starts at the wave-uniform key kb
   // (the group lies inside one block and inside the context)
-  auto group_row = [&](int kb) __attribute__((always_inline)) -> long {
+  auto group_row = [&](int kb, int* blk_out) __attribute__((always_inline)) -> long {
     if (MODE == 0) return (long)b * p.S + kb;
     int blk = table[kb >> p.block_shift];
     blk = min(max(blk, 0), p.num_blocks - 1);
+    *blk_out = blk;
     return (long)blk * p.block_size + (kb & (p.block_size - 1));
   };
-  // per-lane element offsets inside a 16-key group (constant over the whole loop)
-  const int k_lane_off = (int)((kkey & 3) * kv_row_stride) + kchunk * 8;
-  const int v_lane_off = (int)((vkey0 & 15) * kv_row_stride) + kchunk * 8;
+  // per-lane byte offsets inside a 16-key group (constant over the whole loop): 8 elements per piece
+  const int k_lane_off = (int)((kkey & 3) * kv_row_stride) + kchunk * 8 * ESZ;
+  const int v_lane_off = (int)((vkey0 & 15) * kv_row_stride) + kchunk * 8 * ESZ;
 
   typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-  u32x4_t kreg[4], vreg[4];
+  u32x4_t kreg[4], vreg[4];          // FP8: raw codes in .xy until store_tile expands them
+  float kss[4], vss[4];              // FP8: scale of each piece's block
+  auto fetch8 = [&](const char* src) __attribute__((always_inline)) -> u32x4_t {
+    if (FP8) { const uint2 v = *(const uint2*)src; return u32x4_t{v.x, v.y, 0u, 0u}; }
+    return *(const u32x4_t*)src;
+  };
   auto load_tile = [&](int kt) __attribute__((always_inline)) {
     const int key0 = kt * BN;
+    int blk = 0;
     if (MODE != 2 && key0 + BN <= ctx) {         // whole tile inside the context: uniform addressing
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint16_t* g = kbase + group_row(key0 + 16 * i + 4 * wave) * kv_row_stride;
-        kreg[i] = *(const u32x4_t*)(g + k_lane_off);
+        const char* g = kbase + group_row(key0 + 16 * i + 4 * wave, &blk) * kv_row_stride;
+        kreg[i] = fetch8(g + k_lane_off);
+        if (FP8) kss[i] = p.k_scale[(long)blk * p.Hkv + hk];
       }
-      const uint16_t* g = vbase + group_row(key0 + 32 * (wave >> 1) + 16 * (wave & 1)) * kv_row_stride;
+      const char* g = vbase + group_row(key0 + 32 * (wave >> 1) + 16 * (wave & 1), &blk) * kv_row_stride;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) vreg[i] = *(const u32x4_t*)(g + v_lane_off + i * kv_row_stride);
+      for (int i = 0; i < 4; ++i) {
+        vreg[i] = fetch8(g + v_lane_off + i * kv_row_stride);
+        if (FP8) vss[i] = p.v_scale[(long)blk * p.Hkv + hk];
+      }
     } else {                                      // last tile of a context, or odd block sizes
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        kreg[i] = *(const u32x4_t*)(kbase + pool_row(key0 + 16 * i + kkey) * kv_row_stride + kchunk * 8);
+      for (int i = 0; i < 4; ++i) {
+        kreg[i] = fetch8(kbase + pool_row(key0 + 16 * i + kkey, &blk) * kv_row_stride + kchunk * 8 * ESZ);
+        if (FP8) kss[i] = p.k_scale[(long)blk * p.Hkv + hk];
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = key0 + vkey0 + i;
-        vreg[i] = *(const u32x4_t*)(vbase + pool_row(key) * kv_row_stride + kchunk * 8);
+        vreg[i] = fetch8(vbase + pool_row(key, &blk) * kv_row_stride + kchunk * 8 * ESZ);
+        if (FP8) vss[i] = p.v_scale[(long)blk * p.Hkv + hk];
         // rows past the context may hold anything (NaN patterns too); their weight is an
         // exact zero, which only helps if the value is finite
         if (key >= ctx) vreg[i] = u32x4_t{0u, 0u, 0u, 0u};
       }
     }
   };
+  // FP8: 8 codes -> 8 bf16 values times the block's scale (rounded to nearest even)
+  auto expand = [&](u32x4_t& r, float sc8) __attribute__((always_inline)) {
+    float f[8];
+    fp8x4_to_float(r[0], f);
+    fp8x4_to_float(r[1], f + 4);
+    r = u32x4_t{pack_bf16x2(f[0] * sc8, f[1] * sc8), pack_bf16x2(f[2] * sc8, f[3] * sc8),
+                pack_bf16x2(f[4] * sc8, f[5] * sc8), pack_bf16x2(f[6] * sc8, f[7] * sc8)};
+  };
   auto store_tile = [&](char* ks, char* vts) __attribute__((always_inline)) {
+    if (FP8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { expand(kreg[i], kss[i]); expand(vreg[i], vss[i]); }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) *(u32x4_t*)(ks + (16 * i + kkey) * K_ROW_BYTES + kchunk * 16) = kreg[i];
 #pragma unroll
@@ -304,6 +335,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
 
   // ---- normalise and write this lane's query row ---------------------------------
   l_run += __shfl_xor(l_run, 32, 64);
+  // attention sink: a per-head logit that joins the softmax as one more column with no value
+  if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq] * kLog2e - m_run);
   if (qrow < p.T && wq_lo < p.T) {
     uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq * HD;
     const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
@@ -321,16 +354,16 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
 
 constexpr int kPrefillLdsBytes = 2 * (BN * K_ROW_BYTES + VT_BYTES);
 
-template <bool SPARSE, int MODE>
+template <bool SPARSE, int MODE, bool FP8 = false>
 hipError_t launch_prefill_typed(const PrefillParams& p, dim3 grid, hipStream_t s) {
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_kernel<SPARSE, MODE>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_kernel<SPARSE, MODE, FP8>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kPrefillLdsBytes);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
   }
-  hipLaunchKernelGGL((prefill_kernel<SPARSE, MODE>), grid, dim3(256), kPrefillLdsBytes, s, p);
+  hipLaunchKernelGGL((prefill_kernel<SPARSE, MODE, FP8>), grid, dim3(256), kPrefillLdsBytes, s, p);
   return hipGetLastError();
 }
 
@@ -343,10 +376,16 @@ bool prefill_supported(const PrefillParams& p) {
 }
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s) {
-  if (p.impl != 1 && prefill_async_supported(p)) return launch_prefill_async(p, p.impl == 4 || p.impl == 8 ? p.impl : 0, s);
+  if (!p.kv_fp8 && p.impl != 1 && prefill_async_supported(p))
+    return launch_prefill_async(p, p.impl == 4 || p.impl == 8 ? p.impl : 0, s);
   const int nqt = (p.T + BM - 1) / BM;
   if (nqt > 65535 * 32 || p.Hq > 65535 || p.B > 65535) return hipErrorInvalidValue;
   dim3 grid(nqt, p.Hq, p.B);
+  if (p.kv_fp8) {      // fp8 pools: the register-staged kernel expands the codes on their way into LDS
+    if (!p.block_tables || p.sparse_stride > 0 || !p.k_scale || !p.v_scale) return hipErrorInvalidValue;
+    if (p.block_shift >= 4) return launch_prefill_typed<false, 1, true>(p, grid, s);
+    return launch_prefill_typed<false, 2, true>(p, grid, s);
+  }
   if (p.sparse_stride > 0) return launch_prefill_typed<true, 0>(p, grid, s);
   if (!p.block_tables) return launch_prefill_typed<false, 0>(p, grid, s);
   if (p.block_shift >= 4) return launch_prefill_typed<false, 1>(p, grid, s);

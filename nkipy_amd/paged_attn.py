@@ -196,6 +196,7 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
 # crossover against the tiled kernel (rows packed over the kv group, key tiles split over workgroups when
 # the grid is small) lies between 16 and 48 rows for batches of 1 to 64 sequences
 VERIFY_MAX_ROWS = 32
+VERIFY_MAX_ROWS_FP8 = 256     # fp8 pools: the tiled route is the slower register-staged kernel (B = 64: T = 64 774 vs 990 us)
 
 
 def verify_supported(T, D, block_size) -> bool:
@@ -216,8 +217,9 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query rows
     (HBM-bound: the context is read once per kv head); everything else through the tiled
     matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
-    (float8_e4m3fn / uint8 codes with k_scale, v_scale) are the verify kernel's only; sinks and
-    sliding_window (as in `decode`, the window counted back from each query token) work on both.
+    (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both; behind the tiled route they
+    take the register-staged kernel (codes expanded to bf16 on their way into LDS) and no sliding
+    window.  sinks and sliding_window are as in `decode`, the window counted back from each query token.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -247,12 +249,14 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     can_verify = verify_supported(T, D, block_size)
     if route is None:
         # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
-        route = "verify" if can_verify and (kv_code == FP8 or D != 128 or T * (Hq // Hkv) <= VERIFY_MAX_ROWS) else "tiled"
+        rows = T * (Hq // Hkv)
+        route = "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
+                                            or (kv_code == FP8 and (win > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")
     else:
-        _check(kv_code == BF16, "fp8 KV caches are read by the verify kernel only (T <= 64, head_dim 64 or 128)")
+        _check(not (kv_code == FP8 and win > 0), "a sliding window over an fp8 KV cache needs the verify kernel (T <= 64)")
     _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
                  query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out)
     if validate_tables:
@@ -286,9 +290,10 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
             _need_device("workspace", workspace)
             _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
         ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
-        rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), _ptr(seq_lens),
+        rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+                            _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
-                            block_tables.shape[1], num_blocks, float(scale), BF16, _ptr(sinks), win,
+                            block_tables.shape[1], num_blocks, float(scale), BF16, kv_code, _ptr(sinks), win,
                             _ptr(workspace), ws_bytes, _stream_ptr(q.device))
     _raise_on(rc, "pa_prefill")
     return out

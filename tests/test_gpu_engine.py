@@ -126,7 +126,7 @@ def test_serving_loop_fp8_pool(rng):
     dequantised pool within the fp8 bar."""
     from nkipy_amd.engine import PagedAttention, PagedKVCache
     S, Hq, Hkv, D, bs = 2, 8, 2, 128, 16
-    cache = PagedKVCache(num_blocks=12, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=4,
+    cache = PagedKVCache(num_blocks=12, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=5,
                          dtype=torch.float8_e4m3fn)
     layer = PagedAttention(cache, Hq)
     for step in range(40):
@@ -146,7 +146,12 @@ def test_serving_loop_fp8_pool(rng):
                            layer.scale, k_scale=cache.k_scale.cpu().numpy(), v_scale=cache.v_scale.cpu().numpy(), q_dtype="bf16")
     assert_close_abs(got, want, 5e-2)
     assert cache.lens == [43, 42] and np.all(got[1, 2] == 0)
-    with pytest.raises(NotImplementedError):     # longer runs would need the tiled kernel, which reads bf16 pools only
-        layer.step(bf16_to_dev(_rand(rng, (S, 65, Hq, D))), bf16_to_dev(_rand(rng, (S, 65, Hkv, D))),
-                   bf16_to_dev(_rand(rng, (S, 65, Hkv, D))), [2, 2])
-    assert cache.lens == [43, 42]
+    # a longer chunk goes through the tiled kernel, which expands the fp8 codes on their way into LDS
+    cache.release(1)
+    xq, xk, xv = _rand(rng, (S, 70, Hq, D)), _rand(rng, (S, 70, Hkv, D)), _rand(rng, (S, 70, Hkv, D))
+    got = dev_to_f32(layer.step(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv), [0, 70]))
+    want = O.paged_prefill(xq, cache.k_cache.view(torch.uint8).cpu().numpy(), cache.v_cache.view(torch.uint8).cpu().numpy(),
+                           cache.block_tables.cpu().numpy(), cache.seq_lens.cpu().numpy(), np.array([0, 70], np.int32),
+                           layer.scale, k_scale=cache.k_scale.cpu().numpy(), v_scale=cache.v_scale.cpu().numpy(), q_dtype="bf16")
+    assert_close_abs(got, want, 5e-2)
+    assert cache.lens == [43, 70] and np.all(got[0] == 0)

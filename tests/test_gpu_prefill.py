@@ -298,3 +298,36 @@ def test_prefill_split_over_key_tiles(pa, T, Hq, Hkv, window):
     assert np.all(got[1, 5:] == 0)
     with pytest.raises(ValueError):
         pa.prefill(*args, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"), **kw)
+
+
+@pytest.mark.parametrize("bs", [16, 64, 24])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (4, 4)])
+def test_prefill_fp8_pool(pa, bs, Hq, Hkv):
+    """Long chunks over an fp8 pool: codes times their block's scale become bf16 on the way into LDS
+    (block sizes that are and are not a power of two; chunks that start inside a block)."""
+    rng = np.random.default_rng(bs + Hq)
+    T, D = 200, 128
+    qlens, prefixes = [200, 77, 1, 130], [0, 300, 65, 1000]
+    B = len(qlens)
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    k *= rng.uniform(0.2, 3.0, size=(k.shape[0], 1, Hkv, 1)).astype(np.float32)     # different scales per block and head
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_prefill(q, kq, vq, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale,
+                           k_scale=ks, v_scale=vs, q_dtype="bf16", sinks=sinks)
+    got = pa.prefill(bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+                     torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(qlens), scale,
+                     k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(), sinks=bf16_to_dev(sinks),
+                     route="tiled")
+    torch.cuda.synchronize()
+    got = dev_to_f32(got)
+    assert_close_abs(got, want, 5e-2)
+    assert np.all(got[1, 77:] == 0) and np.all(got[2, 1:] == 0)
+    with pytest.raises(ValueError):
+        pa.prefill(bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+                   torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(qlens), scale,
+                   k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(), sliding_window=50, route="tiled")

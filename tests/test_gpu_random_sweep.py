@@ -28,8 +28,10 @@ def _draw(case):
     if kind == "tiled" and D != 128:
         kind = "verify"
     T = 1 if kind == "decode" else int(rng.integers(2, 20)) if kind == "verify" else int(rng.integers(65, 300))
-    fp8 = bool(rng.integers(0, 2)) and kind != "tiled"
+    fp8 = bool(rng.integers(0, 2))
     window = None if rng.integers(0, 2) else int(rng.choice([1, 7, 32, 33, 100, 700]))
+    if fp8 and kind == "tiled":
+        window = None                      # a window over an fp8 pool is the verify kernel's only
     sinks = bool(rng.integers(0, 2))
     long_ctx = rng.integers(0, 4) == 0
     prefixes = [int(rng.integers(0, 3000 if long_ctx else 300)) for _ in range(B)]
