@@ -116,6 +116,43 @@ def main():
     out.update(bsp_q=qb, bsp_k=kb, bsp_v=vb, bsp_scale=np.float32(sc), bsp_local=np.int32(1),
                bsp_stride=np.int32(2), bsp_expected=exp)
 
+    # 6. the gpt-oss variant on a verify-sized chunk: bf16, D=64, 8 q heads on one kv head, 4 query tokens
+    #    (ragged), sliding window 20 and per-head sinks
+    B, T, Hq, Hkv, D, bs = 2, 4, 8, 1, 64, 16
+    qlens, prefixes, window = [4, 3], [37, 5], 20
+    ctxs = [p_ + n for p_, n in zip(prefixes, qlens)]
+    k, v, t = paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, T, Hq, D)).astype(np.float32)
+    sinks = O.bf16_bits_to_f32(O.f32_to_bf16_bits(rng.standard_normal(Hq).astype(np.float32) * 2))
+    qb, kb, vb = O.f32_to_bf16_bits(q), O.f32_to_bf16_bits(k), O.f32_to_bf16_bits(v)
+    qf, kf, vf = O.bf16_bits_to_f32(qb), O.bf16_bits_to_f32(kb), O.bf16_bits_to_f32(vb)
+    sc6 = float(np.float32(1 / np.sqrt(D)))
+    exp = np.zeros((B, T, Hq, D))
+    for b in range(B):
+        exp[b, :qlens[b]] = O.attention_bruteforce_f64(qf[b, :qlens[b]], rows(kf, t[b], ctxs[b], bs), rows(vf, t[b], ctxs[b], bs),
+                                                       sc6, prefix=prefixes[b], window=window, sinks=sinks)
+    out.update(ver_q=qb, ver_k=kb, ver_v=vb, ver_tables=t, ver_ctx=np.array(ctxs, np.int32),
+               ver_qlens=np.array(qlens, np.int32), ver_scale=np.float32(sc6), ver_window=np.int32(window),
+               ver_sinks=sinks.astype(np.float32), ver_expected=exp)
+
+    # 7. fp8 KV decode with a sliding window of 48 and sinks, D=128, block 32
+    B, Hq, Hkv, D, bs = 2, 4, 2, 128, 32
+    ctxs, window = [50, 130], 48
+    k, v, t = paged(rng, B, Hkv, D, bs, ctxs)
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    sinks = rng.standard_normal(Hq).astype(np.float32)
+    qb = O.f32_to_bf16_bits(q)
+    qf = O.bf16_bits_to_f32(qb)
+    kd = O.FP8_E4M3FN_LUT[kq].astype(np.float64) * ks[:, None, :, None]
+    vd = O.FP8_E4M3FN_LUT[vq].astype(np.float64) * vs[:, None, :, None]
+    exp = np.stack([O.attention_bruteforce_f64(qf[b][None], rows(kd, t[b], ctxs[b], bs), rows(vd, t[b], ctxs[b], bs), sc,
+                                               prefix=ctxs[b] - 1, window=window, sinks=sinks)[0] for b in range(B)])
+    out.update(win8_q=qb, win8_k=kq, win8_v=vq, win8_kscale=ks, win8_vscale=vs, win8_tables=t,
+               win8_ctx=np.array(ctxs, np.int32), win8_scale=np.float32(sc), win8_window=np.int32(window),
+               win8_sinks=sinks, win8_expected=exp)
+
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "paged_attention_golden.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes")

@@ -49,6 +49,16 @@ def test_oracle_blocksparse_golden():
     _bf16_close(got, G["bsp_expected"])
 
 
+def test_oracle_window_and_sinks_golden():
+    got = O.paged_prefill(G["ver_q"], G["ver_k"], G["ver_v"], G["ver_tables"], G["ver_ctx"], G["ver_qlens"],
+                          float(G["ver_scale"]), sliding_window=int(G["ver_window"]), sinks=G["ver_sinks"])
+    _bf16_close(got, G["ver_expected"])
+    got = O.paged_decode(G["win8_q"], G["win8_k"], G["win8_v"], G["win8_tables"], G["win8_ctx"], float(G["win8_scale"]),
+                         k_scale=G["win8_kscale"], v_scale=G["win8_vscale"], q_dtype="bf16",
+                         sliding_window=int(G["win8_window"]), sinks=G["win8_sinks"])
+    _bf16_close(got, G["win8_expected"])
+
+
 # ------------------------------------------------------------------------- HIP ops (GPU)
 def _bf(bits):
     return torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16)
@@ -96,3 +106,19 @@ def test_hip_prefill_and_blocksparse_golden():
     got = pa.blocksparse_prefill(_bf(G["bsp_q"]), _bf(G["bsp_k"]), _bf(G["bsp_v"]), float(G["bsp_scale"]),
                                  block=64, local_blocks=int(G["bsp_local"]), vert_stride=int(G["bsp_stride"]))
     assert np.max(np.abs(got.float().cpu().numpy() - G["bsp_expected"])) <= 2e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("route", ["verify", None])
+def test_hip_window_and_sinks_golden(route):
+    import nkipy_amd as pa
+    got = pa.prefill(_bf(G["ver_q"]), _bf(G["ver_k"]), _bf(G["ver_v"]), _i32(G["ver_tables"]), _i32(G["ver_ctx"]),
+                     _i32(G["ver_qlens"]), float(G["ver_scale"]), sliding_window=int(G["ver_window"]),
+                     sinks=torch.from_numpy(G["ver_sinks"]).cuda(), route=route).float().cpu().numpy()
+    assert np.max(np.abs(got - G["ver_expected"])) <= 2e-2
+    got8 = pa.decode(_bf(G["win8_q"]), torch.from_numpy(G["win8_k"]).cuda().view(torch.float8_e4m3fn),
+                     torch.from_numpy(G["win8_v"]).cuda().view(torch.float8_e4m3fn), _i32(G["win8_tables"]),
+                     _i32(G["win8_ctx"]), float(G["win8_scale"]), k_scale=torch.from_numpy(G["win8_kscale"]).cuda(),
+                     v_scale=torch.from_numpy(G["win8_vscale"]).cuda(), sliding_window=int(G["win8_window"]),
+                     sinks=torch.from_numpy(G["win8_sinks"]).cuda()).float().cpu().numpy()
+    assert np.max(np.abs(got8 - G["win8_expected"])) <= 5e-2
