@@ -376,14 +376,14 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
   p.scale_log2e = scale * kLog2e;
   if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
-  if (sliding_window > 0 && (fp8 || p.impl == 1 || !prefill_async_supported(p)))
-    return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (bf16 pool, block_size a power of two >= 16)");
+  if (sliding_window > 0 && (p.impl == 1 || !prefill_async_supported(p)))
+    return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
   p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
   // few workgroups and a long table: split the key tiles of a query tile over several workgroups when the
   // caller brought the workspace for it (without one the call runs unsplit)
   p.splits = 1;
-  if (workspace && !fp8) {
+  if (workspace) {
     if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
     const int want = g_prefill_split.load() ? prefill_async_splits(p, current_num_cus()) : 1;
     if (want > 1 && workspace_bytes >= prefill_split_bytes(p, want)) {

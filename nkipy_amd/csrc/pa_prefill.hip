@@ -376,7 +376,7 @@ bool prefill_supported(const PrefillParams& p) {
 }
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s) {
-  if (!p.kv_fp8 && p.impl != 1 && prefill_async_supported(p))
+  if (p.impl != 1 && prefill_async_supported(p))
     return launch_prefill_async(p, p.impl == 4 || p.impl == 8 ? p.impl : 0, s);
   const int nqt = (p.T + BM - 1) / BM;
   if (nqt > 65535 * 32 || p.Hq > 65535 || p.B > 65535) return hipErrorInvalidValue;

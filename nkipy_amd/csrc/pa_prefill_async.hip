@@ -84,7 +84,13 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 // SPLIT (few workgroups, long contexts): p.splits workgroups share the key tiles of one query tile
 // and leave unnormalised partial results (m, l, O) in the workspace for prefill_split_reduce_kernel:
 // a lone workgroup walks its tiles at about a microsecond each, whatever the rest of the chip does.
-template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT>
+// FP8 (8 waves, paged): the pool holds e4m3fn codes with a float32 scale per (block, kv head).  The
+// copies bring raw codes into a ring of four 16 KB stages; every wave then expands the 8 rows it
+// copied itself (codes x their block's scale -> bf16, once per workgroup, not once per reader) into one
+// of two bf16 stages in exactly the layout the bf16 path copies into, one tile ahead of the
+// compute, so everything from the fragment reads on is shared.  Raw rows are private to the wave that
+// copies and expands them, so the raw ring needs no barrier; the bf16 stages use the one per tile.
+template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT, bool FP8>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -93,8 +99,13 @@ void prefill_async_kernel(PrefillParams p) {
   constexpr int STAGE_B = 2 * TILE_B;        // K then V
   constexpr int UK = BN / 4;                 // 1 KB copy units per tensor tile
   constexpr int BMW = 32 * NW;               // query rows per workgroup
-  constexpr int NST = NW == 8 ? 4 : 2;   // LDS stages
-  constexpr int UPW = 2 * UK / NW;           // copy units per wave per tile
+  constexpr int NST = NW == 8 ? 4 : 2;   // LDS stages the copies land in
+  constexpr int UPW = FP8 ? 2 : 2 * UK / NW; // copy units per wave per tile (FP8: 8 raw rows of K, 8 of V)
+  static_assert(!FP8 || (NW == 8 && MODE == 1 && !SPARSE && !PACK && TT == 2), "fp8 pools: 8-wave paged dense form only");
+  constexpr int EB = FP8 ? 1 : 2;            // bytes per pool element
+  constexpr int RAW_TILE_B = BN * HD;        // FP8: one tensor's raw tile
+  constexpr int RAW_STAGE_B = 2 * RAW_TILE_B;
+  constexpr int BFS = FP8 ? 2 : NST;         // stages that hold bf16 tiles (FP8: the raw ring lies behind them)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -178,9 +189,9 @@ void prefill_async_kernel(PrefillParams p) {
   // with the global chunk  position ^ (row & 7).
   const const_i32_ptr table = MODE != 0 ? (const_i32_ptr)(uintptr_t)(p.block_tables + (long)b * p.max_blocks) : nullptr;
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
-  const long kv_row_bytes = (long)p.Hkv * ROW_B;
-  const char* kbase = (const char*)p.k + (long)hk * ROW_B;
-  const char* vbase = (const char*)p.v + (long)hk * ROW_B;
+  const long kv_row_bytes = (long)p.Hkv * HD * EB;
+  const char* kbase = (const char*)p.k + (long)hk * HD * EB;
+  const char* vbase = (const char*)p.v + (long)hk * HD * EB;
   const int dma_rr = lane >> 4, dma_pos = lane & 15;
   // every unit of a wave starts at the same row modulo 16 (NW is a multiple of 4), hence the
   // same swizzle: K rows use row & 15, V rows 4 * (row & 3) (what their read patterns want)
@@ -190,6 +201,8 @@ void prefill_async_kernel(PrefillParams p) {
   const uint32_t block_bytes_u = MODE != 0 ? (uint32_t)p.block_size * kv_row_bytes_u : 0u;
   const int dma_lane_off_k = (int)(dma_rr * kv_row_bytes) + dma_chunk_k * 16;
   const int dma_lane_off_v = (int)(dma_rr * kv_row_bytes) + dma_chunk_v * 16;
+  // FP8: a unit is 8 raw rows of 128 B, copied as they lie: lane i -> row i / 8, 16-byte piece i % 8
+  const int dma_lane_off_raw = (int)((lane >> 3) * kv_row_bytes) + (lane & 7) * 16;
 
   auto lane_row = [&](int key) __attribute__((always_inline)) -> long {   // same, per lane, clamped
     key = min(key, ctx - 1);
@@ -206,7 +219,7 @@ void prefill_async_kernel(PrefillParams p) {
     if (MODE == 0) return;
 #pragma unroll
     for (int i = 0; i < UPW / 2; ++i) {
-      const int r0 = 4 * ((wave + NW * i) & (UK - 1));
+      const int r0 = FP8 ? 8 * wave : 4 * ((wave + NW * i) & (UK - 1));
       blk_pf[i] = table[min((kt * BN + r0) >> p.block_shift, p.max_blocks - 1)];
     }
   };
@@ -214,6 +227,20 @@ void prefill_async_kernel(PrefillParams p) {
   // the K (j < UPW/2) or V tile, u = (wave + NW j) mod UK.
   auto issue_tile = [&](int kt, int stage) __attribute__((always_inline)) {
     const int key0 = kt * BN;
+    if (FP8) {       // this wave's 8 rows of K and of V, raw, into its own 1 KB of the raw stage
+      const uint32_t rbase = smem_base + BFS * STAGE_B + stage * RAW_STAGE_B + wave * 1024;
+      if (key0 + BN <= ctx) {
+        const uint32_t blk = (uint32_t)min(max(blk_pf[0], 0), p.num_blocks - 1);
+        const uint64_t off = (uint64_t)blk * block_bytes_u + (uint32_t)((key0 + 8 * wave) & (p.block_size - 1)) * kv_row_bytes_u;
+        dma16_uniform(kbase + off, dma_lane_off_raw, rbase);
+        dma16_uniform(vbase + off, dma_lane_off_raw, rbase + RAW_TILE_B);
+      } else {
+        const long src = lane_row(key0 + 8 * wave + (lane >> 3)) * kv_row_bytes + (lane & 7) * 16;
+        dma16_lane(kbase + src, rbase);
+        dma16_lane(vbase + src, rbase + RAW_TILE_B);
+      }
+      return;
+    }
     const uint32_t sbase = smem_base + stage * STAGE_B;
     if (key0 + BN <= ctx) {                       // whole tile inside the context: one row base per unit
       // byte offset of a unit's first row = block * (block bytes) + in-block row * (row bytes):
@@ -324,10 +351,45 @@ void prefill_async_kernel(PrefillParams p) {
   // scalar load in flight turns every LDS wait into a wait for everything.
   auto prefetch_next = [&]() __attribute__((always_inline)) { prefetch_table(w_i.kt < ntiles ? w_i.kt : kt_first); };
   prefetch_table(kt_first);
+  // FP8: scales of this wave's rows in the tiles in flight (its 8 rows lie in one block); a request
+  // puts the new pair in slot 3, a shift per tile brings it to slot 0 when the tile is expanded
+  typedef const __attribute__((address_space(4))) float* const_f32_ptr;
+  float ksq[4] = {0.f, 0.f, 0.f, 0.f}, vsq[4] = {0.f, 0.f, 0.f, 0.f};
   auto request_next = [&]() __attribute__((always_inline)) {
     issue_tile(w_i.kt < ntiles ? w_i.kt : kt_first, stage_i);
+    if (FP8) {
+      const long si = (long)min(max(blk_pf[0], 0), p.num_blocks - 1) * p.Hkv + hk;
+      ksq[3] = ((const_f32_ptr)(uintptr_t)p.k_scale)[si];
+      vsq[3] = ((const_f32_ptr)(uintptr_t)p.v_scale)[si];
+    }
     if (w_i.kt < ntiles) walk_step(w_i);
     stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
+  };
+  auto shift_scales = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) { ksq[i] = ksq[i + 1]; vsq[i] = vsq[i + 1]; }
+  };
+  // FP8: codes of tile kt in raw stage rs -> bf16 values in stage bs, this wave's 8 rows; rows past the
+  // context get the scale 0 (their codes are a copy of the last valid row, their block may not exist)
+  auto expand = [&](int kt, int rs, int bs, float ks, float vs) __attribute__((always_inline)) {
+    const char* raw = smem + BFS * STAGE_B + rs * RAW_STAGE_B + wave * 1024 + lane * 16;
+    const int row = 8 * wave + (lane >> 3), c16 = lane & 7;
+    const bool live = kt * BN + row < ctx;
+    const float sk = live ? ks : 0.f, sv = live ? vs : 0.f;
+    const uint4 rk = *(const uint4*)raw, rv = *(const uint4*)(raw + RAW_TILE_B);
+    auto half = [&](uint32_t a, uint32_t b2, float scl) __attribute__((always_inline)) -> uint4 {
+      float f[8];
+      fp8x4_to_float(a, f);
+      fp8x4_to_float(b2, f + 4);
+      return make_uint4(pack_bf16x2(f[0] * scl, f[1] * scl), pack_bf16x2(f[2] * scl, f[3] * scl),
+                        pack_bf16x2(f[4] * scl, f[5] * scl), pack_bf16x2(f[6] * scl, f[7] * scl));
+    };
+    char* kd = smem + bs * STAGE_B + row * ROW_B;
+    *(uint4*)(kd + (((2 * c16) ^ (row & 15)) << 4)) = half(rk.x, rk.y, sk);
+    *(uint4*)(kd + (((2 * c16 + 1) ^ (row & 15)) << 4)) = half(rk.z, rk.w, sk);
+    char* vd = kd + TILE_B;
+    *(uint4*)(vd + (((2 * c16) ^ (4 * (row & 3))) << 4)) = half(rv.x, rv.y, sv);
+    *(uint4*)(vd + (((2 * c16 + 1) ^ (4 * (row & 3))) << 4)) = half(rv.z, rv.w, sv);
   };
 
   // ---- fragment loads and matrix steps, one "group" at a time -------------------------
@@ -478,17 +540,36 @@ void prefill_async_kernel(PrefillParams p) {
   }
 #pragma unroll
   for (int s = 1; s < NST - 1; ++s) {
+    if (FP8) shift_scales();
     request_next();
     prefetch_next();
+  }
+  if (FP8) {     // the raw ring holds four tiles; the first one is expanded before the loop
+    shift_scales();
+    request_next();
+    prefetch_next();
+    wait_vmcnt<3 * UPW>();
+    expand(kt_first, 0, 0, ksq[0], vsq[0]);
   }
 
   {
     Walk w_c = w_first;
     int stage_c = 0;
+    int rs_n = 1;                                  // FP8: raw stage of the tile after the current one
     while (w_c.kt < ntiles) {
-      wait_vmcnt<(NST - 2) * UPW>();               // this wave's part of the current tile has landed
+      if (FP8) {
+        wait_vmcnt<2 * UPW>();                     // this wave's raw rows of the next tile have landed
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its bf16 rows of the current one are written
+      } else {
+        wait_vmcnt<(NST - 2) * UPW>();             // this wave's part of the current tile has landed
+      }
       __builtin_amdgcn_s_barrier();                // ... and everyone's; all waves are done with the previous tile
+      if (FP8) shift_scales();
       request_next();
+      if (FP8) {
+        if (w_c.kt + 1 < ntiles) expand(w_c.kt + 1, rs_n, stage_c ^ 1, ksq[0], vsq[0]);
+        rs_n = (rs_n + 1) & 3;
+      }
       if (tile_active(w_c)) {
         f32x16_t sacc[TT];
         uint32_t pw[TT][8];
@@ -501,7 +582,7 @@ void prefill_async_kernel(PrefillParams p) {
         prefetch_next();
       }
       walk_step(w_c);
-      stage_c = stage_c + 1 == NST ? 0 : stage_c + 1;
+      stage_c = stage_c + 1 == BFS ? 0 : stage_c + 1;
     }
   }
   wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
@@ -571,12 +652,12 @@ __global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams
   *(uint2*)dst = make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
 }
 
-template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false>
+template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false, bool FP8 = false>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
@@ -587,7 +668,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   const long groups = (long)p.B * p.Hkv;
   const long total = 8 * ((groups + 7) / 8) * per_group * (SPLIT ? p.splits : 1);
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   if (SPLIT) {
     const long items = (long)p.B * p.T * p.Hq * (HD / 4);
     hipLaunchKernelGGL(prefill_split_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, p);
@@ -614,7 +695,7 @@ bool prefill_async_supported(const PrefillParams& p) {
 static bool prefill_packs(const PrefillParams& p) {
   const bool sparse = p.sparse_stride > 0, paged = p.block_tables != nullptr;
   // chunks shorter than a 4-wave tile of a GQA model: rows packed over the heads of a kv group
-  return paged && !sparse && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
+  return paged && !sparse && !p.kv_fp8 && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
 }
 static int prefill_waves(const PrefillParams& p, int waves) {
   const bool sparse = p.sparse_stride > 0;
@@ -622,6 +703,7 @@ static int prefill_waves(const PrefillParams& p, int waves) {
   // 256 rows, 4-stage ring: half the copy requests per FLOP).  Measured within a few per cent of
   // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
   // and for the sparse form.
+  if (p.kv_fp8) return 8;              // fp8 pools: the 8-wave form only
   if (prefill_packs(p)) return 4;
   if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
   return waves;
@@ -645,6 +727,16 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   const bool paged = p.block_tables != nullptr;
   const bool pack = prefill_packs(p);
   waves = prefill_waves(p, waves);
+  if (p.kv_fp8) {
+    if (sparse || !paged || !p.k_scale || !p.v_scale) return hipErrorInvalidValue;
+    if (p.splits > 1) {
+      if (!p.ws_o || !p.ws_ml) return hipErrorInvalidValue;
+      return p.window > 0 ? launch_typed<false, 1, 8, 2, true, false, true, true>(p, s)
+                          : launch_typed<false, 1, 8, 2, false, false, true, true>(p, s);
+    }
+    return p.window > 0 ? launch_typed<false, 1, 8, 2, true, false, false, true>(p, s)
+                        : launch_typed<false, 1, 8, 2, false, false, false, true>(p, s);
+  }
   if (p.splits > 1) {
     if (sparse || !paged || !p.ws_o || !p.ws_ml) return hipErrorInvalidValue;
     if (p.window > 0) {

@@ -216,9 +216,6 @@ class PagedAttention:
             raise ValueError(f"expected one row per slot ({c.max_seqs}), got {B} rows and {len(query_lens)} lengths")
         if any(n < 0 or n > T for n in query_lens):
             raise ValueError("query_lens must lie in [0, T]")
-        if T > 64 and c.k_scale is not None and self.sliding_window:
-            raise NotImplementedError("a sliding window over an fp8 pool is read by the verify kernel only: feed the "
-                                      "prompt in chunks of at most 64 tokens")
         active = [s for s in range(B) if query_lens[s] > 0]
         c.extend(active, [query_lens[s] for s in active])
         self._qlens.copy_(torch.tensor(list(query_lens), dtype=torch.int32))

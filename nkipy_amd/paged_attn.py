@@ -217,9 +217,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query rows
     (HBM-bound: the context is read once per kv head); everything else through the tiled
     matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
-    (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both; behind the tiled route they
-    take the register-staged kernel (codes expanded to bf16 on their way into LDS) and no sliding
-    window.  sinks and sliding_window are as in `decode`, the window counted back from each query token.
+    (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both.  sinks and sliding_window are
+    as in `decode`, the window counted back from each query token.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -255,8 +254,6 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")
-    else:
-        _check(not (kv_code == FP8 and win > 0), "a sliding window over an fp8 KV cache needs the verify kernel (T <= 64)")
     _same_device(q, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
                  query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out)
     if validate_tables:

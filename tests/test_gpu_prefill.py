@@ -327,7 +327,49 @@ def test_prefill_fp8_pool(pa, bs, Hq, Hkv):
     got = dev_to_f32(got)
     assert_close_abs(got, want, 5e-2)
     assert np.all(got[1, 77:] == 0) and np.all(got[2, 1:] == 0)
-    with pytest.raises(ValueError):
-        pa.prefill(bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
-                   torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(qlens), scale,
-                   k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(), sliding_window=50, route="tiled")
+    # with a sliding window: the asynchronous-copy kernel (power-of-two blocks) takes it, the register-staged one does not
+    wargs = (bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+             torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(qlens), scale)
+    wkw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(), sliding_window=50, route="tiled")
+    if bs == 24:
+        with pytest.raises(RuntimeError):
+            pa.prefill(*wargs, **wkw)
+    else:
+        want = O.paged_prefill(q, kq, vq, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale,
+                               k_scale=ks, v_scale=vs, q_dtype="bf16", sliding_window=50)
+        assert_close_abs(dev_to_f32(pa.prefill(*wargs, **wkw)), want, 5e-2)
+
+
+def test_prefill_fp8_pool_kernels_agree(pa):
+    """The asynchronous-copy kernel (raw ring + expansion pass) and the register-staged kernel on the same fp8 pool."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(77)
+    T, D, Hq, Hkv, bs = 300, 128, 4, 2, 32
+    qlens, prefixes = [300, 150, 64], [700, 0, 33]
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, 3, Hkv, D, bs, ctxs)
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    # unused pool rows and the scales of unused blocks may hold anything
+    used = np.zeros(k.shape[0], bool)
+    for b in range(3):
+        used[tables[b, :(ctxs[b] + bs - 1) // bs]] = True
+    ks[~used] = np.nan
+    vs[~used] = np.nan
+    q = O.round_to_bf16(rng.standard_normal((3, T, Hq, D)).astype(np.float32))
+    args = (bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+            torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(qlens), 0.09)
+    kw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(), route="tiled")
+    a = dev_to_f32(pa.prefill(*args, **kw))
+    lib.pa_debug_set(3, 1)
+    try:
+        b_ = dev_to_f32(pa.prefill(*args, **kw))
+    finally:
+        lib.pa_debug_set(3, 0)
+    assert np.isfinite(a).all() and np.isfinite(b_).all()
+    assert np.max(np.abs(a - b_)) <= 2 ** -5
+    ks0, vs0 = np.nan_to_num(ks, nan=1.0), np.nan_to_num(vs, nan=1.0)
+    want = O.paged_prefill(q, kq, vq, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), 0.09,
+                           k_scale=ks0, v_scale=vs0, q_dtype="bf16")
+    assert_close_abs(a, want, 5e-2)

@@ -155,7 +155,5 @@ def test_verify_argument_errors(pa):
     big = bf16_to_dev(np.zeros((1, 65, 4, 128), np.float32))
     with pytest.raises(ValueError):
         pa.verify(big, *args[1:])
-    with pytest.raises(ValueError):     # a sliding window over an fp8 pool needs the verify kernel, which stops at 64 tokens
-        pa.prefill(big, args[1].view(torch.uint8)[..., :128].contiguous(), args[2].view(torch.uint8)[..., :128].contiguous(),
-                   *args[3:], k_scale=torch.ones(k.shape[0], 2, device="cuda"), v_scale=torch.ones(k.shape[0], 2, device="cuda"),
-                   sliding_window=16)
+    with pytest.raises(ValueError):     # forced onto the verify kernel, which stops at 64 tokens
+        pa.prefill(big, *args[1:], route="verify")
