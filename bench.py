@@ -229,14 +229,19 @@ def _mfma_ceiling(lib, sample):
     return round(best, 1)
 
 
-def bench_prefill(steps, warmup, lib, pa, W):
+def bench_prefill(steps, warmup, lib, pa, W, fp8=False):
+    """config 3; with fp8=True the same workload over the pool quantised to e4m3 with per-(block, kv head) scales."""
     from oracle import paged_attention_oracle as O
     from tests.pa_testlib import dev_bits
     w = W.make_prefill()
     out = torch.empty_like(w.q)
+    kc, vc, ks, vs = w.k_cache, w.v_cache, None, None
+    if fp8:
+        kc, ks = W.quantize_pool_fp8(w.k_cache)
+        vc, vs = W.quantize_pool_fp8(w.v_cache)
 
     def step():
-        pa.prefill(w.q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens, w.scale, out=out)
+        pa.prefill(w.q, kc, vc, w.block_tables, w.seq_lens, w.query_lens, w.scale, out=out, k_scale=ks, v_scale=vs)
 
     sec = _time_steps(step, steps, warmup)
     lib.pa_profile_enable(1)
@@ -249,21 +254,24 @@ def bench_prefill(steps, warmup, lib, pa, W):
 
     def cpu():
         heads = [0, 1, 2, 3]
-        O.paged_prefill(dev_bits(w.q), dev_bits(w.k_cache), dev_bits(w.v_cache), w.block_tables.cpu().numpy(),
-                        w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy(), w.scale, seqs=[7], heads=heads)
+        O.paged_prefill(dev_bits(w.q), dev_bits(kc), dev_bits(vc), w.block_tables.cpu().numpy(),
+                        w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy(), w.scale, seqs=[7], heads=heads,
+                        k_scale=None if ks is None else ks.cpu().numpy(), v_scale=None if vs is None else vs.cpu().numpy())
         return 4 * D * len(heads) * (T * int(w.prefix[7]) + T * (T + 1) // 2)
 
     res = {
         "metric": "prefill attn TFLOP/s (% MFMA peak)",
         "value": round(fl / sec / 1e12, 2), "unit": "TFLOP/s",
         "pct_of_bf16_peak": round(100.0 * fl / sec / 1e12 / BF16_PEAK_TFLOPS, 2),
-        "ms_per_step": round(sec * 1e3, 5), "dtype": "bf16, fp32 accumulate",
-        "config": {"workload": f"C3 paged chunked prefill: B={B}, T={T}, Hq={Hq}, Hkv={w.k_cache.shape[2]}, "
+        "ms_per_step": round(sec * 1e3, 5),
+        "dtype": "fp8-e4m3 KV expanded to bf16 in LDS / bf16 q, fp32 accumulate" if fp8 else "bf16, fp32 accumulate",
+        "config": {"workload": f"C3 paged chunked prefill{' over the fp8-quantised pool' if fp8 else ''}: B={B}, T={T}, "
+                               f"Hq={Hq}, Hkv={w.k_cache.shape[2]}, "
                                f"D={D}, block_size={w.k_cache.shape[1]}, prefix={w.prefix.tolist()}",
                    "flops": fl},
         "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
-                     "traffic": _traffic(3)[0], "traffic_source": _traffic(3)[1],
+                     "traffic": None if fp8 else _traffic(3)[0], "traffic_source": None if fp8 else _traffic(3)[1],
                      "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms),
                      "mfma_only_loop_same_data": _mfma_ceiling(lib, w.k_cache)},
@@ -410,7 +418,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8, 9])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -439,6 +447,8 @@ def main():
         res = bench_pre_attention(args.steps, args.warmup, lib, pa, W)
     elif args.config == 8:
         res = bench_verify(args.steps, args.warmup, lib, pa, W)
+    elif args.config == 9:
+        res = bench_prefill(args.steps, args.warmup, lib, pa, W, fp8=True)
     else:
         res = bench_blocksparse(args.steps, args.warmup, lib, pa, W)
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"),
