@@ -341,7 +341,10 @@ size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int bloc
   memset(&p, 0, sizeof(p));
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, 1);
   p.block_tables = (const int32_t*)16;     // paged form (only tested for null)
-  return prefill_split_bytes(p, prefill_async_splits(p, current_num_cus()));
+  const size_t plain = prefill_split_bytes(p, prefill_async_splits(p, current_num_cus()));
+  p.kv_fp8 = 1;                            // fp8 pools use another workgroup shape: cover both
+  const size_t fp8 = prefill_split_bytes(p, prefill_async_splits(p, current_num_cus()));
+  return plain > fp8 ? plain : fp8;
 }
 
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,

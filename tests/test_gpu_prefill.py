@@ -373,3 +373,31 @@ def test_prefill_fp8_pool_kernels_agree(pa):
     want = O.paged_prefill(q, kq, vq, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), 0.09,
                            k_scale=ks0, v_scale=vs0, q_dtype="bf16")
     assert_close_abs(a, want, 5e-2)
+
+
+def test_prefill_fp8_pool_split_over_key_tiles(pa):
+    """One long fp8 context, one chunk: the split form of the fp8 kernel, with and without a window."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(91)
+    T, D, Hq, Hkv, bs = 200, 128, 4, 1, 32
+    ctxs, qlens = [5200], [200]
+    k, v, tables = make_paged(rng, 1, Hkv, D, bs, ctxs)
+    kq, ks = O.quantize_kv_fp8(k)
+    vq, vs = O.quantize_kv_fp8(v)
+    q = O.round_to_bf16(rng.standard_normal((1, T, Hq, D)).astype(np.float32))
+    assert lib.pa_prefill_workspace_bytes(1, T, Hq, Hkv, D, bs, tables.shape[1]) > 0
+    args = (bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+            torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(tables), _i32(ctxs), _i32(qlens), 0.09)
+    for window in (None, 900):
+        want = O.paged_prefill(q, kq, vq, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), 0.09,
+                               k_scale=ks, v_scale=vs, q_dtype="bf16", sliding_window=window)
+        kw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda(), sliding_window=window, route="tiled")
+        got = dev_to_f32(pa.prefill(*args, **kw))
+        lib.pa_debug_set(6, 0)
+        try:
+            unsplit = dev_to_f32(pa.prefill(*args, **kw))
+        finally:
+            lib.pa_debug_set(6, 1)
+        assert_close_abs(got, want, 5e-2)
+        assert np.max(np.abs(got - unsplit)) <= 2 ** -6
