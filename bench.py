@@ -105,6 +105,7 @@ MEASURED_TRAFFIC_BYTES = {
     2: {"bytes": 1_098_900_000, "source": "profiles/decode_balanced_kernel_C2.md"},
     3: {"bytes": 385_200_000, "source": "profiles/prefill_async_kernel_C3.md"},
     4: {"bytes": 743_900_000, "source": "profiles/prefill_async_kernel_C4.md"},
+    5: {"bytes": 2_402_400_000, "source": "profiles/decode_balanced_kernel_C5.md"},
     8: {"bytes": 1_123_600_000, "source": "profiles/decode_balanced_kernel_verify_T4.md"},
 }
 
