@@ -230,6 +230,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
       return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     p.ws_out = (float*)workspace;
     p.ws_ml = p.ws_out + (size_t)Hq * ((size_t)B + p.bal_gv) * D;
+    p.ws_start = (int32_t*)(p.ws_ml + (size_t)Hq * ((size_t)B + p.bal_gv) * 2);
     profile_begin(s);
     hipError_t e = launch_decode_balanced(p, kv_dtype, s);
     profile_end(s);
@@ -314,6 +315,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
     return fail_arg("pa_verify: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   p.ws_out = (float*)workspace;
   p.ws_ml = p.ws_out + (size_t)Hq * T * ((size_t)B + p.bal_gv) * D;
+  p.ws_start = (int32_t*)(p.ws_ml + (size_t)Hq * T * ((size_t)B + p.bal_gv) * 2);
   hipStream_t s = (hipStream_t)stream;
   profile_begin(s);
   hipError_t e = launch_decode_balanced(p, kv_dtype, s);

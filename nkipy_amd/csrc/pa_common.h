@@ -81,6 +81,7 @@ struct DecodeParams {
   void* out;                // shaped like q
   float* ws_out;            // [B, Hq, P, D]
   float* ws_ml;             // [B, Hq, P, 2]
+  int32_t* ws_start;        // balanced schedule: [B + 1] tiles before each sequence, and the total
   int B, Hq, Hkv, D;
   int T;                    // query tokens per sequence (1: decode)
   int window;               // sliding window in tokens (balanced schedule only), 0 = none

@@ -639,6 +639,22 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 
   int dummy_b = 0, dummy_s = 0;
   const int N = scan_tiles(p, lane, -1, &dummy_b, &dummy_s);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
+    // tiles before each sequence (and the total), for the merge kernel: it then needs no scan of its own
+    int base = 0;
+    for (int bb = 0; bb < p.B; bb += 64) {
+      const int t = (bb + lane < p.B) ? span_tiles(p, bb + lane) : 0;
+      int incl = t;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int v = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += v;
+      }
+      if (bb + lane < p.B) p.ws_start[bb + lane] = base + incl - t;
+      base += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) p.ws_start[p.B] = base;
+  }
   if (N == 0) return;
   const int L = (N + gv - 1) / gv;
   int f = cv * L;
@@ -677,10 +693,9 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 template <int D, int G>
 __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParams p) {
   const int b = blockIdx.x;
-  const int lane = threadIdx.x & 63;
-  int bb = 0, start = 0;
-  const int N = scan_tiles(p, lane, -1, &bb, &start);
-  const int T = span_tiles(p, b);
+  const int start = p.ws_start[b];                   // tiles before this sequence, written by the streaming kernel
+  const int T = p.ws_start[b + 1] - start;
+  const int N = p.ws_start[p.B];
   constexpr int QUADS = D / 4;
   const int item = blockIdx.y * (256 / G) + threadIdx.x / G;
   const int g = threadIdx.x % G;
@@ -700,16 +715,6 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   }
   const int gv = p.bal_gv;
   const int L = (N + gv - 1) / gv;
-  {   // tiles before sequence b = flattened index of its first tile
-    int base = 0;
-    for (int x = 0; x < b; x += 64) {
-      int t = (x + lane < b) ? span_tiles(p, x + lane) : 0;
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
-      base += t;
-    }
-    start = base;
-  }
   const int c_first = start / L, c_last = (start + T - 1) / L;
   if (c_first == c_last || !mine) return;   // single piece: written by the streaming kernel
   const long base_slot = (long)hq * (p.B + gv) + b;
@@ -802,7 +807,8 @@ void plan_decode_balanced(DecodeParams& p, int num_cus) {
 }
 
 size_t decode_balanced_workspace_bytes(int B, int Hq, int D, int gv) {
-  return (size_t)Hq * ((size_t)B + gv) * ((size_t)D + 2) * sizeof(float);
+  // partials [Hq][B + gv][D + 2] floats, then B + 1 tile prefix sums
+  return (size_t)Hq * ((size_t)B + gv) * ((size_t)D + 2) * sizeof(float) + ((size_t)B + 1) * sizeof(int32_t);
 }
 
 hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream_t s) {
