@@ -637,8 +637,30 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
   const int cv = blockIdx.x * p.bal_ns + wave / p.bal_hsw;   // chunk of this wave
   const int gv = p.bal_gv;
 
-  int dummy_b = 0, dummy_s = 0;
-  const int N = scan_tiles(p, lane, -1, &dummy_b, &dummy_s);
+  // Total number of tiles and the sequence that holds this wave's first tile.  Up to 512 sequences
+  // the lengths are fetched once, all loads in flight together, and scanned in registers; beyond
+  // that, two passes over seq_lens.
+  constexpr int SCAN_STEPS = 8;
+  const bool scan_in_regs = p.B <= 64 * SCAN_STEPS;
+  int N = 0, tl[SCAN_STEPS], incl[SCAN_STEPS];
+  if (scan_in_regs) {
+#pragma unroll
+    for (int i = 0; i < SCAN_STEPS; ++i) tl[i] = (64 * i + lane < p.B) ? span_tiles(p, 64 * i + lane) : 0;
+#pragma unroll
+    for (int i = 0; i < SCAN_STEPS; ++i) {
+      int x = tl[i];
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int v = __shfl_up(x, off, 64);
+        if (lane >= off) x += v;
+      }
+      incl[i] = x;
+      N += __shfl(x, 63, 64);
+    }
+  } else {
+    int dummy_b = 0, dummy_s = 0;
+    N = scan_tiles(p, lane, -1, &dummy_b, &dummy_s);
+  }
   if (blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
     // tiles before each sequence (and the total), for the merge kernel: it then needs no scan of its own
     int base = 0;
@@ -661,7 +683,24 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
   if (f >= N) return;
   const int f_end = min(N, f + L);
   int b = 0, start = 0;
-  scan_tiles(p, lane, f, &b, &start);
+  if (scan_in_regs) {
+    int base = 0;
+    bool found = false;
+#pragma unroll
+    for (int i = 0; i < SCAN_STEPS; ++i) {
+      const int total = __shfl(incl[i], 63, 64);
+      if (!found && f < base + total) {
+        const unsigned long long m = __ballot(base + incl[i] > f);
+        const int idx = __ffsll((long long)m) - 1;
+        b = 64 * i + idx;
+        start = base + __shfl(incl[i] - tl[i], idx, 64);
+        found = true;
+      }
+      base += total;
+    }
+  } else {
+    scan_tiles(p, lane, f, &b, &start);
+  }
   b = __builtin_amdgcn_readfirstlane(b);
   start = __builtin_amdgcn_readfirstlane(start);
 
