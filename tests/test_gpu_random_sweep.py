@@ -1,6 +1,8 @@
 """GPU parity over seeded random combinations of every option of the attention ops (shape, GQA ratio,
 block size, fp8 pool, ragged query lengths, sliding window, sinks, kernel route): each case against the
 oracle.  The cases are drawn from a fixed seed, so a failure names a reproducible case."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -10,7 +12,7 @@ from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_to_f32, make_pag
 
 pytestmark = pytest.mark.gpu
 
-N_CASES = 60
+N_CASES = int(os.environ.get("PA_SWEEP_CASES", "60"))      # more cases for an occasional longer soak of the same generator
 
 
 def _i32(x):
