@@ -7,9 +7,12 @@ role needs three small pieces:
 
 * `BlockAllocator`  -- free list with reference counts (a block shared by a forked prefix
                        is freed when its last user goes);
-* `PagedKVCache`    -- the K/V pool of one layer (bf16, or fp8-e4m3 with per-(block, kv
-                       head) scales), the per-slot block lists and the device-resident
-                       `block_tables` / `seq_lens` the kernels read;
+* `PagedKVCache`    -- the K/V pools of the model's layers (bf16, or fp8-e4m3 with
+                       per-(block, kv head) scales), the per-slot block lists and the
+                       device-resident `block_tables` / `seq_lens` the kernels read; the
+                       layers share the tables, as the reference's layers share start_pos
+                       (examples/models/qwen3/qwen3.py:310-336), so a step reserves blocks
+                       and publishes lengths once, not once per layer;
 * `PagedAttention`  -- one layer's step: optional QK RMSNorm + RoPE, KV write, then
                        prefill or decode attention, all into preallocated outputs
                        (the order of examples/models/qwen3/kernels/attention.py:78-144).
@@ -79,31 +82,44 @@ class BlockAllocator:
 
 
 class PagedKVCache:
-    """K/V pool of one attention layer plus the tables the kernels read.
+    """K/V pools of `num_layers` attention layers plus the tables the kernels read.
 
     Slots 0 .. max_seqs-1 are the rows of `block_tables` / `seq_lens`; a slot with
-    seq_len 0 is idle.  `dtype` torch.bfloat16, or torch.float8_e4m3fn (then
-    `k_scale` / `v_scale` [num_blocks, Hkv] float32 exist and are maintained by the write
-    kernel).
+    seq_len 0 is idle.  Every layer has its own pool `k_caches[l]` / `v_caches[l]`; block ids, tables
+    and lengths are common to all layers.  `dtype` torch.bfloat16, or torch.float8_e4m3fn (then
+    `k_scales[l]` / `v_scales[l]` [num_blocks, Hkv] float32 exist and are maintained by the write
+    kernel).  `k_cache`, `v_cache`, `k_scale`, `v_scale` name layer 0.
     """
 
     def __init__(self, num_blocks: int, block_size: int, n_kv_heads: int, head_dim: int, *, max_seqs: int,
-                 max_blocks_per_seq: int, dtype=torch.bfloat16, device="cuda"):
+                 max_blocks_per_seq: int, dtype=torch.bfloat16, device="cuda", num_layers: int = 1):
         if dtype not in (torch.bfloat16, torch.float8_e4m3fn):
             raise ValueError(f"unsupported pool dtype {dtype}")
+        if num_layers < 1:
+            raise ValueError("num_layers must be at least 1")
         self.block_size, self.n_kv_heads, self.head_dim = block_size, n_kv_heads, head_dim
-        self.max_seqs, self.max_blocks_per_seq = max_seqs, max_blocks_per_seq
+        self.max_seqs, self.max_blocks_per_seq, self.num_layers = max_seqs, max_blocks_per_seq, num_layers
         self.device = torch.device(device)
         shape = (num_blocks, block_size, n_kv_heads, head_dim)
-        if dtype == torch.float8_e4m3fn:
-            self.k_cache = torch.zeros(shape, dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
-            self.v_cache = torch.zeros(shape, dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
-            self.k_scale = torch.zeros((num_blocks, n_kv_heads), dtype=torch.float32, device=device)
-            self.v_scale = torch.zeros((num_blocks, n_kv_heads), dtype=torch.float32, device=device)
-        else:
-            self.k_cache = torch.zeros(shape, dtype=dtype, device=device)
-            self.v_cache = torch.zeros(shape, dtype=dtype, device=device)
-            self.k_scale = self.v_scale = None
+        fp8 = dtype == torch.float8_e4m3fn
+
+        def pool():
+            if fp8:
+                return torch.zeros(shape, dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
+            return torch.zeros(shape, dtype=dtype, device=device)
+
+        def scales():
+            return torch.zeros((num_blocks, n_kv_heads), dtype=torch.float32, device=device) if fp8 else None
+
+        self.k_caches = [pool() for _ in range(num_layers)]
+        self.v_caches = [pool() for _ in range(num_layers)]
+        self.k_scales = [scales() for _ in range(num_layers)]
+        self.v_scales = [scales() for _ in range(num_layers)]
+        self.k_cache, self.v_cache = self.k_caches[0], self.v_caches[0]
+        self.k_scale, self.v_scale = self.k_scales[0], self.v_scales[0]
+        # state of the step in flight (begin_step): query lengths on the device, tokens per slot
+        self.query_lens = torch.zeros(max_seqs, dtype=torch.int32, device=device)
+        self.step_tokens = 0
         self.allocator = BlockAllocator(num_blocks)
         self.blocks: List[List[int]] = [[] for _ in range(max_seqs)]
         self.lens = [0] * max_seqs
@@ -156,16 +172,30 @@ class PagedKVCache:
         self.allocator.share(shared)
         mine = self.allocator.alloc(len(tail))
         for a, b in zip(tail, mine):
-            self.k_cache.view(torch.uint8)[b].copy_(self.k_cache.view(torch.uint8)[a])
-            self.v_cache.view(torch.uint8)[b].copy_(self.v_cache.view(torch.uint8)[a])
-            if self.k_scale is not None:
-                self.k_scale[b].copy_(self.k_scale[a])
-                self.v_scale[b].copy_(self.v_scale[a])
+            for l in range(self.num_layers):
+                self.k_caches[l].view(torch.uint8)[b].copy_(self.k_caches[l].view(torch.uint8)[a])
+                self.v_caches[l].view(torch.uint8)[b].copy_(self.v_caches[l].view(torch.uint8)[a])
+                if self.k_scales[l] is not None:
+                    self.k_scales[l][b].copy_(self.k_scales[l][a])
+                    self.v_scales[l][b].copy_(self.v_scales[l][a])
         self.blocks[dst] = list(shared) + mine
         self.lens[dst] = self.lens[src]
         self._host_tables[dst] = -1
         self._host_tables[dst, :len(self.blocks[dst])] = self.blocks[dst]
         self._publish([dst])
+
+    def begin_step(self, query_lens: Sequence[int], tokens: int) -> None:
+        """Open a step in which slot b appends query_lens[b] <= tokens tokens (0: idle): reserves the
+        blocks, publishes tables and lengths, and puts the query lengths on the device for every
+        layer's `PagedAttention.attend` of this step.  All or nothing, like `extend`."""
+        if len(query_lens) != self.max_seqs:
+            raise ValueError(f"expected one length per slot ({self.max_seqs}), got {len(query_lens)}")
+        if any(n < 0 or n > tokens for n in query_lens):
+            raise ValueError("query_lens must lie in [0, tokens]")
+        active = [s for s in range(self.max_seqs) if query_lens[s] > 0]
+        self.extend(active, [query_lens[s] for s in active])
+        self.query_lens.copy_(torch.tensor(list(query_lens), dtype=torch.int32))
+        self.step_tokens = tokens
 
     def _publish(self, slots: Sequence[int]) -> None:
         idx = torch.as_tensor(list(slots), dtype=torch.long, device=self.device)
@@ -179,19 +209,24 @@ class PagedKVCache:
 
 
 class PagedAttention:
-    """One attention layer's serving step over a `PagedKVCache`.
+    """One attention layer's serving step over layer `layer` of a `PagedKVCache`.
 
-    `step(xq, xk, xv, query_lens)` takes the projected q/k/v of every slot, [max_seqs, T, H, D]
-    bfloat16 (slot b contributes its first query_lens[b] rows; idle slots 0), reserves the
-    blocks, applies the optional QK RMSNorm + RoPE, writes K/V into the pool and runs the
-    prefill / verify kernel (T > 1) or the decode kernel (T == 1).  Returns [max_seqs, T, Hq, D]
-    (a preallocated buffer, overwritten by the next step of the same T).
+    A model step is `cache.begin_step(query_lens, T)` once, then `attend(xq, xk, xv)` on every
+    layer; `step(xq, xk, xv, query_lens)` does both for a single-layer use.  xq/xk/xv are the
+    projected q/k/v of every slot, [max_seqs, T, H, D] bfloat16 (slot b contributes its first
+    query_lens[b] rows; idle slots 0).  `attend` applies the optional QK RMSNorm + RoPE, writes K/V
+    into the layer's pool and runs the prefill / verify kernel (T > 1) or the decode kernel
+    (T == 1).  Returns [max_seqs, T, Hq, D] (a preallocated buffer, overwritten by the next step of
+    the same T).
     """
 
-    def __init__(self, cache: PagedKVCache, n_heads: int, *, scale: Optional[float] = None, rope_base: Optional[float] = None,
-                 max_positions: int = 0, q_norm_weight=None, k_norm_weight=None, norm_eps: float = 1e-6,
-                 partition_size: int = 512, sinks=None, sliding_window: Optional[int] = None):
-        self.cache, self.n_heads = cache, n_heads
+    def __init__(self, cache: PagedKVCache, n_heads: int, *, layer: int = 0, scale: Optional[float] = None,
+                 rope_base: Optional[float] = None, max_positions: int = 0, q_norm_weight=None, k_norm_weight=None,
+                 norm_eps: float = 1e-6, partition_size: int = 512, sinks=None, sliding_window: Optional[int] = None,
+                 rope_tables=None):
+        if not 0 <= layer < cache.num_layers:
+            raise ValueError(f"layer {layer} outside the cache's {cache.num_layers} layers")
+        self.cache, self.n_heads, self.layer = cache, n_heads, layer
         self.scale = paged_attn.default_scale(cache.head_dim) if scale is None else float(scale)
         self.partition_size = partition_size
         self.q_norm_weight, self.k_norm_weight, self.norm_eps = q_norm_weight, k_norm_weight, norm_eps
@@ -199,46 +234,51 @@ class PagedAttention:
         # logits [n_heads] and a sliding window, fixed per layer
         self.sinks = None if sinks is None else sinks.to(torch.float32).contiguous()
         self.sliding_window = sliding_window
+        # RoPE tables: built from `rope_base`, or handed in as (cos, sin) [max_positions, D/2] bfloat16 — the
+        # way to share one pair between layers and to bring scaled frequencies (gpt_oss/kernels/rope.py:4-24)
         self.rope = None
-        if rope_base is not None:
+        if rope_tables is not None:
+            self.rope = (rope_tables[0], rope_tables[1])
+        elif rope_base is not None:
             if max_positions <= 0:
                 raise ValueError("RoPE needs max_positions")
             self.rope = paged_attn.rope_tables(cache.head_dim, max_positions, rope_base, device=cache.device)
         elif q_norm_weight is not None or k_norm_weight is not None:
             raise ValueError("the fused pre-attention kernel applies the norm together with RoPE: give rope_base")
         self._out: Dict[int, torch.Tensor] = {}
-        self._qlens = torch.zeros(cache.max_seqs, dtype=torch.int32, device=cache.device)
 
     def step(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, query_lens: Sequence[int]) -> torch.Tensor:
-        c = self.cache
+        if xq.shape[0] != self.cache.max_seqs or len(query_lens) != xq.shape[0]:
+            raise ValueError(f"expected one row per slot ({self.cache.max_seqs}), got {xq.shape[0]} rows and "
+                             f"{len(query_lens)} lengths")
+        self.cache.begin_step(query_lens, xq.shape[1])
+        return self.attend(xq, xk, xv)
+
+    def attend(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor) -> torch.Tensor:
+        c, l = self.cache, self.layer
         B, T = xq.shape[:2]
-        if B != c.max_seqs or len(query_lens) != B:
-            raise ValueError(f"expected one row per slot ({c.max_seqs}), got {B} rows and {len(query_lens)} lengths")
-        if any(n < 0 or n > T for n in query_lens):
-            raise ValueError("query_lens must lie in [0, T]")
-        active = [s for s in range(B) if query_lens[s] > 0]
-        c.extend(active, [query_lens[s] for s in active])
-        self._qlens.copy_(torch.tensor(list(query_lens), dtype=torch.int32))
+        if B != c.max_seqs or T != c.step_tokens:
+            raise ValueError(f"expected [{c.max_seqs}, {c.step_tokens}, ...] as opened by begin_step, got [{B}, {T}, ...]")
+        kc, vc, ks, vs = c.k_caches[l], c.v_caches[l], c.k_scales[l], c.v_scales[l]
         out = self._out.get(T)
         if out is None:
             out = self._out[T] = torch.empty((B, T, self.n_heads, c.head_dim), dtype=torch.bfloat16, device=c.device)
         if self.rope is not None:
-            q = paged_attn.qk_norm_rope_kv_write(xq, xk, xv, c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self._qlens,
+            q = paged_attn.qk_norm_rope_kv_write(xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens,
                                                  self.rope[0], self.rope[1], q_norm_weight=self.q_norm_weight,
                                                  k_norm_weight=self.k_norm_weight, eps=self.norm_eps,
-                                                 k_scale=c.k_scale, v_scale=c.v_scale, out=xq)
+                                                 k_scale=ks, v_scale=vs, out=xq)
         else:
-            paged_attn.kv_write(xk, xv, c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self._qlens,
-                                k_scale=c.k_scale, v_scale=c.v_scale)
+            paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq
         if T == 1:
-            paged_attn.decode(q[:, 0], c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self.scale,
-                              k_scale=c.k_scale, v_scale=c.v_scale, partition_size=self.partition_size,
+            paged_attn.decode(q[:, 0], kc, vc, c.block_tables, c.seq_lens, self.scale,
+                              k_scale=ks, v_scale=vs, partition_size=self.partition_size,
                               max_seq_len=max(c.max_seq_len, 1), out=out[:, 0],
                               sinks=self.sinks, sliding_window=self.sliding_window)
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:
-            paged_attn.prefill(q, c.k_cache, c.v_cache, c.block_tables, c.seq_lens, self._qlens, self.scale,
-                               k_scale=c.k_scale, v_scale=c.v_scale, out=out,
+            paged_attn.prefill(q, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
+                               k_scale=ks, v_scale=vs, out=out,
                                sinks=self.sinks, sliding_window=self.sliding_window)
         return out

@@ -77,3 +77,27 @@ def test_cache_fork_shares_full_blocks_and_copies_the_tail():
         c.fork(1, 1)
     c.release(1)
     assert c.allocator.num_free == 10
+
+
+def test_begin_step_is_all_or_nothing_and_layers_share_tables():
+    c = _cache(num_layers=3)
+    assert len(c.k_caches) == 3 and c.k_caches[1].data_ptr() != c.k_caches[2].data_ptr()
+    c.begin_step([5, 0, 2], 5)
+    assert c.lens == [5, 0, 2] and c.step_tokens == 5 and c.query_lens.tolist() == [5, 0, 2]
+    assert c.allocator.num_free == 10 - 2 - 1                    # one reservation for all layers
+    with pytest.raises(ValueError):
+        c.begin_step([1, 1], 1)                                  # one length per slot
+    with pytest.raises(ValueError):
+        c.begin_step([2, 0, 0], 1)                               # longer than the step's token count
+    with pytest.raises(OutOfBlocks):
+        c.begin_step([0, 20, 12], 20)                            # 5 + 3 blocks wanted, 7 free
+    assert c.lens == [5, 0, 2] and c.query_lens.tolist() == [5, 0, 2]   # nothing changed
+    # a fork copies the partial tail block in every layer's pool
+    for l in range(3):
+        c.k_caches[l][c.blocks[0][1]] = float(l + 1)
+    c.fork(0, 1)
+    assert c.blocks[1][0] == c.blocks[0][0] and c.blocks[1][1] != c.blocks[0][1]
+    for l in range(3):
+        assert torch.all(c.k_caches[l][c.blocks[1][1]] == float(l + 1))
+    with pytest.raises(ValueError):
+        _cache(num_layers=0)

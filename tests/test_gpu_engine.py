@@ -155,3 +155,41 @@ def test_serving_loop_fp8_pool(rng):
                            layer.scale, k_scale=cache.k_scale.cpu().numpy(), v_scale=cache.v_scale.cpu().numpy(), q_dtype="bf16")
     assert_close_abs(got, want, 5e-2)
     assert cache.lens == [43, 70] and np.all(got[0] == 0)
+
+
+def test_two_layers_share_tables(rng):
+    """A model step opens once (`begin_step`) and every layer attends into its own pool through the shared
+    block tables; a fork copies the partial tail block of every layer."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    S, Hq, Hkv, D, bs, L = 3, 8, 2, 128, 16, 2
+    cache = PagedKVCache(num_blocks=30, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=8,
+                         num_layers=L)
+    cos, sin = O.rope_tables(D, 128, 10000.0)
+    tables = (bf16_to_dev(cos), bf16_to_dev(sin))                   # one pair of RoPE tables for both layers
+    layers = [PagedAttention(cache, Hq, layer=l, rope_tables=tables) for l in range(L)]
+    mirrors = [_Mirror(S, cos, sin, None, None, 1e-6) for _ in range(L)]
+    assert cache.k_caches[0].data_ptr() != cache.k_caches[1].data_ptr()
+
+    def run(T, qlens):
+        free_before = cache.allocator.num_free
+        cache.begin_step(qlens, T)
+        for l in range(L):
+            xq, xk, xv = _rand(rng, (S, T, Hq, D)), _rand(rng, (S, T, Hkv, D)), _rand(rng, (S, T, Hkv, D))
+            got = dev_to_f32(layers[l].attend(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv)))
+            want = mirrors[l].step(xq, xk, xv, qlens, layers[l].scale)
+            for b in range(S):
+                if qlens[b]:
+                    assert_close_abs(got[b, :qlens[b]], want[b, :qlens[b]], 3e-2)
+        return free_before - cache.allocator.num_free
+
+    used = run(21, [21, 9, 0])
+    assert used == 2 + 1                                             # blocks are reserved once per step, not per layer
+    run(1, [1, 1, 0])
+    cache.fork(0, 2)
+    for m in mirrors:
+        m.k[2], m.v[2] = m.k[0].copy(), m.v[0].copy()
+    for _ in range(3):
+        run(1, [1, 1, 1])
+    with pytest.raises(ValueError):
+        layers[0].attend(bf16_to_dev(_rand(rng, (S, 2, Hq, D))), bf16_to_dev(_rand(rng, (S, 2, Hkv, D))),
+                         bf16_to_dev(_rand(rng, (S, 2, Hkv, D))))   # not the step begin_step opened
