@@ -607,8 +607,13 @@ void prefill_async_kernel(PrefillParams p) {
   }
   // attention sink: a per-head logit that joins the softmax as one more column with no value
   if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq_l] * kLog2e - m_ref);
-  if (qrow < p.T && wq_lo < p.T) {
-    uint16_t* op = out + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * HD;
+  // The rows go out through LDS: a lane holds 4 consecutive d of one row at 16 places, which as direct
+  // stores would be 8-byte pieces of 64 different rows per instruction; staged row-major in a
+  // wave-private patch of the (now idle) tile ring they leave as whole 256-byte rows, 16 bytes a lane.
+  __builtin_amdgcn_s_barrier();                  // every wave is done reading the ring
+  {
+    constexpr int OROW_B = ROW_B + 8;            // row pitch: the 8 bytes spread a column of rows over the banks
+    char* patch = smem + wave * (32 * OROW_B);
     const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
 #pragma unroll
     for (int c = 0; c < HD / 32; ++c)
@@ -617,8 +622,18 @@ void prefill_async_kernel(PrefillParams p) {
         const int d = 32 * c + 8 * i4 + 4 * h;
         const uint32_t w0 = qvalid ? pack_bf16x2(oacc[c][4 * i4] * inv, oacc[c][4 * i4 + 1] * inv) : 0u;
         const uint32_t w1 = qvalid ? pack_bf16x2(oacc[c][4 * i4 + 2] * inv, oacc[c][4 * i4 + 3] * inv) : 0u;
-        *(uint2*)(op + d) = make_uint2(w0, w1);
+        *(uint2*)(patch + n * OROW_B + 2 * d) = make_uint2(w0, w1);
       }
+    // the wave reads back what its own lanes wrote: no barrier, the compiler orders the LDS accesses
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int r = 4 * j + (lane >> 4), ch = lane & 15;
+      const uint2 lo = *(const uint2*)(patch + r * OROW_B + 16 * ch), hi = *(const uint2*)(patch + r * OROW_B + 16 * ch + 8);
+      const int tok = row_token(wave * 32 + r);
+      if (tok < p.T)
+        *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)row_head(wave * 32 + r) * HD + 8 * ch) =
+            make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
   }
 }
 
