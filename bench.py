@@ -414,12 +414,64 @@ def bench_pre_attention(steps, warmup, lib, pa, W):
     return res
 
 
+def bench_prefill_layer_step(steps, warmup, lib, pa, W):
+    """config 10: what one attention layer of a prefill step does on config 3's workload: QK RMSNorm +
+    RoPE, K/V rows into the pool, attention.  The Q half of the transform rides on the attention
+    kernel's Q load; the two-step form (Q transformed by a kernel of its own) is timed beside it."""
+    w = W.make_prefill()
+    B, T, Hq, D = w.q.shape
+    Hkv = w.k_cache.shape[2]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1010)
+    xk = torch.randn((B, T, Hkv, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    xv = torch.randn((B, T, Hkv, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    wq = (1.0 + 0.1 * torch.randn(D, generator=gen, device="cuda")).to(torch.bfloat16)
+    wk = (1.0 + 0.1 * torch.randn(D, generator=gen, device="cuda")).to(torch.bfloat16)
+    cos, sin = pa.rope_tables(D, int(w.seq_lens.max().item()), 1000000.0)
+    out, q2 = torch.empty_like(w.q), torch.empty_like(w.q)
+    qt = pa.QTransform(cos, sin, wq, 1e-6)
+    common = (w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens)
+
+    def fused():
+        pa.qk_norm_rope_kv_write(None, xk, xv, *common, cos, sin, k_norm_weight=wk, eps=1e-6)
+        pa.prefill(w.q, *common, w.scale, out=out, q_transform=qt)
+
+    def two_step():
+        pa.qk_norm_rope_kv_write(w.q, xk, xv, *common, cos, sin, q_norm_weight=wq, k_norm_weight=wk, eps=1e-6, out=q2)
+        pa.prefill(q2, *common, w.scale, out=out)
+
+    sec2 = _time_steps(two_step, steps, warmup)
+    ref = out.clone()
+    sec = _time_steps(fused, steps, warmup)
+    same = bool(torch.equal(out, ref))
+    lib.pa_profile_enable(1)
+    _time_steps(fused, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = [x for x in _collect_kernel_ms(lib, 2 * steps)]
+    katt = float(np.mean(sorted(kms)[len(kms) // 2:]))      # the attention launches are the longer half
+    fl = w.flops()
+    return {
+        "metric": "prefill layer step (QK-norm + RoPE + KV write + attention) attn TFLOP/s",
+        "value": round(fl / sec / 1e12, 2), "unit": "TFLOP/s",
+        "ms_per_step": round(sec * 1e3, 5),
+        "two_step_ms_per_step": round(sec2 * 1e3, 5), "fused_equals_two_step_bits": same,
+        "dtype": "bf16, float32 norm, bf16 rotation, fp32 accumulate",
+        "config": {"workload": f"C3 prefill layer step: B={B}, T={T}, Hq={Hq}, Hkv={Hkv}, D={D}, "
+                               f"block_size={w.k_cache.shape[1]}, prefix={w.prefix.tolist()}", "flops": fl},
+        "roofline": {"bound": "mfma", "achieved": round(fl / (katt * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(fl / (katt * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "prefill_async_kernel with the Q transform in its prologue", "kernel_avg_ms": round(katt, 5),
+                     "launches_timed": len(kms) // 2},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8, 9])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8, 9, 10])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -450,6 +502,8 @@ def main():
         res = bench_verify(args.steps, args.warmup, lib, pa, W)
     elif args.config == 9:
         res = bench_prefill(args.steps, args.warmup, lib, pa, W, fp8=True)
+    elif args.config == 10:
+        res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
     else:
         res = bench_blocksparse(args.steps, args.warmup, lib, pa, W)
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"),

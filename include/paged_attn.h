@@ -55,6 +55,21 @@ int pa_version(void);
  * status strings of spike/src/include/error.h:23-43. */
 const char* pa_last_error(void);
 
+/* Optional last step of the reference's pre-attention code, done by the attention kernels
+ * themselves as they load the Q rows: QK RMSNorm of Q (examples/models/qwen3/kernels/rmsnorm.py:4-21,
+ * applied at qwen3/kernels/attention.py:78-80) and RoPE at the row's absolute position
+ * (rope.py:23-48; attention.py:83-97), the position being seq_lens[b] - query_lens[b] + t
+ * (seq_lens[b] - 1 for pa_decode).  Results are bit for bit those of pa_qk_norm_rope_kv_write's
+ * Q pass followed by the attention call, without that pass's read and rewrite of Q.
+ * Tables as for pa_qk_norm_rope_kv_write; norm_weight NULL = rotation only. */
+typedef struct pa_q_transform {
+  const void* norm_weight;   /* [D] bf16 or NULL */
+  const void* rope_cos;      /* [rope_max_pos, D/2] bf16 */
+  const void* rope_sin;
+  int rope_max_pos;
+  float norm_eps;
+} pa_q_transform;
+
 /* Bytes of scratch that is enough for pa_decode whichever kernel it picks: split-K
  * partials of D floats of normalised output plus (max, sum) each — one per
  * (sequence, q head, partition) for the fixed-partition kernels, one per
@@ -82,6 +97,8 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
  *   keys (p - W, p] (attention.py:118-125).  Both need the MFMA kernel's shapes (bf16 q, bf16 or
  *   fp8 KV, D in {64, 128}, block_size a power of two >= 16); tiles wholly outside the window are
  *   not read.
+ * q_transform: NULL, or the norm and rotation to apply to the Q rows on load (same shapes).
+ *   pa_verify and pa_prefill (tiled kernel with asynchronous copies) take it too.
  */
 int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               const float* k_scale, const float* v_scale,
@@ -90,7 +107,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               int B, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks, int max_seq_len,
               float scale, int partition_size, int q_dtype, int kv_dtype,
-              const float* sinks, int sliding_window, void* stream);
+              const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream);
 
 /*
  * Speculative verify: a few query tokens per sequence against the paged context, causal among
@@ -115,7 +132,8 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
               void* out, void* workspace, size_t workspace_bytes,
               int B, int T, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks,
-              float scale, int kv_dtype, const float* sinks, int sliding_window, void* stream);
+              float scale, int kv_dtype, const float* sinks, int sliding_window,
+              const pa_q_transform* q_transform, void* stream);
 
 /*
  * Paged chunked prefill with a cached prefix, causal: query token i of sequence
@@ -141,7 +159,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
                float scale, int dtype, int kv_dtype, const float* sinks, int sliding_window,
-               void* workspace, size_t workspace_bytes, void* stream);
+               void* workspace, size_t workspace_bytes, const pa_q_transform* q_transform, void* stream);
 
 /*
  * Block-sparse causal prefill over dense q [B, S, Hq, D], k/v [B, S, Hkv, D]:
@@ -192,7 +210,9 @@ int pa_kv_write(const void* k_new, const void* v_new, void* k_cache, void* v_cac
  * (examples/models/qwen3/kernels/rmsnorm.py:4-21, applied at qwen3/kernels/attention.py:78-80),
  * RoPE at the tokens' absolute positions start_pos + t, start_pos = seq_lens[b] -
  * query_lens[b] (rope.py:23-48; attention.py:83-97; gpt_oss/kernels/attention.py:85-90), then
- * pa_kv_write of the rotated K and of V.  Two launches: Q rows, then the K/V scatter.
+ * pa_kv_write of the rotated K and of V.  Two launches: Q rows, then the K/V scatter; with xq
+ * and q_out both NULL only the second (for callers that hand the Q part to the attention call
+ * as a pa_q_transform).
  *   xq [B, T, Hq, D], xk, xv [B, T, Hkv, D]  bf16; q_out [B, T, Hq, D] bf16 (may be xq); rows
  *                 t >= query_lens[b] of q_out are zero
  *   q_norm_weight, k_norm_weight [D] bf16, or NULL for no norm on that tensor

@@ -19,15 +19,23 @@ _lib = None
 
 c_int, c_float, c_void_p, c_size_t = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 
+
+
+class QTransformStruct(ctypes.Structure):
+    """`pa_q_transform` of include/paged_attn.h."""
+    _fields_ = [("norm_weight", c_void_p), ("rope_cos", c_void_p), ("rope_sin", c_void_p),
+                ("rope_max_pos", c_int), ("norm_eps", c_float)]
+
+
 SIGNATURES = {
     "pa_version": (c_int, []),
     "pa_last_error": (ctypes.c_char_p, []),
     "pa_decode_workspace_bytes": (c_size_t, [c_int] * 5),
-    "pa_decode": (c_int, [c_void_p] * 9 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p]),
+    "pa_decode": (c_int, [c_void_p] * 9 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "pa_verify_workspace_bytes": (c_size_t, [c_int] * 4),
-    "pa_verify": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 8 + [c_float, c_int, c_void_p, c_int, c_void_p]),
+    "pa_verify": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 8 + [c_float, c_int, c_void_p, c_int, c_void_p, c_void_p]),
     "pa_prefill_workspace_bytes": (c_size_t, [c_int] * 7),
-    "pa_prefill": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "pa_prefill": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p, c_void_p]),
     "pa_blocksparse_prefill": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_float, c_int, c_void_p]),
     "pa_gather_kv": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_void_p]),
     "pa_kv_write": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_void_p]),

@@ -154,6 +154,24 @@ int pa_probe_mfma(const void* operands, void* sink, int blocks, int iters, float
   return check_hip(e, "pa_probe_mfma");
 }
 
+// Checks an optional Q transform and copies it into the kernel parameters; returns 0 or -1.
+static int take_q_transform(const char* who, const pa_q_transform* qt, int D, bool kernel_ok, QTransform& dst) {
+  memset(&dst, 0, sizeof(dst));
+  if (!qt) return 0;
+  if (!kernel_ok)
+    return fail_arg("%s: q_transform needs the matrix-core kernels (bf16 q, head_dim 64 or 128 for decode and verify, "
+                    "128 for tiled prefill, block_size a power of two >= 16)", who);
+  if (!qt->rope_cos || !qt->rope_sin || qt->rope_max_pos <= 0)
+    return fail_arg("%s: q_transform needs rope_cos, rope_sin and rope_max_pos > 0", who);
+  if (!aligned16(qt->rope_cos) || !aligned16(qt->rope_sin) || !aligned16(qt->norm_weight))
+    return fail_arg("%s: q_transform tables must be 16-byte aligned", who);
+  (void)D;
+  dst.norm_weight = (const uint16_t*)qt->norm_weight;
+  dst.cos = (const uint16_t*)qt->rope_cos; dst.sin = (const uint16_t*)qt->rope_sin;
+  dst.max_pos = qt->rope_max_pos; dst.eps = qt->norm_eps;
+  return 0;
+}
+
 static int num_partitions_for(int max_seq_len, int partition_size) {
   if (max_seq_len <= 0) return 1;
   return (max_seq_len + partition_size - 1) / partition_size;
@@ -176,7 +194,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               int B, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks, int max_seq_len,
               float scale, int partition_size, int q_dtype, int kv_dtype,
-              const float* sinks, int sliding_window, void* stream) {
+              const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream) {
   tl_error[0] = 0;
   if (sliding_window < 0) return fail_arg("pa_decode: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
   if (B < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_decode: bad sizes B=%d Hq=%d Hkv=%d D=%d", B, Hq, Hkv, D);
@@ -221,6 +239,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
     return fail_arg("pa_decode: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
                     "head_dim 64 or 128, block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
+  if (take_q_transform("pa_decode", q_transform, D, kind != 1, p.qt)) return -1;
   if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
   if (kind == 3) {
     plan_decode_balanced(p, current_num_cus());
@@ -268,7 +287,8 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
               void* out, void* workspace, size_t workspace_bytes,
               int B, int T, int Hq, int Hkv, int D, int block_size,
               int max_blocks_per_seq, int num_blocks,
-              float scale, int kv_dtype, const float* sinks, int sliding_window, void* stream) {
+              float scale, int kv_dtype, const float* sinks, int sliding_window,
+              const pa_q_transform* q_transform, void* stream) {
   tl_error[0] = 0;
   if (sliding_window < 0) return fail_arg("pa_verify: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
   if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_verify: bad sizes B=%d T=%d Hq=%d Hkv=%d D=%d", B, T, Hq, Hkv, D);
@@ -308,6 +328,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
   p.scale_log2e = scale * kLog2e;
   if (!decode_mfma_supported(p, PA_BF16, kv_dtype))
     return fail_arg("pa_verify: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", D, block_size);
+  if (take_q_transform("pa_verify", q_transform, D, true, p.qt)) return -1;
   plan_decode_balanced(p, current_num_cus());
   p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
   const size_t need = decode_balanced_workspace_bytes(B, Hq * T, D, p.bal_gv);
@@ -356,7 +377,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                int B, int T, int Hq, int Hkv, int D, int block_size,
                int max_blocks_per_seq, int num_blocks,
                float scale, int dtype, int kv_dtype, const float* sinks, int sliding_window,
-               void* workspace, size_t workspace_bytes, void* stream) {
+               void* workspace, size_t workspace_bytes, const pa_q_transform* q_transform, void* stream) {
   tl_error[0] = 0;
   if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_prefill: bad sizes");
   if (sliding_window < 0) return fail_arg("pa_prefill: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
@@ -384,6 +405,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   if (sliding_window > 0 && (p.impl == 1 || !prefill_async_supported(p)))
     return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
+  if (take_q_transform("pa_prefill", q_transform, D, p.impl != 1 && prefill_async_supported(p), p.qt)) return -1;
   p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
   // few workgroups and a long table: split the key tiles of a query tile over several workgroups when the
   // caller brought the workspace for it (without one the call runs unsplit)
@@ -488,8 +510,10 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
   if ((long)max_blocks_per_seq * block_size > 0x7fffffffL) return fail_arg("pa_qk_norm_rope_kv_write: table capacity exceeds 2^31 tokens");
   if (B == 0 || T == 0) return 0;
   if (B > 65535 || Hkv > 65535) return fail_arg("pa_qk_norm_rope_kv_write: B and Hkv are limited to 65535 (grid dimensions)");
-  if (!xq || !xk || !xv || !q_out || !rope_cos || !rope_sin || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens)
+  if (!xk || !xv || !rope_cos || !rope_sin || !k_cache || !v_cache || !block_tables || !seq_lens || !query_lens)
     return fail_arg("pa_qk_norm_rope_kv_write: null pointer argument");
+  if ((xq == nullptr) != (q_out == nullptr))
+    return fail_arg("pa_qk_norm_rope_kv_write: xq and q_out must both be given, or both be NULL (K and V only)");
   if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_qk_norm_rope_kv_write: fp8 pools need k_scale and v_scale");
   if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache))
     return fail_arg("pa_qk_norm_rope_kv_write: xq, xk, xv, q_out, k_cache and v_cache must be 16-byte aligned");

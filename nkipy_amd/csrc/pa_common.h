@@ -68,6 +68,88 @@ template <> struct Store<uint16_t> {
   }
 };
 
+// ---- Q transform on load ---------------------------------------------------------
+// The reference's pre-attention step on Q (QK RMSNorm, examples/models/qwen3/kernels/rmsnorm.py:4-21;
+// RoPE at the token's absolute position, rope.py:23-48) applied by the attention kernel to the Q
+// rows as it loads them, instead of by a kernel of its own that reads and rewrites Q.
+struct QTransform {
+  const uint16_t* norm_weight;  // [D] bf16 or null (no norm)
+  const uint16_t* cos;          // [max_pos, D/2] bf16; null: no transform at all
+  const uint16_t* sin;
+  int max_pos;
+  float eps;
+};
+
+// A lane holds NS chunks of 8 consecutive elements of one row of 8 * CPR elements; the other
+// chunks of the row are held by lanes whose number differs in bits of L's choosing.  L says
+// where chunk index bit `bit` lives: in the lane's slot number s (L::slot_xor(bit) != 0) or in
+// the lane number (L::lane_xor(bit) != 0), and L::chunk(s, part) numbers the chunk held in slot
+// s by a lane whose part number is `part`.  The arithmetic and its order are those of the
+// stand-alone transform kernel (mean of squares as a butterfly over the chunk index, norm in
+// float32 rounded once to bf16, every product and sum of the rotation rounded to bf16), so
+// the two give the same bits.
+template <int CPR, int NS, class L>
+__device__ __forceinline__ void q_norm_rope_lane(float (&x)[NS][8], const QTransform& t, int pos, int part) {
+  constexpr int D = 8 * CPR;
+  auto r16 = [](float f) __attribute__((always_inline)) { return __uint_as_float(pack_bf16x2(f, 0.f) << 16); };
+  auto unpack = [](const uint4& v, float (&f)[8]) __attribute__((always_inline)) {
+    const uint32_t a[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = bf16_bits_to_float(a[j] & 0xffffu);
+      f[2 * j + 1] = bf16_bits_to_float(a[j] >> 16);
+    }
+  };
+  if (t.norm_weight) {
+    float ss[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      ss[s] = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss[s] += x[s][j] * x[s][j];
+    }
+#pragma unroll
+    for (int bit = 1; bit < CPR; bit <<= 1) {
+      float nx[NS];
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        nx[s] = ss[s] + (L::slot_xor(bit) ? ss[s ^ L::slot_xor(bit)] : __shfl_xor(ss[s], L::lane_xor(bit)));
+#pragma unroll
+      for (int s = 0; s < NS; ++s) ss[s] = nx[s];
+    }
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const float inv = __builtin_amdgcn_rsqf(__fdiv_rn(ss[s], (float)D) + t.eps);
+      float w[8];
+      unpack(*(const uint4*)(t.norm_weight + 8 * L::chunk(s, part)), w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[s][j] = r16((x[s][j] * inv) * w[j]);
+    }
+  }
+  constexpr int hc = CPR / 2;
+  const uint16_t* cos_row = t.cos + (long)pos * (D / 2);
+  const uint16_t* sin_row = t.sin + (long)pos * (D / 2);
+  float y[NS][8];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int c = L::chunk(s, part);
+    const bool first = c < hc;
+    const int fi = 8 * (first ? c : c - hc);
+    float cs[8], sn[8];
+    unpack(*(const uint4*)(cos_row + fi), cs);
+    unpack(*(const uint4*)(sin_row + fi), sn);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float other = L::slot_xor(hc) ? x[s ^ L::slot_xor(hc)][j] : __shfl_xor(x[s][j], L::lane_xor(hc));
+      y[s][j] = first ? r16(r16(x[s][j] * cs[j]) - r16(other * sn[j])) : r16(r16(other * sn[j]) + r16(x[s][j] * cs[j]));
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[s][j] = y[s][j];
+}
+
 // ---- decode ------------------------------------------------------------------------
 struct DecodeParams {
   const void* q;            // [B, Hq, D]; [B, T, Hq, D] for a multi-token call
@@ -94,6 +176,7 @@ struct DecodeParams {
   int head_major;           // fixed-partition grid order: kv head fastest (1) or partition fastest (0)
   int bal_hsw, bal_ns, bal_gv;  // balanced schedule: head slots and chunks per workgroup, total chunks
   int bal_lockstep;         // keep the head waves of a workgroup on the same tile with a barrier
+  QTransform qt;            // balanced schedule only: Q rows are normed and rotated as they are loaded
 };
 
 hipError_t launch_decode_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
@@ -129,6 +212,7 @@ struct PrefillParams {
   int splits;               // same: workgroups sharing the key tiles of one query tile (1: no split)
   float* ws_o;              // splits > 1: [B * T * Hq, splits, D] partial outputs
   float* ws_ml;             // splits > 1: [B * T * Hq, splits, 2] partial (max, sum)
+  QTransform qt;            // asynchronous kernel only: Q rows are normed and rotated as they are loaded
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);

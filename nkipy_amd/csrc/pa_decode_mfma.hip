@@ -96,6 +96,16 @@ struct VTile {
 // 256 registers otherwise): the Q fragments live in LDS, each lane reading back
 // the 16-byte pieces it wrote itself (no conflicts, no barrier), and V is single-
 // buffered: the next tile's V is requested right after the current P.V.
+// Where the 8-element chunks of a Q row sit in the Q^T operand: lane (g, r) holds, in k-step s,
+// chunk 4 s + g (bf16 pools) or 8 (s >> 1) + 2 g + (s & 1) (fp8 pools, whose K loads cover 16
+// elements of a row per lane).  g is lane >> 4.
+template <bool FP8>
+struct QOperandLayout {
+  static __device__ __forceinline__ int chunk(int s, int g) { return FP8 ? 8 * (s >> 1) + 2 * g + (s & 1) : 4 * s + g; }
+  static constexpr int slot_xor(int bit) { return FP8 ? (bit == 1 ? 1 : bit == 8 ? 2 : 0) : (bit >> 2); }
+  static constexpr int lane_xor(int bit) { return FP8 ? (bit == 2 ? 16 : bit == 4 ? 32 : 0) : (bit == 1 ? 16 : bit == 2 ? 32 : 0); }
+};
+
 template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false>
 struct DecodeWave {
   using KT = KTile<D, FP8>;
@@ -165,14 +175,39 @@ struct DecodeWave {
       } else {
         qrow = (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
       }
+      uint4 qraw[KSTEPS];
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
         // d range of k-slots 8g..8g+7 in step s (must mirror the K loads below)
         const int d0 = FP8 ? ((4 * (s >> 1) + g) * 16 + (s & 1) * 8) : ((4 * s + g) * 8);
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (row_valid) v = *(const uint4*)(qrow + d0);
-        if (LEAN) qlds[(rg * KSTEPS + s) * 64 + qlane] = v;
-        else qf[rg][s] = __builtin_bit_cast(bf16x8_t, v);
+        qraw[s] = make_uint4(0, 0, 0, 0);
+        if (row_valid) qraw[s] = *(const uint4*)(qrow + d0);
+      }
+      if (p.qt.cos) {
+        // norm and rotation of the row on the way in; every lane takes part (a row is spread
+        // over the four lanes r, r + 16, r + 32, r + 48), padded rows carry zeros
+        float x[KSTEPS][8];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          const uint32_t w[4] = {qraw[s].x, qraw[s].y, qraw[s].z, qraw[s].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[s][2 * j] = bf16_bits_to_float(w[j] & 0xffffu);
+            x[s][2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+          }
+        }
+        const int qpos = MULTI ? row_end[rg] - 1 : last;
+        q_norm_rope_lane<D / 8, KSTEPS, QOperandLayout<FP8>>(x, p.qt, min(max(qpos, 0), p.qt.max_pos - 1), g);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          qraw[s].x = pack_bf16x2(x[s][0], x[s][1]); qraw[s].y = pack_bf16x2(x[s][2], x[s][3]);
+          qraw[s].z = pack_bf16x2(x[s][4], x[s][5]); qraw[s].w = pack_bf16x2(x[s][6], x[s][7]);
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        if (LEAN) qlds[(rg * KSTEPS + s) * 64 + qlane] = qraw[s];
+        else qf[rg][s] = __builtin_bit_cast(bf16x8_t, qraw[s]);
       }
 #pragma unroll
       for (int e = 0; e < VEC; ++e) oacc[rg][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};

@@ -281,7 +281,7 @@ __global__ __launch_bounds__(WG) void q_norm_rope_kernel(KvWriteParams p) {
 
 template <int CPR>
 void launch_xform(const KvWriteParams& p, dim3 grid, hipStream_t s) {
-  hipLaunchKernelGGL(q_norm_rope_kernel<CPR>, dim3(p.T, p.B), dim3(WG), 0, s, p);
+  if (p.q_in) hipLaunchKernelGGL(q_norm_rope_kernel<CPR>, dim3(p.T, p.B), dim3(WG), 0, s, p);
   if (p.kv_dtype == PA_FP8_E4M3FN) hipLaunchKernelGGL((kv_write_kernel<1, CPR>), grid, dim3(WG), 0, s, p);
   else hipLaunchKernelGGL((kv_write_kernel<2, CPR>), grid, dim3(WG), 0, s, p);
 }

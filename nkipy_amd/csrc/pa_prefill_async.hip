@@ -42,6 +42,13 @@ namespace {
 
 constexpr int HD = 128;                // head dim
 constexpr int ROW_B = HD * 2;          // bytes per K/V row
+// Where the 8-element chunks of a Q row sit: lane (n, h) holds chunk 2 s + h in slot s, so the
+// lowest chunk-index bit is the half-wave and the others are the slot number.
+struct QRowLayout {
+  static __device__ __forceinline__ int chunk(int s, int h) { return 2 * s + h; }
+  static constexpr int slot_xor(int bit) { return bit >> 1; }
+  static constexpr int lane_xor(int bit) { return bit == 1 ? 32 : 0; }
+};
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -519,10 +526,36 @@ void prefill_async_kernel(PrefillParams p) {
   prefetch_next();
   {
     const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * HD;
+    uint4 qraw[HD / 16];
 #pragma unroll
     for (int s = 0; s < HD / 16; ++s) {
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (qvalid) v = *(const uint4*)(qp + 16 * s + 8 * h);
+      qraw[s] = make_uint4(0, 0, 0, 0);
+      if (qvalid) qraw[s] = *(const uint4*)(qp + 16 * s + 8 * h);
+    }
+    if (!SPARSE && p.qt.cos) {
+      // norm and rotation of the row on the way in; every lane takes part (the row's other
+      // half sits in lane ^ 32), rows past the query length carry zeros
+      float x[HD / 16][8];
+#pragma unroll
+      for (int s = 0; s < HD / 16; ++s) {
+        const uint32_t w[4] = {qraw[s].x, qraw[s].y, qraw[s].z, qraw[s].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[s][2 * j] = bf16_bits_to_float(w[j] & 0xffffu);
+          x[s][2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+        }
+      }
+      const int pos = min(max(prefix + qrow, 0), p.qt.max_pos - 1);
+      q_norm_rope_lane<HD / 8, HD / 16, QRowLayout>(x, p.qt, pos, h);
+#pragma unroll
+      for (int s = 0; s < HD / 16; ++s) {
+        qraw[s].x = pack_bf16x2(x[s][0], x[s][1]); qraw[s].y = pack_bf16x2(x[s][2], x[s][3]);
+        qraw[s].z = pack_bf16x2(x[s][4], x[s][5]); qraw[s].w = pack_bf16x2(x[s][6], x[s][7]);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < HD / 16; ++s) {
+      const uint4 v = qraw[s];
       // scale * log2(e) goes into Q once (rounded to bf16 again: a relative 2^-9 per element,
       // below the rounding of the probabilities), so that the scores leave the matrix cores
       // ready for exp2

@@ -263,11 +263,18 @@ class PagedAttention:
         out = self._out.get(T)
         if out is None:
             out = self._out[T] = torch.empty((B, T, self.n_heads, c.head_dim), dtype=torch.bfloat16, device=c.device)
+        qt = None
         if self.rope is not None:
-            q = paged_attn.qk_norm_rope_kv_write(xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens,
-                                                 self.rope[0], self.rope[1], q_norm_weight=self.q_norm_weight,
+            # the Q half of the norm and rotation rides on the attention kernel's Q load where that
+            # kernel can do it (no pass over Q of its own); K is transformed on its way into the pool
+            fused = paged_attn.q_transform_supported(T, c.head_dim, c.block_size)
+            q = paged_attn.qk_norm_rope_kv_write(None if fused else xq, xk, xv, kc, vc, c.block_tables, c.seq_lens,
+                                                 c.query_lens, self.rope[0], self.rope[1],
+                                                 q_norm_weight=None if fused else self.q_norm_weight,
                                                  k_norm_weight=self.k_norm_weight, eps=self.norm_eps,
-                                                 k_scale=ks, v_scale=vs, out=xq)
+                                                 k_scale=ks, v_scale=vs, out=None if fused else xq)
+            if fused:
+                q, qt = xq, paged_attn.QTransform(self.rope[0], self.rope[1], self.q_norm_weight, self.norm_eps)
         else:
             paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq
@@ -275,10 +282,10 @@ class PagedAttention:
             paged_attn.decode(q[:, 0], kc, vc, c.block_tables, c.seq_lens, self.scale,
                               k_scale=ks, v_scale=vs, partition_size=self.partition_size,
                               max_seq_len=max(c.max_seq_len, 1), out=out[:, 0],
-                              sinks=self.sinks, sliding_window=self.sliding_window)
+                              sinks=self.sinks, sliding_window=self.sliding_window, q_transform=qt)
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:
             paged_attn.prefill(q, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
                                k_scale=ks, v_scale=vs, out=out,
-                               sinks=self.sinks, sliding_window=self.sliding_window)
+                               sinks=self.sinks, sliding_window=self.sliding_window, q_transform=qt)
         return out

@@ -124,9 +124,54 @@ def _workspace(device, nbytes):
     return buf
 
 
+class QTransform:
+    """Norm and rotation of the Q rows done by the attention kernel as it loads them: the Q half of
+    the reference's pre-attention step (QK RMSNorm, examples/models/qwen3/kernels/rmsnorm.py:4-21;
+    RoPE at the row's absolute position, rope.py:23-48), bit for bit what `qk_norm_rope_kv_write`
+    writes for Q, without that kernel's pass over Q.  rope_cos / rope_sin [max_pos, D/2] bfloat16
+    (`rope_tables`); norm_weight [D] bfloat16 or None for rotation only."""
+
+    def __init__(self, rope_cos, rope_sin, norm_weight=None, eps=1e-6):
+        self.rope_cos, self.rope_sin, self.norm_weight, self.eps = rope_cos, rope_sin, norm_weight, float(eps)
+
+    def _struct(self, D, q):
+        for n, t in (("rope_cos", self.rope_cos), ("rope_sin", self.rope_sin)):
+            _need_device(n, t)
+            _check(t.dim() == 2 and t.shape[1] == D // 2 and t.dtype == torch.bfloat16 and t.shape[0] > 0,
+                   f"q_transform.{n} must be bfloat16 [max_pos, D/2]")
+        _check(self.rope_sin.shape == self.rope_cos.shape, "q_transform.rope_sin must match rope_cos")
+        if self.norm_weight is not None:
+            _need_device("norm_weight", self.norm_weight)
+            _check(tuple(self.norm_weight.shape) == (D,) and self.norm_weight.dtype == torch.bfloat16,
+                   "q_transform.norm_weight must be bfloat16 [D]")
+        _check(q.dtype == torch.bfloat16, "q_transform needs bfloat16 q")
+        _same_device(q, rope_cos=self.rope_cos, rope_sin=self.rope_sin, norm_weight=self.norm_weight)
+        return _lib.QTransformStruct(None if self.norm_weight is None else self.norm_weight.data_ptr(),
+                                     self.rope_cos.data_ptr(), self.rope_sin.data_ptr(),
+                                     self.rope_cos.shape[0], self.eps)
+
+
+def q_transform_supported(T, D, block_size) -> bool:
+    """Whether the kernel that `decode` (T = 1) or `prefill` picks for bfloat16 q of this shape can
+    take a `QTransform`: the matrix-core kernels, which need a power-of-two block size >= 16 and
+    head_dim 128 (decode and verify: 64 too)."""
+    if block_size < 16 or block_size & (block_size - 1):
+        return False
+    return D == 128 or (D == 64 and T <= 64)
+
+
+def _qt_arg(q_transform, D, q):
+    """(struct kept alive by the caller, pointer value or None) for a C call."""
+    if q_transform is None:
+        return None, None
+    _check(isinstance(q_transform, QTransform), "q_transform must be a QTransform")
+    st = q_transform._struct(D, q)
+    return st, ctypes.addressof(st)
+
+
 def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, v_scale=None,
            partition_size=512, max_seq_len=None, out=None, workspace=None, validate_tables=False,
-           sinks=None, sliding_window=None):
+           sinks=None, sliding_window=None, q_transform=None):
     """out[b, h] = softmax(q[b, h] . K_b^T * scale) V_b over the paged context.
 
     q [B, Hq, D] (float32 or bfloat16); k_cache/v_cache [num_blocks, block_size, Hkv, D]
@@ -136,6 +181,7 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
     without a device sync; default = table capacity).
     sinks [Hq]: per-head logits that join the softmax as one more column and carry no value;
     sliding_window W: only the last W keys are visible (bf16 / fp8 pools, head_dim 64 or 128).
+    q_transform: a `QTransform`; q then holds the rows before norm and rotation (same shapes).
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache),
@@ -183,11 +229,13 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
         _need_device("workspace", workspace)
         _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    qt_keep, qt_ptr = _qt_arg(q_transform, D, q)
     with torch.cuda.device(q.device):
         rc = lib.pa_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                            _ptr(block_tables), _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes,
                            B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
-                           float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, _stream_ptr(q.device))
+                           float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, qt_ptr,
+                           _stream_ptr(q.device))
     _raise_on(rc, "pa_decode")
     return out
 
@@ -205,7 +253,8 @@ def verify_supported(T, D, block_size) -> bool:
 
 
 def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
-            out=None, workspace=None, route=None, validate_tables=False, sinks=None, sliding_window=None):
+            out=None, workspace=None, route=None, validate_tables=False, sinks=None, sliding_window=None,
+            q_transform=None):
     """Chunked prefill against a cached prefix (causal).
 
     q [B, T, Hq, D] bfloat16 holds the last query_lens[b] tokens of each sequence
@@ -218,7 +267,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     (HBM-bound: the context is read once per kv head); everything else through the tiled
     matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
     (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both.  sinks and sliding_window are
-    as in `decode`, the window counted back from each query token.
+    as in `decode`, the window counted back from each query token; so is q_transform, the position of
+    row t being seq_lens[b] - query_lens[b] + t.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -263,6 +313,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     else:
         _need_device("out", out)
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
+    qt_keep, qt_ptr = _qt_arg(q_transform, D, q)
     if route == "verify":
         need = int(lib.pa_verify_workspace_bytes(B, T, Hq, D))
         if workspace is None:
@@ -276,7 +327,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
                                _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), _ptr(out),
                                _ptr(workspace), ws_bytes, B, T, Hq, Hkv, D, block_size,
                                block_tables.shape[1], num_blocks, float(scale), kv_code, _ptr(sinks), win,
-                               _stream_ptr(q.device))
+                               qt_ptr, _stream_ptr(q.device))
         _raise_on(rc, "pa_verify")
         return out
     with torch.cuda.device(q.device):
@@ -291,7 +342,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
                             _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
                             block_tables.shape[1], num_blocks, float(scale), BF16, kv_code, _ptr(sinks), win,
-                            _ptr(workspace), ws_bytes, _stream_ptr(q.device))
+                            _ptr(workspace), ws_bytes, qt_ptr, _stream_ptr(q.device))
     _raise_on(rc, "pa_prefill")
     return out
 
@@ -428,18 +479,26 @@ def qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, 
     xk / xv [B, T, Hkv, D] bfloat16; rope_cos / rope_sin [max_pos, D/2] bfloat16 (`rope_tables`).
     Returns the transformed q (`out`, which may be xq itself; padding rows are zero); the pool
     (and its scales for float8) is updated in place.
+
+    xq None: only K and V are done and None is returned; the Q half then rides on the attention
+    call as its `q_transform` (a `QTransform` with the same tables), which saves a pass over Q.
     """
     lib = _lib.load()
-    for n, t in (("xq", xq), ("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
+    for n, t in (("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
                  ("block_tables", block_tables), ("seq_lens", seq_lens), ("query_lens", query_lens),
                  ("rope_cos", rope_cos), ("rope_sin", rope_sin)):
         _need_device(n, t)
-    _check(xq.dim() == 4 and xq.dtype == torch.bfloat16, "xq must be bfloat16 [B, T, Hq, D]")
-    B, T, Hq, D = xq.shape
-    _check(xk.dim() == 4 and xk.dtype == torch.bfloat16 and xk.shape[:2] == (B, T) and xk.shape[3] == D,
-           "xk must be bfloat16 [B, T, Hkv, D]")
-    Hkv = xk.shape[2]
+    _check(xk.dim() == 4 and xk.dtype == torch.bfloat16, "xk must be bfloat16 [B, T, Hkv, D]")
+    B, T, Hkv, D = xk.shape
     _check(xv.shape == xk.shape and xv.dtype == torch.bfloat16, "xv must match xk")
+    if xq is None:
+        _check(out is None and q_norm_weight is None, "without xq there is neither out nor q_norm_weight")
+        Hq = Hkv
+    else:
+        _need_device("xq", xq)
+        _check(xq.dim() == 4 and xq.dtype == torch.bfloat16 and xq.shape[:2] == (B, T) and xq.shape[3] == D,
+               "xq must be bfloat16 [B, T, Hq, D] with xk's B, T and D")
+        Hq = xq.shape[2]
     _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
     _check(D in (64, 128, 256), f"head_dim {D} must be 64, 128 or 256")
     _check(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (Hkv, D), "k_cache must be [num_blocks, block_size, Hkv, D]")
@@ -465,20 +524,21 @@ def qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, 
             _check(t.dtype == torch.float32 and tuple(t.shape) == (num_blocks, Hkv), f"{n} must be float32 [num_blocks, Hkv]")
     else:
         _check(k_scale is None and v_scale is None, "k_scale / v_scale are for float8 pools only")
-    if out is None:
-        out = torch.empty_like(xq)
-    else:
-        _need_device("out", out)
-        _check(out.shape == xq.shape and out.dtype == xq.dtype, "out must match xq")
-    _same_device(xq, xk=xk, xv=xv, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
+    if xq is not None:
+        if out is None:
+            out = torch.empty_like(xq)
+        else:
+            _need_device("out", out)
+            _check(out.shape == xq.shape and out.dtype == xq.dtype, "out must match xq")
+    _same_device(xk, xq=xq, xv=xv, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
                  query_lens=query_lens, rope_cos=rope_cos, rope_sin=rope_sin, q_norm_weight=q_norm_weight,
                  k_norm_weight=k_norm_weight, k_scale=k_scale, v_scale=v_scale, out=out)
-    with torch.cuda.device(xq.device):
+    with torch.cuda.device(xk.device):
         rc = lib.pa_qk_norm_rope_kv_write(
             _ptr(xq), _ptr(xk), _ptr(xv), _ptr(out), _ptr(q_norm_weight), _ptr(k_norm_weight), ctypes.c_float(eps),
             _ptr(rope_cos), _ptr(rope_sin), rope_cos.shape[0], _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
             _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), B, T, Hq, Hkv, D, block_size, block_tables.shape[1],
-            num_blocks, kv_dtype, _stream_ptr(xq.device))
+            num_blocks, kv_dtype, _stream_ptr(xk.device))
     _raise_on(rc, "pa_qk_norm_rope_kv_write")
     return out
 

@@ -28,22 +28,32 @@ def _win(w: int):
     return None if w <= 0 else int(w)
 
 
+def _qt(rope_cos, rope_sin, q_norm_weight, eps):
+    return None if rope_cos is None else paged_attn.QTransform(rope_cos, rope_sin, q_norm_weight, eps)
+
+
 @torch.library.custom_op(f"{_NS}::paged_decode", mutates_args=("out",), device_types="cuda")
 def paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                  seq_lens: torch.Tensor, scale: float, out: torch.Tensor,
                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
-                 max_seq_len: int = 0, sinks: Optional[torch.Tensor] = None, sliding_window: int = 0) -> None:
+                 max_seq_len: int = 0, sinks: Optional[torch.Tensor] = None, sliding_window: int = 0,
+                 rope_cos: Optional[torch.Tensor] = None, rope_sin: Optional[torch.Tensor] = None,
+                 q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6) -> None:
     paged_attn.decode(q, k_cache, v_cache, block_tables, seq_lens, scale, k_scale=k_scale, v_scale=v_scale,
-                      max_seq_len=max_seq_len or None, out=out, sinks=sinks, sliding_window=_win(sliding_window))
+                      max_seq_len=max_seq_len or None, out=out, sinks=sinks, sliding_window=_win(sliding_window),
+                      q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps))
 
 
 @torch.library.custom_op(f"{_NS}::paged_prefill", mutates_args=("out",), device_types="cuda")
 def paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                   seq_lens: torch.Tensor, query_lens: torch.Tensor, scale: float, out: torch.Tensor,
                   k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
-                  sinks: Optional[torch.Tensor] = None, sliding_window: int = 0) -> None:
+                  sinks: Optional[torch.Tensor] = None, sliding_window: int = 0,
+                  rope_cos: Optional[torch.Tensor] = None, rope_sin: Optional[torch.Tensor] = None,
+                  q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6) -> None:
     paged_attn.prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, k_scale=k_scale,
-                       v_scale=v_scale, out=out, sinks=sinks, sliding_window=_win(sliding_window))
+                       v_scale=v_scale, out=out, sinks=sinks, sliding_window=_win(sliding_window),
+                       q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps))
 
 
 @torch.library.custom_op(f"{_NS}::blocksparse_prefill", mutates_args=("out",), device_types="cuda")
@@ -95,6 +105,28 @@ def qk_norm_rope_kv_write_fp8(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tens
                                      k_scale=k_scale, v_scale=v_scale, out=q_out)
 
 
+# K and V only: the Q half of the transform then rides on paged_decode / paged_prefill (rope_cos, rope_sin,
+# q_norm_weight arguments), which saves the pass over Q
+@torch.library.custom_op(f"{_NS}::k_norm_rope_kv_write", mutates_args=("k_cache", "v_cache"), device_types="cuda")
+def k_norm_rope_kv_write(xk: torch.Tensor, xv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                         block_tables: torch.Tensor, seq_lens: torch.Tensor, query_lens: torch.Tensor,
+                         rope_cos: torch.Tensor, rope_sin: torch.Tensor,
+                         k_norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> None:
+    paged_attn.qk_norm_rope_kv_write(None, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, rope_cos,
+                                     rope_sin, k_norm_weight=k_norm_weight, eps=eps)
+
+
+@torch.library.custom_op(f"{_NS}::k_norm_rope_kv_write_fp8", mutates_args=("k_cache", "v_cache", "k_scale", "v_scale"),
+                         device_types="cuda")
+def k_norm_rope_kv_write_fp8(xk: torch.Tensor, xv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                             k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor,
+                             seq_lens: torch.Tensor, query_lens: torch.Tensor, rope_cos: torch.Tensor,
+                             rope_sin: torch.Tensor, k_norm_weight: Optional[torch.Tensor] = None,
+                             eps: float = 1e-6) -> None:
+    paged_attn.qk_norm_rope_kv_write(None, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, rope_cos,
+                                     rope_sin, k_norm_weight=k_norm_weight, eps=eps, k_scale=k_scale, v_scale=v_scale)
+
+
 def _no_cpu(name):
     def impl(*args, **kwargs):
         raise NotImplementedError(f"{_NS}::{name} runs hand-written HIP kernels and has no CPU path; "
@@ -105,9 +137,10 @@ def _no_cpu(name):
 for _op, _name in ((paged_decode, "paged_decode"), (paged_prefill, "paged_prefill"),
                    (blocksparse_prefill, "blocksparse_prefill"), (paged_kv_write, "paged_kv_write"),
                    (paged_kv_write_fp8, "paged_kv_write_fp8"), (qk_norm_rope_kv_write, "qk_norm_rope_kv_write"),
-                   (qk_norm_rope_kv_write_fp8, "qk_norm_rope_kv_write_fp8")):
+                   (qk_norm_rope_kv_write_fp8, "qk_norm_rope_kv_write_fp8"),
+                   (k_norm_rope_kv_write, "k_norm_rope_kv_write"), (k_norm_rope_kv_write_fp8, "k_norm_rope_kv_write_fp8")):
     _op.register_kernel("cpu")(_no_cpu(_name))
     _op.register_fake(lambda *args, **kwargs: None)      # outputs are caller-allocated: nothing to infer
 
 OPS = ("paged_decode", "paged_prefill", "blocksparse_prefill", "paged_kv_write", "paged_kv_write_fp8",
-       "qk_norm_rope_kv_write", "qk_norm_rope_kv_write_fp8")
+       "qk_norm_rope_kv_write", "qk_norm_rope_kv_write_fp8", "k_norm_rope_kv_write", "k_norm_rope_kv_write_fp8")

@@ -47,7 +47,7 @@ def test_c_abi_argument_errors_without_gpu(lib):
         a = dict(B=2, Hq=8, Hkv=2, D=128, bs=16, mb=4, nb=8, msl=0, scale=1.0, part=512, qd=1, kd=1)
         a.update(kw)
         return lib.pa_decode(z, z, z, z, z, z, z, z, z, 0, a["B"], a["Hq"], a["Hkv"], a["D"], a["bs"],
-                             a["mb"], a["nb"], a["msl"], a["scale"], a["part"], a["qd"], a["kd"], z, a.get("win", 0), z)
+                             a["mb"], a["nb"], a["msl"], a["scale"], a["part"], a["qd"], a["kd"], z, a.get("win", 0), z, z)
     assert dec(Hq=7) == -1 and b"multiple" in lib.pa_last_error()
     assert dec(D=96) == -1 and b"head_dim" in lib.pa_last_error()
     assert dec(qd=0, kd=1) == -1 and b"dtype" in lib.pa_last_error()
@@ -57,9 +57,9 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert dec(B=0) == 0                                        # empty batch is a no-op
     assert lib.pa_blocksparse_prefill(z, z, z, z, 1, 64, 4, 4, 128, 32, 4, 8, 1.0, 1, z) == -1
     assert b"block must be 64" in lib.pa_last_error()
-    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 0, 1, z, 0, z, 0, z) == -1
-    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 1, 1, z, -1, z, 0, z) == -1 and b"sliding_window" in lib.pa_last_error()
-    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 1, 0, z, 0, z, 0, z) == -1 and b"kv_dtype" in lib.pa_last_error()
+    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 0, 1, z, 0, z, 0, z, z) == -1
+    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 1, 1, z, -1, z, 0, z, z) == -1 and b"sliding_window" in lib.pa_last_error()
+    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 1, 0, z, 0, z, 0, z, z) == -1 and b"kv_dtype" in lib.pa_last_error()
     assert lib.pa_gather_kv(z, z, z, z, 1, 2, 64, 16, 2, 8, 100, 2, z) == -1  # beyond table capacity
     def kvw(**kw):
         a = dict(B=2, T=4, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1)
@@ -84,7 +84,7 @@ def test_c_abi_argument_errors_without_gpu(lib):
         a = dict(B=2, T=4, Hq=8, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1)
         a.update(kw)
         return lib.pa_verify(z, z, z, z, z, z, z, z, z, z, 0, a["B"], a["T"], a["Hq"], a["Hkv"], a["D"], a["bs"],
-                             a["mb"], a["nb"], 1.0, a["kd"], z, a.get("win", 0), z)
+                             a["mb"], a["nb"], 1.0, a["kd"], z, a.get("win", 0), z, z)
     assert ver(Hq=7) == -1 and b"multiple" in lib.pa_last_error()
     assert ver(kd=0) == -1 and b"kv_dtype" in lib.pa_last_error()
     assert ver(T=65) == -1 and b"pa_prefill" in lib.pa_last_error()

@@ -81,3 +81,16 @@ def test_ops_match_the_python_ops_and_replay_in_a_graph():
         step()                               # the program's own eager work between replays
         torch.cuda.synchronize()
         assert np.array_equal(got, dev_bits(o))
+
+    # the Q half of the pre-attention transform on the attention operator, K and V through the write operator
+    cos, sin = pa.rope_tables(D, 4096)
+    wn = bf16_to_dev(1.0 + 0.1 * rng.standard_normal(D).astype(np.float32))
+    torch.ops.nkipy_amd.k_norm_rope_kv_write(xk, xv, kd, vd, td, sd, qlens, cos, sin, wn)
+    want = pa.prefill(xq, kd, vd, td, sd, qlens, 0.09, q_transform=pa.QTransform(cos, sin, wn))
+    torch.ops.nkipy_amd.paged_prefill(xq, kd, vd, td, sd, qlens, 0.09, o, rope_cos=cos, rope_sin=sin, q_norm_weight=wn)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(o), dev_bits(want))
+    two = pa.prefill(pa.qk_norm_rope_kv_write(xq, xk, xv, kd, vd, td, sd, qlens, cos, sin, q_norm_weight=wn,
+                                              k_norm_weight=wn), kd, vd, td, sd, qlens, 0.09)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(o), dev_bits(two))
