@@ -1,6 +1,6 @@
 """GPU parity over seeded random combinations of every option of the attention ops (shape, GQA ratio,
-block size, fp8 pool, ragged query lengths, sliding window, sinks, kernel route): each case against the
-oracle.  The cases are drawn from a fixed seed, so a failure names a reproducible case."""
+block size, fp8 pool, ragged query lengths, sliding window, sinks, Q transform on load, kernel route): each
+case against the oracle.  The cases are drawn from a fixed seed, so a failure names a reproducible case."""
 import os
 
 import numpy as np
@@ -32,15 +32,14 @@ def _draw(case):
     T = 1 if kind == "decode" else int(rng.integers(2, 20)) if kind == "verify" else int(rng.integers(65, 300))
     fp8 = bool(rng.integers(0, 2))
     window = None if rng.integers(0, 2) else int(rng.choice([1, 7, 32, 33, 100, 700]))
-    if fp8 and kind == "tiled":
-        window = None                      # a window over an fp8 pool is the verify kernel's only
     sinks = bool(rng.integers(0, 2))
     long_ctx = rng.integers(0, 4) == 0
     prefixes = [int(rng.integers(0, 3000 if long_ctx else 300)) for _ in range(B)]
     qlens = [int(rng.integers(0 if kind != "decode" and B > 1 else 1, T + 1)) for _ in range(B)]
     if kind != "decode" and max(qlens) == 0:
         qlens[0] = T
-    return dict(rng=rng, D=D, Hkv=Hkv, Hq=Hkv * n_rep, bs=bs, B=B, kind=kind, T=T, fp8=fp8, window=window,
+    qt = int(rng.integers(0, 3))           # 0: q as given; 1: rotated on load; 2: normed and rotated on load
+    return dict(qt=qt, rng=rng, D=D, Hkv=Hkv, Hq=Hkv * n_rep, bs=bs, B=B, kind=kind, T=T, fp8=fp8, window=window,
                 sinks=sinks, prefixes=prefixes, qlens=qlens)
 
 
@@ -70,16 +69,25 @@ def test_random_case(case):
         kc_d, vc_d = bf16_to_dev(k), bf16_to_dev(v)
     sinks_d = None if sinks is None else bf16_to_dev(sinks)
     tol = 5e-2 if c["fp8"] else 2e-2
+    q_dev, qt = q, None
+    if c["qt"]:
+        w = O.round_to_bf16(1.0 + 0.2 * rng.standard_normal(D).astype(np.float32)) if c["qt"] == 2 else None
+        max_pos = max(ctxs) + 1
+        cos, sin = O.rope_tables(D, max_pos, 10000.0)
+        dcos, dsin = pa.rope_tables(D, max_pos, 10000.0)
+        qt = pa.QTransform(dcos, dsin, None if w is None else bf16_to_dev(w), 1e-6)
+        q, _ = O.qk_norm_rope(q_dev, q_dev[:, :, :Hkv], np.asarray(ctxs), np.asarray(qlens), cos, sin,
+                              q_norm_weight=w, eps=1e-6)          # what the oracle's attention sees
     if c["kind"] == "decode":
         want = O.paged_decode(q[:, 0], kc_o, vc_o, tables, np.asarray(ctxs, np.int32), scale, q_dtype="bf16",
                               sliding_window=c["window"], sinks=sinks, **kw_o)
-        got = pa.decode(bf16_to_dev(q[:, 0]), kc_d, vc_d, _i32(tables), _i32(ctxs), scale,
-                        sliding_window=c["window"], sinks=sinks_d, **kw_d)
+        got = pa.decode(bf16_to_dev(q_dev[:, 0]), kc_d, vc_d, _i32(tables), _i32(ctxs), scale,
+                        sliding_window=c["window"], sinks=sinks_d, q_transform=qt, **kw_d)
     else:
         want = O.paged_prefill(q, kc_o, vc_o, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale,
                                q_dtype="bf16", sliding_window=c["window"], sinks=sinks, **kw_o)
-        got = pa.prefill(bf16_to_dev(q), kc_d, vc_d, _i32(tables), _i32(ctxs), _i32(qlens), scale,
-                         sliding_window=c["window"], sinks=sinks_d, route=c["kind"], **kw_d)
+        got = pa.prefill(bf16_to_dev(q_dev), kc_d, vc_d, _i32(tables), _i32(ctxs), _i32(qlens), scale,
+                         sliding_window=c["window"], sinks=sinks_d, route=c["kind"], q_transform=qt, **kw_d)
     torch.cuda.synchronize()
     got = dev_to_f32(got)
     assert_close_abs(got, want, tol)
