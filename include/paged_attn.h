@@ -141,11 +141,13 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * (examples/models/gpt_oss/kernels/attention.py:85,127-135: "query at
  * start_pos+i attends to keys <= start_pos+i").  The new tokens' K/V are
  * already in the pool.  dtype: BF16 for q and out; kv_dtype PA_BF16, or PA_FP8_E4M3FN with
- * k_scale / v_scale [num_blocks, Hkv] (NULL otherwise): fp8 pools go through the register-staged
- * kernel, which expands the codes times their block's scale to bf16 on the way into LDS, and take no
- * sliding window.  sinks / sliding_window as for pa_decode, the
+ * k_scale / v_scale [num_blocks, Hkv] (NULL otherwise): the codes are copied into LDS as they are
+ * and expanded there, times their block's scale, to bf16.  sinks / sliding_window as for pa_decode, the
  * window counted back from each query token's own position; key tiles outside every row's
  * window are skipped.
+ * D = 128 runs the tiled matrix-core kernel (any block_size; the sliding window, the split and
+ * q_transform need a power of two >= 16).  D = 64 (block_size a power of two >= 16) runs as
+ * launches of pa_verify's kernel over 64 query tokens each and needs the workspace.
  * workspace: NULL, or pa_prefill_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed).  With
  * it, a call with too few query tiles to fill the device (one long-context request prefilled in
  * chunks) splits the key tiles of each query tile over up to 16 workgroups and merges their partial

@@ -276,6 +276,55 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   return 0;
 }
 
+// Query tokens [t0, t0 + Tc) of the T tokens per sequence through the decode-shaped kernel (pa_verify: all
+// of them in one launch; pa_prefill for shapes the tiled kernel does not take: 64 at a time).
+static int verify_launch(const char* who, const void* q, const void* k_cache, const void* v_cache,
+                         const float* k_scale, const float* v_scale,
+                         const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
+                         void* out, void* workspace, size_t workspace_bytes,
+                         int B, int T, int t0, int Tc, int Hq, int Hkv, int D, int block_size,
+                         int max_blocks_per_seq, int num_blocks, float scale, int kv_dtype,
+                         const float* sinks, int sliding_window, const pa_q_transform* q_transform, hipStream_t s) {
+  const long cap = (long)max_blocks_per_seq * block_size;
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
+  p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens; p.out = out;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = Tc; p.T_stride = T; p.t0 = t0;
+  {
+    // One wave carries 16 query rows of a kv head, or 32 where that measured faster: with more than 16 rows
+    // and a batch large enough to be bandwidth-bound, for D = 64 and for fp8 pools (which fit the registers),
+    // and for bf16 at D = 128 (which spills a little) only from four 16-row groups on.
+    const int n_rows = (Hq / Hkv) * Tc, forced = g_verify_rows.load();
+    const bool wide = n_rows > 16 && B >= 16 && (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
+    p.rows_per_wave = forced == 16 || forced == 32 ? forced : (wide ? 32 : 16);
+  }
+  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
+  p.block_shift = ilog2_exact(block_size);
+  p.max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
+  p.sinks = sinks; p.window = sliding_window;
+  p.partition_size = p.max_seq_len;
+  p.num_partitions = 1;
+  p.scale_log2e = scale * kLog2e;
+  if (!decode_mfma_supported(p, PA_BF16, kv_dtype))
+    return fail_arg("%s: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", who, D, block_size);
+  if (take_q_transform(who, q_transform, D, true, p.qt)) return -1;
+  plan_decode_balanced(p, current_num_cus());
+  p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
+  const size_t need = decode_balanced_workspace_bytes(B, Hq * Tc, D, p.bal_gv);
+  if (!workspace || workspace_bytes < need)
+    return fail_arg("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  p.ws_out = (float*)workspace;
+  p.ws_ml = p.ws_out + (size_t)Hq * Tc * ((size_t)B + p.bal_gv) * D;
+  p.ws_start = (int32_t*)(p.ws_ml + (size_t)Hq * Tc * ((size_t)B + p.bal_gv) * 2);
+  profile_begin(s);
+  hipError_t e = launch_decode_balanced(p, kv_dtype, s);
+  profile_end(s);
+  if (e != hipSuccess) return check_hip(e, "verify kernel launch");
+  e = launch_decode_balanced_reduce(p, s);
+  return check_hip(e, "verify merge launch");
+}
+
 size_t pa_verify_workspace_bytes(int B, int T, int Hq, int D) {
   if (B <= 0 || T <= 0 || Hq <= 0 || D <= 0 || (long)Hq * T > 0x7fffffffL) return 0;
   return decode_balanced_workspace_bytes(B, Hq * T, D, 8 * current_num_cus());
@@ -304,46 +353,9 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
   if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_verify: fp8 KV needs k_scale and v_scale");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out) || !aligned16(workspace))
     return fail_arg("pa_verify: q, k_cache, v_cache, out and workspace must be 16-byte aligned");
-  const long cap = (long)max_blocks_per_seq * block_size;
-
-  DecodeParams p;
-  memset(&p, 0, sizeof(p));
-  p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
-  p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens; p.out = out;
-  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = T;
-  {
-    // One wave carries 16 query rows of a kv head, or 32 where that measured faster: with more than 16 rows
-    // and a batch large enough to be bandwidth-bound, for D = 64 and for fp8 pools (which fit the registers),
-    // and for bf16 at D = 128 (which spills a little) only from four 16-row groups on.
-    const int n_rows = (Hq / Hkv) * T, forced = g_verify_rows.load();
-    const bool wide = n_rows > 16 && B >= 16 && (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
-    p.rows_per_wave = forced == 16 || forced == 32 ? forced : (wide ? 32 : 16);
-  }
-  p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
-  p.block_shift = ilog2_exact(block_size);
-  p.max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
-  p.sinks = sinks; p.window = sliding_window;
-  p.partition_size = p.max_seq_len;
-  p.num_partitions = 1;
-  p.scale_log2e = scale * kLog2e;
-  if (!decode_mfma_supported(p, PA_BF16, kv_dtype))
-    return fail_arg("pa_verify: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", D, block_size);
-  if (take_q_transform("pa_verify", q_transform, D, true, p.qt)) return -1;
-  plan_decode_balanced(p, current_num_cus());
-  p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
-  const size_t need = decode_balanced_workspace_bytes(B, Hq * T, D, p.bal_gv);
-  if (!workspace || workspace_bytes < need)
-    return fail_arg("pa_verify: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-  p.ws_out = (float*)workspace;
-  p.ws_ml = p.ws_out + (size_t)Hq * T * ((size_t)B + p.bal_gv) * D;
-  p.ws_start = (int32_t*)(p.ws_ml + (size_t)Hq * T * ((size_t)B + p.bal_gv) * 2);
-  hipStream_t s = (hipStream_t)stream;
-  profile_begin(s);
-  hipError_t e = launch_decode_balanced(p, kv_dtype, s);
-  profile_end(s);
-  if (e != hipSuccess) return check_hip(e, "pa_verify launch");
-  e = launch_decode_balanced_reduce(p, s);
-  return check_hip(e, "pa_verify reduce launch");
+  return verify_launch("pa_verify", q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens, out,
+                       workspace, workspace_bytes, B, T, 0, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks,
+                       scale, kv_dtype, sinks, sliding_window, q_transform, (hipStream_t)stream);
 }
 
 static void fill_prefill_shape(PrefillParams& p, int B, int T, int Hq, int Hkv, int D, int block_size,
@@ -360,6 +372,8 @@ static size_t prefill_split_bytes(const PrefillParams& p, int splits) {
 
 size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq) {
   if (B <= 0 || T <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || block_size <= 0 || max_blocks_per_seq <= 0 || Hq % Hkv) return 0;
+  if (D != 128)     // not the tiled kernel's: the call runs as launches of the decode-shaped kernel, 64 query tokens each
+    return pa_verify_workspace_bytes(B, T < PA_VERIFY_MAX_TOKENS ? T : PA_VERIFY_MAX_TOKENS, Hq, D);
   PrefillParams p;
   memset(&p, 0, sizeof(p));
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, 1);
@@ -401,7 +415,22 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.query_lens = query_lens; p.out = out;
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
   p.scale_log2e = scale * kLog2e;
-  if (!prefill_supported(p)) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
+  if (!prefill_supported(p)) {
+    // head_dim 64 (the tiled kernel is built for 128): the decode-shaped kernel takes the query tokens 64 at a
+    // time; each launch reads the context up to its last token once per kv head
+    if (D != 64) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
+    if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
+    if (B > 65535) return fail_arg("pa_prefill: B=%d exceeds 65535", B);
+    for (int t0 = 0; t0 < T; t0 += PA_VERIFY_MAX_TOKENS) {
+      const int tc = T - t0 < PA_VERIFY_MAX_TOKENS ? T - t0 : PA_VERIFY_MAX_TOKENS;
+      const int rc = verify_launch("pa_prefill", q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens,
+                                   out, workspace, workspace_bytes, B, T, t0, tc, Hq, Hkv, D, block_size,
+                                   max_blocks_per_seq, num_blocks, scale, kv_dtype, sinks, sliding_window, q_transform,
+                                   (hipStream_t)stream);
+      if (rc) return rc;
+    }
+    return 0;
+  }
   if (sliding_window > 0 && (p.impl == 1 || !prefill_async_supported(p)))
     return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;

@@ -165,7 +165,8 @@ struct DecodeParams {
   float* ws_ml;             // [B, Hq, P, 2]
   int32_t* ws_start;        // balanced schedule: [B + 1] tiles before each sequence, and the total
   int B, Hq, Hkv, D;
-  int T;                    // query tokens per sequence (1: decode)
+  int T;                    // query tokens per sequence in this launch (1: decode)
+  int T_stride, t0;         // multi-token launches: tokens per sequence in q / out, and the first one this launch covers
   int window;               // sliding window in tokens (balanced schedule only), 0 = none
   const float* sinks;       // [Hq] per-head sink logits (balanced schedule only) or null
   int rows_per_wave;        // query rows of a kv head carried by one wavefront: 16, or 32 (multi-token calls only)

@@ -154,7 +154,7 @@ struct DecodeWave {
     const int t = j / n_rep;
     *t_out = t;
     *head_out = hk * n_rep + (j - t * n_rep);
-    return (((long)b * p.T + t) * p.Hq + *head_out) * D;
+    return (((long)b * p.T_stride + p.t0 + t) * p.Hq + *head_out) * D;
   }
 
   // Start on sequence b (context ctx >= 1, of which the last tq tokens are the
@@ -524,13 +524,24 @@ struct DecodeWave {
   }
 };
 
-__device__ __forceinline__ int clamp_ctx(const DecodeParams& p, int b) {
-  return min(max(p.seq_lens[b], 0), p.max_seq_len);
+// Keys and query rows of sequence b in this launch.  Decode: the whole context and one row.  A
+// multi-token launch covers query tokens [t0, t0 + T) of the T_stride tokens per sequence in q:
+// its rows are the tq of them that lie below the sequence's query length, and its context ends
+// with the last of those (a launch none of whose tokens the sequence has streams nothing).
+struct SeqSpan { int ctx, tq; };
+__device__ __forceinline__ SeqSpan seq_span(const DecodeParams& p, int b) {
+  const int c = min(max(p.seq_lens[b], 0), p.max_seq_len);
+  if (!p.query_lens) return {c, 1};
+  const int qfull = min(min(max(p.query_lens[b], 0), p.T_stride), c);
+  const int tq = min(max(qfull - p.t0, 0), p.T);
+  return {tq > 0 ? c - qfull + p.t0 + tq : 0, tq};
 }
+__device__ __forceinline__ int clamp_ctx(const DecodeParams& p, int b) { return seq_span(p, b).ctx; }
 
-// Query tokens of sequence b (decode: 1)
+// Query tokens of sequence b in this launch (decode: 1)
 __device__ __forceinline__ int query_len(const DecodeParams& p, int b, int ctx) {
-  return p.query_lens ? min(min(max(p.query_lens[b], 0), p.T), ctx) : 1;
+  (void)ctx;
+  return seq_span(p, b).tq;
 }
 // First 32-token tile that any query row of sequence b sees (0 without a sliding window)
 __device__ __forceinline__ int first_tile(const DecodeParams& p, int b, int ctx) {
@@ -746,7 +757,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
     if (T == 0) { ++b; continue; }
     const int ti = f - start + first_tile(p, b, ctx);
     const int n = min(T - (f - start), f_end - f);
-    w.begin(b, ctx, MULTI ? min(min(max(p.query_lens[b], 0), p.T), ctx) : 1);
+    w.begin(b, ctx, MULTI ? query_len(p, b, ctx) : 1);
     w.stream(ti << 5, 32, n, ctx, p.bal_lockstep != 0);
     const int c_first = start / L, c_last = (start + T - 1) / L;
     if (c_first == c_last) w.store_final(b);
@@ -777,11 +788,11 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int hq = item / QUADS, q4 = item % QUADS;     // hq: virtual head when p.T > 1
   uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hq) * D + 4 * q4;
   int head = hq;                                      // the real q head of this item
-  if (p.T > 1) {
+  if (p.query_lens) {
     const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
     const int hk = hq / n_rows, j = hq % n_rows, t = j / n_rep;
     head = hk * n_rep + (j - t * n_rep);
-    dst = (uint16_t*)p.out + (((long)b * p.T + t) * p.Hq + head) * D + 4 * q4;
+    dst = (uint16_t*)p.out + (((long)b * p.T_stride + p.t0 + t) * p.Hq + head) * D + 4 * q4;
   }
   if (T == 0) {
     if (mine && g == 0) *(uint2*)dst = make_uint2(0u, 0u);

@@ -154,10 +154,10 @@ class QTransform:
 def q_transform_supported(T, D, block_size) -> bool:
     """Whether the kernel that `decode` (T = 1) or `prefill` picks for bfloat16 q of this shape can
     take a `QTransform`: the matrix-core kernels, which need a power-of-two block size >= 16 and
-    head_dim 128 (decode and verify: 64 too)."""
+    head_dim 128 or 64."""
     if block_size < 16 or block_size & (block_size - 1):
         return False
-    return D == 128 or (D == 64 and T <= 64)
+    return D in (64, 128)
 
 
 def _qt_arg(q_transform, D, q):
@@ -265,7 +265,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     Two kernels stand behind it.  Short query runs -- speculative verify: T * (Hq / Hkv) <=
     VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query rows
     (HBM-bound: the context is read once per kv head); everything else through the tiled
-    matrix-core prefill kernel.  `route` = "verify" or "tiled" forces one.  fp8 pools
+    matrix-core prefill kernel (head_dim 128; with head_dim 64 a long query run goes through the
+    verify kernel 64 tokens at a time).  `route` = "verify" or "tiled" forces one.  fp8 pools
     (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both.  sinks and sliding_window are
     as in `decode`, the window counted back from each query token; so is q_transform, the position of
     row t being seq_lens[b] - query_lens[b] + t.

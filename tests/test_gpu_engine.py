@@ -95,13 +95,14 @@ def test_serving_loop_bf16_pool(rng, rope):
 
 def test_serving_loop_gpt_oss_variant(rng):
     """head_dim 64, RoPE, per-head sinks and a 24-token sliding window (shorter than the prompts): prompt
-    chunks, verify-sized steps and decode steps all go through the decode-shaped kernel."""
+    chunks (one of them longer than a launch of that kernel takes), verify-sized steps and decode steps all go
+    through the decode-shaped kernel."""
     from nkipy_amd.engine import PagedAttention, PagedKVCache
     S, Hq, Hkv, D, bs = 3, 8, 2, 64, 16
-    cache = PagedKVCache(num_blocks=30, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=8)
+    cache = PagedKVCache(num_blocks=40, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=12)
     sinks = _rand(rng, Hq)
-    cos, sin = O.rope_tables(D, 128, 150000.0)
-    layer = PagedAttention(cache, Hq, rope_base=150000.0, max_positions=128, sinks=bf16_to_dev(sinks), sliding_window=24)
+    cos, sin = O.rope_tables(D, 192, 150000.0)
+    layer = PagedAttention(cache, Hq, rope_base=150000.0, max_positions=192, sinks=bf16_to_dev(sinks), sliding_window=24)
     mirror = _Mirror(S, cos, sin, None, None, 1e-6, window=24, sinks=sinks)
 
     def run(T, qlens):
@@ -119,6 +120,8 @@ def test_serving_loop_gpt_oss_variant(rng):
     run(30, [0, 0, 30])
     for _ in range(20):
         run(1, [1, 1, 1])
+    run(100, [0, 100, 70])          # a long chunk at head_dim 64: the verify kernel, 64 tokens per launch
+    run(1, [1, 1, 1])
 
 
 def test_serving_loop_fp8_pool(rng):

@@ -157,3 +157,51 @@ def test_verify_argument_errors(pa):
         pa.verify(big, *args[1:])
     with pytest.raises(ValueError):     # forced onto the verify kernel, which stops at 64 tokens
         pa.prefill(big, *args[1:], route="verify")
+
+
+@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
+@pytest.mark.parametrize("T,Hq,Hkv,bs", [(65, 4, 4, 16), (200, 8, 2, 32), (129, 64, 8, 64)])
+def test_head_dim_64_long_prefill_runs_in_64_token_launches(pa, fp8, T, Hq, Hkv, bs):
+    """head_dim 64 has no tiled kernel: pa_prefill covers the query tokens with launches of the verify
+    kernel, 64 tokens each.  Ragged lengths put chunk boundaries inside, at the end of and past a sequence's
+    query run; the sliding window and the sinks ride along."""
+    rng = np.random.default_rng(T + Hq)
+    D = 64
+    qlens = [T, 64, 65, 0, T - 1, 1]
+    prefixes = [0, 300, 65, 40, 1533, 31]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    okw, dkw = {}, {}
+    kd, vd = bf16_to_dev(k), bf16_to_dev(v)
+    if fp8:
+        k, ks = O.quantize_kv_fp8(k)
+        v, vs = O.quantize_kv_fp8(v)
+        okw = dict(k_scale=ks, v_scale=vs)
+        dkw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda())
+        kd = torch.from_numpy(k).cuda().view(torch.float8_e4m3fn)
+        vd = torch.from_numpy(v).cuda().view(torch.float8_e4m3fn)
+    for win, snk in ((None, None), (100, sinks)):
+        want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.125, q_dtype="bf16", sliding_window=win, sinks=snk, **okw)
+        got = pa.prefill(bf16_to_dev(q), kd, vd, _i32(tables), _i32(ctxs), _i32(ql), 0.125, sliding_window=win,
+                         sinks=None if snk is None else bf16_to_dev(snk), **dkw)
+        torch.cuda.synchronize()
+        got = dev_to_f32(got)
+        assert_close_abs(got, want, FP8_TOL if fp8 else BF16_TOL)
+        for b, n in enumerate(qlens):
+            assert np.all(got[b, n:] == 0)
+
+
+def test_head_dim_64_long_prefill_with_q_transform(pa):
+    rng = np.random.default_rng(77)
+    T, Hq, Hkv, bs, D = 150, 8, 2, 32, 64
+    qlens, prefixes = [150, 70, 3], [200, 0, 900]
+    xq, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    w = O.round_to_bf16(1.0 + 0.2 * rng.standard_normal(D).astype(np.float32))
+    cos, sin = O.rope_tables(D, 1200, 10000.0)
+    dcos, dsin = pa.rope_tables(D, 1200, 10000.0)
+    oq, _ = O.qk_norm_rope(xq, xq[:, :, :Hkv], ctxs, ql, cos, sin, q_norm_weight=w, eps=1e-6)
+    want = O.paged_prefill(oq, k, v, tables, ctxs, ql, 0.125, q_dtype="bf16")
+    got = pa.prefill(bf16_to_dev(xq), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.125,
+                     q_transform=pa.QTransform(dcos, dsin, bf16_to_dev(w)))
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)
