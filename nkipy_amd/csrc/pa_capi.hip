@@ -293,10 +293,13 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = Tc; p.T_stride = T; p.t0 = t0;
   {
     // One wave carries 16 query rows of a kv head, or 32 where that measured faster: with more than 16 rows
-    // and a batch large enough to be bandwidth-bound, for D = 64 and for fp8 pools (which fit the registers),
-    // and for bf16 at D = 128 (which spills a little) only from four 16-row groups on.
+    // and enough waves either way (a batch of 16 or more, or 128 rows per kv head as in the 64-token launches
+    // of a long prefill), for D = 64 and for fp8 pools (which fit the registers), and for bf16 at D = 128
+    // (which spills a little) only from four 16-row groups on.
     const int n_rows = (Hq / Hkv) * Tc, forced = g_verify_rows.load();
-    const bool wide = n_rows > 16 && B >= 16 && (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
+    // (not under a sliding window: the few tiles a launch then sees are better spread over more waves)
+    const bool wide = n_rows > 16 && (B >= 16 || (n_rows >= 128 && sliding_window == 0)) &&
+                      (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
     p.rows_per_wave = forced == 16 || forced == 32 ? forced : (wide ? 32 : 16);
   }
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
