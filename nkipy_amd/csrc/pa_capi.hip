@@ -155,7 +155,7 @@ int pa_probe_mfma(const void* operands, void* sink, int blocks, int iters, float
 }
 
 // Checks an optional Q transform and copies it into the kernel parameters; returns 0 or -1.
-static int take_q_transform(const char* who, const pa_q_transform* qt, int D, bool kernel_ok, QTransform& dst) {
+static int take_q_transform(const char* who, const pa_q_transform* qt, bool kernel_ok, QTransform& dst) {
   memset(&dst, 0, sizeof(dst));
   if (!qt) return 0;
   if (!kernel_ok)
@@ -165,7 +165,6 @@ static int take_q_transform(const char* who, const pa_q_transform* qt, int D, bo
     return fail_arg("%s: q_transform needs rope_cos, rope_sin and rope_max_pos > 0", who);
   if (!aligned16(qt->rope_cos) || !aligned16(qt->rope_sin) || !aligned16(qt->norm_weight))
     return fail_arg("%s: q_transform tables must be 16-byte aligned", who);
-  (void)D;
   dst.norm_weight = (const uint16_t*)qt->norm_weight;
   dst.cos = (const uint16_t*)qt->rope_cos; dst.sin = (const uint16_t*)qt->rope_sin;
   dst.max_pos = qt->rope_max_pos; dst.eps = qt->norm_eps;
@@ -239,7 +238,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
     return fail_arg("pa_decode: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
                     "head_dim 64 or 128, block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
-  if (take_q_transform("pa_decode", q_transform, D, kind != 1, p.qt)) return -1;
+  if (take_q_transform("pa_decode", q_transform, kind != 1, p.qt)) return -1;
   if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
   if (kind == 3) {
     plan_decode_balanced(p, current_num_cus());
@@ -311,7 +310,7 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   p.scale_log2e = scale * kLog2e;
   if (!decode_mfma_supported(p, PA_BF16, kv_dtype))
     return fail_arg("%s: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", who, D, block_size);
-  if (take_q_transform(who, q_transform, D, true, p.qt)) return -1;
+  if (take_q_transform(who, q_transform, true, p.qt)) return -1;
   plan_decode_balanced(p, current_num_cus());
   p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
   const size_t need = decode_balanced_workspace_bytes(B, Hq * Tc, D, p.bal_gv);
@@ -437,7 +436,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   if (sliding_window > 0 && (p.impl == 1 || !prefill_async_supported(p)))
     return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
-  if (take_q_transform("pa_prefill", q_transform, D, p.impl != 1 && prefill_async_supported(p), p.qt)) return -1;
+  if (take_q_transform("pa_prefill", q_transform, p.impl != 1 && prefill_async_supported(p), p.qt)) return -1;
   p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
   // few workgroups and a long table: split the key tiles of a query tile over several workgroups when the
   // caller brought the workspace for it (without one the call runs unsplit)

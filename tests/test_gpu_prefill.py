@@ -228,8 +228,8 @@ def test_prefill_argument_errors(pa):
         pa.prefill(q[:, :, :3].contiguous(), kc, kc, bt, one, one, 1.0)
     with pytest.raises(ValueError):
         pa.blocksparse_prefill(q, q, q, 1.0, block=32)
-    with pytest.raises(RuntimeError):      # the tiled kernel is built for head_dim 128 only
-        pa.prefill(q[..., :64].contiguous(), kc[..., :64].contiguous(), kc[..., :64].contiguous(), bt, one, one, 1.0,
+    with pytest.raises(RuntimeError):      # head_dim 128 (tiled kernel) or 64 (verify kernel, 64 tokens per launch) only
+        pa.prefill(q[..., :32].contiguous(), kc[..., :32].contiguous(), kc[..., :32].contiguous(), bt, one, one, 1.0,
                    route="tiled")
     with pytest.raises(ValueError):
         pa.prefill(q, kc, kc, bt, one, one, 1.0, route="fast")
