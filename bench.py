@@ -230,11 +230,14 @@ def _mfma_ceiling(lib, sample):
     return round(best, 1)
 
 
-def bench_prefill(steps, warmup, lib, pa, W, fp8=False):
-    """config 3; with fp8=True the same workload over the pool quantised to e4m3 with per-(block, kv head) scales."""
+def bench_prefill(steps, warmup, lib, pa, W, fp8=False, gpt_oss=False):
+    """config 3; with fp8=True the same workload over the pool quantised to e4m3 with per-(block, kv head) scales;
+    with gpt_oss=True the same tokens and tables at that model's attention shape (64 q heads and 8 kv heads of 64,
+    per-head sinks; examples/models/gpt_oss/kernels/attention.py:117-148)."""
     from oracle import paged_attention_oracle as O
     from tests.pa_testlib import dev_bits
-    w = W.make_prefill()
+    w = W.make_prefill(heads=(64, 8), head_dim=64, name="C3 tokens, gpt-oss heads") if gpt_oss else W.make_prefill()
+    sinks = torch.linspace(-1.0, 1.0, w.q.shape[2], device="cuda") if gpt_oss else None
     out = torch.empty_like(w.q)
     kc, vc, ks, vs = w.k_cache, w.v_cache, None, None
     if fp8:
@@ -242,7 +245,8 @@ def bench_prefill(steps, warmup, lib, pa, W, fp8=False):
         vc, vs = W.quantize_pool_fp8(w.v_cache)
 
     def step():
-        pa.prefill(w.q, kc, vc, w.block_tables, w.seq_lens, w.query_lens, w.scale, out=out, k_scale=ks, v_scale=vs)
+        pa.prefill(w.q, kc, vc, w.block_tables, w.seq_lens, w.query_lens, w.scale, out=out, k_scale=ks, v_scale=vs,
+                   sinks=sinks)
 
     sec = _time_steps(step, steps, warmup)
     lib.pa_profile_enable(1)
@@ -257,7 +261,8 @@ def bench_prefill(steps, warmup, lib, pa, W, fp8=False):
         heads = [0, 1, 2, 3]
         O.paged_prefill(dev_bits(w.q), dev_bits(kc), dev_bits(vc), w.block_tables.cpu().numpy(),
                         w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy(), w.scale, seqs=[7], heads=heads,
-                        k_scale=None if ks is None else ks.cpu().numpy(), v_scale=None if vs is None else vs.cpu().numpy())
+                        k_scale=None if ks is None else ks.cpu().numpy(), v_scale=None if vs is None else vs.cpu().numpy(),
+                        sinks=None if sinks is None else sinks.cpu().numpy())
         return 4 * D * len(heads) * (T * int(w.prefix[7]) + T * (T + 1) // 2)
 
     res = {
@@ -266,13 +271,15 @@ def bench_prefill(steps, warmup, lib, pa, W, fp8=False):
         "pct_of_bf16_peak": round(100.0 * fl / sec / 1e12 / BF16_PEAK_TFLOPS, 2),
         "ms_per_step": round(sec * 1e3, 5),
         "dtype": "fp8-e4m3 KV expanded to bf16 in LDS / bf16 q, fp32 accumulate" if fp8 else "bf16, fp32 accumulate",
-        "config": {"workload": f"C3 paged chunked prefill{' over the fp8-quantised pool' if fp8 else ''}: B={B}, T={T}, "
+        "config": {"workload": f"{'gpt-oss-shape' if gpt_oss else 'C3'} paged chunked prefill{' over the fp8-quantised pool' if fp8 else ''}"
+                               f"{' with sinks' if gpt_oss else ''}: B={B}, T={T}, "
                                f"Hq={Hq}, Hkv={w.k_cache.shape[2]}, "
                                f"D={D}, block_size={w.k_cache.shape[1]}, prefix={w.prefix.tolist()}",
                    "flops": fl},
         "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
-                     "traffic": None if fp8 else _traffic(3)[0], "traffic_source": None if fp8 else _traffic(3)[1],
+                     "traffic": None if fp8 or gpt_oss else _traffic(3)[0],
+                     "traffic_source": None if fp8 or gpt_oss else _traffic(3)[1],
                      "kernel": "prefill_async_kernel", "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms),
                      "mfma_only_loop_same_data": _mfma_ceiling(lib, w.k_cache)},
@@ -471,7 +478,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8, 9, 10])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7, 8, 9, 10, 11])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -502,6 +509,8 @@ def main():
         res = bench_verify(args.steps, args.warmup, lib, pa, W)
     elif args.config == 9:
         res = bench_prefill(args.steps, args.warmup, lib, pa, W, fp8=True)
+    elif args.config == 11:
+        res = bench_prefill(args.steps, args.warmup, lib, pa, W, gpt_oss=True)
     elif args.config == 10:
         res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
     else:

@@ -146,8 +146,10 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * window counted back from each query token's own position; key tiles outside every row's
  * window are skipped.
  * D = 128 runs the tiled matrix-core kernel (any block_size; the sliding window, the split and
- * q_transform need a power of two >= 16).  D = 64 (block_size a power of two >= 16) runs as
- * launches of pa_verify's kernel over 64 query tokens each and needs the workspace.
+ * q_transform need a power of two >= 16).  D = 64 needs block_size a power of two >= 16 and the
+ * workspace: bf16 pools with an even Hkv and T > 64 run the same tiled kernel (two adjacent kv
+ * heads share its 256-byte rows), anything else launches of pa_verify's kernel over 64 query
+ * tokens each.
  * workspace: NULL, or pa_prefill_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed).  With
  * it, a call with too few query tiles to fill the device (one long-context request prefilled in
  * chunks) splits the key tiles of each query tile over up to 16 workgroups and merges their partial

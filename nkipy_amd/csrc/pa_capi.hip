@@ -374,13 +374,15 @@ static size_t prefill_split_bytes(const PrefillParams& p, int splits) {
 
 size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq) {
   if (B <= 0 || T <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || block_size <= 0 || max_blocks_per_seq <= 0 || Hq % Hkv) return 0;
-  if (D != 128)     // not the tiled kernel's: the call runs as launches of the decode-shaped kernel, 64 query tokens each
-    return pa_verify_workspace_bytes(B, T < PA_VERIFY_MAX_TOKENS ? T : PA_VERIFY_MAX_TOKENS, Hq, D);
   PrefillParams p;
   memset(&p, 0, sizeof(p));
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, 1);
   p.block_tables = (const int32_t*)16;     // paged form (only tested for null)
   const size_t plain = prefill_split_bytes(p, prefill_async_splits(p, current_num_cus()));
+  if (D != 128) {   // what the tiled kernel does not take runs as launches of the decode-shaped kernel, 64 query tokens each
+    const size_t chunks = pa_verify_workspace_bytes(B, T < PA_VERIFY_MAX_TOKENS ? T : PA_VERIFY_MAX_TOKENS, Hq, D);
+    return plain > chunks ? plain : chunks;
+  }
   p.kv_fp8 = 1;                            // fp8 pools use another workgroup shape: cover both
   const size_t fp8 = prefill_split_bytes(p, prefill_async_splits(p, current_num_cus()));
   return plain > fp8 ? plain : fp8;
@@ -417,9 +419,12 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.query_lens = query_lens; p.out = out;
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
   p.scale_log2e = scale * kLog2e;
-  if (!prefill_supported(p)) {
-    // head_dim 64 (the tiled kernel is built for 128): the decode-shaped kernel takes the query tokens 64 at a
-    // time; each launch reads the context up to its last token once per kv head
+  p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
+  // head_dim 64: the tiled kernel takes bf16 pools with an even number of kv heads (two heads share its 256-byte
+  // rows); short query runs and everything else go to the decode-shaped kernel, 64 query tokens per launch, each
+  // launch reading the context up to its last token once per kv head
+  const bool tiled64 = D == 64 && T > PA_VERIFY_MAX_TOKENS && p.impl != 1 && prefill_async_supported(p);
+  if (!prefill_supported(p) && !tiled64) {
     if (D != 64) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
     if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
     if (B > 65535) return fail_arg("pa_prefill: B=%d exceeds 65535", B);
@@ -437,7 +442,6 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
     return fail_arg("pa_prefill: sliding_window needs the asynchronous-copy kernel (block_size a power of two >= 16)");
   p.sinks = sinks; p.window = sliding_window;
   if (take_q_transform("pa_prefill", q_transform, p.impl != 1 && prefill_async_supported(p), p.qt)) return -1;
-  p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
   // few workgroups and a long table: split the key tiles of a query tile over several workgroups when the
   // caller brought the workspace for it (without one the call runs unsplit)
   p.splits = 1;

@@ -97,7 +97,7 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 // of two bf16 stages in exactly the layout the bf16 path copies into, one tile ahead of the
 // compute, so everything from the fragment reads on is shared.  Raw rows are private to the wave that
 // copies and expands them, so the raw ring needs no barrier; the bf16 stages use the one per tile.
-template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT, bool FP8>
+template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT, bool FP8, int DH>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -106,6 +106,16 @@ void prefill_async_kernel(PrefillParams p) {
   constexpr int STAGE_B = 2 * TILE_B;        // K then V
   constexpr int UK = BN / 4;                 // 1 KB copy units per tensor tile
   constexpr int BMW = 32 * NW;               // query rows per workgroup
+  // Head dim 64 (PAIR): a 256-byte row of the pool then holds two adjacent kv heads, and the LDS tile
+  // layout, the copies and the fragment maps stay those of 256-byte rows.  The first half of the waves
+  // works for a q head of the even kv head on the rows' first 128 bytes, the second half for the q head
+  // at the same place in the odd kv head's group on the other 128 bytes; both halves take the same
+  // TOKW query tokens, so every byte copied is used.
+  constexpr bool PAIR = DH == 64;
+  static_assert(DH == HD || (PAIR && NW == 8 && MODE == 1 && !SPARSE && !PACK && !FP8), "head dim 64: 8-wave paged dense bf16 form only");
+  constexpr int KS = DH / 16;                // k-steps of the score product
+  constexpr int VC = DH / 32;                // 32-wide d chunks of the output
+  constexpr int TOKW = PAIR ? BMW / 2 : BMW; // query tokens per workgroup (plain form)
   constexpr int NST = NW == 8 ? 4 : 2;   // LDS stages the copies land in
   constexpr int UPW = FP8 ? 2 : 2 * UK / NW; // copy units per wave per tile (FP8: 8 raw rows of K, 8 of V)
   static_assert(!FP8 || (NW == 8 && MODE == 1 && !SPARSE && !PACK && TT == 2), "fp8 pools: 8-wave paged dense form only");
@@ -124,22 +134,24 @@ void prefill_async_kernel(PrefillParams p) {
   // that share one kv head run on one XCD, back to back, heavy tiles first: their K/V
   // stays in that XCD's L2.
   const int n_rep = p.Hq / p.Hkv;
-  const int nqt = PACK ? (p.T * n_rep + BMW - 1) / BMW : (p.T + BMW - 1) / BMW;
+  const int nqt = PACK ? (p.T * n_rep + BMW - 1) / BMW : (p.T + TOKW - 1) / TOKW;
+  const int kvg = PAIR ? p.Hkv / 2 : p.Hkv;    // K/V row groups: kv heads, or pairs of them
   const int per_group = PACK ? nqt : nqt * n_rep;
-  const int groups = p.B * p.Hkv;
+  const int groups = p.B * kvg;
   const int xcd = blockIdx.x & 7;
   const int part = SPLIT ? (int)(blockIdx.x >> 3) % p.splits : 0;      // which share of the key tiles
   const int slot = SPLIT ? (int)(blockIdx.x >> 3) / p.splits : (int)(blockIdx.x >> 3);
   const int grp = xcd + 8 * (slot / per_group);
   if (grp >= groups) return;
   const int rr_ = slot % per_group;
-  const int b = grp / p.Hkv, hk = grp % p.Hkv;
+  const int b = grp / kvg, hk = grp % kvg;     // PAIR: hk numbers the pair
   const int qt = PACK ? nqt - 1 - rr_ : nqt - 1 - rr_ / n_rep;
-  const int hq = PACK ? hk * n_rep : hk * n_rep + rr_ % n_rep;     // PACK: first head of the group
+  const int hq = PACK ? hk * n_rep : (PAIR ? 2 * hk : hk) * n_rep + rr_ % n_rep;     // PACK: first head of the group; PAIR: the even kv head's
   // row r of the workgroup (0 .. BMW-1) -> query token and q head
-  const int v0 = qt * BMW;
-  auto row_token = [&](int r) __attribute__((always_inline)) { return PACK ? (v0 + r) / n_rep : v0 + r; };
-  auto row_head = [&](int r) __attribute__((always_inline)) { return PACK ? hq + (v0 + r) % n_rep : hq; };
+  const int v0 = qt * TOKW;
+  auto row_token = [&](int r) __attribute__((always_inline)) { return PACK ? (v0 + r) / n_rep : v0 + (PAIR ? (r & (TOKW - 1)) : r); };
+  auto row_head = [&](int r) __attribute__((always_inline)) { return PACK ? hq + (v0 + r) % n_rep : hq + (PAIR && r >= TOKW ? n_rep : 0); };
+  const int par = PAIR ? wave / (NW / 2) : 0;   // which 128 bytes of the rows this wave works on
 
   int tq = p.query_lens ? p.query_lens[b] : p.T;
   int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
@@ -149,14 +161,14 @@ void prefill_async_kernel(PrefillParams p) {
   const int prefix = ctx - tq;
   const int q0 = row_token(0);                                    // first query token of the workgroup
   uint16_t* out = (uint16_t*)p.out;
-  const long q_row_stride = (long)p.Hq * HD;
+  const long q_row_stride = (long)p.Hq * DH;
 
   if (q0 >= tq) {   // only padding rows here: zeros (written by the reduce kernel when splitting)
     if (SPLIT) return;
-    for (int i = tid; i < BMW * (HD / 8); i += NW * 64) {
-      const int r = i / (HD / 8);
+    for (int i = tid; i < BMW * (DH / 8); i += NW * 64) {
+      const int r = i / (DH / 8);
       const int row = row_token(r);
-      if (row < p.T) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)row_head(r) * HD + (i % (HD / 8)) * 8) = make_uint4(0, 0, 0, 0);
+      if (row < p.T) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)row_head(r) * DH + (i % (DH / 8)) * 8) = make_uint4(0, 0, 0, 0);
     }
     return;
   }
@@ -167,7 +179,7 @@ void prefill_async_kernel(PrefillParams p) {
   const bool qvalid = qrow < tq;
   const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
   const float sc = p.scale_log2e;
-  bf16x8_t qf[HD / 16];           // loaded below, between the first copy requests
+  bf16x8_t qf[KS];                // loaded below, between the first copy requests
   const int wq_lo = row_token(wave * 32);                         // first token of this wave
   const int wq_hi = min(row_token(wave * 32 + 31), tq - 1);       // last valid token (may be < wq_lo)
   const bool wave_has_rows = wq_lo < tq;
@@ -196,8 +208,8 @@ void prefill_async_kernel(PrefillParams p) {
   // with the global chunk  position ^ (row & 7).
   const const_i32_ptr table = MODE != 0 ? (const_i32_ptr)(uintptr_t)(p.block_tables + (long)b * p.max_blocks) : nullptr;
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
-  const long kv_row_bytes = (long)p.Hkv * HD * EB;
-  const char* kbase = (const char*)p.k + (long)hk * HD * EB;
+  const long kv_row_bytes = (long)p.Hkv * DH * EB;
+  const char* kbase = (const char*)p.k + (long)hk * HD * EB;     // PAIR: 256 bytes per pair
   const char* vbase = (const char*)p.v + (long)hk * HD * EB;
   const int dma_rr = lane >> 4, dma_pos = lane & 15;
   // every unit of a wave starts at the same row modulo 16 (NW is a multiple of 4), hence the
@@ -278,22 +290,22 @@ void prefill_async_kernel(PrefillParams p) {
   };
 
   // ---- LDS read maps (lane constants) -------------------------------------------------
-  int k_off[HD / 16];                 // K fragment of k-step s: row n, chunk 2s + h
+  int k_off[KS];                      // K fragment of k-step s: row n, chunk 2s + h (PAIR: of this wave's half)
 #pragma unroll
-  for (int s = 0; s < HD / 16; ++s) k_off[s] = n * ROW_B + (((2 * s + h) ^ (n & 15)) << 4);
-  int v_off[HD / 32];                 // V^T fragment source of d-chunk c
+  for (int s = 0; s < KS; ++s) k_off[s] = n * ROW_B + (((2 * (KS * par + s) + h) ^ (n & 15)) << 4);
+  int v_off[VC];                      // V^T fragment source of d-chunk c
   {
     const int g = lane >> 4, sl = lane & 15;
     const int row = 4 * h + (sl >> 2);                       // key row inside a 16-key window (also row & 7)
     const int y = 2 * (g & 1) + ((sl & 3) >> 1);             // 16-byte chunk inside the 64-byte d window
 #pragma unroll
-    for (int c = 0; c < HD / 32; ++c) v_off[c] = row * ROW_B + (((4 * c + y) ^ (4 * (row & 3))) << 4) + (sl & 1) * 8;
+    for (int c = 0; c < VC; ++c) v_off[c] = row * ROW_B + (((4 * (VC * par + c) + y) ^ (4 * (row & 3))) << 4) + (sl & 1) * 8;
   }
 
   // ---- accumulators ------------------------------------------------------------
-  f32x16_t oacc[HD / 32];
+  f32x16_t oacc[VC];
 #pragma unroll
-  for (int c = 0; c < HD / 32; ++c)
+  for (int c = 0; c < VC; ++c)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[c][i] = 0.f;
   // Softmax state of this lane's query row.  Scores come out of the matrix cores already
@@ -404,15 +416,15 @@ void prefill_async_kernel(PrefillParams p) {
   // a 16-key slice (4 MFMAs).  The loads of group g+1 are written before the MFMAs of group
   // g; where exactly they issue is left to the compiler's scheduler (pinning the order with
   // scheduling barriers measured 3 % slower).
-  auto load_k = [&](bf16x8_t (&kf)[HD / 16], int stage, int tt) __attribute__((always_inline)) {
+  auto load_k = [&](bf16x8_t (&kf)[KS], int stage, int tt) __attribute__((always_inline)) {
     const char* ks = smem + stage * STAGE_B + 32 * tt * ROW_B;
 #pragma unroll
-    for (int s = 0; s < HD / 16; ++s) kf[s] = *(const bf16x8_t*)(ks + k_off[s]);
+    for (int s = 0; s < KS; ++s) kf[s] = *(const bf16x8_t*)(ks + k_off[s]);
   };
-  auto load_v = [&](bf16x8_t (&vf)[HD / 32], int stage, int g) __attribute__((always_inline)) {   // g = 2 tt + kk
+  auto load_v = [&](bf16x8_t (&vf)[VC], int stage, int g) __attribute__((always_inline)) {   // g = 2 tt + kk
     const char* vs = smem + stage * STAGE_B + TILE_B + 16 * g * ROW_B;
 #pragma unroll
-    for (int c = 0; c < HD / 32; ++c) {
+    for (int c = 0; c < VC; ++c) {
       const lds_char* src = (const lds_char*)(vs + v_off[c]);
       const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
       const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 8 * ROW_B));
@@ -420,22 +432,22 @@ void prefill_async_kernel(PrefillParams p) {
       vf[c] = __builtin_bit_cast(bf16x8_t, pair);
     }
   };
-  auto mma_qk = [&](f32x16_t& sacc, const bf16x8_t (&kf)[HD / 16]) __attribute__((always_inline)) {
+  auto mma_qk = [&](f32x16_t& sacc, const bf16x8_t (&kf)[KS]) __attribute__((always_inline)) {
     sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[0], cinit, 0, 0, 0);
 #pragma unroll
-    for (int s = 1; s < HD / 16; ++s)
+    for (int s = 1; s < KS; ++s)
       sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[s], sacc, 0, 0, 0);
   };
-  auto mma_pv = [&](const bf16x8_t (&vf)[HD / 32], const uint32_t (&pw)[TT][8], int g) __attribute__((always_inline)) {
+  auto mma_pv = [&](const bf16x8_t (&vf)[VC], const uint32_t (&pw)[TT][8], int g) __attribute__((always_inline)) {
     const int tt = g >> 1, kk = g & 1;
     const bf16x8_t pf = make_frag(pw[tt][4 * kk], pw[tt][4 * kk + 1], pw[tt][4 * kk + 2], pw[tt][4 * kk + 3]);
 #pragma unroll
-    for (int c = 0; c < HD / 32; ++c)
+    for (int c = 0; c < VC; ++c)
       oacc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[c], pf, oacc[c], 0, 0, 0);
   };
   // S^T = K Q^T for the tile in `stage`; leaves the first V^T group of `vstage` in flight
-  auto scores = [&](f32x16_t (&sacc)[TT], int stage, bf16x8_t (&v0)[HD / 32], int vstage) __attribute__((always_inline)) {
-    bf16x8_t ka[HD / 16], kb[HD / 16];
+  auto scores = [&](f32x16_t (&sacc)[TT], int stage, bf16x8_t (&v0)[VC], int vstage) __attribute__((always_inline)) {
+    bf16x8_t ka[KS], kb[KS];
     load_k(ka, stage, 0);
     if (TT == 2) {
       load_k(kb, stage, 1);
@@ -448,8 +460,8 @@ void prefill_async_kernel(PrefillParams p) {
     }
   };
   // O^T += V^T P^T for the tile in `stage`; group 0's fragments were loaded by scores()
-  auto accumulate = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[HD / 32]) __attribute__((always_inline)) {
-    bf16x8_t v1[HD / 32];
+  auto accumulate = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[VC]) __attribute__((always_inline)) {
+    bf16x8_t v1[VC];
 #pragma unroll
     for (int g = 0; g < 2 * TT; g += 2) {
       load_v(v1, stage, g + 1);
@@ -500,7 +512,7 @@ void prefill_async_kernel(PrefillParams p) {
       slack = move ? REF_SLACK : slack;
       l_run *= alpha;
 #pragma unroll
-      for (int c = 0; c < HD / 32; ++c) oacc[c] *= alpha;
+      for (int c = 0; c < VC; ++c) oacc[c] *= alpha;
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
@@ -525,19 +537,19 @@ void prefill_async_kernel(PrefillParams p) {
   request_next();
   prefetch_next();
   {
-    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * HD;
-    uint4 qraw[HD / 16];
+    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * DH;
+    uint4 qraw[KS];
 #pragma unroll
-    for (int s = 0; s < HD / 16; ++s) {
+    for (int s = 0; s < KS; ++s) {
       qraw[s] = make_uint4(0, 0, 0, 0);
       if (qvalid) qraw[s] = *(const uint4*)(qp + 16 * s + 8 * h);
     }
     if (!SPARSE && p.qt.cos) {
       // norm and rotation of the row on the way in; every lane takes part (the row's other
       // half sits in lane ^ 32), rows past the query length carry zeros
-      float x[HD / 16][8];
+      float x[KS][8];
 #pragma unroll
-      for (int s = 0; s < HD / 16; ++s) {
+      for (int s = 0; s < KS; ++s) {
         const uint32_t w[4] = {qraw[s].x, qraw[s].y, qraw[s].z, qraw[s].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -546,15 +558,15 @@ void prefill_async_kernel(PrefillParams p) {
         }
       }
       const int pos = min(max(prefix + qrow, 0), p.qt.max_pos - 1);
-      q_norm_rope_lane<HD / 8, HD / 16, QRowLayout>(x, p.qt, pos, h);
+      q_norm_rope_lane<DH / 8, KS, QRowLayout>(x, p.qt, pos, h);
 #pragma unroll
-      for (int s = 0; s < HD / 16; ++s) {
+      for (int s = 0; s < KS; ++s) {
         qraw[s].x = pack_bf16x2(x[s][0], x[s][1]); qraw[s].y = pack_bf16x2(x[s][2], x[s][3]);
         qraw[s].z = pack_bf16x2(x[s][4], x[s][5]); qraw[s].w = pack_bf16x2(x[s][6], x[s][7]);
       }
     }
 #pragma unroll
-    for (int s = 0; s < HD / 16; ++s) {
+    for (int s = 0; s < KS; ++s) {
       const uint4 v = qraw[s];
       // scale * log2(e) goes into Q once (rounded to bf16 again: a relative 2^-9 per element,
       // below the rounding of the probabilities), so that the scores leave the matrix cores
@@ -569,7 +581,7 @@ void prefill_async_kernel(PrefillParams p) {
     // the Q loads must be complete (and known to the compiler to be) before the loop, or the
     // first use of a fragment inside it would drain the ring with a full wait
 #pragma unroll
-    for (int s = 0; s < HD / 16; ++s) asm volatile("" ::"v"(qf[s]));
+    for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qf[s]));
   }
 #pragma unroll
   for (int s = 1; s < NST - 1; ++s) {
@@ -606,7 +618,7 @@ void prefill_async_kernel(PrefillParams p) {
       if (tile_active(w_c)) {
         f32x16_t sacc[TT];
         uint32_t pw[TT][8];
-        bf16x8_t v0[HD / 32];
+        bf16x8_t v0[VC];
         scores(sacc, stage_c, v0, stage_c);
         prefetch_next();
         softmax(sacc, pw, w_c.kt);
@@ -627,9 +639,9 @@ void prefill_async_kernel(PrefillParams p) {
   }
   if (SPLIT) {     // partial result relative to m_ref; the sink and the division belong to the merge
     if (qvalid) {
-      float* po = p.ws_o + (row_g * p.splits + part) * HD;
+      float* po = p.ws_o + (row_g * p.splits + part) * DH;
 #pragma unroll
-      for (int c = 0; c < HD / 32; ++c)
+      for (int c = 0; c < VC; ++c)
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4)
           *(float4*)(po + 32 * c + 8 * i4 + 4 * h) =
@@ -645,11 +657,12 @@ void prefill_async_kernel(PrefillParams p) {
   // wave-private patch of the (now idle) tile ring they leave as whole 256-byte rows, 16 bytes a lane.
   __builtin_amdgcn_s_barrier();                  // every wave is done reading the ring
   {
-    constexpr int OROW_B = ROW_B + 8;            // row pitch: the 8 bytes spread a column of rows over the banks
+    constexpr int OROW_B = 2 * DH + 8;           // row pitch: the 8 bytes spread a column of rows over the banks
+    constexpr int OCH = DH / 8, ORI = 64 / OCH;  // 16-byte pieces per row; rows a wave stores per instruction
     char* patch = smem + wave * (32 * OROW_B);
     const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
 #pragma unroll
-    for (int c = 0; c < HD / 32; ++c)
+    for (int c = 0; c < VC; ++c)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int d = 32 * c + 8 * i4 + 4 * h;
@@ -659,12 +672,12 @@ void prefill_async_kernel(PrefillParams p) {
       }
     // the wave reads back what its own lanes wrote: no barrier, the compiler orders the LDS accesses
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int r = 4 * j + (lane >> 4), ch = lane & 15;
+    for (int j = 0; j < 32 / ORI; ++j) {
+      const int r = ORI * j + lane / OCH, ch = lane % OCH;
       const uint2 lo = *(const uint2*)(patch + r * OROW_B + 16 * ch), hi = *(const uint2*)(patch + r * OROW_B + 16 * ch + 8);
       const int tok = row_token(wave * 32 + r);
       if (tok < p.T)
-        *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)row_head(wave * 32 + r) * HD + 8 * ch) =
+        *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)row_head(wave * 32 + r) * DH + 8 * ch) =
             make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
   }
@@ -673,21 +686,22 @@ void prefill_async_kernel(PrefillParams p) {
 // Merge of the split form: one thread per (query row, 4 consecutive d); rows past query_lens become zeros.
 __global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams p) {
   const long item = (long)blockIdx.x * 256 + threadIdx.x;
-  const long row = item / (HD / 4);
-  const int q4 = (int)(item % (HD / 4));
+  const int D = p.D;
+  const long row = item / (D / 4);
+  const int q4 = (int)(item % (D / 4));
   if (row >= (long)p.B * p.T * p.Hq) return;
   const int hq = (int)(row % p.Hq);
   const long bt = row / p.Hq;
   const int t = (int)(bt % p.T), b = (int)(bt / p.T);
   const int tq = min(max(p.query_lens[b], 0), p.T);
-  uint16_t* dst = (uint16_t*)p.out + row * HD + 4 * q4;
+  uint16_t* dst = (uint16_t*)p.out + row * D + 4 * q4;
   if (t >= tq) { *(uint2*)dst = make_uint2(0u, 0u); return; }
   float m = -INFINITY, l = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   for (int c = 0; c < p.splits; ++c) {
     const float2 ml = *(const float2*)(p.ws_ml + (row * p.splits + c) * 2);
     if (ml.y == 0.f) continue;                 // a share in which the row saw no key (its O may be unwritten)
-    const float4 o = *(const float4*)(p.ws_o + (row * p.splits + c) * HD + 4 * q4);
+    const float4 o = *(const float4*)(p.ws_o + (row * p.splits + c) * D + 4 * q4);
     const float m_new = fmaxf(m, ml.x);
     const float a = exp2f(m - m_new), w = exp2f(ml.x - m_new);
     l = l * a + ml.y * w;
@@ -700,25 +714,26 @@ __global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams
   *(uint2*)dst = make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
 }
 
-template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false, bool FP8 = false>
+template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false, bool FP8 = false, int DH = HD>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
+  constexpr int TOKW = DH == 64 ? 16 * NW : 32 * NW;      // query tokens per workgroup (plain form)
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
   }
   const int n_rep = p.Hq / p.Hkv;
   const long per_group = PACK ? ((long)p.T * n_rep + 32 * NW - 1) / (32 * NW)
-                              : (long)((p.T + 32 * NW - 1) / (32 * NW)) * n_rep;
-  const long groups = (long)p.B * p.Hkv;
+                              : (long)((p.T + TOKW - 1) / TOKW) * n_rep;
+  const long groups = (long)p.B * (DH == 64 ? p.Hkv / 2 : p.Hkv);
   const long total = 8 * ((groups + 7) / 8) * per_group * (SPLIT ? p.splits : 1);
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   if (SPLIT) {
-    const long items = (long)p.B * p.T * p.Hq * (HD / 4);
+    const long items = (long)p.B * p.T * p.Hq * (DH / 4);
     hipLaunchKernelGGL(prefill_split_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, p);
   }
   return hipGetLastError();
@@ -727,6 +742,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
 // workgroups of the paged dense form for a given choice of waves and packing
 long prefill_workgroups(const PrefillParams& p, int waves, bool pack) {
   const int n_rep = p.Hq / p.Hkv;
+  if (p.D == 64) return (long)p.B * (p.Hkv / 2) * ((p.T + 16 * waves - 1) / (16 * waves)) * n_rep;
   const long per_group = pack ? ((long)p.T * n_rep + 32 * waves - 1) / (32 * waves)
                               : (long)((p.T + 32 * waves - 1) / (32 * waves)) * n_rep;
   return (long)p.B * p.Hkv * per_group;
@@ -735,15 +751,16 @@ long prefill_workgroups(const PrefillParams& p, int waves, bool pack) {
 }  // namespace
 
 bool prefill_async_supported(const PrefillParams& p) {
-  if (p.D != HD) return false;
   if (p.block_tables && p.block_shift < 4) return false;   // paged: power-of-two block size >= 16
-  return true;
+  if (p.D == HD) return true;
+  // head dim 64: two adjacent kv heads share the 256-byte rows the kernel is laid out for
+  return p.D == 64 && p.Hkv % 2 == 0 && p.block_tables && p.sparse_stride == 0 && !p.kv_fp8;
 }
 
 static bool prefill_packs(const PrefillParams& p) {
   const bool sparse = p.sparse_stride > 0, paged = p.block_tables != nullptr;
   // chunks shorter than a 4-wave tile of a GQA model: rows packed over the heads of a kv group
-  return paged && !sparse && !p.kv_fp8 && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
+  return paged && !sparse && !p.kv_fp8 && p.D == HD && p.Hq > p.Hkv && p.T < 128 && (p.impl == 0 || p.impl == 5);
 }
 static int prefill_waves(const PrefillParams& p, int waves) {
   const bool sparse = p.sparse_stride > 0;
@@ -751,7 +768,7 @@ static int prefill_waves(const PrefillParams& p, int waves) {
   // 256 rows, 4-stage ring: half the copy requests per FLOP).  Measured within a few per cent of
   // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
   // and for the sparse form.
-  if (p.kv_fp8) return 8;              // fp8 pools: the 8-wave form only
+  if (p.kv_fp8 || p.D == 64) return 8; // fp8 pools and head dim 64: the 8-wave form only
   if (prefill_packs(p)) return 4;
   if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
   return waves;
@@ -775,6 +792,16 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   const bool paged = p.block_tables != nullptr;
   const bool pack = prefill_packs(p);
   waves = prefill_waves(p, waves);
+  if (p.D == 64) {
+    if (sparse || !paged || p.kv_fp8 || p.Hkv % 2) return hipErrorInvalidValue;
+    if (p.splits > 1) {
+      if (!p.ws_o || !p.ws_ml) return hipErrorInvalidValue;
+      return p.window > 0 ? launch_typed<false, 1, 8, 2, true, false, true, false, 64>(p, s)
+                          : launch_typed<false, 1, 8, 2, false, false, true, false, 64>(p, s);
+    }
+    return p.window > 0 ? launch_typed<false, 1, 8, 2, true, false, false, false, 64>(p, s)
+                        : launch_typed<false, 1, 8, 2, false, false, false, false, 64>(p, s);
+  }
   if (p.kv_fp8) {
     if (sparse || !paged || !p.k_scale || !p.v_scale) return hipErrorInvalidValue;
     if (p.splits > 1) {

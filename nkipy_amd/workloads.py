@@ -207,13 +207,14 @@ def make_decode(config: int, device="cuda", shrink: int = 1) -> DecodeWorkload:
         partition_size=part, max_seq_len=int(ctx.max()), k_scale=ks, v_scale=vs, ctx=ctx)
 
 
-def make_prefill(device="cuda", shrink: int = 1) -> PrefillWorkload:
+def make_prefill(device="cuda", shrink: int = 1, heads=(32, 8), head_dim: int = 128, name: str = "C3") -> PrefillWorkload:
     """config 3: bf16 causal chunked prefill, B=8, T=2048 new tokens, prefix U[0,4096],
     bs=32, 32/8 heads, D=128; sequences 0-3 share one prefix (same length, a multiple of
-    the block size, same physical blocks), 4-7 have private prefixes."""
+    the block size, same physical blocks), 4-7 have private prefixes.  `heads` and `head_dim` give the
+    same tokens and tables another attention shape (the gpt-oss layers: 64/8 heads of 64)."""
     rng = np.random.default_rng(1003)
     gen = _gen(1003, device)
-    B, Hq, Hkv, D, bs = 8, 32, 8, 128, 32
+    B, (Hq, Hkv), D, bs = 8, heads, head_dim, 32
     T = max(2048 // shrink, 1)
     prefix = rng.integers(0, 4096 // shrink + 1, size=B).astype(np.int64)
     shared = (int(prefix[0]) // bs) * bs
@@ -240,7 +241,7 @@ def make_prefill(device="cuda", shrink: int = 1) -> PrefillWorkload:
     k = _randn((pool_blocks, bs, Hkv, D), torch.bfloat16, gen, device)
     v = _randn((pool_blocks, bs, Hkv, D), torch.bfloat16, gen, device)
     return PrefillWorkload(
-        name="C3" + (f"/shrink{shrink}" if shrink > 1 else ""), q=q, k_cache=k, v_cache=v,
+        name=name + (f"/shrink{shrink}" if shrink > 1 else ""), q=q, k_cache=k, v_cache=v,
         block_tables=torch.from_numpy(tables).to(device),
         seq_lens=torch.from_numpy(seq.astype(np.int32)).to(device),
         query_lens=torch.full((B,), T, dtype=torch.int32, device=device),

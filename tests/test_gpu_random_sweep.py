@@ -27,8 +27,6 @@ def _draw(case):
     bs = int(rng.choice([16, 32, 64, 128]))
     B = int(rng.integers(1, 7))
     kind = rng.choice(["decode", "verify", "tiled"])
-    if kind == "tiled" and D != 128:
-        kind = "verify"
     T = 1 if kind == "decode" else int(rng.integers(2, 20)) if kind == "verify" else int(rng.integers(65, 300))
     fp8 = bool(rng.integers(0, 2))
     window = None if rng.integers(0, 2) else int(rng.choice([1, 7, 32, 33, 100, 700]))

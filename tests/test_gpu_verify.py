@@ -159,12 +159,23 @@ def test_verify_argument_errors(pa):
         pa.prefill(big, *args[1:], route="verify")
 
 
+@pytest.fixture(params=["tiled", "chunks"])
+def d64_path(request):
+    """head_dim 64 beyond 64 query tokens: bf16 pools with an even number of kv heads take the tiled kernel
+    (two kv heads share its 256-byte rows); with the tiled kernel switched off, as for fp8 pools and odd head
+    counts, pa_prefill covers the query tokens with launches of the verify kernel, 64 tokens each."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    lib.pa_debug_set(3, 1 if request.param == "chunks" else 0)
+    yield request.param
+    lib.pa_debug_set(3, 0)
+
+
 @pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
-@pytest.mark.parametrize("T,Hq,Hkv,bs", [(65, 4, 4, 16), (200, 8, 2, 32), (129, 64, 8, 64)])
-def test_head_dim_64_long_prefill_runs_in_64_token_launches(pa, fp8, T, Hq, Hkv, bs):
-    """head_dim 64 has no tiled kernel: pa_prefill covers the query tokens with launches of the verify
-    kernel, 64 tokens each.  Ragged lengths put chunk boundaries inside, at the end of and past a sequence's
-    query run; the sliding window and the sinks ride along."""
+@pytest.mark.parametrize("T,Hq,Hkv,bs", [(65, 4, 4, 16), (200, 8, 2, 32), (129, 64, 8, 64), (300, 3, 1, 32), (530, 12, 6, 16)])
+def test_head_dim_64_long_prefill(pa, d64_path, fp8, T, Hq, Hkv, bs):
+    """Ragged lengths put tile and launch boundaries inside, at the end of and past a sequence's query run;
+    the sliding window and the sinks ride along."""
     rng = np.random.default_rng(T + Hq)
     D = 64
     qlens = [T, 64, 65, 0, T - 1, 1]
@@ -191,7 +202,7 @@ def test_head_dim_64_long_prefill_runs_in_64_token_launches(pa, fp8, T, Hq, Hkv,
             assert np.all(got[b, n:] == 0)
 
 
-def test_head_dim_64_long_prefill_with_q_transform(pa):
+def test_head_dim_64_long_prefill_with_q_transform(pa, d64_path):
     rng = np.random.default_rng(77)
     T, Hq, Hkv, bs, D = 150, 8, 2, 32, 64
     qlens, prefixes = [150, 70, 3], [200, 0, 900]
@@ -205,3 +216,24 @@ def test_head_dim_64_long_prefill_with_q_transform(pa):
                      q_transform=pa.QTransform(dcos, dsin, bf16_to_dev(w)))
     torch.cuda.synchronize()
     assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+
+
+def test_head_dim_64_tiled_split_matches_unsplit(pa):
+    """One long-context request at head_dim 64: the key tiles of its query tiles are split over workgroups."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(91)
+    T, Hq, Hkv, bs, D = 256, 4, 2, 32, 64
+    q, k, v, tables, ctxs, ql = _case(rng, T, [T], [6000], Hq, Hkv, bs, D)
+    sinks = bf16_to_dev(O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32)))
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.125)
+    want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.125, q_dtype="bf16", sinks=dev_to_f32(sinks))
+    got = dev_to_f32(pa.prefill(*args, sinks=sinks))
+    lib.pa_debug_set(6, 0)
+    try:
+        unsplit = dev_to_f32(pa.prefill(*args, sinks=sinks))
+    finally:
+        lib.pa_debug_set(6, 1)
+    torch.cuda.synchronize()
+    assert_close_abs(got, want, BF16_TOL)
+    assert np.max(np.abs(got - unsplit)) <= 2 ** -6
