@@ -40,7 +40,7 @@
 namespace pa {
 namespace {
 
-constexpr int HD = 128;                // head dim
+constexpr int HD = 128;                // elements of a 256-byte row: the head dim, or two heads of 64
 constexpr int ROW_B = HD * 2;          // bytes per K/V row
 // Where the 8-element chunks of a Q row sit: lane (n, h) holds chunk 2 s + h in slot s, so the
 // lowest chunk-index bit is the half-wave and the others are the slot number.
@@ -97,6 +97,8 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 // of two bf16 stages in exactly the layout the bf16 path copies into, one tile ahead of the
 // compute, so everything from the fragment reads on is shared.  Raw rows are private to the wave that
 // copies and expands them, so the raw ring needs no barrier; the bf16 stages use the one per tile.
+// DH: head dim, 128 or 64.  At 64 a 256-byte piece of a pool row is two adjacent kv heads: the tile
+// layout stays that of 256-byte rows and the two halves of the workgroup's waves work for the two heads.
 template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT, bool FP8, int DH>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
