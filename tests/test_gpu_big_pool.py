@@ -193,3 +193,30 @@ def test_kv_write(pa, big_bf16, big_fp8, mode):
     if fp8:
         assert np.array_equal(u8(scales[0]), dev_bits(_take(big[2], dev_ids)))
         assert np.array_equal(u8(scales[1]), dev_bits(_take(big[3], dev_ids)))
+
+
+@pytest.mark.parametrize("T", [4, 300], ids=["verify", "tiled"])
+def test_head_dim_64(pa, big_fp8, T):
+    """The same memory seen as a bf16 pool of head dim 64 (a row of 8 heads x 64 x 2 B is as long as one of
+    8 x 128 fp8 codes): the decode kernels and the tiled prefill kernel's two-heads-per-row form."""
+    rng = np.random.default_rng(81 + T)
+    D64 = 64
+    big = tuple(t.view(torch.uint8).view(torch.bfloat16) for t in big_fp8[:2])        # [BIG_FP8, BS, HKV, 64]
+    assert big[0].shape == (BIG_FP8, BS, HKV, D64)
+    prefixes = [2500, 0, 77]
+    ctxs = [p + T for p in prefixes]
+    k, v, tables = make_paged(rng, len(ctxs), HKV, D64, BS, ctxs)
+    small = (bf16_to_dev(k), bf16_to_dev(v))
+    ids = _spread(small[0].shape[0], BIG_FP8)
+    _place(small[0], big[0], ids)
+    _place(small[1], big[1], ids)
+    q = bf16_to_dev(rng.standard_normal((len(ctxs), T, 16, D64)).astype(np.float32))
+    run = lambda kk, vv, t: pa.prefill(q, kk, vv, t, _i32(ctxs), _i32([T] * len(ctxs)), 0.125)   # noqa: E731
+    a = run(small[0], small[1], _i32(tables))
+    b = run(big[0], big[1], _i32(_remap(tables, ids)))
+    qd = q[:, 0].contiguous()
+    c = pa.decode(qd, small[0], small[1], _i32(tables), _i32(ctxs), 0.125)
+    d = pa.decode(qd, big[0], big[1], _i32(_remap(tables, ids)), _i32(ctxs), 0.125)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(a), dev_bits(b))
+    assert np.array_equal(dev_bits(c), dev_bits(d))
