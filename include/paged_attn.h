@@ -147,7 +147,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * window are skipped.
  * D = 128 runs the tiled matrix-core kernel (any block_size; the sliding window, the split and
  * q_transform need a power of two >= 16).  D = 64 needs block_size a power of two >= 16 and the
- * workspace: bf16 pools with an even Hkv and T > 64 run the same tiled kernel (two adjacent kv
+ * workspace: an even Hkv and T > 64 run the same tiled kernel (two adjacent kv
  * heads share its 256-byte rows), anything else launches of pa_verify's kernel over 64 query
  * tokens each.
  * workspace: NULL, or pa_prefill_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed).  With

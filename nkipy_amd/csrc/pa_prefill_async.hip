@@ -114,7 +114,7 @@ void prefill_async_kernel(PrefillParams p) {
   // at the same place in the odd kv head's group on the other 128 bytes; both halves take the same
   // TOKW query tokens, so every byte copied is used.
   constexpr bool PAIR = DH == 64;
-  static_assert(DH == HD || (PAIR && NW == 8 && MODE == 1 && !SPARSE && !PACK && !FP8), "head dim 64: 8-wave paged dense bf16 form only");
+  static_assert(DH == HD || (PAIR && NW == 8 && MODE == 1 && !SPARSE && !PACK), "head dim 64: 8-wave paged dense form only");
   constexpr int KS = DH / 16;                // k-steps of the score product
   constexpr int VC = DH / 32;                // 32-wide d chunks of the output
   constexpr int TOKW = PAIR ? BMW / 2 : BMW; // query tokens per workgroup (plain form)
@@ -376,26 +376,36 @@ void prefill_async_kernel(PrefillParams p) {
   // puts the new pair in slot 3, a shift per tile brings it to slot 0 when the tile is expanded
   typedef const __attribute__((address_space(4))) float* const_f32_ptr;
   float ksq[4] = {0.f, 0.f, 0.f, 0.f}, vsq[4] = {0.f, 0.f, 0.f, 0.f};
+  float ksq2[4] = {0.f, 0.f, 0.f, 0.f}, vsq2[4] = {0.f, 0.f, 0.f, 0.f};      // PAIR: the odd kv head's
   auto request_next = [&]() __attribute__((always_inline)) {
     issue_tile(w_i.kt < ntiles ? w_i.kt : kt_first, stage_i);
     if (FP8) {
-      const long si = (long)min(max(blk_pf[0], 0), p.num_blocks - 1) * p.Hkv + hk;
+      const long si = (long)min(max(blk_pf[0], 0), p.num_blocks - 1) * p.Hkv + (PAIR ? 2 * hk : hk);
       ksq[3] = ((const_f32_ptr)(uintptr_t)p.k_scale)[si];
       vsq[3] = ((const_f32_ptr)(uintptr_t)p.v_scale)[si];
+      if (PAIR) {
+        ksq2[3] = ((const_f32_ptr)(uintptr_t)p.k_scale)[si + 1];
+        vsq2[3] = ((const_f32_ptr)(uintptr_t)p.v_scale)[si + 1];
+      }
     }
     if (w_i.kt < ntiles) walk_step(w_i);
     stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
   };
   auto shift_scales = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) { ksq[i] = ksq[i + 1]; vsq[i] = vsq[i + 1]; }
+    for (int i = 0; i < 3; ++i) {
+      ksq[i] = ksq[i + 1]; vsq[i] = vsq[i + 1];
+      if (PAIR) { ksq2[i] = ksq2[i + 1]; vsq2[i] = vsq2[i + 1]; }
+    }
   };
   // FP8: codes of tile kt in raw stage rs -> bf16 values in stage bs, this wave's 8 rows; rows past the
   // context get the scale 0 (their codes are a copy of the last valid row, their block may not exist)
-  auto expand = [&](int kt, int rs, int bs, float ks, float vs) __attribute__((always_inline)) {
+  auto expand = [&](int kt, int rs, int bs) __attribute__((always_inline)) {
     const char* raw = smem + BFS * STAGE_B + rs * RAW_STAGE_B + wave * 1024 + lane * 16;
     const int row = 8 * wave + (lane >> 3), c16 = lane & 7;
     const bool live = kt * BN + row < ctx;
+    // PAIR: the first 64 codes of a raw row belong to the even kv head, the others to the odd one
+    const float ks = PAIR && c16 >= 4 ? ksq2[0] : ksq[0], vs = PAIR && c16 >= 4 ? vsq2[0] : vsq[0];
     const float sk = live ? ks : 0.f, sv = live ? vs : 0.f;
     const uint4 rk = *(const uint4*)raw, rv = *(const uint4*)(raw + RAW_TILE_B);
     auto half = [&](uint32_t a, uint32_t b2, float scl) __attribute__((always_inline)) -> uint4 {
@@ -596,7 +606,7 @@ void prefill_async_kernel(PrefillParams p) {
     request_next();
     prefetch_next();
     wait_vmcnt<3 * UPW>();
-    expand(kt_first, 0, 0, ksq[0], vsq[0]);
+    expand(kt_first, 0, 0);
   }
 
   {
@@ -614,7 +624,7 @@ void prefill_async_kernel(PrefillParams p) {
       if (FP8) shift_scales();
       request_next();
       if (FP8) {
-        if (w_c.kt + 1 < ntiles) expand(w_c.kt + 1, rs_n, stage_c ^ 1, ksq[0], vsq[0]);
+        if (w_c.kt + 1 < ntiles) expand(w_c.kt + 1, rs_n, stage_c ^ 1);
         rs_n = (rs_n + 1) & 3;
       }
       if (tile_active(w_c)) {
@@ -756,7 +766,7 @@ bool prefill_async_supported(const PrefillParams& p) {
   if (p.block_tables && p.block_shift < 4) return false;   // paged: power-of-two block size >= 16
   if (p.D == HD) return true;
   // head dim 64: two adjacent kv heads share the 256-byte rows the kernel is laid out for
-  return p.D == 64 && p.Hkv % 2 == 0 && p.block_tables && p.sparse_stride == 0 && !p.kv_fp8;
+  return p.D == 64 && p.Hkv % 2 == 0 && p.block_tables && p.sparse_stride == 0;
 }
 
 static bool prefill_packs(const PrefillParams& p) {
@@ -795,14 +805,19 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   const bool pack = prefill_packs(p);
   waves = prefill_waves(p, waves);
   if (p.D == 64) {
-    if (sparse || !paged || p.kv_fp8 || p.Hkv % 2) return hipErrorInvalidValue;
-    if (p.splits > 1) {
-      if (!p.ws_o || !p.ws_ml) return hipErrorInvalidValue;
-      return p.window > 0 ? launch_typed<false, 1, 8, 2, true, false, true, false, 64>(p, s)
-                          : launch_typed<false, 1, 8, 2, false, false, true, false, 64>(p, s);
+    if (sparse || !paged || p.Hkv % 2 || (p.kv_fp8 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
+    if (p.splits > 1 && (!p.ws_o || !p.ws_ml)) return hipErrorInvalidValue;
+    const int form = (p.kv_fp8 ? 4 : 0) + (p.splits > 1 ? 2 : 0) + (p.window > 0 ? 1 : 0);
+    switch (form) {
+      case 0: return launch_typed<false, 1, 8, 2, false, false, false, false, 64>(p, s);
+      case 1: return launch_typed<false, 1, 8, 2, true, false, false, false, 64>(p, s);
+      case 2: return launch_typed<false, 1, 8, 2, false, false, true, false, 64>(p, s);
+      case 3: return launch_typed<false, 1, 8, 2, true, false, true, false, 64>(p, s);
+      case 4: return launch_typed<false, 1, 8, 2, false, false, false, true, 64>(p, s);
+      case 5: return launch_typed<false, 1, 8, 2, true, false, false, true, 64>(p, s);
+      case 6: return launch_typed<false, 1, 8, 2, false, false, true, true, 64>(p, s);
+      default: return launch_typed<false, 1, 8, 2, true, false, true, true, 64>(p, s);
     }
-    return p.window > 0 ? launch_typed<false, 1, 8, 2, true, false, false, false, 64>(p, s)
-                        : launch_typed<false, 1, 8, 2, false, false, false, false, 64>(p, s);
   }
   if (p.kv_fp8) {
     if (sparse || !paged || !p.k_scale || !p.v_scale) return hipErrorInvalidValue;

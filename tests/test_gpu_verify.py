@@ -161,8 +161,8 @@ def test_verify_argument_errors(pa):
 
 @pytest.fixture(params=["tiled", "chunks"])
 def d64_path(request):
-    """head_dim 64 beyond 64 query tokens: bf16 pools with an even number of kv heads take the tiled kernel
-    (two kv heads share its 256-byte rows); with the tiled kernel switched off, as for fp8 pools and odd head
+    """head_dim 64 beyond 64 query tokens: an even number of kv heads takes the tiled kernel
+    (two kv heads share its 256-byte rows); with the tiled kernel switched off, as for odd head
     counts, pa_prefill covers the query tokens with launches of the verify kernel, 64 tokens each."""
     from nkipy_amd import _lib
     lib = _lib.load()
