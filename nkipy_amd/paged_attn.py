@@ -58,6 +58,23 @@ def _stream_ptr(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on(device):
+    """Context in which `device` is the current one for a launch; nothing to switch when it already is
+    (the usual case, and the switch costs a few microseconds of a call that launches ten-microsecond kernels)."""
+    return _NO_GUARD if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
@@ -115,8 +132,8 @@ def decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size) -> int:
     return int(_lib.load().pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size))
 
 
-def _workspace(device, nbytes):
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+def _workspace(device, nbytes, stream=None):
+    key = (device, (stream or _stream_ptr(device)).value)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
@@ -223,19 +240,19 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
         _need_device("out", out)
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
     need = int(lib.pa_decode_workspace_bytes(B, Hq, D, msl, partition_size))
+    stream = _stream_ptr(q.device)
     if workspace is None:
-        workspace = _workspace(q.device, need) if need else None
+        workspace = _workspace(q.device, need, stream) if need else None
     else:
         _need_device("workspace", workspace)
         _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     qt_keep, qt_ptr = _qt_arg(q_transform, D, q)
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = lib.pa_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                            _ptr(block_tables), _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes,
                            B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
-                           float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, qt_ptr,
-                           _stream_ptr(q.device))
+                           float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, qt_ptr, stream)
     _raise_on(rc, "pa_decode")
     return out
 
@@ -316,26 +333,27 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
         _need_device("out", out)
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
     qt_keep, qt_ptr = _qt_arg(q_transform, D, q)
+    stream = _stream_ptr(q.device)
     if route == "verify":
         need = int(lib.pa_verify_workspace_bytes(B, T, Hq, D))
         if workspace is None:
-            workspace = _workspace(q.device, need)
+            workspace = _workspace(q.device, need, stream)
         else:
             _need_device("workspace", workspace)
             _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
         ws_bytes = workspace.numel() * workspace.element_size()
-        with torch.cuda.device(q.device):
+        with _on(q.device):
             rc = lib.pa_verify(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                                _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), _ptr(out),
                                _ptr(workspace), ws_bytes, B, T, Hq, Hkv, D, block_size,
                                block_tables.shape[1], num_blocks, float(scale), kv_code, _ptr(sinks), win,
-                               qt_ptr, _stream_ptr(q.device))
+                               qt_ptr, stream)
         _raise_on(rc, "pa_verify")
         return out
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         need = int(lib.pa_prefill_workspace_bytes(B, T, Hq, Hkv, D, block_size, block_tables.shape[1]))
         if workspace is None:
-            workspace = _workspace(q.device, need) if need else None
+            workspace = _workspace(q.device, need, stream) if need else None
         else:
             _need_device("workspace", workspace)
             _check(workspace.numel() * workspace.element_size() >= need, f"workspace needs {need} bytes")
@@ -344,7 +362,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
                             _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
                             block_tables.shape[1], num_blocks, float(scale), BF16, kv_code, _ptr(sinks), win,
-                            _ptr(workspace), ws_bytes, qt_ptr, _stream_ptr(q.device))
+                            _ptr(workspace), ws_bytes, qt_ptr, stream)
     _raise_on(rc, "pa_prefill")
     return out
 
@@ -380,7 +398,7 @@ def blocksparse_prefill(q, k, v, scale, *, block=64, local_blocks=4, vert_stride
     else:
         _need_device("out", out)
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = lib.pa_blocksparse_prefill(_ptr(q), _ptr(k), _ptr(v), _ptr(out), B, S, Hq, Hkv, D, block,
                                         int(local_blocks), int(vert_stride), float(scale), BF16,
                                         _stream_ptr(q.device))
@@ -402,7 +420,7 @@ def gather_kv(cache, block_tables, seq_lens, max_seq_len=None):
     msl = cap if max_seq_len is None else int(max_seq_len)
     _check(0 <= msl <= cap, f"max_seq_len {msl} outside [0, {cap}]")
     out = torch.empty((B, msl, Hkv, D), dtype=cache.dtype, device=cache.device)
-    with torch.cuda.device(cache.device):
+    with _on(cache.device):
         rc = lib.pa_gather_kv(_ptr(cache), _ptr(block_tables), _ptr(seq_lens), _ptr(out), B, Hkv, D,
                               block_size, block_tables.shape[1], num_blocks, msl, cache.element_size(),
                               _stream_ptr(cache.device))
@@ -451,7 +469,7 @@ def kv_write(k_new, v_new, k_cache, v_cache, block_tables, seq_lens, query_lens,
         _check(k_scale is None and v_scale is None, "k_scale / v_scale are for float8 pools only")
     _same_device(k_new, v_new=v_new, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables,
                  seq_lens=seq_lens, query_lens=query_lens, k_scale=k_scale, v_scale=v_scale)
-    with torch.cuda.device(k_new.device):
+    with _on(k_new.device):
         rc = lib.pa_kv_write(_ptr(k_new), _ptr(v_new), _ptr(k_cache), _ptr(v_cache),
                              _ptr(k_scale) if k_scale is not None else None,
                              _ptr(v_scale) if v_scale is not None else None,
@@ -535,7 +553,7 @@ def qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, 
     _same_device(xk, xq=xq, xv=xv, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
                  query_lens=query_lens, rope_cos=rope_cos, rope_sin=rope_sin, q_norm_weight=q_norm_weight,
                  k_norm_weight=k_norm_weight, k_scale=k_scale, v_scale=v_scale, out=out)
-    with torch.cuda.device(xk.device):
+    with _on(xk.device):
         rc = lib.pa_qk_norm_rope_kv_write(
             _ptr(xq), _ptr(xk), _ptr(xv), _ptr(out), _ptr(q_norm_weight), _ptr(k_norm_weight), ctypes.c_float(eps),
             _ptr(rope_cos), _ptr(rope_sin), rope_cos.shape[0], _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
