@@ -243,7 +243,8 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * workgroup packed over the q heads of a kv head, which is what short chunks get by default); key 4:
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
  * the same tile (1 = on, the default); key 5: query rows per wavefront of pa_verify (0 =
- * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never). */
+ * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never);
+ * key 7: query tokens from which pa_prefill at head dim 64 takes the tiled kernel (0 = the default, 65). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

@@ -42,6 +42,7 @@ static std::atomic<int> g_prefill_impl{0};
 static std::atomic<int> g_lockstep{1};
 static std::atomic<int> g_verify_rows{0};
 static std::atomic<int> g_prefill_split{1};
+static std::atomic<int> g_d64_tiled_from{PA_VERIFY_MAX_TOKENS + 1};   // query tokens from which head dim 64 takes the tiled kernel
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 static std::atomic<int> g_profile{0};
@@ -111,6 +112,7 @@ int pa_debug_set(int key, int value) {
   if (key == 4) { g_lockstep = value; return 0; }
   if (key == 5) { g_verify_rows = value; return 0; }
   if (key == 6) { g_prefill_split = value; return 0; }
+  if (key == 7) { g_d64_tiled_from = value > 0 ? value : PA_VERIFY_MAX_TOKENS + 1; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -423,7 +425,10 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   // head_dim 64: the tiled kernel takes bf16 pools with an even number of kv heads (two heads share its 256-byte
   // rows); short query runs and everything else go to the decode-shaped kernel, 64 query tokens per launch, each
   // launch reading the context up to its last token once per kv head
-  const bool tiled64 = D == 64 && T > PA_VERIFY_MAX_TOKENS && p.impl != 1 && prefill_async_supported(p);
+  // (measured crossover for runs of up to 64 tokens: 320 query rows per kv head in a batch of 8 or more)
+  const int from64 = g_d64_tiled_from.load();
+  const bool many_rows = from64 == PA_VERIFY_MAX_TOKENS + 1 && B >= 8 && (long)T * (Hq / Hkv) >= 320;
+  const bool tiled64 = D == 64 && (T >= from64 || many_rows) && p.impl != 1 && prefill_async_supported(p);
   if (!prefill_supported(p) && !tiled64) {
     if (D != 64) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);
     if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");

@@ -318,8 +318,13 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     if route is None:
         # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
         rows = T * (Hq // Hkv)
-        route = "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
-                                            or (kv_code == FP8 and (win > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"
+        if D == 64:
+            # the tiled kernel takes head dim 64 two kv heads at a time; below 320 rows per kv head, and for small
+            # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself)
+            route = "tiled" if not can_verify or (Hkv % 2 == 0 and B >= 8 and rows >= 320) else "verify"
+        else:
+            route = "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
+                                                or (kv_code == FP8 and (win > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")

@@ -237,3 +237,23 @@ def test_head_dim_64_tiled_split_matches_unsplit(pa):
     torch.cuda.synchronize()
     assert_close_abs(got, want, BF16_TOL)
     assert np.max(np.abs(got - unsplit)) <= 2 ** -6
+
+
+def test_head_dim_64_many_rows_of_a_short_run_take_the_tiled_kernel(pa):
+    """48 tokens x 8 q heads per kv head in a batch of 8: past the measured crossover the default route is the
+    tiled kernel; the verify kernel gives the same result."""
+    rng = np.random.default_rng(93)
+    T, Hq, Hkv, bs, D = 48, 16, 2, 32, 64
+    qlens = [48, 48, 7, 48, 0, 48, 33, 48]
+    prefixes = [100, 0, 900, 31, 5, 2000, 64, 333]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.125)
+    want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.125, q_dtype="bf16")
+    got = dev_to_f32(pa.prefill(*args))
+    via_verify = dev_to_f32(pa.prefill(*args, route="verify"))
+    torch.cuda.synchronize()
+    assert_close_abs(got, want, BF16_TOL)
+    assert_close_abs(via_verify, want, BF16_TOL)
+    assert not np.array_equal(got, via_verify)          # two kernels: different summation orders
+    for b, n in enumerate(qlens):
+        assert np.all(got[b, n:] == 0)
