@@ -261,7 +261,7 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
 # crossover against the tiled kernel (rows packed over the kv group, key tiles split over workgroups when
 # the grid is small) lies between 16 and 48 rows for batches of 1 to 64 sequences
 VERIFY_MAX_ROWS = 32
-VERIFY_MAX_ROWS_FP8 = 256     # fp8 pools: the tiled route is the slower register-staged kernel (B = 64: T = 64 774 vs 990 us)
+VERIFY_MAX_ROWS_FP8 = 256     # fp8 pools: the tiled kernel has no packed-rows form for them (B = 64, 4 K prefix: T = 64 718 vs 810 us)
 
 
 def verify_supported(T, D, block_size) -> bool:
