@@ -153,6 +153,24 @@ def main():
                win8_ctx=np.array(ctxs, np.int32), win8_scale=np.float32(sc), win8_window=np.int32(window),
                win8_sinks=sinks, win8_expected=exp)
 
+    # 8. a long chunk of the gpt-oss variant: bf16, D=64, 8 q heads on 2 kv heads, 100 query tokens (ragged)
+    #    behind cached prefixes, sliding window 50 and per-head sinks
+    B, T, Hq, Hkv, D, bs = 2, 100, 8, 2, 64, 16
+    qlens, prefixes, window = [100, 70], [30, 200], 50
+    ctxs = [p_ + n for p_, n in zip(prefixes, qlens)]
+    k, v, t = paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, T, Hq, D)).astype(np.float32)
+    sinks = O.bf16_bits_to_f32(O.f32_to_bf16_bits(rng.standard_normal(Hq).astype(np.float32) * 2))
+    qb, kb, vb = O.f32_to_bf16_bits(q), O.f32_to_bf16_bits(k), O.f32_to_bf16_bits(v)
+    qf, kf, vf = O.bf16_bits_to_f32(qb), O.bf16_bits_to_f32(kb), O.bf16_bits_to_f32(vb)
+    exp = np.zeros((B, T, Hq, D))
+    for b in range(B):
+        exp[b, :qlens[b]] = O.attention_bruteforce_f64(qf[b, :qlens[b]], rows(kf, t[b], ctxs[b], bs), rows(vf, t[b], ctxs[b], bs),
+                                                       sc6, prefix=prefixes[b], window=window, sinks=sinks)
+    out.update(long64_q=qb, long64_k=kb, long64_v=vb, long64_tables=t, long64_ctx=np.array(ctxs, np.int32),
+               long64_qlens=np.array(qlens, np.int32), long64_scale=np.float32(sc6), long64_window=np.int32(window),
+               long64_sinks=sinks.astype(np.float32), long64_expected=exp.astype(np.float32))   # float32: 2^-24 of the values, far below the bf16 bar
+
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "paged_attention_golden.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes")

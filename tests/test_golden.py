@@ -68,6 +68,12 @@ def _i32(x):
     return torch.from_numpy(np.asarray(x, np.int32)).cuda()
 
 
+def test_oracle_long_head_dim_64_chunk_golden():
+    got = O.paged_prefill(G["long64_q"], G["long64_k"], G["long64_v"], G["long64_tables"], G["long64_ctx"], G["long64_qlens"],
+                          float(G["long64_scale"]), sliding_window=int(G["long64_window"]), sinks=G["long64_sinks"])
+    _bf16_close(got, G["long64_expected"])
+
+
 @pytest.mark.gpu
 def test_hip_decode_fp32_golden():
     import nkipy_amd as pa
@@ -122,3 +128,22 @@ def test_hip_window_and_sinks_golden(route):
                      v_scale=torch.from_numpy(G["win8_vscale"]).cuda(), sliding_window=int(G["win8_window"]),
                      sinks=torch.from_numpy(G["win8_sinks"]).cuda()).float().cpu().numpy()
     assert np.max(np.abs(got8 - G["win8_expected"])) <= 5e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", ["tiled", "chunks"])
+def test_hip_long_head_dim_64_chunk_golden(path):
+    """100 query tokens at head dim 64: the tiled kernel's two-heads-per-row form, and the verify kernel's
+    64-token launches (tiled kernel switched off)."""
+    import nkipy_amd as pa
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    lib.pa_debug_set(3, 1 if path == "chunks" else 0)
+    try:
+        got = pa.prefill(_bf(G["long64_q"]), _bf(G["long64_k"]), _bf(G["long64_v"]), _i32(G["long64_tables"]),
+                         _i32(G["long64_ctx"]), _i32(G["long64_qlens"]), float(G["long64_scale"]),
+                         sliding_window=int(G["long64_window"]), sinks=torch.from_numpy(G["long64_sinks"]).cuda()).float().cpu().numpy()
+    finally:
+        lib.pa_debug_set(3, 0)
+    assert np.max(np.abs(got - G["long64_expected"])) <= 2e-2
+    assert np.all(got[1, 70:] == 0)
