@@ -13,6 +13,7 @@ from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_to_f32, make_pag
 pytestmark = pytest.mark.gpu
 
 N_CASES = int(os.environ.get("PA_SWEEP_CASES", "60"))      # more cases for an occasional longer soak of the same generator
+FIRST_CASE = int(os.environ.get("PA_SWEEP_FIRST", "0"))
 
 
 def _i32(x):
@@ -41,7 +42,7 @@ def _draw(case):
                 sinks=sinks, prefixes=prefixes, qlens=qlens)
 
 
-@pytest.mark.parametrize("case", range(N_CASES))
+@pytest.mark.parametrize("case", range(FIRST_CASE, FIRST_CASE + N_CASES))
 def test_random_case(case):
     import nkipy_amd as pa
     c = _draw(case)
@@ -88,6 +89,11 @@ def test_random_case(case):
                          sliding_window=c["window"], sinks=sinks_d, route=c["kind"], q_transform=qt, **kw_d)
     torch.cuda.synchronize()
     got = dev_to_f32(got)
+    # The absolute bar holds for outputs of the usual size (a softmax average of N(0,1) rows).  A window of one
+    # key hands a single V row through, and a rare row reaches |v| > 4, where one bf16 step is 2^-5: the device
+    # rounds the output once and the oracle its probabilities once, so allow 2^-7 of the largest output (case
+    # 4765 of this generator: 4.28 -> 0.031, reproduced by the device arithmetic written out in NumPy).
+    tol = max(tol, 2.0 ** -7 * float(np.abs(want).max()))
     assert_close_abs(got, want, tol)
     if c["kind"] != "decode":
         for b, n in enumerate(qlens):
