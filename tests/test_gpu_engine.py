@@ -196,3 +196,80 @@ def test_two_layers_share_tables(rng):
     with pytest.raises(ValueError):
         layers[0].attend(bf16_to_dev(_rand(rng, (S, 2, Hq, D))), bf16_to_dev(_rand(rng, (S, 2, Hkv, D))),
                          bf16_to_dev(_rand(rng, (S, 2, Hkv, D))))   # not the step begin_step opened
+
+
+@pytest.mark.parametrize("seed,variant", [(0, "qwen"), (1, "qwen"), (2, "gpt_oss"), (3, "gpt_oss")])
+def test_serving_loop_random_schedule(seed, variant):
+    """A random schedule of prompt chunks, verify-sized steps, decode steps, forks and releases over two
+    layers' worth of history (one layer computed), every step against the oracle's dense attention; the pool
+    is small enough that slots must be released to make room."""
+    from nkipy_amd.engine import OutOfBlocks, PagedAttention, PagedKVCache
+    rng = np.random.default_rng(500 + seed)
+    S, bs = 5, 16
+    if variant == "qwen":
+        Hq, Hkv, D, window, base, cap = 8, 2, 128, None, 1000000.0, 400
+    else:
+        Hq, Hkv, D, window, base, cap = 16, 2, 64, 40, 150000.0, 400
+    max_blocks = cap // bs
+    cache = PagedKVCache(num_blocks=70, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=max_blocks)
+    cos, sin = O.rope_tables(D, cap, base)
+    wq = O.round_to_bf16(1.0 + 0.1 * rng.standard_normal(D).astype(np.float32)) if variant == "qwen" else None
+    wk = O.round_to_bf16(1.0 + 0.1 * rng.standard_normal(D).astype(np.float32)) if variant == "qwen" else None
+    sinks = _rand(rng, Hq) if variant == "gpt_oss" else None
+    layer = PagedAttention(cache, Hq, rope_base=base, max_positions=cap,
+                           q_norm_weight=None if wq is None else bf16_to_dev(wq),
+                           k_norm_weight=None if wk is None else bf16_to_dev(wk), norm_eps=1e-6,
+                           sinks=None if sinks is None else bf16_to_dev(sinks), sliding_window=window)
+    mirror = _Mirror(S, cos, sin, wq, wk, 1e-6, window=window, sinks=sinks)
+    steps = 0
+    for it in range(70):
+        action = rng.choice(["prompt", "decode", "decode", "decode", "verify", "fork", "release"])
+        live = [s for s in range(S) if cache.lens[s] > 0]
+        idle = [s for s in range(S) if cache.lens[s] == 0]
+        if action == "fork" and live and idle:
+            src, dst = int(rng.choice(live)), int(rng.choice(idle))
+            try:
+                cache.fork(src, dst)
+            except OutOfBlocks:
+                continue
+            mirror.k[dst], mirror.v[dst] = mirror.k[src].copy(), mirror.v[src].copy()
+            continue
+        if action == "release" and live:
+            s = int(rng.choice(live))
+            cache.release(s)
+            mirror.k[s] = mirror.v[s] = None
+            continue
+        if action == "prompt":
+            T = int(rng.integers(5, 90))
+            qlens = [int(rng.integers(1, T + 1)) if (s in idle or rng.integers(0, 3) == 0) else 0 for s in range(S)]
+        elif action == "verify":
+            T = int(rng.integers(2, 6))
+            qlens = [int(rng.integers(1, T + 1)) if s in live else 0 for s in range(S)]
+        else:
+            T = 1
+            qlens = [1 if s in live else 0 for s in range(S)]
+        qlens = [n if cache.lens[s] + n <= cap else 0 for s, n in enumerate(qlens)]
+        if max(qlens) == 0:
+            continue
+        T = max(T, max(qlens))
+        xq, xk, xv = _rand(rng, (S, T, Hq, D)), _rand(rng, (S, T, Hkv, D)), _rand(rng, (S, T, Hkv, D))
+        try:
+            got = dev_to_f32(layer.step(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv), qlens))
+        except OutOfBlocks:
+            victim = max(range(S), key=lambda s: cache.lens[s])        # make room: drop the longest sequence
+            cache.release(victim)
+            mirror.k[victim] = mirror.v[victim] = None
+            continue
+        want = mirror.step(xq, xk, xv, qlens, layer.scale)
+        steps += 1
+        for b in range(S):
+            if qlens[b]:
+                assert_close_abs(got[b, :qlens[b]], want[b, :qlens[b]], 3e-2)
+    assert steps >= 25
+    # bookkeeping stays consistent: every block is free or owned, shared ones counted once per owner
+    owned = {}
+    for s in range(S):
+        for blk in cache.blocks[s]:
+            owned[blk] = owned.get(blk, 0) + 1
+    assert all(cache.allocator.refcount(blk) == n for blk, n in owned.items())
+    assert cache.allocator.num_free + len(owned) == 70
