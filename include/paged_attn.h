@@ -76,6 +76,15 @@ typedef struct pa_q_transform {
  * (q head, sequence + chunk) for the balanced MFMA schedule. */
 size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int partition_size);
 
+/* The same for a known shape and dtype pair: exactly what the kernel pa_decode picks for it
+ * needs (the balanced schedule's [Hq][B + chunks][D + 2] floats for bf16 / fp8 pools at head
+ * dim 64 or 128 and a power-of-two block size >= 16, whatever max_seq_len is; the fixed
+ * partitions' B x Hq x ceil(max_seq_len / partition_size) slots otherwise).  Never more than
+ * pa_decode_workspace_bytes.  Sizing helper next to the output allocation of
+ * nkipy/src/nkipy/runtime/device_tensor.py:51-74. */
+size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len,
+                                     int partition_size, int q_dtype, int kv_dtype);
+
 /*
  * Paged decode attention: one query token per sequence.
  *   out[b, h, :] = softmax(q[b, h, :] . K_b^T * scale) V_b,  K_b/V_b = the first

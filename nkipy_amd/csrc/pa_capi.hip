@@ -188,6 +188,31 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
   return fixed > balanced ? fixed : balanced;
 }
 
+// Which kernel pa_decode takes for a shape: 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced;
+// -1 when a forced kernel (debug switch 0) does not take the shape.
+static int decode_kind(const DecodeParams& p, int q_dtype, int kv_dtype) {
+  const int impl = g_decode_impl.load();
+  const bool mfma_ok = decode_mfma_supported(p, q_dtype, kv_dtype);
+  if ((impl == 2 || impl == 3) && !mfma_ok) return -1;
+  return !mfma_ok || impl == 1 ? 1 : (impl == 2 ? 2 : 3);
+}
+
+size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len,
+                                     int partition_size, int q_dtype, int kv_dtype) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0 || partition_size <= 0) return 0;
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = 1; p.rows_per_wave = 16;
+  p.block_size = block_size; p.block_shift = ilog2_exact(block_size);
+  const int kind = decode_kind(p, q_dtype, kv_dtype);
+  if (kind == 3) {
+    plan_decode_balanced(p, current_num_cus());
+    return decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
+  }
+  const int np = num_partitions_for(max_seq_len, partition_size);
+  return np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+}
+
 int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               const float* k_scale, const float* v_scale,
               const int32_t* block_tables, const int32_t* seq_lens,
@@ -231,11 +256,9 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   if (p.num_partitions > 65535 || B > 65535) return fail_arg("pa_decode: grid too large (partitions=%d B=%d)", p.num_partitions, B);
   hipStream_t s = (hipStream_t)stream;
   // kernel choice: 0 automatic, 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced
-  const int impl = g_decode_impl.load();
-  const bool mfma_ok = decode_mfma_supported(p, q_dtype, kv_dtype);
-  if ((impl == 2 || impl == 3) && !mfma_ok) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
-  if (impl == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
-  const int kind = !mfma_ok || impl == 1 ? 1 : (impl == 2 ? 2 : 3);
+  const int kind = decode_kind(p, q_dtype, kv_dtype);
+  if (kind < 0) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
+  if (kind == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
   if ((sinks || sliding_window > 0) && kind != 3)
     return fail_arg("pa_decode: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
                     "head_dim 64 or 128, block_size a power of two >= 16)");
@@ -557,6 +580,8 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
   if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_qk_norm_rope_kv_write: fp8 pools need k_scale and v_scale");
   if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache))
     return fail_arg("pa_qk_norm_rope_kv_write: xq, xk, xv, q_out, k_cache and v_cache must be 16-byte aligned");
+  if (!aligned16(rope_cos) || !aligned16(rope_sin) || !aligned16(q_norm_weight) || !aligned16(k_norm_weight))
+    return fail_arg("pa_qk_norm_rope_kv_write: rope_cos, rope_sin and the norm weights must be 16-byte aligned");
   KvWriteParams p;
   memset(&p, 0, sizeof(p));
   p.k_new = xk; p.v_new = xv; p.k_cache = k_cache; p.v_cache = v_cache;

@@ -76,7 +76,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillParams p) {
   int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
   tq = min(max(tq, 0), p.T);
   if (MODE != 0) ctx = min(ctx, p.max_blocks * p.block_size);
-  ctx = max(ctx, tq);
+  ctx = max(ctx, 0);
+  tq = min(tq, ctx);          // more query tokens than context: the first ctx of them count, without a prefix (as pa_verify)
   const int prefix = ctx - tq;
   const int q0 = qt * BM;
   uint16_t* out = (uint16_t*)p.out;

@@ -159,7 +159,8 @@ void prefill_async_kernel(PrefillParams p) {
   int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
   tq = min(max(tq, 0), p.T);
   if (MODE != 0) ctx = min(ctx, p.max_blocks * p.block_size);
-  ctx = max(ctx, tq);
+  ctx = max(ctx, 0);
+  tq = min(tq, ctx);          // more query tokens than context: the first ctx of them count, without a prefix (as pa_verify)
   const int prefix = ctx - tq;
   const int q0 = row_token(0);                                    // first query token of the workgroup
   uint16_t* out = (uint16_t*)p.out;
@@ -705,7 +706,8 @@ __global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams
   const int hq = (int)(row % p.Hq);
   const long bt = row / p.Hq;
   const int t = (int)(bt % p.T), b = (int)(bt / p.T);
-  const int tq = min(max(p.query_lens[b], 0), p.T);
+  const int ctx = max(min(p.seq_lens[b], p.max_blocks * p.block_size), 0);
+  const int tq = min(min(max(p.query_lens[b], 0), p.T), ctx);
   uint16_t* dst = (uint16_t*)p.out + row * D + 4 * q4;
   if (t >= tq) { *(uint2*)dst = make_uint2(0u, 0u); return; }
   float m = -INFINITY, l = 0.f;

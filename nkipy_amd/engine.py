@@ -245,6 +245,14 @@ class PagedAttention:
             self.rope = paged_attn.rope_tables(cache.head_dim, max_positions, rope_base, device=cache.device)
         elif q_norm_weight is not None or k_norm_weight is not None:
             raise ValueError("the fused pre-attention kernel applies the norm together with RoPE: give rope_base")
+        if self.rope is not None:
+            # the kernels clamp positions past the table to its last row: a table shorter than what the
+            # block tables can hold would silently rotate late tokens by the wrong angle
+            cap = cache.max_blocks_per_seq * cache.block_size
+            if self.rope[0].shape[0] < cap:
+                raise ValueError(f"RoPE tables cover {self.rope[0].shape[0]} positions, the cache holds sequences of up "
+                                 f"to {cap} tokens ({cache.max_blocks_per_seq} blocks of {cache.block_size}): give "
+                                 f"max_positions >= {cap}")
         self._out: Dict[int, torch.Tensor] = {}
 
     def step(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, query_lens: Sequence[int]) -> torch.Tensor:

@@ -132,12 +132,27 @@ def decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size) -> int:
     return int(_lib.load().pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size))
 
 
+_WORKSPACE_SLOTS = 16     # (device, stream) pairs whose workspace is kept; the least recently used goes first
+_retired = []             # buffers a captured graph may still write to: kept until the process ends
+
+
 def _workspace(device, nbytes, stream=None):
+    """Scratch for split-K partials, cached per (device, stream) so that calls on one stream reuse one
+    buffer and calls on different streams never share one.  The cache holds at most _WORKSPACE_SLOTS
+    entries (a server that cycles streams does not accumulate device memory); dropping an entry returns
+    its memory to torch's allocator, which reuses it in stream order.  While the stream is being
+    captured into a HIP graph a buffer that is too small is retired, not dropped: graphs captured
+    earlier on that stream have its address baked in.  Callers that replay graphs should pass a
+    `workspace=` of their own, sized with the *_workspace_bytes functions, and keep it alive."""
     key = (device, (stream or _stream_ptr(device)).value)
-    buf = _workspaces.get(key)
+    buf = _workspaces.pop(key, None)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None and buf.is_cuda and torch.cuda.is_current_stream_capturing():
+            _retired.append(buf)
         buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
-        _workspaces[key] = buf
+    _workspaces[key] = buf              # (re)inserted last: dict order is the LRU order
+    while len(_workspaces) > _WORKSPACE_SLOTS:
+        _workspaces.pop(next(iter(_workspaces)))
     return buf
 
 
@@ -239,7 +254,8 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
     else:
         _need_device("out", out)
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
-    need = int(lib.pa_decode_workspace_bytes(B, Hq, D, msl, partition_size))
+    with _on(q.device):
+        need = int(lib.pa_decode_workspace_bytes_for(B, Hq, Hkv, D, block_size, msl, partition_size, q_code, kv_code))
     stream = _stream_ptr(q.device)
     if workspace is None:
         workspace = _workspace(q.device, need, stream) if need else None

@@ -126,6 +126,17 @@ class KvWriteWorkload:
         return 2 * rows * hkv * d * (self.k_new.element_size() + self.k_cache.element_size()) + scales + 4 * touched + 8 * B
 
 
+def storage_bits(t: torch.Tensor) -> np.ndarray:
+    """Raw storage bits of a device tensor as a NumPy unsigned array (uint16 for bf16, uint8 for
+    fp8 codes, uint32 for float32): the form in which host-side checkers take device data."""
+    t = t.detach().contiguous().cpu()
+    if t.element_size() == 2:
+        return t.view(torch.int16).numpy().view(np.uint16)
+    if t.element_size() == 1:
+        return t.view(torch.uint8).numpy()
+    return t.view(torch.int32).numpy().view(np.uint32)
+
+
 def _randn(shape, dtype, gen, device, chunk=1 << 27):
     """N(0,1) drawn in float32 and rounded to `dtype`, in bounded chunks."""
     out = torch.empty(shape, dtype=dtype, device=device)

@@ -543,11 +543,13 @@ def blocksparse_block_mask(n_blocks: int, head: int, local_blocks: int, vert_str
 
 
 def blocksparse_prefill(q, k, v, scale, *, block=64, local_blocks=4, vert_stride=8,
-                        q_dtype="bf16", acc=np.float32, items=None) -> np.ndarray:
+                        q_dtype="bf16", acc=np.float32, items=None, head_ids=None) -> np.ndarray:
     """Block-sparse causal self-attention over dense q/k/v [B, S, H(kv), D].
 
     Equals dense attention under the block mask expanded to tokens, ANDed with
     token-level causality.  `items` = iterable of (b, h) to compute (default all).
+    `head_ids[h]` = the head number that sets head h's phase offset (default h itself):
+    lets a caller pass a slice of the heads of a larger tensor.
     """
     qf, kf, vf = to_f32(q), to_f32(k), to_f32(v)
     B, S, Hq, D = qf.shape
@@ -557,7 +559,7 @@ def blocksparse_prefill(q, k, v, scale, *, block=64, local_blocks=4, vert_stride
     out = np.zeros((B, S, Hq, D), dtype=np.float32)
     todo = [(b, h) for b in range(B) for h in range(Hq)] if items is None else list(items)
     for b, h in todo:
-        bm = blocksparse_block_mask(nb, h, local_blocks, vert_stride)
+        bm = blocksparse_block_mask(nb, h if head_ids is None else int(head_ids[h]), local_blocks, vert_stride)
         tok = np.repeat(np.repeat(bm, block, axis=0), block, axis=1)[:S, :S]
         hk = h // n_rep
         o = dense_attention(qf[b][:, h:h + 1], kf[b][:, hk:hk + 1], vf[b][:, hk:hk + 1],

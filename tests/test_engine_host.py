@@ -101,3 +101,34 @@ def test_begin_step_is_all_or_nothing_and_layers_share_tables():
         assert torch.all(c.k_caches[l][c.blocks[1][1]] == float(l + 1))
     with pytest.raises(ValueError):
         _cache(num_layers=0)
+
+
+def test_rope_table_must_cover_the_cache_capacity():
+    """Positions past the RoPE table are clamped by the kernels, so the layer refuses a table that is
+    shorter than the longest sequence the block tables can hold."""
+    import torch
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    cache = PagedKVCache(num_blocks=8, block_size=16, n_kv_heads=2, head_dim=64, max_seqs=2, max_blocks_per_seq=4,
+                         device="cpu")
+    short = (torch.zeros(63, 32, dtype=torch.bfloat16), torch.zeros(63, 32, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="max_positions >= 64"):
+        PagedAttention(cache, 4, rope_tables=short)
+    exact = (torch.zeros(64, 32, dtype=torch.bfloat16), torch.zeros(64, 32, dtype=torch.bfloat16))
+    PagedAttention(cache, 4, rope_tables=exact)
+
+
+def test_workspace_cache_is_bounded():
+    """The per-(device, stream) scratch cache keeps the most recently used entries only."""
+    import ctypes
+    import torch
+    from nkipy_amd import paged_attn
+    paged_attn._workspaces.clear()
+    dev = torch.device("cpu")
+    bufs = [paged_attn._workspace(dev, 64, ctypes.c_void_p(1000 + i)) for i in range(paged_attn._WORKSPACE_SLOTS + 5)]
+    assert len(paged_attn._workspaces) == paged_attn._WORKSPACE_SLOTS
+    assert (dev, 1000) not in paged_attn._workspaces and (dev, 1000 + len(bufs) - 1) in paged_attn._workspaces
+    again = paged_attn._workspace(dev, 32, ctypes.c_void_p(1000 + len(bufs) - 1))
+    assert again is bufs[-1]                                  # reused, not reallocated
+    bigger = paged_attn._workspace(dev, 4096, ctypes.c_void_p(1000 + len(bufs) - 1))
+    assert bigger.numel() >= 4096 and len(paged_attn._workspaces) == paged_attn._WORKSPACE_SLOTS
+    paged_attn._workspaces.clear()

@@ -76,6 +76,13 @@ def test_config1_fp32_exact_config(pa):
         torch.cuda.synchronize()
         assert_close_fp32(dev_to_f32(got), want, FP32_REL)
         assert_close_fp32(dev_to_f32(got), truth, FP32_REL)
+        # element-wise as well (the form of the reference's own comparisons, tests/utils.py:17-26):
+        # |got - truth| <= atol + rtol |truth| for every element, against the float64 result
+        g = dev_to_f32(got).astype(np.float64)
+        excess = np.abs(g - truth) - (1e-6 + 1e-5 * np.abs(truth))
+        worst = float((np.abs(g - truth) / np.maximum(np.abs(truth), 1e-30)).max())
+        print(f"config 1, partition {part}: max abs err {np.abs(g - truth).max():.3e}, max element-wise rel err {worst:.3e}")
+        assert excess.max() <= 0, f"element-wise rtol=1e-5, atol=1e-6 exceeded by {excess.max():.3e}"
 
 
 @pytest.mark.parametrize("D", [32, 64, 128, 256])

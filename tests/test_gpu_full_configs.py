@@ -43,7 +43,9 @@ def test_config5_full_size_sampled_sequences(pa):
     got = dev_to_f32(_decode(pa, w))
     assert np.isfinite(got).all()
     order = np.argsort(w.ctx)
-    sample = sorted({int(order[0]), int(order[-1]), int(order[len(order) // 2]), 3, 77})
+    # shortest, median and longest context, plus every 9th sequence: 18 of 128
+    sample = sorted({int(order[0]), int(order[-1]), int(order[len(order) // 2])} | set(range(3, 128, 9)))
+    assert len(sample) >= 16
     kc, vc = dev_bits(w.k_cache), dev_bits(w.v_cache)
     ks, vs = w.k_scale.cpu().numpy(), w.v_scale.cpu().numpy()
     tables = w.block_tables.cpu().numpy()
@@ -66,6 +68,8 @@ def test_config5_full_size_sampled_sequences(pa):
 
 
 def test_config3_full_size_sampled(pa):
+    """Every sequence, one q head of every kv group (the head's place in its group varies with the
+    sequence), against the oracle; the rest of the output through the hull property."""
     from nkipy_amd import workloads as W
     w = W.make_prefill()
     got = pa.prefill(w.q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens, w.scale,
@@ -73,20 +77,42 @@ def test_config3_full_size_sampled(pa):
     torch.cuda.synchronize()
     g = dev_to_f32(got)
     assert np.isfinite(g).all()
-    heads = [0, 13, 31]
-    want = O.paged_prefill(dev_bits(w.q), dev_bits(w.k_cache), dev_bits(w.v_cache), w.block_tables.cpu().numpy(),
-                           w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy(), w.scale, seqs=[0, 6], heads=heads)
-    for b in (0, 6):
+    qb, kb, vb = dev_bits(w.q), dev_bits(w.k_cache), dev_bits(w.v_cache)
+    tables, lens, qlens = w.block_tables.cpu().numpy(), w.seq_lens.cpu().numpy(), w.query_lens.cpu().numpy()
+    B, T, Hq, D = w.q.shape
+    n_rep = Hq // w.k_cache.shape[2]
+    for b in range(B):
+        heads = [hk * n_rep + (b + hk) % n_rep for hk in range(w.k_cache.shape[2])]     # 8 heads, one per kv group
+        want = O.paged_prefill(qb, kb, vb, tables, lens, qlens, w.scale, seqs=[b], heads=heads)
         assert_close_abs(g[b][:, heads], want[b][:, heads], 2e-2)
-    # sequences 0-3 alias the same prefix blocks: with identical new tokens and queries they
-    # must agree bit for bit; with their own (different) tokens they must not
-    assert not np.array_equal(dev_bits(got[0]), dev_bits(got[1]))
-    # first query row of a no-prefix sequence would equal V[0]; here check the property that
-    # holds for every row: output inside the hull of V
     assert np.abs(g).max() <= float(w.v_cache.float().abs().max()) + 1e-3
 
 
+def test_config3_aliased_prefix_blocks_give_identical_bits(pa):
+    """Sequences 0-3 of config 3 read their shared prefix through the same physical blocks.  Give
+    sequence 1 the queries and the new tokens' K/V of sequence 0 (copied into its own private
+    blocks): everything it attends to is then equal, part of it through aliased blocks and part
+    through its own, and its output must equal sequence 0's bit for bit, at full size."""
+    from nkipy_amd import workloads as W
+    w = W.make_prefill()
+    bs = w.k_cache.shape[1]
+    shared = int(w.prefix[0]) // bs
+    n0 = (int(w.prefix[0]) + w.q.shape[1] + bs - 1) // bs
+    assert int(w.prefix[0]) % bs == 0 and int(w.prefix[1]) == int(w.prefix[0]) and shared > 0
+    t0, t1 = w.block_tables[0, shared:n0].long(), w.block_tables[1, shared:n0].long()
+    assert torch.equal(w.block_tables[0, :shared], w.block_tables[1, :shared])        # aliased prefix
+    assert not bool((t0 == t1).any())                                                  # private tails
+    w.k_cache[t1] = w.k_cache[t0]
+    w.v_cache[t1] = w.v_cache[t0]
+    w.q[1] = w.q[0]
+    got = pa.prefill(w.q, w.k_cache, w.v_cache, w.block_tables, w.seq_lens, w.query_lens, w.scale)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(got[0]), dev_bits(got[1]))
+    assert not np.array_equal(dev_bits(got[0]), dev_bits(got[2]))      # sequence 2 kept its own tokens
+
+
 def test_config4_full_size_sampled(pa):
+    """Eight (batch, head) pairs, one for every phase offset h mod 8, both batches, against the oracle."""
     from nkipy_amd import workloads as W
     w = W.make_blocksparse()
     got = pa.blocksparse_prefill(w.q, w.k, w.v, w.scale, block=w.block, local_blocks=w.local_blocks,
@@ -94,11 +120,13 @@ def test_config4_full_size_sampled(pa):
     torch.cuda.synchronize()
     g = dev_to_f32(got)
     assert np.isfinite(g).all()
-    items = [(0, 0), (1, 13)]
-    want = O.blocksparse_prefill(dev_bits(w.q), dev_bits(w.k), dev_bits(w.v), w.scale, block=w.block,
-                                 local_blocks=w.local_blocks, vert_stride=w.vert_stride, items=items)
+    items = [(0, 0), (1, 9), (0, 18), (1, 27), (0, 4), (1, 13), (0, 22), (1, 31)]
+    assert sorted(h % 8 for _, h in items) == list(range(8))
     for b, h in items:
-        assert_close_abs(g[b][:, h], want[b][:, h], 2e-2)
+        sl = tuple(dev_bits(x[b:b + 1, :, h:h + 1].contiguous()) for x in (w.q, w.k, w.v))
+        want = O.blocksparse_prefill(*sl, w.scale, block=w.block, local_blocks=w.local_blocks,
+                                     vert_stride=w.vert_stride, head_ids=[h])[0, :, 0]
+        assert_close_abs(g[b][:, h], want, 2e-2)
     # the first 64 rows only see block 0: plain causal attention there, for every head
     first = O.blocksparse_prefill(dev_bits(w.q[:, :64]), dev_bits(w.k[:, :64]), dev_bits(w.v[:, :64]), w.scale,
                                   block=64, local_blocks=1, vert_stride=1)

@@ -171,3 +171,30 @@ def test_argument_validation(pa):
                     pool.view(torch.uint8)[..., :128].contiguous().view(torch.float8_e4m3fn), t, one, one)   # fp8 without scales
     with pytest.raises(NotImplementedError):
         pa.kv_write(z.cpu().float().numpy(), z, pool, pool, t, one, one)
+
+
+def test_device_kernel_alias_convention_writes_in_place(pa, rng):
+    """The write through the name-keyed call convention with the reference's aliasing names
+    (examples/models/qwen3/qwen3.py:289-301: "cache_k.must_alias_input" in, "cache_k" out, same
+    buffer) gives the bits of the direct call."""
+    from nkipy_amd.runtime import DeviceKernel, DeviceTensor
+    B, T, Hkv, D, bs = 3, 40, 2, 128, 32
+    nb, tables, seqs, qlens, xk, xv = _case(rng, B, T, Hkv, D, bs, seqs=[40, 97, 5], qlens=[40, 33, 0])
+    pk = rng.integers(0, 65536, size=(nb, bs, Hkv, D), dtype=np.uint16)
+    pv = rng.integers(0, 65536, size=(nb, bs, Hkv, D), dtype=np.uint16)
+    mk = lambda a: torch.from_numpy(a.view(np.int16).copy()).cuda().view(torch.bfloat16)  # noqa: E731
+    dk, dv, dk2, dv2 = mk(pk), mk(pv), mk(pk), mk(pv)
+    ins = dict(k_new=bf16_to_dev(xk), v_new=bf16_to_dev(xv), block_tables=_i32(tables), seq_lens=_i32(seqs),
+               query_lens=_i32(qlens))
+    pa.kv_write(ins["k_new"], ins["v_new"], dk, dv, ins["block_tables"], ins["seq_lens"], ins["query_lens"])
+    kern = DeviceKernel.compile_and_load(pa.kv_write, name="kv_write", k_cache=dk2, v_cache=dv2, **ins)
+    ret = kern(inputs={**{n: DeviceTensor(t) for n, t in ins.items()},
+                       "k_cache.must_alias_input": DeviceTensor(dk2), "v_cache.must_alias_input": DeviceTensor(dv2)},
+               outputs={"k_cache": DeviceTensor(dk2), "v_cache": DeviceTensor(dv2)})
+    torch.cuda.synchronize()
+    assert ret is None
+    assert np.array_equal(dev_bits(dk2), dev_bits(dk)) and np.array_equal(dev_bits(dv2), dev_bits(dv))
+    assert not np.array_equal(dev_bits(dk2), pk)            # something was written
+    with pytest.raises(AssertionError):                     # alias output must be the aliased input's buffer
+        kern(inputs={**ins, "k_cache.must_alias_input": dk2, "v_cache.must_alias_input": dv2},
+             outputs={"k_cache": dk, "v_cache": dv2})

@@ -401,3 +401,34 @@ def test_prefill_fp8_pool_split_over_key_tiles(pa):
             lib.pa_debug_set(6, 1)
         assert_close_abs(got, want, 5e-2)
         assert np.max(np.abs(got - unsplit)) <= 2 ** -6
+
+
+@pytest.mark.parametrize("T,impl", [(40, 0), (200, 0), (200, 1)])
+def test_query_lens_beyond_seq_lens_counts_the_first_rows(pa, T, impl):
+    """query_lens[b] > seq_lens[b] (a caller's slip): every kernel clamps the query length to the
+    context, so the first seq_lens[b] rows of q are the sequence's tokens, without a prefix, and the
+    other rows are padding -- the tiled kernels (asynchronous and register-staged) and the verify
+    kernel agree with each other and with the oracle on the clamped lengths."""
+    from nkipy_amd import _lib
+    rng = np.random.default_rng(40 + T)
+    B, Hq, Hkv, D, bs = 3, 8, 2, 128, 32
+    ctxs = [25, T + 30, 7]
+    qlens = [T, T, 9]                 # sequences 0 and 2 claim more query tokens than they have context
+    clamped = [min(a, c) for a, c in zip(qlens, ctxs)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, T, Hq, D)).astype(np.float32)
+    want = O.paged_prefill(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                           np.asarray(ctxs, np.int32), np.asarray(clamped, np.int32), 0.09)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), 0.09)
+    _lib.load().pa_debug_set(3, impl)
+    try:
+        tiled = pa.prefill(*args, route="tiled")
+        torch.cuda.synchronize()
+    finally:
+        _lib.load().pa_debug_set(3, 0)
+    assert_close_abs(dev_to_f32(tiled), want, BF16_TOL)
+    assert np.all(dev_to_f32(tiled)[0, 25:] == 0) and np.all(dev_to_f32(tiled)[2, 7:] == 0)
+    if T <= 64:
+        ver = pa.prefill(*args, route="verify")
+        torch.cuda.synchronize()
+        assert_close_abs(dev_to_f32(ver), want, BF16_TOL)

@@ -40,6 +40,14 @@ def test_version_and_workspace_formula(lib):
     assert lib.pa_decode_workspace_bytes(0, 32, 128, 512, 512) == 0
 
 
+def test_decode_workspace_for_shape(lib):
+    """The exact size query never exceeds the upper bound."""
+    upper = lib.pa_decode_workspace_bytes(64, 32, 128, 1 << 20, 512)
+    exact = lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 1, 1)     # bf16: balanced schedule
+    assert 0 < exact <= upper and exact < 64 << 20          # no term that grows with max_seq_len
+    assert lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 0, 0) == 64 * 32 * 2048 * 130 * 4   # fp32
+
+
 def test_c_abi_argument_errors_without_gpu(lib):
     """Argument errors are found on the host before anything touches a device."""
     z = ctypes.c_void_p(0)
@@ -171,3 +179,43 @@ def test_device_kernel_name_validation_without_gpu(lib):
         DeviceKernel.compile_and_load(print)
     with pytest.raises(NotImplementedError):      # host tensors: no CPU path behind the op
         k(inputs=good)
+
+
+def test_device_kernel_alias_names_without_gpu(lib):
+    """In-place state travels under the reference's aliasing names (trace.py:218-256,
+    tests/unit/test_alias.py:236-349): input "k_cache.must_alias_input", output "k_cache" bound to
+    the same buffer; the plain parameter name is not an input name of such a kernel."""
+    import nkipy_amd
+    from nkipy_amd.runtime import ALIAS_SUFFIX, DeviceKernel
+    assert ALIAS_SUFFIX == ".must_alias_input"
+    kn = torch.zeros(2, 3, 2, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16)
+    vc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 2, dtype=torch.int32)
+    sl = torch.full((2,), 3, dtype=torch.int32)
+    k = DeviceKernel.compile_and_load("kv_write", name="write", k_new=kn, v_new=kn, k_cache=kc, v_cache=vc,
+                                      block_tables=bt, seq_lens=sl, query_lens=sl)
+    assert k.output_names == ["k_cache", "v_cache"]          # no positional output: the op returns nothing
+    assert set(k.input_names) == {"k_new", "v_new", "k_cache.must_alias_input", "v_cache.must_alias_input",
+                                  "block_tables", "seq_lens", "query_lens"}
+    good = {"k_new": kn, "v_new": kn, "k_cache.must_alias_input": kc, "v_cache.must_alias_input": vc,
+            "block_tables": bt, "seq_lens": sl, "query_lens": sl}
+    with pytest.raises(ValueError):                           # the un-suffixed name is not an input
+        k(inputs={**{n: t for n, t in good.items() if n != "k_cache.must_alias_input"}, "k_cache": kc})
+    with pytest.raises(ValueError):
+        k(inputs=good, outputs={"output0": kc})
+    with pytest.raises(AssertionError):                       # alias output bound to another buffer
+        k(inputs=good, outputs={"k_cache": vc, "v_cache": vc})
+    with pytest.raises(NotImplementedError):                  # names and aliases fine; host tensors have no path
+        k(inputs=good, outputs={"k_cache": kc, "v_cache": vc})
+    # the fused pre-attention step returns the transformed q as output0 and aliases the pool
+    xq = torch.zeros(2, 3, 4, 128, dtype=torch.bfloat16)
+    cs = torch.zeros(8, 64, dtype=torch.bfloat16)
+    k2 = DeviceKernel.compile_and_load("qk_norm_rope_kv_write", xq=xq, xk=kn, xv=kn, k_cache=kc, v_cache=vc,
+                                       block_tables=bt, seq_lens=sl, query_lens=sl, rope_cos=cs, rope_sin=cs, eps=1e-6)
+    assert k2.output_names == ["output0", "k_cache", "v_cache"] and k2.static_kwargs == {"eps": 1e-6}
+    k3 = DeviceKernel.compile_and_load("qk_norm_rope_kv_write", xq=None, xk=kn, xv=kn, k_cache=kc, v_cache=vc,
+                                       block_tables=bt, seq_lens=sl, query_lens=sl, rope_cos=cs, rope_sin=cs)
+    assert k3.output_names == ["k_cache", "v_cache"]
+    with pytest.raises(ValueError):
+        DeviceKernel.compile_and_load("no_such_op")
