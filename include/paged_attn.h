@@ -119,6 +119,26 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
               const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream);
 
 /*
+ * pa_decode for callers that cannot allocate device memory or bring a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference (its runtime allocates every tensor up front, nkipy/src/nkipy/runtime/device_tensor.py:51-74).
+ * Arguments, validation, kernels and results are pa_decode's (bit for bit); the split-K partials go
+ * to a static array of PA_DECODE_NOALLOC_SCRATCH_BYTES inside the library's device code, one copy per
+ * GPU, held until the process ends.  A call whose partials need more (see
+ * pa_decode_workspace_bytes_for) fails with an argument error before any launch.  The call itself
+ * allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that overlap in
+ * time on one GPU (different streams, or threads) race; calls on one stream are ordered.
+ */
+#define PA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
+int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
+                      const float* k_scale, const float* v_scale,
+                      const int32_t* block_tables, const int32_t* seq_lens, void* out,
+                      int B, int Hq, int Hkv, int D, int block_size,
+                      int max_blocks_per_seq, int num_blocks, int max_seq_len,
+                      float scale, int partition_size, int q_dtype, int kv_dtype,
+                      const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream);
+
+/*
  * Speculative verify: a few query tokens per sequence against the paged context, causal among
  * themselves -- the non-prefill branch of examples/models/gpt_oss/kernels/attention.py:80-100,
  * 127-135 with seq_len = K+1 ("query at start_pos+i attends to keys <= start_pos+i"), driven by

@@ -33,6 +33,7 @@ SIGNATURES = {
     "pa_decode_workspace_bytes": (c_size_t, [c_int] * 5),
     "pa_decode_workspace_bytes_for": (c_size_t, [c_int] * 9),
     "pa_decode": (c_int, [c_void_p] * 9 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
+    "pa_decode_noalloc": (c_int, [c_void_p] * 8 + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "pa_verify_workspace_bytes": (c_size_t, [c_int] * 4),
     "pa_verify": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 8 + [c_float, c_int, c_void_p, c_int, c_void_p, c_void_p]),
     "pa_prefill_workspace_bytes": (c_size_t, [c_int] * 7),

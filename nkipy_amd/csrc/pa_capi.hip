@@ -300,6 +300,60 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   return 0;
 }
 
+// ---- pa_decode for callers that cannot allocate ------------------------------------------------
+// Split-K partials of pa_decode_noalloc live in this array instead of a caller's workspace.  Every
+// device the library runs on holds its own copy, at its own address, for the life of the process.
+static __device__ __align__(256) unsigned char scratch[PA_DECODE_NOALLOC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device, looked up once per device (in host code the
+// array's name is not a device address).  Returns nullptr with the error text set on failure.
+static void* noalloc_scratch_ptr() {
+  static std::mutex mu;
+  static void* ptrs[64] = {nullptr};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { check_hip(e, "pa_decode_noalloc: hipGetDevice"); return nullptr; }
+  if (dev < 0 || dev >= 64) { set_error("pa_decode_noalloc: device index %d outside [0, 64)", dev); return nullptr; }
+  std::lock_guard<std::mutex> lk(mu);
+  if (!ptrs[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      check_hip(e == hipSuccess ? hipErrorInvalidSymbol : e, "pa_decode_noalloc: hipGetSymbolAddress(scratch)");
+      return nullptr;
+    }
+    ptrs[dev] = ptr;
+  }
+  return ptrs[dev];
+}
+
+int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
+                      const float* k_scale, const float* v_scale,
+                      const int32_t* block_tables, const int32_t* seq_lens, void* out,
+                      int B, int Hq, int Hkv, int D, int block_size,
+                      int max_blocks_per_seq, int num_blocks, int max_seq_len,
+                      float scale, int partition_size, int q_dtype, int kv_dtype,
+                      const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream) {
+  tl_error[0] = 0;
+  if (B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && D > 0 && block_size > 0 && max_blocks_per_seq > 0 && partition_size > 0) {
+    const long cap = (long)max_blocks_per_seq * block_size;
+    int msl = max_seq_len;
+    if (msl <= 0 || msl > cap) msl = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
+    const size_t need = pa_decode_workspace_bytes_for(B, Hq, Hkv, D, block_size, msl, partition_size, q_dtype, kv_dtype);
+    if (need > (size_t)PA_DECODE_NOALLOC_SCRATCH_BYTES)
+      return fail_arg("pa_decode_noalloc: this call needs %zu bytes for its split-K partials, the library's static "
+                      "scratch holds %zu (PA_DECODE_NOALLOC_SCRATCH_BYTES); use pa_decode with a workspace of the caller's",
+                      need, (size_t)PA_DECODE_NOALLOC_SCRATCH_BYTES);
+  }
+  void* ws = noalloc_scratch_ptr();
+  if (!ws) return 1;
+  // same validation, kernels and launches as pa_decode; the partials are rewritten by every call before they are
+  // read, so nothing in the scratch has to start at zero
+  return pa_decode(q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, out, ws,
+                   (size_t)PA_DECODE_NOALLOC_SCRATCH_BYTES, B, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks,
+                   max_seq_len, scale, partition_size, q_dtype, kv_dtype, sinks, sliding_window, q_transform, stream);
+}
+
 // Query tokens [t0, t0 + Tc) of the T tokens per sequence through the decode-shaped kernel (pa_verify: all
 // of them in one launch; pa_prefill for shapes the tiled kernel does not take: 64 at a time).
 static int verify_launch(const char* who, const void* q, const void* k_cache, const void* v_cache,

@@ -40,12 +40,16 @@ def test_version_and_workspace_formula(lib):
     assert lib.pa_decode_workspace_bytes(0, 32, 128, 512, 512) == 0
 
 
-def test_decode_workspace_for_shape(lib):
-    """The exact size query never exceeds the upper bound."""
+def test_decode_workspace_for_shape_and_noalloc_limit(lib):
+    """The exact size query never exceeds the upper bound, and the entry point that uses the
+    library's static scratch refuses, on the host, a call whose partials do not fit it."""
     upper = lib.pa_decode_workspace_bytes(64, 32, 128, 1 << 20, 512)
     exact = lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 1, 1)     # bf16: balanced schedule
     assert 0 < exact <= upper and exact < 64 << 20          # no term that grows with max_seq_len
     assert lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 0, 0) == 64 * 32 * 2048 * 130 * 4   # fp32
+    z = ctypes.c_void_p(0)
+    rc = lib.pa_decode_noalloc(z, z, z, z, z, z, z, z, 8192, 64, 8, 128, 32, 4, 64, 0, 1.0, 512, 1, 1, z, 0, z, z)
+    assert rc == -1 and b"static" in lib.pa_last_error()
 
 
 def test_c_abi_argument_errors_without_gpu(lib):
