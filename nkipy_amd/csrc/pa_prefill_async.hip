@@ -313,12 +313,14 @@ void prefill_async_kernel(PrefillParams p) {
     for (int i = 0; i < 16; ++i) oacc[c][i] = 0.f;
   // Softmax state of this lane's query row.  Scores come out of the matrix cores already
   // relative to a reference m_ref (the accumulator starts at -m_ref), in log2 units.  The
-  // reference only follows the running maximum when a tile exceeds it by more than
-  // REF_SLACK, so in the steady state there is no per-element subtraction and no
-  // rescaling of the output accumulators; probabilities stay below 2^REF_SLACK.
+  // reference is set to the row maximum of the first tile in which the row sees a key and
+  // after that moves only when float range is at stake (see softmax below), so in the steady
+  // state there is no row maximum, no per-element subtraction and no rescaling of the output
+  // accumulators.  When it does move it goes to the tile's maximum.
   constexpr float REF_SLACK = 8.f;
   float m_ref = 0.f, l_run = 0.f;
   float slack = -INFINITY;            // -inf until the row has seen a finite score (m_ref is arbitrary till then)
+  bool fresh_rows = true;             // wave-uniform: some row of the wave still has slack == -inf
   f32x16_t cinit;                     // -m_ref in every accumulator slot
 #pragma unroll
   for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
@@ -507,6 +509,28 @@ void prefill_async_kernel(PrefillParams p) {
           sacc[tt][i] = key >= qlo ? sacc[tt][i] : -INFINITY;
         }
     }
+    // Steady state: every row of the wave has a reference already (slack is finite), the scores
+    // arrive relative to it, and nothing but a float overflow can go wrong with a reference that is
+    // too low: bf16 and float32 keep their relative precision whatever the magnitude.  So the
+    // probabilities are taken at once and the row maximum is never formed; only if a row's sum
+    // comes out beyond 2^OVF_LOG2 (or not a number) is the tile redone the careful way below.
+    constexpr float OVF_LIMIT = 0x1p+64f;
+    if (!fresh_rows) {
+      float psum = 0.f;
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(sacc[tt][i]);
+          const float p1 = __builtin_amdgcn_exp2f(sacc[tt][i + 1]);
+          psum += p0 + p1;
+          pw[tt][i >> 1] = pack_bf16x2(p0, p1);
+        }
+      if (__builtin_amdgcn_ballot_w64(!(psum < OVF_LIMIT)) == 0) {
+        l_run += psum;
+        return;
+      }
+    }
     float tmax = -INFINITY;
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt)
@@ -516,7 +540,8 @@ void prefill_async_kernel(PrefillParams p) {
       const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(tmax), __float_as_uint(tmax), false, false);
       tmax = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
     }
-    // move the reference only for the first finite tile of a row or a jump beyond the slack
+    // move the reference for the first finite tile of a row, or when a score lies more than the
+    // slack above it
     const bool move = tmax > slack;
     if (__builtin_amdgcn_ballot_w64(move) != 0) {
       const float shift = move ? tmax : 0.f;
@@ -544,6 +569,7 @@ void prefill_async_kernel(PrefillParams p) {
         pw[tt][i >> 1] = pack_bf16x2(p0, p1);
       }
     l_run += psum;
+    fresh_rows = __builtin_amdgcn_ballot_w64(slack == -INFINITY) != 0;
   };
   // ---- prologue: the first tile's copies, then Q, then the rest of the ring: the Q loads and
   // the first tile travel together instead of one memory latency after the other
