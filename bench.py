@@ -9,7 +9,8 @@ resident in HBM.  Prints ONE JSON line.  Without --config the line is config 2
 carries, under "configs", one record each for config 3 (paged chunked prefill),
 config 4 (blocksparse prefill) and config 5 (fp8-KV long-context decode), timed in
 the same run with the same protocol: both halves of the headline metric and every
-benchmark-sized configuration.  --config N prints that configuration alone.
+benchmark-sized configuration, plus "o_proj", the output projection behind config 3's
+attention.  --config N prints that configuration alone.
 
 value      whole-step throughput: algorithmic HBM bytes / step time for the decode
            configs (GB/s), attention FLOPs / step time for the prefill configs
@@ -389,6 +390,58 @@ def bench_blocksparse(steps, warmup, lib, pa, W):
     return res
 
 
+def bench_o_proj(steps, warmup, lib, pa, W, M=None):
+    """config 12: the output projection behind config 3's attention (examples/models/qwen3/kernels/
+    attention.py:143-147): out [B * T, hidden] = attention output [B * T, Hq * D] @ o_weight [Hq * D, hidden],
+    Llama-3-8B / Qwen3-8B sizes (32 heads of 128, hidden 4096), N(0,1) activations, N(0, 1/K) weights."""
+    from oracle import paged_attention_oracle as O
+    from nkipy_amd.workloads import storage_bits as dev_bits
+    B, T, Hq, D, N = 8, 2048, 32, 128, 4096
+    K = Hq * D
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1012)
+    x = torch.randn((B, T, Hq, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((K, N), generator=gen, device="cuda", dtype=torch.float32) / K ** 0.5).to(torch.bfloat16)
+    out = torch.empty((B, T, N), dtype=torch.bfloat16, device="cuda")
+
+    def step():
+        pa.o_proj(x, w, out=out)
+
+    sec = _time_steps(step, steps, warmup)
+    lib.pa_profile_enable(1)
+    _time_steps(step, steps, 0)
+    lib.pa_profile_enable(0)
+    kms = _collect_kernel_ms(lib, steps)
+    kavg = float(np.mean(kms))
+    fl = 2 * B * T * K * N
+    res = {
+        "metric": "post-attention output projection TFLOP/s (% MFMA peak)",
+        "value": round(fl / sec / 1e12, 2), "unit": "TFLOP/s",
+        "pct_of_bf16_peak": round(100.0 * fl / sec / 1e12 / BF16_PEAK_TFLOPS, 2),
+        "ms_per_step": round(sec * 1e3, 5), "dtype": "bf16, fp32 accumulate",
+        "config": {"workload": f"C12 o_proj behind config 3: tokens M={B * T} (B={B}, T={T}), K=Hq*D={K}, N=hidden={N}", "flops": fl},
+        "roofline": {"bound": "mfma", "achieved": round(fl / (kavg * 1e-3) / 1e12, 2), "peak": BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(fl / (kavg * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "o_proj_kernel", "kernel_avg_ms": round(kavg, 5), "launches_timed": len(kms),
+                     "mfma_only_loop_same_data": _mfma_ceiling(lib, x)},
+    }
+    res["cpu_baseline"] = res["parity"] = None
+    if not _NO_CPU:
+        rows = 512
+        torch.cuda.synchronize()
+        xh, wh = dev_bits(x.reshape(B * T, K)[:rows].contiguous()), dev_bits(w)
+        dt, want = _median3(lambda: O.o_proj(xh, wh))
+        res["cpu_baseline"] = {"value": round(2 * rows * K * N / dt / 1e12, 5), "unit": "TFLOP/s", "cores": _host_info(), "kind": "port",
+                               "sample": f"NumPy oracle (float32 matmul), first {rows} of {B * T} token rows of the same workload, "
+                                         f"1 warm-up + 3 runs, median {dt:.2f} s, numpy {np.__version__} default BLAS threading"}
+        got = out.reshape(B * T, N)[:rows].float().cpu().numpy()
+        err = np.abs(got.astype(np.float64) - want)
+        tol = 2.0 ** -7 * np.abs(want) + 1e-5 * float(np.abs(want).max())
+        res["parity"] = {"max_abs_err": round(float(err.max()), 6), "tol": "2^-7 |want| + 1e-5 max|want| per element (one bf16 step + float32 summation order)",
+                         "pass": bool(np.isfinite(got).all() and np.all(err <= tol))}
+    return res
+
+
 def bench_kv_write(steps, warmup, lib, pa, W):
     """Paged KV write with fp8 quantise-on-write (the step in front of the attention call).
     The kernel mutates the pool; every step rewrites the same rows with the same values, so the
@@ -536,7 +589,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11],
+    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     args = ap.parse_args()
@@ -574,6 +627,8 @@ def main():
             res = bench_prefill(args.steps, args.warmup, lib, pa, W, fp8=True)
         elif cfg == 11:
             res = bench_prefill(args.steps, args.warmup, lib, pa, W, gpt_oss=True)
+        elif cfg == 12:
+            res = bench_o_proj(args.steps, args.warmup, lib, pa, W)
         else:
             res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
         gc.collect()
@@ -593,10 +648,10 @@ def main():
         # headline metric (config 3), the blocksparse form (config 4) and the fp8-KV decode (config 5)
         line["metric"] = "decode attn HBM GB/s (% peak) + tok/s; prefill attn TFLOP/s (% MFMA peak)"
         subs = {}
-        for cfg in (3, 4, 5):
+        for cfg in (3, 4, 5, 12):
             r = run(cfg)
             r["steps"], r["warmup"] = args.steps, args.warmup
-            subs[f"C{cfg}"] = r
+            subs["o_proj" if cfg == 12 else f"C{cfg}"] = r
         line["configs"] = subs
         line["prefill_value"] = subs["C3"]["value"]
         line["prefill_unit"] = subs["C3"]["unit"]

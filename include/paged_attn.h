@@ -207,6 +207,22 @@ int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* ou
                            float scale, int dtype, void* stream);
 
 /*
+ * Post-attention output projection, the step behind the attention call:
+ *   out[m, :] = x[m, :] @ w (+ bias)
+ * `output_to_be_reduced = np.matmul(output, o_weight)` of examples/models/qwen3/kernels/attention.py:143-147
+ * and, with the bias, examples/models/gpt_oss/kernels/attention.py:155-163 (`+ o_bias`, which the
+ * reference adds on rank 0 only; the all-reduce behind it, attention.py:150-154, is the caller's).
+ *   x    [M, K] bf16: the attention output [B, T, Hq, D] (or [B, Hq, D]) viewed as [tokens, Hq * D],
+ *        padding rows included (they project to bias)
+ *   w    [K, N] bf16 row-major, i.e. o_proj.weight transposed as the reference stores it
+ *        (examples/models/qwen3/tensor_preparation.py:148-156); a tensor-parallel rank passes its K rows
+ *   bias [N] bf16 or NULL;  out [M, N] bf16
+ * Products and sums in float32 on the matrix cores, one rounding to bf16 on the way out.
+ * K a multiple of 64, N a multiple of 8; dtype PA_BF16.
+ */
+int pa_o_proj(const void* x, const void* w, const void* bias, void* out, int M, int K, int N, int dtype, void* stream);
+
+/*
  * Test hook: materialise the block-table gather.  out [B, max_seq_len, Hkv, D]
  * (elem_bytes per element, bits copied verbatim); rows >= seq_lens[b] are zero.
  * Bit-exact counterpart of np.take(pool, table, axis=0)
@@ -277,7 +293,7 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel
- * of pa_decode / pa_prefill / pa_blocksparse_prefill is bracketed by HIP events
+ * of pa_decode / pa_prefill / pa_blocksparse_prefill / pa_o_proj is bracketed by HIP events
  * on its own stream.  pa_profile_collect synchronises those events, writes up
  * to `cap` durations (milliseconds, oldest first) and clears the list; returns
  * the number written.  The counterpart of the reference's device-side timing,

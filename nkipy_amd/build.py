@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpaged_attn.so")
 
-SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip", "pa_prefill_async.hip", "pa_kv_write.hip", "pa_probe.hip"]
+SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip", "pa_prefill_async.hip", "pa_kv_write.hip", "pa_o_proj.hip", "pa_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -654,6 +654,28 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
   return check_hip(e, "pa_qk_norm_rope_kv_write launch");
 }
 
+int pa_o_proj(const void* x, const void* w, const void* bias, void* out, int M, int K, int N, int dtype, void* stream) {
+  tl_error[0] = 0;
+  if (M < 0 || K <= 0 || N <= 0) return fail_arg("pa_o_proj: bad sizes M=%d K=%d N=%d", M, K, N);
+  if (dtype != PA_BF16) return fail_arg("pa_o_proj: only bf16 is supported (dtype=%d)", dtype);
+  if (K % 64) return fail_arg("pa_o_proj: K=%d (Hq * head_dim) must be a multiple of 64", K);
+  if (N % 8) return fail_arg("pa_o_proj: N=%d must be a multiple of 8", N);
+  if (M == 0) return 0;
+  if ((long)N * 2 * 64 > 0xffffffffL || (long)K * 2 * 256 > 0xffffffffL)
+    return fail_arg("pa_o_proj: row of %d (K) or %d (N) elements too long for 32-bit tile offsets", K, N);
+  if (!x || !w || !out) return fail_arg("pa_o_proj: null pointer argument");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(out) || !aligned16(bias))
+    return fail_arg("pa_o_proj: x, w, bias and out must be 16-byte aligned");
+  OProjParams p;
+  memset(&p, 0, sizeof(p));
+  p.x = x; p.w = w; p.bias = bias; p.out = out; p.M = M; p.K = K; p.N = N;
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipError_t e = launch_o_proj(p, s);
+  profile_end(s);
+  return check_hip(e, "pa_o_proj launch");
+}
+
 int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,
                  void* out, int B, int Hkv, int D, int block_size,
                  int max_blocks_per_seq, int num_blocks, int max_seq_len,

@@ -249,6 +249,16 @@ struct KvWriteParams {
 hipError_t launch_kv_write(const KvWriteParams& p, hipStream_t s);
 bool kv_write_xform_supported(int D);   // head dims the fused RMSNorm + RoPE write is built for
 
+// ---- post-attention output projection ---------------------------------------------------
+struct OProjParams {
+  const void* x;            // [M, K] bf16: attention output, tokens x (Hq * D)
+  const void* w;            // [K, N] bf16, row-major
+  const void* bias;         // [N] bf16 or null
+  void* out;                // [M, N] bf16
+  int M, K, N;
+};
+hipError_t launch_o_proj(const OProjParams& p, hipStream_t s);
+
 // matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats
 hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s);
 hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,

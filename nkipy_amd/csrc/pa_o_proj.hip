@@ -1,0 +1,228 @@
+// Post-attention output projection on the gfx950 matrix cores:
+//   out[m, :] = x[m, :] @ w (+ bias),   x [M, K] = the attention output viewed as [tokens, Hq * D],
+//   w [K, N] row-major (the reference stores o_proj.weight transposed: examples/models/qwen3/
+//   tensor_preparation.py:148-156), bias [N] (examples/models/gpt_oss/kernels/attention.py:155-163).
+// Reference lines: examples/models/qwen3/kernels/attention.py:143-147.  bf16 in, float32 accumulate,
+// one rounding to bf16 on the way out.
+//
+// One workgroup of 8 wavefronts owns a 256 x 256 tile of out; wavefront (wm, wn) owns rows
+// 64 wm .. +63 and columns 128 wn .. +127 of it (two 32-row blocks x four 32-column chunks = eight
+// 32 x 32 accumulators).  K is walked in steps of 64.  The product is formed transposed,
+// out^T[n, m] += w^T[n, k] x^T[k, m] on v_mfma_f32_32x32x16_bf16: the A operand (w^T, 32 n x 16 k)
+// comes from the w tile, stored row-major [k][n] exactly as in memory, through the transposing LDS
+// read ds_read_b64_tr_b16; the B operand (x^T, 16 k x 32 m) is a plain 16-byte read of a row of the
+// x tile.  A lane's accumulator column is one row m of out, as in the attention kernels, so the
+// store path is theirs too.
+//
+// Both tiles travel HBM/L2 -> LDS with global_load_lds_dwordx4 (no registers) into a ring of two
+// 64 KB stages: the copies of k-step j + 1 are in flight while step j is multiplied.
+//   stage = x tile [256 m][128 B]  +  w tile, columns 0-127 [64 k][256 B]  +  w tile, columns 128-255
+// 16-byte chunk g of x row r sits at position g ^ (r & 7); chunk g of w row r at g ^ 4 (r & 3): the
+// reads of both kinds then spread over the banks (the copy lane fetches whatever chunk belongs in
+// its fixed LDS slot, so the swizzle costs nothing).
+#include <atomic>
+
+#include "pa_common.h"
+
+namespace pa {
+namespace {
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) char lds_char;
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int XT_B = BM * BK * 2;          // x tile bytes (32 KB)
+constexpr int WH_B = BK * 128 * 2;         // half a w tile: 64 k x 128 n (16 KB)
+constexpr int STAGE_B = XT_B + 2 * WH_B;   // 64 KB
+constexpr int LDS_B = 2 * STAGE_B;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// lane i's 16 bytes land at lds_base + 16 i; issued as inline assembly so that the waits are placed by hand
+__device__ __forceinline__ void dma16(const char* base, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+
+template <bool BIAS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void o_proj_kernel(OProjParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int wm = wave & 3, wn = wave >> 2;
+
+  // tile of this workgroup: consecutive workgroup ids go to consecutive XCDs; an XCD takes row tiles
+  // xcd, xcd + 8, ... and runs the column tiles of one row tile back to back, so that the x rows they
+  // share stay in that XCD's L2
+  const int MT = (p.M + BM - 1) / BM, NT = (p.N + BN - 1) / BN;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int mt = xcd + 8 * (slot / NT), nt = slot % NT;
+  if (mt >= MT) return;
+  const int m0 = mt * BM, n0 = nt * BN;
+
+  // ---- copy maps ---------------------------------------------------------------------------------
+  // x tile: 32 units of 1 KB = 8 rows x 128 B; lane i fills (row 8u + i/8, position i%8) with chunk
+  // (i%8) ^ (row & 7).  w half tile: 16 units of 4 rows x 256 B; lane i fills (row 4u + i/16, position
+  // i%16) with chunk (i%16) ^ 4 (row & 3).  Wave w issues x units w, w+8, w+16, w+24 and w units w,
+  // w+8 of both halves.  Rows past M and columns past N are clamped to the last valid ones (their
+  // products are never stored).
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
+  const long x_row_b = (long)p.K * 2, w_row_b = (long)p.N * 2;
+  uint32_t xoff[4], woff[2][2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = min(8 * (wave + 8 * j) + (lane >> 3), p.M - 1 - m0);
+    xoff[j] = (uint32_t)(r * x_row_b) + (uint32_t)(((lane & 7) ^ (lane >> 3)) << 4);
+  }
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = 4 * (wave + 8 * j) + (lane >> 4);
+      const int chunk = (lane & 15) ^ (4 * ((lane >> 4) & 3));
+      const int col = min(n0 + 128 * hf + 8 * chunk, p.N - 8);
+      woff[hf][j] = (uint32_t)(r * w_row_b) + (uint32_t)(col * 2);
+    }
+  const char* xbase = (const char*)p.x + (long)m0 * x_row_b;      // advanced by 128 B per k-step
+  const char* wbase = (const char*)p.w;                           // advanced by 64 rows per k-step
+  auto request = [&](int stage) __attribute__((always_inline)) {
+    const uint32_t sb = smem_base + stage * STAGE_B;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma16(xbase, xoff[j], sb + (wave + 8 * j) * 1024);
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) dma16(wbase, woff[hf][j], sb + XT_B + hf * WH_B + (wave + 8 * j) * 1024);
+    xbase += BK * 2;
+    wbase += (long)BK * w_row_b;
+  };
+
+  // ---- fragment read maps (lane constants) ---------------------------------------------------------
+  int x_off[4];                       // x^T fragment of k16-step s: row n of a 32-row block, chunk 2s + h
+#pragma unroll
+  for (int s = 0; s < 4; ++s) x_off[s] = (64 * wm + n) * 128 + (((2 * s + h) ^ (n & 7)) << 4);
+  // w^T fragment of 32-column chunk c.  ds_read_b64_tr_b16, per group of 16 lanes: lane i receives, for
+  // j = 0..3, the (i%4)-th 16-bit element of the 8 bytes addressed by lane (i/4) + 4j.  Source lane sl
+  // therefore points at k row (sl/4) of its half-wave's eight rows (8h .. 8h+3 for the first read, 4 rows
+  // further for the second: k-slot 8h + j of the operand is k row 8h + j, the same order as the x^T
+  // fragment) and at columns 4 (sl%4) .. +3 of the group's 16-column window.
+  int w_off[4];
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int row = 8 * h + (sl >> 2);
+    const int y = 2 * (g & 1) + ((sl & 3) >> 1);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) w_off[c] = XT_B + wn * WH_B + row * 256 + (((4 * c + y) ^ (4 * (row & 3))) << 4) + (sl & 1) * 8;
+  }
+
+  f32x16_t acc[2][4];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mb][c][i] = 0.f;
+
+  auto load_x = [&](bf16x8_t (&xf)[2], int stage, int s) __attribute__((always_inline)) {
+    const char* b = smem + stage * STAGE_B + x_off[s];
+    xf[0] = *(const bf16x8_t*)b;
+    xf[1] = *(const bf16x8_t*)(b + 32 * 128);
+  };
+  auto load_w = [&](bf16x8_t (&wf)[4], int stage, int s) __attribute__((always_inline)) {
+    const char* b = smem + stage * STAGE_B + 16 * s * 256;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const lds_char* src = (const lds_char*)(b + w_off[c]);
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 4 * 256));
+      struct { s16x4_t a, b; } pair = {lo, hi};
+      wf[c] = __builtin_bit_cast(bf16x8_t, pair);
+    }
+  };
+  auto mma = [&](const bf16x8_t (&wf)[4], const bf16x8_t (&xf)[2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        acc[mb][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[c], xf[mb], acc[mb][c], 0, 0, 0);
+  };
+
+  const int ktiles = p.K / BK;
+  request(0);
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int stage = kt & 1;
+    wait_vmcnt<0>();                       // this wave's part of step kt has landed
+    __builtin_amdgcn_s_barrier();          // ... and everyone's; all waves are done with step kt - 1
+    if (kt + 1 < ktiles) request(stage ^ 1);
+    bf16x8_t wa[4], wb[4], xa[2], xb[2];
+    load_w(wa, stage, 0); load_x(xa, stage, 0);
+    load_w(wb, stage, 1); load_x(xb, stage, 1);
+    mma(wa, xa);
+    load_w(wa, stage, 2); load_x(xa, stage, 2);
+    mma(wb, xb);
+    load_w(wb, stage, 3); load_x(xb, stage, 3);
+    mma(wa, xa);
+    mma(wb, xb);
+  }
+
+  // ---- bias, rounding, store: rows go out through a wave-private patch of the (now idle) ring so that
+  // they leave as whole 256-byte pieces, 16 bytes a lane --------------------------------------------------
+  __builtin_amdgcn_s_barrier();            // every wave is done reading the ring
+  uint16_t* out = (uint16_t*)p.out;
+  constexpr int PROW_B = 256 + 8;          // patch row pitch: the 8 bytes spread a column of rows over the banks
+  char* patch = smem + wave * (32 * PROW_B);
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int col = 32 * c + 8 * i4 + 4 * h;           // column inside the wave's 128
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (BIAS) {
+          const int gc = min(n0 + 128 * wn + col, p.N - 4);
+          const uint2 bw = *(const uint2*)((const uint16_t*)p.bias + gc);
+          b0 = bf16_bits_to_float(bw.x & 0xffffu); b1 = bf16_bits_to_float(bw.x >> 16);
+          b2 = bf16_bits_to_float(bw.y & 0xffffu); b3 = bf16_bits_to_float(bw.y >> 16);
+        }
+        const uint32_t w0 = pack_bf16x2(acc[mb][c][4 * i4] + b0, acc[mb][c][4 * i4 + 1] + b1);
+        const uint32_t w1 = pack_bf16x2(acc[mb][c][4 * i4 + 2] + b2, acc[mb][c][4 * i4 + 3] + b3);
+        *(uint2*)(patch + n * PROW_B + 2 * col) = make_uint2(w0, w1);
+      }
+    // the wave reads back what its own lanes wrote: no barrier, the compiler orders the LDS accesses
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int r = 4 * j + (lane >> 4), ch = lane & 15;
+      const uint2 lo = *(const uint2*)(patch + r * PROW_B + 16 * ch), hi = *(const uint2*)(patch + r * PROW_B + 16 * ch + 8);
+      const int m = m0 + 64 * wm + 32 * mb + r, col = n0 + 128 * wn + 8 * ch;
+      if (m < p.M && col < p.N) *(uint4*)(out + (long)m * p.N + col) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute((const void*)o_proj_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_B);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_B);
+    if (e != hipSuccess) return e;
+    configured.store(1, std::memory_order_release);
+  }
+  const long MT = (p.M + BM - 1) / BM, NT = (p.N + BN - 1) / BN;
+  const long total = 8 * ((MT + 7) / 8) * NT;
+  if (total > 0x7fffffffL) return hipErrorInvalidValue;
+  if (p.bias) hipLaunchKernelGGL(o_proj_kernel<true>, dim3((unsigned)total), dim3(512), LDS_B, s, p);
+  else hipLaunchKernelGGL(o_proj_kernel<false>, dim3((unsigned)total), dim3(512), LDS_B, s, p);
+  return hipGetLastError();
+}
+
+}  // namespace pa

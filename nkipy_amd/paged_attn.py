@@ -584,6 +584,47 @@ def qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, 
     return out
 
 
+def o_proj(x, o_weight, bias=None, *, out=None):
+    """Output projection behind the attention call: `np.matmul(output, o_weight)` (+ `o_bias`) of
+    examples/models/qwen3/kernels/attention.py:143-147 and examples/models/gpt_oss/kernels/attention.py:155-163.
+
+    x: the attention output, bfloat16, [..., Hq, D] (as `decode` / `prefill` return it) or already
+    [..., K]; o_weight [K, N] bfloat16 with K = Hq * D (the reference's transposed o_proj.weight; a
+    tensor-parallel rank passes its own K rows and all-reduces the result itself); bias [N]
+    bfloat16 or None.  Returns [..., N] bfloat16 (`out`, if given, is written in place).  Products
+    and sums are float32; the result is rounded to bfloat16 once.
+    """
+    lib = _lib.load()
+    for n, t in (("x", x), ("o_weight", o_weight)):
+        _need_device(n, t)
+    _check(x.dtype == torch.bfloat16 and o_weight.dtype == torch.bfloat16, "o_proj supports bfloat16 only")
+    _check(o_weight.dim() == 2, "o_weight must be [K, N]")
+    K, N = o_weight.shape
+    if x.dim() >= 2 and x.shape[-1] != K and x.shape[-1] * x.shape[-2] == K:
+        lead = tuple(x.shape[:-2])            # [..., Hq, D] -> [..., Hq * D]
+    else:
+        _check(x.dim() >= 1 and x.shape[-1] == K, f"x's last dimension(s) {tuple(x.shape[-2:])} do not give K={K}")
+        lead = tuple(x.shape[:-1])
+    M = 1
+    for d in lead:
+        M *= d
+    _check(K % 64 == 0, f"K={K} must be a multiple of 64")
+    _check(N % 8 == 0, f"N={N} must be a multiple of 8")
+    if bias is not None:
+        _need_device("bias", bias)
+        _check(bias.dtype == torch.bfloat16 and tuple(bias.shape) == (N,), "bias must be bfloat16 [N]")
+    _same_device(x, o_weight=o_weight, bias=bias, out=out)
+    if out is None:
+        out = torch.empty(lead + (N,), dtype=torch.bfloat16, device=x.device)
+    else:
+        _need_device("out", out)
+        _check(tuple(out.shape) == lead + (N,) and out.dtype == torch.bfloat16, f"out must be bfloat16 {lead + (N,)}")
+    with _on(x.device):
+        rc = lib.pa_o_proj(_ptr(x), _ptr(o_weight), _ptr(bias), _ptr(out), M, K, N, BF16, _stream_ptr(x.device))
+    _raise_on(rc, "pa_o_proj")
+    return out
+
+
 def default_scale(head_dim: int) -> float:
     """1 / sqrt(head_dim) in float32, as examples/models/qwen3/kernels/attention.py:119."""
     return float(np.float32(1.0) / np.float32(math.sqrt(head_dim)))

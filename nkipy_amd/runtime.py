@@ -25,7 +25,7 @@ import torch
 
 from . import _lib, paged_attn
 
-_TENSOR_PARAMS = {"q", "k_cache", "v_cache", "block_tables", "seq_lens", "query_lens", "k", "v",
+_TENSOR_PARAMS = {"x", "o_weight", "bias", "q", "k_cache", "v_cache", "block_tables", "seq_lens", "query_lens", "k", "v",
                   "k_scale", "v_scale", "k_new", "v_new", "xq", "xk", "xv", "rope_cos", "rope_sin",
                   "q_norm_weight", "k_norm_weight", "sinks"}
 ALIAS_SUFFIX = ".must_alias_input"      # nkipy/src/nkipy/core/trace.py:222
@@ -81,7 +81,8 @@ class DeviceKernel:
 
     _OPS = {"decode": paged_attn.decode, "prefill": paged_attn.prefill,
             "blocksparse_prefill": paged_attn.blocksparse_prefill,
-            "kv_write": paged_attn.kv_write, "qk_norm_rope_kv_write": paged_attn.qk_norm_rope_kv_write}
+            "kv_write": paged_attn.kv_write, "qk_norm_rope_kv_write": paged_attn.qk_norm_rope_kv_write,
+            "o_proj": paged_attn.o_proj}
 
     def __init__(self, fn, name, signature, static_kwargs):
         self.fn, self.name = fn, name
@@ -94,6 +95,12 @@ class DeviceKernel:
             self._result_like = None
         else:
             self._result_like = "xq" if fn is paged_attn.qk_norm_rope_kv_write else "q"
+        # shape and dtype of "output0"
+        self._result_sig = self.signature.get(self._result_like) if self._result_like else None
+        if fn is paged_attn.o_proj and "x" in signature and "o_weight" in signature:
+            (xs, xd), (ws, _) = signature["x"], signature["o_weight"]
+            lead = xs[:-1] if xs[-1] == ws[0] else xs[:-2]          # x is [..., K] or [..., Hq, D]
+            self._result_like, self._result_sig = "x", (tuple(lead) + (ws[1],), xd)
         self.output_names = (["output0"] if self._result_like else []) + list(self.aliased)
         # names the caller uses for inputs: mutated parameters carry the alias suffix
         self.input_names = {(k + ALIAS_SUFFIX if k in self.aliased else k): k for k in signature}
@@ -153,9 +160,9 @@ class DeviceKernel:
             if "output0" in outputs:
                 o = outputs["output0"]
                 out = o.tensor if isinstance(o, DeviceTensor) else o
-                qshape, qdtype = self.signature[self._result_like]
+                qshape, qdtype = self._result_sig
                 assert tuple(out.shape) == qshape and out.dtype == qdtype, \
-                    f"output0 must match {self._result_like} in shape and dtype"
+                    f"output0 must be {qdtype} {qshape}"
         if self._result_like is None:
             self.fn(**args, **self.static_kwargs)
             res = None

@@ -127,6 +127,13 @@ def k_norm_rope_kv_write_fp8(xk: torch.Tensor, xv: torch.Tensor, k_cache: torch.
                                      rope_sin, k_norm_weight=k_norm_weight, eps=eps, k_scale=k_scale, v_scale=v_scale)
 
 
+# the projection behind the attention call (examples/models/qwen3/kernels/attention.py:143-147; with the bias
+# examples/models/gpt_oss/kernels/attention.py:155-163); the tensor-parallel all-reduce stays with the caller
+@torch.library.custom_op(f"{_NS}::o_proj", mutates_args=("out",), device_types="cuda")
+def o_proj(x: torch.Tensor, o_weight: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
+    paged_attn.o_proj(x, o_weight, bias, out=out)
+
+
 def _no_cpu(name):
     def impl(*args, **kwargs):
         raise NotImplementedError(f"{_NS}::{name} runs hand-written HIP kernels and has no CPU path; "
@@ -138,9 +145,10 @@ for _op, _name in ((paged_decode, "paged_decode"), (paged_prefill, "paged_prefil
                    (blocksparse_prefill, "blocksparse_prefill"), (paged_kv_write, "paged_kv_write"),
                    (paged_kv_write_fp8, "paged_kv_write_fp8"), (qk_norm_rope_kv_write, "qk_norm_rope_kv_write"),
                    (qk_norm_rope_kv_write_fp8, "qk_norm_rope_kv_write_fp8"),
-                   (k_norm_rope_kv_write, "k_norm_rope_kv_write"), (k_norm_rope_kv_write_fp8, "k_norm_rope_kv_write_fp8")):
+                   (k_norm_rope_kv_write, "k_norm_rope_kv_write"), (k_norm_rope_kv_write_fp8, "k_norm_rope_kv_write_fp8"),
+                   (o_proj, "o_proj")):
     _op.register_kernel("cpu")(_no_cpu(_name))
     _op.register_fake(lambda *args, **kwargs: None)      # outputs are caller-allocated: nothing to infer
 
 OPS = ("paged_decode", "paged_prefill", "blocksparse_prefill", "paged_kv_write", "paged_kv_write_fp8",
-       "qk_norm_rope_kv_write", "qk_norm_rope_kv_write_fp8", "k_norm_rope_kv_write", "k_norm_rope_kv_write_fp8")
+       "qk_norm_rope_kv_write", "qk_norm_rope_kv_write_fp8", "k_norm_rope_kv_write", "k_norm_rope_kv_write_fp8", "o_proj")

@@ -27,6 +27,9 @@ in the one-dynamic-index `np.take` form the reference's tracer supports:
 * QK RMSNorm + RoPE     examples/models/qwen3/kernels/rmsnorm.py:4-21, rope.py:4-48 and
                         their call sites attention.py:78-97 (bf16 tensors: every
                         RoPE product and sum is rounded to bf16, the norm is float32)
+* output projection     examples/models/qwen3/kernels/attention.py:143-147 (`np.matmul(output,
+                        o_weight)` on the BSHD output reshaped to (B, S, H*D)) and, with the
+                        bias, examples/models/gpt_oss/kernels/attention.py:155-163
 * cache update          examples/models/gpt_oss/kernels/attention.py:92-100
                         (`cache_k[:, query_pos] = xk`, query_pos = start_pos +
                         arange(seq_len)), examples/models/qwen3/kernels/attention.py:100-106
@@ -55,6 +58,9 @@ sliding window, sinks  float64 brute force; W >= context == no window; W = 1 ==
 merge_partitions       split-K merge == single pass in float64 for any split
 blocksparse_prefill    == dense attention under the expanded boolean mask;
                        all-active pattern == dense causal
+o_proj                 torch.matmul on CPU (an independent library); float64 row-by-row
+                       dot products on tiny inputs; identity weight returns the input;
+                       linearity in x; the bias shifts every row alike
 rope_tables / rmsnorm / apply_rope   closed forms (position 0 is the identity,
                        rotation preserves the pair norm, angle addition), float64
                        restatement, torch.nn.functional.rms_norm on CPU
@@ -566,6 +572,28 @@ def blocksparse_prefill(q, k, v, scale, *, block=64, local_blocks=4, vert_stride
                             scale, prefix=0, mask=tok[None], acc=acc)
         out[b][:, h:h + 1] = o
     return round_output(out, q_dtype)
+
+
+def o_proj(x, o_weight, bias=None, *, acc=np.float32) -> np.ndarray:
+    """Output projection behind attention: examples/models/qwen3/kernels/attention.py:143-147
+    (`output.reshape(batch, seq, -1)` then `np.matmul(output, o_weight)`), with `+ o_bias` as
+    examples/models/gpt_oss/kernels/attention.py:155-163 adds it (on one rank).
+
+    x [..., Hq, D] or [..., K] (float32 values or uint16 bf16 bits), o_weight [K, N], bias [N] or
+    None.  Products and sums in `acc`, bias added before the single rounding to bf16.  The
+    reference rounds the matmul result to bf16 before it adds the bias; that extra rounding (at most
+    one bf16 step of the result) is not reproduced, like its rounding of the score matrix.
+    Returns [..., N] float32 holding bf16-representable values.
+    """
+    xf, wf = to_f32(x), to_f32(o_weight)
+    K, N = wf.shape
+    if xf.shape[-1] != K:
+        assert xf.ndim >= 2 and xf.shape[-1] * xf.shape[-2] == K, (xf.shape, wf.shape)
+        xf = xf.reshape(xf.shape[:-2] + (K,))
+    y = np.matmul(xf.astype(acc), wf.astype(acc))
+    if bias is not None:
+        y = y + to_f32(bias).astype(acc)
+    return round_to_bf16(y.astype(np.float32))
 
 
 # ---------------------------------------------------------------------------

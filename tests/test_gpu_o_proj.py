@@ -1,0 +1,99 @@
+"""GPU parity: HIP output projection (through the C ABI) vs the NumPy oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_attention_oracle as O
+from tests.pa_testlib import bf16_to_dev, dev_bits, dev_to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pa():
+    import nkipy_amd
+    from nkipy_amd import _lib
+    _lib.load()
+    return nkipy_amd
+
+
+def _close(got, want):
+    """bf16 output of a float32-accumulated dot product: one bf16 step of the result (2^-8 relative)
+    plus the float32 summation-order term, which scales with the size of the terms, not of the sum."""
+    scale = float(np.abs(want).max()) if want.size else 0.0
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bar = 2.0 ** -7 * np.abs(want) + 1e-5 * scale + 1e-6
+    assert np.isfinite(got).all()
+    assert np.all(err <= bar), f"max excess {(err - bar).max():.3e} at scale {scale:.3e}"
+
+
+@pytest.mark.parametrize("M,K,N,bias", [(1, 64, 8, False), (37, 128, 72, True), (256, 4096, 256, False),
+                                        (300, 512, 2880, True), (513, 1024, 520, True), (64, 4096, 4096, False)])
+def test_o_proj_vs_oracle(pa, M, K, N, bias):
+    rng = np.random.default_rng(M + K + N)
+    x = O.round_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = O.round_to_bf16((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32))
+    b = O.round_to_bf16(rng.standard_normal(N).astype(np.float32)) if bias else None
+    want = O.o_proj(x, w, b)
+    print(f"o_proj M={M} K={K} N={N} bias={bias}", flush=True)
+    got = pa.o_proj(bf16_to_dev(x), bf16_to_dev(w), None if b is None else bf16_to_dev(b))
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (M, N)
+    _close(dev_to_f32(got), want)
+
+
+def test_identity_and_permutation_weights_move_bits(pa, rng):
+    """Exact cases: an identity weight returns x bit for bit (which also pins the [.., Hq, D] -> [.., Hq*D]
+    view), a column permutation permutes it, a zero x returns the bias in every row."""
+    B, T, Hq, D = 2, 70, 4, 64
+    K = Hq * D
+    x = bf16_to_dev(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    eye = torch.eye(K, dtype=torch.bfloat16, device="cuda")
+    got = pa.o_proj(x, eye)
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (B, T, K)
+    assert np.array_equal(dev_bits(got), dev_bits(x).reshape(B, T, K))
+    perm = torch.randperm(K, device="cuda")
+    got_p = pa.o_proj(x, eye[:, perm].contiguous())          # out[:, n] = x[:, perm[n]]
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(got_p), dev_bits(x).reshape(B, T, K)[..., perm.cpu().numpy()])
+    b = bf16_to_dev(rng.standard_normal(K).astype(np.float32))
+    got_b = pa.o_proj(torch.zeros_like(x), eye, b)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(got_b), np.broadcast_to(dev_bits(b), (B, T, K)))
+
+
+def test_fed_by_the_attention_output_and_preallocated_out(pa, rng):
+    """decode -> o_proj on the device equals the oracle's decode -> o_proj; `out=` is written in place."""
+    from tests.pa_testlib import make_paged
+    B, Hq, Hkv, D, bs, N = 5, 8, 2, 128, 32, 264
+    ctxs = [3, 200, 64, 900, 33]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    w = O.round_to_bf16((rng.standard_normal((Hq * D, N)) / np.sqrt(Hq * D)).astype(np.float32))
+    i32 = lambda a: torch.from_numpy(np.asarray(a, np.int32)).cuda()  # noqa: E731
+    att = pa.decode(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), i32(tables), i32(ctxs), 0.09)
+    out = torch.empty((B, N), dtype=torch.bfloat16, device="cuda")
+    ret = pa.o_proj(att, bf16_to_dev(w), out=out)
+    torch.cuda.synchronize()
+    assert ret is out
+    want = O.o_proj(dev_bits(att), w)                      # the projection of the device's own attention bits
+    _close(dev_to_f32(out), want)
+    want_all = O.o_proj(O.paged_decode(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables,
+                                       np.asarray(ctxs, np.int32), 0.09, q_dtype="bf16"), w)
+    assert np.abs(dev_to_f32(out) - want_all).max() <= 2e-2
+
+
+def test_argument_errors(pa):
+    x = torch.zeros(4, 96, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        pa.o_proj(x, torch.zeros(96, 64, dtype=torch.bfloat16, device="cuda"))        # K not a multiple of 64
+    x = torch.zeros(4, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        pa.o_proj(x, torch.zeros(128, 20, dtype=torch.bfloat16, device="cuda"))       # N not a multiple of 8
+    with pytest.raises(ValueError):
+        pa.o_proj(x, torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"))        # K mismatch
+    with pytest.raises(ValueError):
+        pa.o_proj(x.float(), torch.zeros(128, 64, dtype=torch.float32, device="cuda"))
+    with pytest.raises(NotImplementedError):
+        pa.o_proj(np.zeros((4, 128), np.float32), np.zeros((128, 64), np.float32))

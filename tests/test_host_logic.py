@@ -223,3 +223,23 @@ def test_device_kernel_alias_names_without_gpu(lib):
     assert k3.output_names == ["k_cache", "v_cache"]
     with pytest.raises(ValueError):
         DeviceKernel.compile_and_load("no_such_op")
+
+
+def test_device_kernel_o_proj_signature_without_gpu(lib):
+    """The projection's positional output has its own shape, [..., N], checked like any other."""
+    import nkipy_amd
+    from nkipy_amd.runtime import DeviceKernel
+    x = torch.zeros(2, 3, 4, 32, dtype=torch.bfloat16)
+    w = torch.zeros(128, 48, dtype=torch.bfloat16)
+    k = DeviceKernel.compile_and_load(nkipy_amd.o_proj, x=x, o_weight=w)
+    assert k.output_names == ["output0"] and k._result_sig == ((2, 3, 48), torch.bfloat16)
+    with pytest.raises(AssertionError):
+        k(inputs={"x": x, "o_weight": w}, outputs={"output0": torch.zeros(2, 3, 128, dtype=torch.bfloat16)})
+    with pytest.raises(NotImplementedError):
+        k(inputs={"x": x, "o_weight": w}, outputs={"output0": torch.zeros(2, 3, 48, dtype=torch.bfloat16)})
+    z = ctypes.c_void_p(0)
+    assert lib.pa_o_proj(z, z, z, z, 4, 96, 64, 1, z) == -1 and b"multiple of 64" in lib.pa_last_error()
+    assert lib.pa_o_proj(z, z, z, z, 4, 128, 20, 1, z) == -1 and b"multiple of 8" in lib.pa_last_error()
+    assert lib.pa_o_proj(z, z, z, z, 4, 128, 64, 0, z) == -1 and b"bf16" in lib.pa_last_error()
+    assert lib.pa_o_proj(z, z, z, z, 0, 128, 64, 1, z) == 0
+    assert lib.pa_o_proj(z, z, z, z, 4, 128, 64, 1, z) == -1 and b"null" in lib.pa_last_error()
