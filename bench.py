@@ -36,6 +36,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 _NO_CPU = False
+_CONST_DATA = False         # --const-data: every Q / K / V element the same value (a power probe, see main)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
@@ -268,6 +269,9 @@ def bench_prefill(steps, warmup, lib, pa, W, fp8=False, gpt_oss=False):
     w = W.make_prefill(heads=(64, 8), head_dim=64, name="C3 tokens, gpt-oss heads") if gpt_oss else W.make_prefill()
     sinks = torch.linspace(-1.0, 1.0, w.q.shape[2], device="cuda") if gpt_oss else None
     out = torch.empty_like(w.q)
+    if _CONST_DATA:
+        for t in (w.q, w.k_cache, w.v_cache):
+            t.fill_(0.011)
     kc, vc, ks, vs = w.k_cache, w.v_cache, None, None
     if fp8:
         kc, ks = W.quantize_pool_fp8(w.k_cache)
@@ -592,6 +596,10 @@ def main():
     ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
+    ap.add_argument("--const-data", action="store_true",
+                    help="prefill configs 3 / 9 / 11: every Q, K and V element is the same value instead of N(0,1).  Same "
+                         "kernel, same instruction stream, far fewer bit flips in the matrix cores' operands: the time "
+                         "difference to the normal run is what the chip's power limit costs on random data")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is measured on ONE GPU (the kernel on one GPU's share at its real "
@@ -609,6 +617,9 @@ def main():
     if args.no_cpu:
         global _NO_CPU
         _NO_CPU = True
+    if args.const_data:
+        global _CONST_DATA
+        _CONST_DATA = True
 
     def run(cfg):
         if cfg in (2, 5):
@@ -658,6 +669,8 @@ def main():
         line["prefill_roofline_frac"] = subs["C3"]["roofline"]["frac"]
         par = [line.get("parity")] + [r.get("parity") for r in subs.values()]
         line["parity_all_pass"] = None if any(x is None for x in par) else all(x["pass"] for x in par)
+    if args.const_data:
+        line["data"] = "synthetic CONSTANT operands (power probe: not a benchmark result)"
     line["device"] = torch.cuda.get_device_name(0)
     line["bench_wall_s"] = round(time.perf_counter() - t_start, 1)
     print(json.dumps(line))

@@ -58,13 +58,16 @@ void o_proj_kernel(OProjParams p) {
   const int n = lane & 31, h = lane >> 5;
   const int wm = wave & 3, wn = wave >> 2;
 
-  // tile of this workgroup: consecutive workgroup ids go to consecutive XCDs; an XCD takes row tiles
-  // xcd, xcd + 8, ... and runs the column tiles of one row tile back to back, so that the x rows they
-  // share stay in that XCD's L2
+  // tile of this workgroup: consecutive workgroup ids go to consecutive XCDs; an XCD owns row tiles xcd,
+  // xcd + 8, ... and walks its tiles in groups of (all its row tiles) x (4 column tiles), so that the
+  // workgroups resident on it at one time (32 on MI355X) share x slabs four ways and w slabs eight ways
+  // through that XCD's L2 instead of streaming all of w once per pair of row tiles
   const int MT = (p.M + BM - 1) / BM, NT = (p.N + BN - 1) / BN;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int mt = xcd + 8 * (slot / NT), nt = slot % NT;
-  if (mt >= MT) return;
+  const int mtx = (MT + 7) / 8;                       // row tiles per XCD (the last ones may not exist)
+  const int grp = slot / (4 * mtx), rem = slot % (4 * mtx);
+  const int mt = xcd + 8 * (rem >> 2), nt = 4 * grp + (rem & 3);
+  if (mt >= MT || nt >= NT) return;
   const int m0 = mt * BM, n0 = nt * BN;
 
   // ---- copy maps ---------------------------------------------------------------------------------
@@ -218,7 +221,7 @@ hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
     configured.store(1, std::memory_order_release);
   }
   const long MT = (p.M + BM - 1) / BM, NT = (p.N + BN - 1) / BN;
-  const long total = 8 * ((MT + 7) / 8) * NT;
+  const long total = 8 * ((MT + 7) / 8) * 4 * ((NT + 3) / 4);
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
   if (p.bias) hipLaunchKernelGGL(o_proj_kernel<true>, dim3((unsigned)total), dim3(512), LDS_B, s, p);
   else hipLaunchKernelGGL(o_proj_kernel<false>, dim3((unsigned)total), dim3(512), LDS_B, s, p);
