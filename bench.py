@@ -407,6 +407,9 @@ def bench_o_proj(steps, warmup, lib, pa, W, M=None):
     x = torch.randn((B, T, Hq, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
     w = (torch.randn((K, N), generator=gen, device="cuda", dtype=torch.float32) / K ** 0.5).to(torch.bfloat16)
     out = torch.empty((B, T, N), dtype=torch.bfloat16, device="cuda")
+    if _CONST_DATA:
+        x.fill_(0.011)
+        w.fill_(0.011)
 
     def step():
         pa.o_proj(x, w, out=out)
@@ -597,7 +600,7 @@ def main():
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     ap.add_argument("--const-data", action="store_true",
-                    help="prefill configs 3 / 9 / 11: every Q, K and V element is the same value instead of N(0,1).  Same "
+                    help="prefill configs 3 / 9 / 11 and the projection 12: every Q, K and V (x and w) element is the same value instead of N(0,1).  Same "
                          "kernel, same instruction stream, far fewer bit flips in the matrix cores' operands: the time "
                          "difference to the normal run is what the chip's power limit costs on random data")
     args = ap.parse_args()

@@ -17,7 +17,8 @@
 // Both tiles travel HBM/L2 -> LDS with global_load_lds_dwordx4 (no registers) into a ring of two
 // 64 KB stages: the copies of k-step j + 1 are in flight while step j is multiplied.
 //   stage = x tile [256 m][128 B]  +  w tile, columns 0-127 [64 k][256 B]  +  w tile, columns 128-255
-// 16-byte chunk g of x row r sits at position g ^ (r & 7); chunk g of w row r at g ^ 4 (r & 3): the
+// 16-byte chunk g of x row r sits at position g ^ ((r >> 1) & 7) (two 128-byte rows fill the 64 banks once,
+// so sixteen consecutive rows must land on sixteen different 16-byte slots); chunk g of w row r at g ^ 4 (r & 3): the
 // reads of both kinds then spread over the banks (the copy lane fetches whatever chunk belongs in
 // its fixed LDS slot, so the swizzle costs nothing).
 #include <atomic>
@@ -72,7 +73,7 @@ void o_proj_kernel(OProjParams p) {
 
   // ---- copy maps ---------------------------------------------------------------------------------
   // x tile: 32 units of 1 KB = 8 rows x 128 B; lane i fills (row 8u + i/8, position i%8) with chunk
-  // (i%8) ^ (row & 7).  w half tile: 16 units of 4 rows x 256 B; lane i fills (row 4u + i/16, position
+  // (i%8) ^ ((row >> 1) & 7).  w half tile: 16 units of 4 rows x 256 B; lane i fills (row 4u + i/16, position
   // i%16) with chunk (i%16) ^ 4 (row & 3).  Wave w issues x units w, w+8, w+16, w+24 and w units w,
   // w+8 of both halves.  Rows past M and columns past N are clamped to the last valid ones (their
   // products are never stored).
@@ -82,7 +83,8 @@ void o_proj_kernel(OProjParams p) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int r = min(8 * (wave + 8 * j) + (lane >> 3), p.M - 1 - m0);
-    xoff[j] = (uint32_t)(r * x_row_b) + (uint32_t)(((lane & 7) ^ (lane >> 3)) << 4);
+    const int lrow = 8 * (wave + 8 * j) + (lane >> 3);          // row of the tile this lane's LDS slot belongs to
+    xoff[j] = (uint32_t)(r * x_row_b) + (uint32_t)(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);
   }
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf)
@@ -110,7 +112,7 @@ void o_proj_kernel(OProjParams p) {
   // ---- fragment read maps (lane constants) ---------------------------------------------------------
   int x_off[4];                       // x^T fragment of k16-step s: row n of a 32-row block, chunk 2s + h
 #pragma unroll
-  for (int s = 0; s < 4; ++s) x_off[s] = (64 * wm + n) * 128 + (((2 * s + h) ^ (n & 7)) << 4);
+  for (int s = 0; s < 4; ++s) x_off[s] = (64 * wm + n) * 128 + (((2 * s + h) ^ ((n >> 1) & 7)) << 4);
   // w^T fragment of 32-column chunk c.  ds_read_b64_tr_b16, per group of 16 lanes: lane i receives, for
   // j = 0..3, the (i%4)-th 16-bit element of the 8 bytes addressed by lane (i/4) + 4j.  Source lane sl
   // therefore points at k row (sl/4) of its half-wave's eight rows (8h .. 8h+3 for the first read, 4 rows
