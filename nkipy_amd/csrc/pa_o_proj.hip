@@ -212,9 +212,142 @@ void o_proj_kernel(OProjParams p) {
   }
 }
 
+// Few rows (decode: M = batch, or a verify step): the work is w's bytes, once.  One workgroup of 4 waves per
+// 64 output columns owns ALL rows (BM = 32 MBT of them) and streams its 128-byte-wide column slab of w through
+// a deep ring of small stages (K step 64: w tile [64 k][128 B] + x tile [BM][128 B]), so that N / 64
+// workgroups keep the memory system busy instead of N / 256.  Same operand layouts and product as above; wave w
+// takes the 32-column block w & 1 and the 32-row blocks of parity w >> 1.
+template <int MBT, bool BIAS>
+__global__ __launch_bounds__(256) void o_proj_skinny_kernel(OProjParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int SBM = 32 * MBT;
+  constexpr int SX_B = SBM * 128, SW_B = 64 * 128, SSTAGE_B = SX_B + SW_B;
+  constexpr int NST = MBT == 2 ? 8 : (MBT == 4 ? 5 : 3);
+  constexpr int XU = SBM / 8, UPW = (XU + 8) / 4;       // 1 KB copy units of the x tile; copy instructions per wave and stage
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int nb = wave & 1, mpar = wave >> 1;
+  const int n0 = blockIdx.x * 64;
+
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
+  const long x_row_b = (long)p.K * 2, w_row_b = (long)p.N * 2;
+  // copy maps: units of 8 rows x 128 B for both tiles; lane i fills (row 8u + i/8, position i%8).  x chunk g of
+  // row r sits at g ^ ((r >> 1) & 7), w chunk g of row r at g ^ 4 ((r >> 1) & 1) (two 128-byte rows per bank cycle)
+  uint32_t xoff[XU / 4], woff[2];
+#pragma unroll
+  for (int j = 0; j < XU / 4; ++j) {
+    const int lrow = 8 * (wave + 4 * j) + (lane >> 3);
+    xoff[j] = (uint32_t)(min(lrow, p.M - 1) * x_row_b) + (uint32_t)(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int lrow = 8 * (wave + 4 * j) + (lane >> 3);
+    const int chunk = (lane & 7) ^ (4 * ((lrow >> 1) & 1));
+    woff[j] = (uint32_t)(lrow * w_row_b) + (uint32_t)(min(n0 + 8 * chunk, p.N - 8) * 2);
+  }
+  const int ktiles = p.K / BK;
+  int kt_req = 0, stage_req = 0;
+  auto request = [&]() __attribute__((always_inline)) {
+    // requests past the end repeat the first step (into a stage nobody reads any more): the wait counts stay exact
+    const int kt = kt_req < ktiles ? kt_req : 0;
+    const char* xb = (const char*)p.x + (long)kt * (BK * 2);
+    const char* wb = (const char*)p.w + (long)kt * BK * w_row_b;
+    const uint32_t sb = smem_base + stage_req * SSTAGE_B;
+#pragma unroll
+    for (int j = 0; j < XU / 4; ++j) dma16(xb, xoff[j], sb + (wave + 4 * j) * 1024);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) dma16(wb, woff[j], sb + SX_B + (wave + 4 * j) * 1024);
+    ++kt_req;
+    stage_req = stage_req + 1 == NST ? 0 : stage_req + 1;
+  };
+
+  int x_off[4], w_off;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) x_off[s] = n * 128 + (((2 * s + h) ^ ((n >> 1) & 7)) << 4);
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int row = 8 * h + (sl >> 2);
+    const int y = 2 * (g & 1) + ((sl & 3) >> 1);
+    w_off = SX_B + row * 128 + (((4 * nb + y) ^ (4 * ((row >> 1) & 1))) << 4) + (sl & 1) * 8;
+  }
+  f32x16_t acc[MBT / 2];
+#pragma unroll
+  for (int i = 0; i < MBT / 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+
+#pragma unroll
+  for (int s = 0; s < NST - 1; ++s) request();
+  int stage = 0;
+  for (int kt = 0; kt < ktiles; ++kt) {
+    wait_vmcnt<(NST - 2) * UPW>();
+    __builtin_amdgcn_s_barrier();
+    request();
+    const char* sb = smem + stage * SSTAGE_B;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const lds_char* src = (const lds_char*)(sb + 16 * s * 128 + w_off);
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 4 * 128));
+      struct { s16x4_t a, b; } pair = {lo, hi};
+      const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, pair);
+#pragma unroll
+      for (int i = 0; i < MBT / 2; ++i) {
+        const bf16x8_t xf = *(const bf16x8_t*)(sb + (2 * i + mpar) * (32 * 128) + x_off[s]);
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[i], 0, 0, 0);
+      }
+    }
+    stage = stage + 1 == NST ? 0 : stage + 1;
+  }
+  wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
+
+  // a lane holds, for its row, 4 consecutive columns at 4 places: 8-byte stores (the output is small here)
+  uint16_t* out = (uint16_t*)p.out;
+#pragma unroll
+  for (int i = 0; i < MBT / 2; ++i) {
+    const int m = 32 * (2 * i + mpar) + n;
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int col = n0 + 32 * nb + 8 * i4 + 4 * h;
+      float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+      if (BIAS) {
+        const uint2 bw = *(const uint2*)((const uint16_t*)p.bias + min(col, p.N - 4));
+        b0 = bf16_bits_to_float(bw.x & 0xffffu); b1 = bf16_bits_to_float(bw.x >> 16);
+        b2 = bf16_bits_to_float(bw.y & 0xffffu); b3 = bf16_bits_to_float(bw.y >> 16);
+      }
+      if (m < p.M && col < p.N)
+        *(uint2*)(out + (long)m * p.N + col) = make_uint2(pack_bf16x2(acc[i][4 * i4] + b0, acc[i][4 * i4 + 1] + b1),
+                                                           pack_bf16x2(acc[i][4 * i4 + 2] + b2, acc[i][4 * i4 + 3] + b3));
+    }
+  }
+}
+
+template <int MBT>
+hipError_t launch_skinny(const OProjParams& p, hipStream_t s) {
+  constexpr int NST = MBT == 2 ? 8 : (MBT == 4 ? 5 : 3);
+  constexpr int lds = NST * (32 * MBT * 128 + 64 * 128);
+  static std::atomic<int> configured{0};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute((const void*)o_proj_skinny_kernel<MBT, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_skinny_kernel<MBT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    configured.store(1, std::memory_order_release);
+  }
+  const unsigned grid = (unsigned)((p.N + 63) / 64);
+  if (p.bias) hipLaunchKernelGGL((o_proj_skinny_kernel<MBT, true>), dim3(grid), dim3(256), lds, s, p);
+  else hipLaunchKernelGGL((o_proj_skinny_kernel<MBT, false>), dim3(grid), dim3(256), lds, s, p);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
+  // up to 256 rows: one workgroup per 64 columns owns every row (the call is bound by w's bytes)
+  if (p.M <= 64) return launch_skinny<2>(p, s);
+  if (p.M <= 128) return launch_skinny<4>(p, s);
+  if (p.M <= 256) return launch_skinny<8>(p, s);
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute((const void*)o_proj_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_B);

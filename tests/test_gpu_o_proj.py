@@ -28,7 +28,9 @@ def _close(got, want):
 
 
 @pytest.mark.parametrize("M,K,N,bias", [(1, 64, 8, False), (37, 128, 72, True), (256, 4096, 256, False),
-                                        (300, 512, 2880, True), (513, 1024, 520, True), (64, 4096, 4096, False)])
+                                        (300, 512, 2880, True), (513, 1024, 520, True), (64, 4096, 4096, False),
+                                        (100, 2048, 2880, True), (129, 512, 200, False), (200, 4096, 1024, True),
+                                        (257, 64, 64, True)])
 def test_o_proj_vs_oracle(pa, M, K, N, bias):
     rng = np.random.default_rng(M + K + N)
     x = O.round_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
