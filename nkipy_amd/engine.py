@@ -217,13 +217,13 @@ class PagedAttention:
     query_lens[b] rows; idle slots 0).  `attend` applies the optional QK RMSNorm + RoPE, writes K/V
     into the layer's pool and runs the prefill / verify kernel (T > 1) or the decode kernel
     (T == 1).  Returns [max_seqs, T, Hq, D] (a preallocated buffer, overwritten by the next step of
-    the same T).
+    the same T), or, when the layer was given `o_weight`, the output projection of it, [max_seqs, T, hidden].
     """
 
     def __init__(self, cache: PagedKVCache, n_heads: int, *, layer: int = 0, scale: Optional[float] = None,
                  rope_base: Optional[float] = None, max_positions: int = 0, q_norm_weight=None, k_norm_weight=None,
                  norm_eps: float = 1e-6, partition_size: int = 512, sinks=None, sliding_window: Optional[int] = None,
-                 rope_tables=None):
+                 rope_tables=None, o_weight=None, o_bias=None):
         if not 0 <= layer < cache.num_layers:
             raise ValueError(f"layer {layer} outside the cache's {cache.num_layers} layers")
         self.cache, self.n_heads, self.layer = cache, n_heads, layer
@@ -253,7 +253,14 @@ class PagedAttention:
                 raise ValueError(f"RoPE tables cover {self.rope[0].shape[0]} positions, the cache holds sequences of up "
                                  f"to {cap} tokens ({cache.max_blocks_per_seq} blocks of {cache.block_size}): give "
                                  f"max_positions >= {cap}")
+        # output projection behind the attention call (examples/models/qwen3/kernels/attention.py:143-147;
+        # with the bias gpt_oss/kernels/attention.py:155-163): o_weight [n_heads * head_dim, hidden] bfloat16 as the
+        # reference stores it, this rank's rows; `attend` then returns [max_seqs, T, hidden] for the caller to all-reduce
+        self.o_weight, self.o_bias = o_weight, o_bias
+        if o_weight is not None and tuple(o_weight.shape[:1]) != (n_heads * cache.head_dim,):
+            raise ValueError(f"o_weight must be [{n_heads * cache.head_dim}, hidden], got {tuple(o_weight.shape)}")
         self._out: Dict[int, torch.Tensor] = {}
+        self._proj: Dict[int, torch.Tensor] = {}
 
     def step(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, query_lens: Sequence[int]) -> torch.Tensor:
         if xq.shape[0] != self.cache.max_seqs or len(query_lens) != xq.shape[0]:
@@ -296,4 +303,9 @@ class PagedAttention:
             paged_attn.prefill(q, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
                                k_scale=ks, v_scale=vs, out=out,
                                sinks=self.sinks, sliding_window=self.sliding_window, q_transform=qt)
-        return out
+        if self.o_weight is None:
+            return out
+        proj = self._proj.get(T)
+        if proj is None:
+            proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
+        return paged_attn.o_proj(out, self.o_weight, self.o_bias, out=proj)

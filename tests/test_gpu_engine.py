@@ -273,3 +273,29 @@ def test_serving_loop_random_schedule(seed, variant):
             owned[blk] = owned.get(blk, 0) + 1
     assert all(cache.allocator.refcount(blk) == n for blk, n in owned.items())
     assert cache.allocator.num_free + len(owned) == 70
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_layer_with_output_projection(rng, bias):
+    """A layer given `o_weight` returns the projected rows: the attention output in its stored bfloat16 rounding
+    times o_weight, float32 accumulation, one rounding (qwen3 attention.py:143-147; with bias gpt_oss
+    attention.py:155-163)."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    S, Hq, Hkv, D, bs, hidden = 3, 8, 2, 128, 16, 512
+    cache = PagedKVCache(num_blocks=30, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=8)
+    w = _rand(rng, (Hq * D, hidden), 0.05)
+    b = _rand(rng, hidden) if bias else None
+    layer = PagedAttention(cache, Hq, o_weight=bf16_to_dev(w), o_bias=None if b is None else bf16_to_dev(b))
+    mirror = _Mirror(S, None, None, None, None, 1e-6)
+    for T, qlens in ((19, [19, 7, 0]), (1, [1, 1, 0]), (1, [1, 1, 0])):
+        cache.begin_step(qlens, T)
+        xq, xk, xv = _rand(rng, (S, T, Hq, D)), _rand(rng, (S, T, Hkv, D)), _rand(rng, (S, T, Hkv, D))
+        got = dev_to_f32(layer.attend(bf16_to_dev(xq), bf16_to_dev(xk), bf16_to_dev(xv)))
+        assert got.shape == (S, T, hidden)
+        attn = mirror.step(xq, xk, xv, qlens, layer.scale)
+        want = O.o_proj(attn.reshape(S, T, Hq * D), w, b)
+        for s in range(S):
+            if qlens[s]:
+                assert_close_abs(got[s, :qlens[s]], want[s, :qlens[s]], 4e-2)
+    with pytest.raises(ValueError):
+        PagedAttention(cache, Hq, o_weight=bf16_to_dev(_rand(rng, (Hq * D - 64, hidden))))
