@@ -499,8 +499,8 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
   p.scale_log2e = scale * kLog2e;
   p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
-  // head_dim 64: the tiled kernel takes bf16 pools with an even number of kv heads (two heads share its 256-byte
-  // rows); short query runs and everything else go to the decode-shaped kernel, 64 query tokens per launch, each
+  // head_dim 64: the tiled kernel takes two or more kv heads (two heads share its 256-byte rows); short
+  // query runs and a single kv head go to the decode-shaped kernel, 64 query tokens per launch, each
   // launch reading the context up to its last token once per kv head
   // (measured crossover for runs of up to 64 tokens: 320 query rows per kv head in a batch of 8 or more)
   const int from64 = g_d64_tiled_from.load();

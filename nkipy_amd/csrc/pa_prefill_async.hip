@@ -112,7 +112,9 @@ void prefill_async_kernel(PrefillParams p) {
   // layout, the copies and the fragment maps stay those of 256-byte rows.  The first half of the waves
   // works for a q head of the even kv head on the rows' first 128 bytes, the second half for the q head
   // at the same place in the odd kv head's group on the other 128 bytes; both halves take the same
-  // TOKW query tokens, so every byte copied is used.
+  // TOKW query tokens, so every byte copied is used.  An odd number of kv heads leaves the last head without
+  // a partner: its workgroups take the 256 bytes that end with it (the pair one head earlier), the second half
+  // of the waves works for it and the first half only copies (`idle_half`).
   constexpr bool PAIR = DH == 64;
   static_assert(DH == HD || (PAIR && NW == 8 && MODE == 1 && !SPARSE && !PACK), "head dim 64: 8-wave paged dense form only");
   constexpr int KS = DH / 16;                // k-steps of the score product
@@ -137,7 +139,7 @@ void prefill_async_kernel(PrefillParams p) {
   // stays in that XCD's L2.
   const int n_rep = p.Hq / p.Hkv;
   const int nqt = PACK ? (p.T * n_rep + BMW - 1) / BMW : (p.T + TOKW - 1) / TOKW;
-  const int kvg = PAIR ? p.Hkv / 2 : p.Hkv;    // K/V row groups: kv heads, or pairs of them
+  const int kvg = PAIR ? (p.Hkv + 1) / 2 : p.Hkv;    // K/V row groups: kv heads, or pairs of them
   const int per_group = PACK ? nqt : nqt * n_rep;
   const int groups = p.B * kvg;
   const int xcd = blockIdx.x & 7;
@@ -148,12 +150,15 @@ void prefill_async_kernel(PrefillParams p) {
   const int rr_ = slot % per_group;
   const int b = grp / kvg, hk = grp % kvg;     // PAIR: hk numbers the pair
   const int qt = PACK ? nqt - 1 - rr_ : nqt - 1 - rr_ / n_rep;
-  const int hq = PACK ? hk * n_rep : (PAIR ? 2 * hk : hk) * n_rep + rr_ % n_rep;     // PACK: first head of the group; PAIR: the even kv head's
+  const int kv0 = PAIR ? min(2 * hk, p.Hkv - 2) : hk;    // first kv head of the rows' 256 bytes (PAIR: Hkv >= 2, checked on the host)
+  const int hq = PACK ? hk * n_rep : kv0 * n_rep + rr_ % n_rep;     // PACK: first head of the group; PAIR: the first kv head's
   // row r of the workgroup (0 .. BMW-1) -> query token and q head
   const int v0 = qt * TOKW;
   auto row_token = [&](int r) __attribute__((always_inline)) { return PACK ? (v0 + r) / n_rep : v0 + (PAIR ? (r & (TOKW - 1)) : r); };
   auto row_head = [&](int r) __attribute__((always_inline)) { return PACK ? hq + (v0 + r) % n_rep : hq + (PAIR && r >= TOKW ? n_rep : 0); };
   const int par = PAIR ? wave / (NW / 2) : 0;   // which 128 bytes of the rows this wave works on
+  const bool lone = PAIR && 2 * hk + 1 >= p.Hkv;          // the unpaired last head of an odd Hkv
+  const bool idle_half = lone && par == 0;                // these waves' head belongs to the pair before: copies only
 
   int tq = p.query_lens ? p.query_lens[b] : p.T;
   int ctx = p.seq_lens ? p.seq_lens[b] : p.S;
@@ -171,7 +176,7 @@ void prefill_async_kernel(PrefillParams p) {
     for (int i = tid; i < BMW * (DH / 8); i += NW * 64) {
       const int r = i / (DH / 8);
       const int row = row_token(r);
-      if (row < p.T) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)row_head(r) * DH + (i % (DH / 8)) * 8) = make_uint4(0, 0, 0, 0);
+      if (row < p.T && !(lone && r < TOKW)) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)row_head(r) * DH + (i % (DH / 8)) * 8) = make_uint4(0, 0, 0, 0);
     }
     return;
   }
@@ -179,13 +184,13 @@ void prefill_async_kernel(PrefillParams p) {
   // ---- this lane's query row (token index qrow, head hq_l) and its Q^T fragments ------------
   const int qrow = row_token(wave * 32 + n);
   const int hq_l = row_head(wave * 32 + n);
-  const bool qvalid = qrow < tq;
+  const bool qvalid = qrow < tq && !idle_half;
   const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
   const float sc = p.scale_log2e;
   bf16x8_t qf[KS];                // loaded below, between the first copy requests
   const int wq_lo = row_token(wave * 32);                         // first token of this wave
   const int wq_hi = min(row_token(wave * 32 + 31), tq - 1);       // last valid token (may be < wq_lo)
-  const bool wave_has_rows = wq_lo < tq;
+  const bool wave_has_rows = wq_lo < tq && !idle_half;
   const int k_end = prefix + min(row_token(BMW - 1) + 1, tq);     // keys the workgroup needs: [0, k_end)
   // sliding window (its own instantiation, so that the plain form carries none of its scalar
   // work): the row at position pos sees keys (pos - win, pos]
@@ -212,8 +217,8 @@ void prefill_async_kernel(PrefillParams p) {
   const const_i32_ptr table = MODE != 0 ? (const_i32_ptr)(uintptr_t)(p.block_tables + (long)b * p.max_blocks) : nullptr;
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
   const long kv_row_bytes = (long)p.Hkv * DH * EB;
-  const char* kbase = (const char*)p.k + (long)hk * HD * EB;     // PAIR: 256 bytes per pair
-  const char* vbase = (const char*)p.v + (long)hk * HD * EB;
+  const char* kbase = (const char*)p.k + (long)kv0 * DH * EB;    // PAIR: 256 bytes from kv head kv0 on
+  const char* vbase = (const char*)p.v + (long)kv0 * DH * EB;
   const int dma_rr = lane >> 4, dma_pos = lane & 15;
   // every unit of a wave starts at the same row modulo 16 (NW is a multiple of 4), hence the
   // same swizzle: K rows use row & 15, V rows 4 * (row & 3) (what their read patterns want)
@@ -383,7 +388,7 @@ void prefill_async_kernel(PrefillParams p) {
   auto request_next = [&]() __attribute__((always_inline)) {
     issue_tile(w_i.kt < ntiles ? w_i.kt : kt_first, stage_i);
     if (FP8) {
-      const long si = (long)min(max(blk_pf[0], 0), p.num_blocks - 1) * p.Hkv + (PAIR ? 2 * hk : hk);
+      const long si = (long)min(max(blk_pf[0], 0), p.num_blocks - 1) * p.Hkv + kv0;
       ksq[3] = ((const_f32_ptr)(uintptr_t)p.k_scale)[si];
       vsq[3] = ((const_f32_ptr)(uintptr_t)p.v_scale)[si];
       if (PAIR) {
@@ -715,7 +720,7 @@ void prefill_async_kernel(PrefillParams p) {
       const int r = ORI * j + lane / OCH, ch = lane % OCH;
       const uint2 lo = *(const uint2*)(patch + r * OROW_B + 16 * ch), hi = *(const uint2*)(patch + r * OROW_B + 16 * ch + 8);
       const int tok = row_token(wave * 32 + r);
-      if (tok < p.T)
+      if (tok < p.T && !idle_half)
         *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)row_head(wave * 32 + r) * DH + 8 * ch) =
             make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
@@ -768,7 +773,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   const int n_rep = p.Hq / p.Hkv;
   const long per_group = PACK ? ((long)p.T * n_rep + 32 * NW - 1) / (32 * NW)
                               : (long)((p.T + TOKW - 1) / TOKW) * n_rep;
-  const long groups = (long)p.B * (DH == 64 ? p.Hkv / 2 : p.Hkv);
+  const long groups = (long)p.B * (DH == 64 ? (p.Hkv + 1) / 2 : p.Hkv);
   const long total = 8 * ((groups + 7) / 8) * per_group * (SPLIT ? p.splits : 1);
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
   hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
@@ -782,7 +787,7 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
 // workgroups of the paged dense form for a given choice of waves and packing
 long prefill_workgroups(const PrefillParams& p, int waves, bool pack) {
   const int n_rep = p.Hq / p.Hkv;
-  if (p.D == 64) return (long)p.B * (p.Hkv / 2) * ((p.T + 16 * waves - 1) / (16 * waves)) * n_rep;
+  if (p.D == 64) return (long)p.B * ((p.Hkv + 1) / 2) * ((p.T + 16 * waves - 1) / (16 * waves)) * n_rep;
   const long per_group = pack ? ((long)p.T * n_rep + 32 * waves - 1) / (32 * waves)
                               : (long)((p.T + 32 * waves - 1) / (32 * waves)) * n_rep;
   return (long)p.B * p.Hkv * per_group;
@@ -794,7 +799,7 @@ bool prefill_async_supported(const PrefillParams& p) {
   if (p.block_tables && p.block_shift < 4) return false;   // paged: power-of-two block size >= 16
   if (p.D == HD) return true;
   // head dim 64: two adjacent kv heads share the 256-byte rows the kernel is laid out for
-  return p.D == 64 && p.Hkv % 2 == 0 && p.block_tables && p.sparse_stride == 0;
+  return p.D == 64 && p.Hkv >= 2 && p.block_tables && p.sparse_stride == 0;
 }
 
 static bool prefill_packs(const PrefillParams& p) {
@@ -833,7 +838,7 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   const bool pack = prefill_packs(p);
   waves = prefill_waves(p, waves);
   if (p.D == 64) {
-    if (sparse || !paged || p.Hkv % 2 || (p.kv_fp8 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
+    if (sparse || !paged || p.Hkv < 2 || (p.kv_fp8 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
     if (p.splits > 1 && (!p.ws_o || !p.ws_ml)) return hipErrorInvalidValue;
     const int form = (p.kv_fp8 ? 4 : 0) + (p.splits > 1 ? 2 : 0) + (p.window > 0 ? 1 : 0);
     switch (form) {

@@ -335,9 +335,9 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
         # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
         rows = T * (Hq // Hkv)
         if D == 64:
-            # the tiled kernel takes head dim 64 two kv heads at a time; below 320 rows per kv head, and for small
+            # the tiled kernel takes head dim 64 two kv heads at a time (not a single kv head); below 320 rows per kv head, and for small
             # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself)
-            route = "tiled" if not can_verify or (Hkv % 2 == 0 and B >= 8 and rows >= 320) else "verify"
+            route = "tiled" if not can_verify or (Hkv >= 2 and B >= 8 and rows >= 320) else "verify"
         else:
             route = "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
                                                 or (kv_code == FP8 and (win > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"

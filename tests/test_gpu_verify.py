@@ -161,9 +161,10 @@ def test_verify_argument_errors(pa):
 
 @pytest.fixture(params=["tiled", "chunks"])
 def d64_path(request):
-    """head_dim 64 beyond 64 query tokens: an even number of kv heads takes the tiled kernel
-    (two kv heads share its 256-byte rows); with the tiled kernel switched off, as for odd head
-    counts, pa_prefill covers the query tokens with launches of the verify kernel, 64 tokens each."""
+    """head_dim 64 beyond 64 query tokens: two or more kv heads take the tiled kernel (two kv heads
+    share its 256-byte rows; the last head of an odd count works alone on the 256 bytes that end with
+    it); with the tiled kernel switched off, as for a single kv head, pa_prefill covers the query
+    tokens with launches of the verify kernel, 64 tokens each."""
     from nkipy_amd import _lib
     lib = _lib.load()
     lib.pa_debug_set(3, 1 if request.param == "chunks" else 0)
@@ -172,7 +173,8 @@ def d64_path(request):
 
 
 @pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
-@pytest.mark.parametrize("T,Hq,Hkv,bs", [(65, 4, 4, 16), (200, 8, 2, 32), (129, 64, 8, 64), (300, 3, 1, 32), (530, 12, 6, 16)])
+@pytest.mark.parametrize("T,Hq,Hkv,bs", [(65, 4, 4, 16), (200, 8, 2, 32), (129, 64, 8, 64), (300, 3, 1, 32), (530, 12, 6, 16),
+                                         (300, 9, 3, 32), (130, 10, 5, 16), (257, 7, 7, 64)])
 def test_head_dim_64_long_prefill(pa, d64_path, fp8, T, Hq, Hkv, bs):
     """Ragged lengths put tile and launch boundaries inside, at the end of and past a sequence's query run;
     the sliding window and the sinks ride along."""
@@ -237,6 +239,36 @@ def test_head_dim_64_tiled_split_matches_unsplit(pa):
     torch.cuda.synchronize()
     assert_close_abs(got, want, BF16_TOL)
     assert np.max(np.abs(got - unsplit)) <= 2 ** -6
+
+
+@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
+def test_head_dim_64_odd_kv_heads_at_the_end_of_the_pool(pa, fp8):
+    """Three kv heads, every sequence's last block the last block of the pool and filled to its last row: the
+    unpaired head's 256-byte window ends exactly with the pool.  Checked against the verify-kernel route too."""
+    rng = np.random.default_rng(97)
+    T, Hq, Hkv, bs, D = 192, 6, 3, 16, 64
+    qlens, prefixes = [192, 100, 64], [64, 12 * 16 - 100, 0]
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    last = k.shape[0] - 1
+    for b in range(len(qlens)):
+        assert ctxs[b] % bs == 0
+        tables[b, ctxs[b] // bs - 1] = last
+    okw, dkw = {}, {}
+    kd, vd = bf16_to_dev(k), bf16_to_dev(v)
+    if fp8:
+        k, ks = O.quantize_kv_fp8(k)
+        v, vs = O.quantize_kv_fp8(v)
+        okw = dict(k_scale=ks, v_scale=vs)
+        dkw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda())
+        kd = torch.from_numpy(k).cuda().view(torch.float8_e4m3fn)
+        vd = torch.from_numpy(v).cuda().view(torch.float8_e4m3fn)
+    want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.125, q_dtype="bf16", **okw)
+    args = (bf16_to_dev(q), kd, vd, _i32(tables), _i32(ctxs), _i32(ql), 0.125)
+    got = dev_to_f32(pa.prefill(*args, route="tiled", **dkw))
+    torch.cuda.synchronize()
+    assert_close_abs(got, want, FP8_TOL if fp8 else BF16_TOL)
+    for b, n in enumerate(qlens):
+        assert np.all(got[b, n:] == 0)
 
 
 def test_head_dim_64_many_rows_of_a_short_run_take_the_tiled_kernel(pa):
