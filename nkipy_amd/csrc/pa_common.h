@@ -204,7 +204,8 @@ struct PrefillParams {
   int S;                    // dense form: keys per sequence
   int sparse_local, sparse_stride;  // blocksparse pattern; sparse_stride == 0 -> plain causal
   float scale_log2e;
-  int impl;                 // 0 automatic, 1 register-staged, 4 / 8 asynchronous (waves per workgroup), 5 asynchronous with packed rows
+  int impl;                 // 0 automatic, 1 register-staged, 4 / 8 asynchronous (waves per workgroup), 5 asynchronous with packed rows,
+                            // 6 asynchronous, head dim 64 with one q head per wave
   int window;               // paged form, asynchronous kernel only: sliding window in tokens, 0 = none
   const float* sinks;       // same: [Hq] per-head sink logits or null
   int kv_fp8;               // paged form: the pool holds e4m3fn codes (register-staged kernel only)

@@ -99,7 +99,11 @@ typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 // copies and expands them, so the raw ring needs no barrier; the bf16 stages use the one per tile.
 // DH: head dim, 128 or 64.  At 64 a 256-byte piece of a pool row is two adjacent kv heads: the tile
 // layout stays that of 256-byte rows and the two halves of the workgroup's waves work for the two heads.
-template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT, bool FP8, int DH>
+// QH (head dim 64 only): q heads of one kv group per wave, 1 or 2.  With 2 a wave carries the same 32 query
+// tokens for two adjacent q heads: every K and V tile then serves twice the matrix work (at head dim 64 a tile
+// otherwise has half the matrix work of head dim 128 against the same copies and barrier), and between two
+// barriers the waves of a SIMD have twice as many matrix and vector phases to slide under one another.
+template <bool SPARSE, int MODE, int NW, int TT, bool WIN, bool PACK, bool SPLIT, bool FP8, int DH, int QH>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_async_kernel(PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -117,6 +121,7 @@ void prefill_async_kernel(PrefillParams p) {
   // of the waves works for it and the first half only copies (`idle_half`).
   constexpr bool PAIR = DH == 64;
   static_assert(DH == HD || (PAIR && NW == 8 && MODE == 1 && !SPARSE && !PACK), "head dim 64: 8-wave paged dense form only");
+  static_assert(QH == 1 || (QH == 2 && PAIR), "two q heads per wave: head dim 64 only");
   constexpr int KS = DH / 16;                // k-steps of the score product
   constexpr int VC = DH / 32;                // 32-wide d chunks of the output
   constexpr int TOKW = PAIR ? BMW / 2 : BMW; // query tokens per workgroup (plain form)
@@ -140,7 +145,8 @@ void prefill_async_kernel(PrefillParams p) {
   const int n_rep = p.Hq / p.Hkv;
   const int nqt = PACK ? (p.T * n_rep + BMW - 1) / BMW : (p.T + TOKW - 1) / TOKW;
   const int kvg = PAIR ? (p.Hkv + 1) / 2 : p.Hkv;    // K/V row groups: kv heads, or pairs of them
-  const int per_group = PACK ? nqt : nqt * n_rep;
+  const int hpg = n_rep / QH;                  // workgroups (per query tile) that cover the q heads of a kv head
+  const int per_group = PACK ? nqt : nqt * hpg;
   const int groups = p.B * kvg;
   const int xcd = blockIdx.x & 7;
   const int part = SPLIT ? (int)(blockIdx.x >> 3) % p.splits : 0;      // which share of the key tiles
@@ -149,9 +155,9 @@ void prefill_async_kernel(PrefillParams p) {
   if (grp >= groups) return;
   const int rr_ = slot % per_group;
   const int b = grp / kvg, hk = grp % kvg;     // PAIR: hk numbers the pair
-  const int qt = PACK ? nqt - 1 - rr_ : nqt - 1 - rr_ / n_rep;
+  const int qt = PACK ? nqt - 1 - rr_ : nqt - 1 - rr_ / hpg;
   const int kv0 = PAIR ? min(2 * hk, p.Hkv - 2) : hk;    // first kv head of the rows' 256 bytes (PAIR: Hkv >= 2, checked on the host)
-  const int hq = PACK ? hk * n_rep : kv0 * n_rep + rr_ % n_rep;     // PACK: first head of the group; PAIR: the first kv head's
+  const int hq = PACK ? hk * n_rep : kv0 * n_rep + QH * (rr_ % hpg);     // PACK: first head of the group; PAIR: the first kv head's; QH 2: and hq + 1
   // row r of the workgroup (0 .. BMW-1) -> query token and q head
   const int v0 = qt * TOKW;
   auto row_token = [&](int r) __attribute__((always_inline)) { return PACK ? (v0 + r) / n_rep : v0 + (PAIR ? (r & (TOKW - 1)) : r); };
@@ -176,18 +182,22 @@ void prefill_async_kernel(PrefillParams p) {
     for (int i = tid; i < BMW * (DH / 8); i += NW * 64) {
       const int r = i / (DH / 8);
       const int row = row_token(r);
-      if (row < p.T && !(lone && r < TOKW)) *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)row_head(r) * DH + (i % (DH / 8)) * 8) = make_uint4(0, 0, 0, 0);
+      if (row < p.T && !(lone && r < TOKW)) {
+#pragma unroll
+        for (int j = 0; j < QH; ++j)
+          *(uint4*)(out + ((long)b * p.T + row) * q_row_stride + (long)(row_head(r) + j) * DH + (i % (DH / 8)) * 8) = make_uint4(0, 0, 0, 0);
+      }
     }
     return;
   }
 
-  // ---- this lane's query row (token index qrow, head hq_l) and its Q^T fragments ------------
+  // ---- this lane's query row (token index qrow, head hq_l; QH 2: also head hq_l + 1) and its Q^T fragments ----
   const int qrow = row_token(wave * 32 + n);
   const int hq_l = row_head(wave * 32 + n);
   const bool qvalid = qrow < tq && !idle_half;
   const int qlim = prefix + min(qrow, tq - 1);     // last visible key of this lane's row
   const float sc = p.scale_log2e;
-  bf16x8_t qf[KS];                // loaded below, between the first copy requests
+  bf16x8_t qf[QH][KS];            // loaded below, between the first copy requests
   const int wq_lo = row_token(wave * 32);                         // first token of this wave
   const int wq_hi = min(row_token(wave * 32 + 31), tq - 1);       // last valid token (may be < wq_lo)
   const bool wave_has_rows = wq_lo < tq && !idle_half;
@@ -198,14 +208,16 @@ void prefill_async_kernel(PrefillParams p) {
   // key tiles of this workgroup: [kt_begin, ntiles)
   int kt_begin = win > 0 ? max(prefix + q0 - win + 1, 0) / BN : 0;   // first tile the first row sees
   int ntiles = (k_end + BN - 1) / BN;
-  const long row_g = ((long)b * p.T + qrow) * p.Hq + hq_l;            // this lane's row among all B * T * Hq
+  const long row_g = ((long)b * p.T + qrow) * p.Hq + hq_l;            // this lane's (first) row among all B * T * Hq
   if (SPLIT) {
     const int n_all = ntiles - kt_begin;
     const int lo = kt_begin + (int)((long)part * n_all / p.splits);
     ntiles = kt_begin + (int)((long)(part + 1) * n_all / p.splits);
     kt_begin = lo;
     if (kt_begin >= ntiles) {                  // nothing for this share: an empty partial
-      if (qvalid && h == 0) *(float2*)(p.ws_ml + (row_g * p.splits + part) * 2) = make_float2(-INFINITY, 0.f);
+#pragma unroll
+      for (int j = 0; j < QH; ++j)
+        if (qvalid && h == 0) *(float2*)(p.ws_ml + ((row_g + j) * p.splits + part) * 2) = make_float2(-INFINITY, 0.f);
       return;
     }
   }
@@ -311,11 +323,13 @@ void prefill_async_kernel(PrefillParams p) {
   }
 
   // ---- accumulators ------------------------------------------------------------
-  f32x16_t oacc[VC];
+  f32x16_t oacc[QH][VC];
 #pragma unroll
-  for (int c = 0; c < VC; ++c)
+  for (int j = 0; j < QH; ++j)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[c][i] = 0.f;
+    for (int c = 0; c < VC; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[j][c][i] = 0.f;
   // Softmax state of this lane's query row.  Scores come out of the matrix cores already
   // relative to a reference m_ref (the accumulator starts at -m_ref), in log2 units.  The
   // reference is set to the row maximum of the first tile in which the row sees a key and
@@ -323,12 +337,16 @@ void prefill_async_kernel(PrefillParams p) {
   // state there is no row maximum, no per-element subtraction and no rescaling of the output
   // accumulators.  When it does move it goes to the tile's maximum.
   constexpr float REF_SLACK = 8.f;
-  float m_ref = 0.f, l_run = 0.f;
-  float slack = -INFINITY;            // -inf until the row has seen a finite score (m_ref is arbitrary till then)
-  bool fresh_rows = true;             // wave-uniform: some row of the wave still has slack == -inf
-  f32x16_t cinit;                     // -m_ref in every accumulator slot
+  float m_ref[QH], l_run[QH];
+  float slack[QH];                    // -inf until the row has seen a finite score (m_ref is arbitrary till then)
+  bool fresh_rows[QH];                // wave-uniform: some row of the wave still has slack == -inf
+  f32x16_t cinit[QH];                 // -m_ref in every accumulator slot
 #pragma unroll
-  for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
+  for (int j = 0; j < QH; ++j) {
+    m_ref[j] = 0.f; l_run[j] = 0.f; slack[j] = -INFINITY; fresh_rows[j] = true;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) cinit[j][i] = 0.f;
+  }
 
   const int head_phase = SPARSE ? hq % p.sparse_stride : 0;
   const int qblk = wq_lo / 64;                    // sparse: q block of this wave
@@ -452,65 +470,71 @@ void prefill_async_kernel(PrefillParams p) {
       vf[c] = __builtin_bit_cast(bf16x8_t, pair);
     }
   };
-  auto mma_qk = [&](f32x16_t& sacc, const bf16x8_t (&kf)[KS]) __attribute__((always_inline)) {
-    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[0], cinit, 0, 0, 0);
+  auto mma_qk = [&](f32x16_t& sacc, const bf16x8_t (&kf)[KS], int j) __attribute__((always_inline)) {
+    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[j][0], cinit[j], 0, 0, 0);
 #pragma unroll
     for (int s = 1; s < KS; ++s)
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[s], sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qf[j][s], sacc, 0, 0, 0);
   };
-  auto mma_pv = [&](const bf16x8_t (&vf)[VC], const uint32_t (&pw)[TT][8], int g) __attribute__((always_inline)) {
-    const int tt = g >> 1, kk = g & 1;
-    const bf16x8_t pf = make_frag(pw[tt][4 * kk], pw[tt][4 * kk + 1], pw[tt][4 * kk + 2], pw[tt][4 * kk + 3]);
+  auto mma_pv = [&](const bf16x8_t (&vf)[VC], const uint32_t (&pw)[8], int kk, int j) __attribute__((always_inline)) {
+    const bf16x8_t pf = make_frag(pw[4 * kk], pw[4 * kk + 1], pw[4 * kk + 2], pw[4 * kk + 3]);
 #pragma unroll
     for (int c = 0; c < VC; ++c)
-      oacc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[c], pf, oacc[c], 0, 0, 0);
+      oacc[j][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[c], pf, oacc[j][c], 0, 0, 0);
   };
-  // S^T = K Q^T for the tile in `stage`; leaves the first V^T group of `vstage` in flight
-  auto scores = [&](f32x16_t (&sacc)[TT], int stage, bf16x8_t (&v0)[VC], int vstage) __attribute__((always_inline)) {
+  // S^T = K Q^T of head j for the tile in `stage`; leaves the first V^T group of `vstage` in flight
+  auto scores = [&](f32x16_t (&sacc)[TT], int stage, bf16x8_t (&v0)[VC], int vstage, int j) __attribute__((always_inline)) {
     bf16x8_t ka[KS], kb[KS];
     load_k(ka, stage, 0);
     if (TT == 2) {
       load_k(kb, stage, 1);
-      mma_qk(sacc[0], ka);
+      mma_qk(sacc[0], ka, j);
       load_v(v0, vstage, 0);
-      mma_qk(sacc[TT - 1], kb);
+      mma_qk(sacc[TT - 1], kb, j);
     } else {
       load_v(v0, vstage, 0);
-      mma_qk(sacc[0], ka);
+      mma_qk(sacc[0], ka, j);
     }
   };
-  // O^T += V^T P^T for the tile in `stage`; group 0's fragments were loaded by scores()
-  auto accumulate = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[VC]) __attribute__((always_inline)) {
+  // O^T += V^T P^T of head j for the tile in `stage`; group 0's fragments were loaded by scores()
+  auto accumulate = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[VC], int j) __attribute__((always_inline)) {
     bf16x8_t v1[VC];
 #pragma unroll
     for (int g = 0; g < 2 * TT; g += 2) {
       load_v(v1, stage, g + 1);
-      mma_pv(v0, pw, g);
+      mma_pv(v0, pw[g >> 1], 0, j);
       if (g + 2 < 2 * TT) load_v(v0, stage, g + 2);
-      mma_pv(v1, pw, g + 1);
+      mma_pv(v1, pw[g >> 1], 1, j);
     }
   };
 
   // online softmax on this lane's column: scores -> packed bf16 probabilities, state update
-  auto softmax = [&](f32x16_t (&sacc)[TT], uint32_t (&pw)[TT][8], int kt) __attribute__((always_inline)) {
-    const int key0 = kt * BN;
-    const bool need_mask = key0 + BN - 1 > prefix + wq_lo;    // tile reaches past the first row's diagonal
+  // (sacc: NS 32-key sub-tiles that start at key key0; j: which head of the wave)
+  auto softmax = [&](auto& sacc, auto& pw, int key0, int j) __attribute__((always_inline)) {
+    constexpr int NS = sizeof(sacc) / sizeof(sacc[0]);
+    const bool need_mask = key0 + 32 * NS - 1 > prefix + wq_lo;    // reaches past the first row's diagonal
     if (need_mask) {
+      int kb = key0;
+      // sub-tile form: keeps the key arithmetic and the compares inside the branch (the compiler hoisted them onto
+      // every tile); the whole-tile forms do not need it, and with it they run out of registers
+      if constexpr (NS == 1) asm volatile("" : "+s"(kb));
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
+      for (int tt = 0; tt < NS; ++tt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
+          const int key = kb + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
           sacc[tt][i] = key <= qlim ? sacc[tt][i] : -INFINITY;
         }
     }
     if (win > 0 && key0 < prefix + wq_hi - win + 1) {         // tile starts below the last row's window
       const int qlo = qlim - win + 1;
+      int kb = key0;
+      if constexpr (NS == 1) asm volatile("" : "+s"(kb));       // (as above)
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
+      for (int tt = 0; tt < NS; ++tt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int key = key0 + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
+          const int key = kb + 32 * tt + 8 * (i >> 2) + 4 * h + (i & 3);
           sacc[tt][i] = key >= qlo ? sacc[tt][i] : -INFINITY;
         }
     }
@@ -520,10 +544,10 @@ void prefill_async_kernel(PrefillParams p) {
     // probabilities are taken at once and the row maximum is never formed; only if a row's sum
     // comes out beyond 2^OVF_LOG2 (or not a number) is the tile redone the careful way below.
     constexpr float OVF_LIMIT = 0x1p+64f;
-    if (!fresh_rows) {
+    if (!fresh_rows[j]) {
       float psum = 0.f;
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
+      for (int tt = 0; tt < NS; ++tt)
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
           const float p0 = __builtin_amdgcn_exp2f(sacc[tt][i]);
@@ -532,13 +556,13 @@ void prefill_async_kernel(PrefillParams p) {
           pw[tt][i >> 1] = pack_bf16x2(p0, p1);
         }
       if (__builtin_amdgcn_ballot_w64(!(psum < OVF_LIMIT)) == 0) {
-        l_run += psum;
+        l_run[j] += psum;
         return;
       }
     }
     float tmax = -INFINITY;
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
+    for (int tt = 0; tt < NS; ++tt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sacc[tt][i]);
     {   // the other half-wave holds the remaining keys of this query row: swap halves in registers
@@ -547,25 +571,30 @@ void prefill_async_kernel(PrefillParams p) {
     }
     // move the reference for the first finite tile of a row, or when a score lies more than the
     // slack above it
-    const bool move = tmax > slack;
+    const bool move = tmax > slack[j];
     if (__builtin_amdgcn_ballot_w64(move) != 0) {
       const float shift = move ? tmax : 0.f;
-      const float alpha = (move && slack != -INFINITY) ? __builtin_amdgcn_exp2f(-shift) : 1.f;   // a fresh row has nothing to rescale
-      m_ref += shift;
-      slack = move ? REF_SLACK : slack;
-      l_run *= alpha;
+      const float alpha = (move && slack[j] != -INFINITY) ? __builtin_amdgcn_exp2f(-shift) : 1.f;   // a fresh row has nothing to rescale
+      m_ref[j] += shift;
+      slack[j] = move ? REF_SLACK : slack[j];
+      l_run[j] *= alpha;
+      // (in-place forms: the accumulators and the reference tuple must come out of this rare branch in the registers
+      // they went in with, or the register allocator may pay for the join with copies on the common path)
 #pragma unroll
-      for (int c = 0; c < VC; ++c) oacc[c] *= alpha;
+      for (int c = 0; c < VC; ++c)
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
+        for (int i = 0; i < 16; ++i) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(oacc[j][c][i]) : "v"(alpha));
+#pragma unroll
+      for (int tt = 0; tt < NS; ++tt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) sacc[tt][i] -= shift;
+      const float neg_ref = -m_ref[j];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) cinit[i] = -m_ref;
+      for (int i = 0; i < 16; ++i) asm volatile("v_mov_b32 %0, %1" : "+v"(cinit[j][i]) : "v"(neg_ref));
     }
     float psum = 0.f;
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
+    for (int tt = 0; tt < NS; ++tt)
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
         const float p0 = __builtin_amdgcn_exp2f(sacc[tt][i]);
@@ -573,15 +602,16 @@ void prefill_async_kernel(PrefillParams p) {
         psum += p0 + p1;
         pw[tt][i >> 1] = pack_bf16x2(p0, p1);
       }
-    l_run += psum;
-    fresh_rows = __builtin_amdgcn_ballot_w64(slack == -INFINITY) != 0;
+    l_run[j] += psum;
+    fresh_rows[j] = __builtin_amdgcn_ballot_w64(slack[j] == -INFINITY) != 0;
   };
   // ---- prologue: the first tile's copies, then Q, then the rest of the ring: the Q loads and
   // the first tile travel together instead of one memory latency after the other
   request_next();
   prefetch_next();
-  {
-    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)hq_l * DH;
+#pragma unroll
+  for (int j = 0; j < QH; ++j) {
+    const uint16_t* qp = (const uint16_t*)p.q + ((long)b * p.T + qrow) * q_row_stride + (long)(hq_l + j) * DH;
     uint4 qraw[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
@@ -620,12 +650,12 @@ void prefill_async_kernel(PrefillParams p) {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         r[j] = pack_bf16x2(bf16_bits_to_float(w[j] & 0xffffu) * sc, bf16_bits_to_float(w[j] >> 16) * sc);
-      qf[s] = make_frag(r[0], r[1], r[2], r[3]);
+      qf[j][s] = make_frag(r[0], r[1], r[2], r[3]);
     }
     // the Q loads must be complete (and known to the compiler to be) before the loop, or the
     // first use of a fragment inside it would drain the ring with a full wait
 #pragma unroll
-    for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qf[s]));
+    for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qf[j][s]));
   }
 #pragma unroll
   for (int s = 1; s < NST - 1; ++s) {
@@ -660,13 +690,44 @@ void prefill_async_kernel(PrefillParams p) {
         rs_n = (rs_n + 1) & 3;
       }
       if (tile_active(w_c)) {
-        f32x16_t sacc[TT];
-        uint32_t pw[TT][8];
-        bf16x8_t v0[VC];
-        scores(sacc, stage_c, v0, stage_c);
-        prefetch_next();
-        softmax(sacc, pw, w_c.kt);
-        accumulate(pw, stage_c, v0);
+        if constexpr (QH == 1) {
+          f32x16_t sacc[TT];
+          uint32_t pw[TT][8];
+          bf16x8_t v0[VC];
+          scores(sacc, stage_c, v0, stage_c, 0);
+          prefetch_next();
+          softmax(sacc, pw, w_c.kt * BN, 0);
+          accumulate(pw, stage_c, v0, 0);
+        } else {
+          // two heads, one 32-key sub-tile at a time: its K fragments and its two groups of V^T fragments are
+          // read once and serve both heads; scores, probabilities and fragments of one sub-tile are all the
+          // registers hold besides the accumulators
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) {
+            bf16x8_t kf[KS];
+            load_k(kf, stage_c, tt);
+            f32x16_t sacc[QH][1];
+            uint32_t pw[QH][1][8];
+#pragma unroll
+            for (int j = 0; j < QH; ++j) mma_qk(sacc[j][0], kf, j);
+            bf16x8_t va[VC], vb[VC];
+            load_v(va, stage_c, 2 * tt);
+            load_v(vb, stage_c, 2 * tt + 1);
+            if (tt == 0) {
+              // the scalar loads must not drift up in front of the wait for the K fragments (LDS reads and scalar
+              // loads share a counter: that wait would then sit out the loads' whole latency)
+              __builtin_amdgcn_sched_barrier(0);
+              prefetch_next();
+            }
+#pragma unroll
+            for (int j = 0; j < QH; ++j) softmax(sacc[j], pw[j], w_c.kt * BN + 32 * tt, j);
+#pragma unroll
+            for (int j = 0; j < QH; ++j) {
+              mma_pv(va, pw[j][0], 0, j);
+              mma_pv(vb, pw[j][0], 1, j);
+            }
+          }
+        }
       } else {
         prefetch_next();
       }
@@ -677,41 +738,49 @@ void prefill_async_kernel(PrefillParams p) {
   wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
 
   // ---- normalise and write this lane's query row ---------------------------------
-  {
-    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
-    l_run = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+#pragma unroll
+  for (int j = 0; j < QH; ++j) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run[j]), __float_as_uint(l_run[j]), false, false);
+    l_run[j] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
   }
   if (SPLIT) {     // partial result relative to m_ref; the sink and the division belong to the merge
     if (qvalid) {
-      float* po = p.ws_o + (row_g * p.splits + part) * DH;
 #pragma unroll
-      for (int c = 0; c < VC; ++c)
+      for (int j = 0; j < QH; ++j) {
+        float* po = p.ws_o + ((row_g + j) * p.splits + part) * DH;
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4)
-          *(float4*)(po + 32 * c + 8 * i4 + 4 * h) =
-              make_float4(oacc[c][4 * i4], oacc[c][4 * i4 + 1], oacc[c][4 * i4 + 2], oacc[c][4 * i4 + 3]);
-      if (h == 0) *(float2*)(p.ws_ml + (row_g * p.splits + part) * 2) = make_float2(slack == -INFINITY ? -INFINITY : m_ref, l_run);
+        for (int c = 0; c < VC; ++c)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            *(float4*)(po + 32 * c + 8 * i4 + 4 * h) =
+                make_float4(oacc[j][c][4 * i4], oacc[j][c][4 * i4 + 1], oacc[j][c][4 * i4 + 2], oacc[j][c][4 * i4 + 3]);
+        if (h == 0)
+          *(float2*)(p.ws_ml + ((row_g + j) * p.splits + part) * 2) = make_float2(slack[j] == -INFINITY ? -INFINITY : m_ref[j], l_run[j]);
+      }
     }
     return;
   }
   // attention sink: a per-head logit that joins the softmax as one more column with no value
-  if (p.sinks && l_run > 0.f) l_run += __builtin_amdgcn_exp2f(p.sinks[hq_l] * kLog2e - m_ref);
+#pragma unroll
+  for (int j = 0; j < QH; ++j)
+    if (p.sinks && l_run[j] > 0.f) l_run[j] += __builtin_amdgcn_exp2f(p.sinks[hq_l + j] * kLog2e - m_ref[j]);
   // The rows go out through LDS: a lane holds 4 consecutive d of one row at 16 places, which as direct
   // stores would be 8-byte pieces of 64 different rows per instruction; staged row-major in a
   // wave-private patch of the (now idle) tile ring they leave as whole 256-byte rows, 16 bytes a lane.
   __builtin_amdgcn_s_barrier();                  // every wave is done reading the ring
-  {
+#pragma unroll
+  for (int hj = 0; hj < QH; ++hj) {
     constexpr int OROW_B = 2 * DH + 8;           // row pitch: the 8 bytes spread a column of rows over the banks
     constexpr int OCH = DH / 8, ORI = 64 / OCH;  // 16-byte pieces per row; rows a wave stores per instruction
-    char* patch = smem + wave * (32 * OROW_B);
-    const float inv = (qvalid && l_run > 0.f) ? 1.f / l_run : 0.f;
+    char* patch = smem + (wave * QH + hj) * (32 * OROW_B);
+    const float inv = (qvalid && l_run[hj] > 0.f) ? 1.f / l_run[hj] : 0.f;
 #pragma unroll
     for (int c = 0; c < VC; ++c)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int d = 32 * c + 8 * i4 + 4 * h;
-        const uint32_t w0 = qvalid ? pack_bf16x2(oacc[c][4 * i4] * inv, oacc[c][4 * i4 + 1] * inv) : 0u;
-        const uint32_t w1 = qvalid ? pack_bf16x2(oacc[c][4 * i4 + 2] * inv, oacc[c][4 * i4 + 3] * inv) : 0u;
+        const uint32_t w0 = qvalid ? pack_bf16x2(oacc[hj][c][4 * i4] * inv, oacc[hj][c][4 * i4 + 1] * inv) : 0u;
+        const uint32_t w1 = qvalid ? pack_bf16x2(oacc[hj][c][4 * i4 + 2] * inv, oacc[hj][c][4 * i4 + 3] * inv) : 0u;
         *(uint2*)(patch + n * OROW_B + 2 * d) = make_uint2(w0, w1);
       }
     // the wave reads back what its own lanes wrote: no barrier, the compiler orders the LDS accesses
@@ -721,7 +790,7 @@ void prefill_async_kernel(PrefillParams p) {
       const uint2 lo = *(const uint2*)(patch + r * OROW_B + 16 * ch), hi = *(const uint2*)(patch + r * OROW_B + 16 * ch + 8);
       const int tok = row_token(wave * 32 + r);
       if (tok < p.T && !idle_half)
-        *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)row_head(wave * 32 + r) * DH + 8 * ch) =
+        *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)(row_head(wave * 32 + r) + hj) * DH + 8 * ch) =
             make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
   }
@@ -759,24 +828,24 @@ __global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams
   *(uint2*)dst = make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
 }
 
-template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false, bool FP8 = false, int DH = HD>
+template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false, bool FP8 = false, int DH = HD, int QH = 1>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   constexpr int TOKW = DH == 64 ? 16 * NW : 32 * NW;      // query tokens per workgroup (plain form)
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH>,
+    hipError_t e = hipFuncSetAttribute((const void*)prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH, QH>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
   }
   const int n_rep = p.Hq / p.Hkv;
   const long per_group = PACK ? ((long)p.T * n_rep + 32 * NW - 1) / (32 * NW)
-                              : (long)((p.T + TOKW - 1) / TOKW) * n_rep;
+                              : (long)((p.T + TOKW - 1) / TOKW) * (n_rep / QH);
   const long groups = (long)p.B * (DH == 64 ? (p.Hkv + 1) / 2 : p.Hkv);
   const long total = 8 * ((groups + 7) / 8) * per_group * (SPLIT ? p.splits : 1);
   if (total > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
+  hipLaunchKernelGGL((prefill_async_kernel<SPARSE, MODE, NW, TT, WIN, PACK, SPLIT, FP8, DH, QH>), dim3((unsigned)total), dim3(NW * 64), lds, s, p);
   if (SPLIT) {
     const long items = (long)p.B * p.T * p.Hq * (DH / 4);
     hipLaunchKernelGGL(prefill_split_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, p);
@@ -784,10 +853,13 @@ hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// head dim 64: q heads per wave (two when the kv group has an even number of them)
+int d64_heads_per_wave(const PrefillParams& p) { return (p.Hq / p.Hkv) % 2 == 0 && p.impl != 6 ? 2 : 1; }
+
 // workgroups of the paged dense form for a given choice of waves and packing
 long prefill_workgroups(const PrefillParams& p, int waves, bool pack) {
   const int n_rep = p.Hq / p.Hkv;
-  if (p.D == 64) return (long)p.B * ((p.Hkv + 1) / 2) * ((p.T + 16 * waves - 1) / (16 * waves)) * n_rep;
+  if (p.D == 64) return (long)p.B * ((p.Hkv + 1) / 2) * ((p.T + 16 * waves - 1) / (16 * waves)) * (n_rep / d64_heads_per_wave(p));
   const long per_group = pack ? ((long)p.T * n_rep + 32 * waves - 1) / (32 * waves)
                               : (long)((p.T + 32 * waves - 1) / (32 * waves)) * n_rep;
   return (long)p.B * p.Hkv * per_group;
@@ -840,15 +912,22 @@ hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s
   if (p.D == 64) {
     if (sparse || !paged || p.Hkv < 2 || (p.kv_fp8 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
     if (p.splits > 1 && (!p.ws_o || !p.ws_ml)) return hipErrorInvalidValue;
-    const int form = (p.kv_fp8 ? 4 : 0) + (p.splits > 1 ? 2 : 0) + (p.window > 0 ? 1 : 0);
+    // Head dim 64 always takes the instantiation that carries the sliding-window tests (window 0: no row is cut).
+    // The one without them, otherwise the same code, leaves the register allocator with spills (two heads per
+    // wave) or with some fifty register copies per key tile on the common path (one head per wave).
+    const int form = (p.kv_fp8 ? 2 : 0) + (p.splits > 1 ? 1 : 0);
+    if (d64_heads_per_wave(p) == 2) {
+      switch (form) {
+        case 0: return launch_typed<false, 1, 8, 2, true, false, false, false, 64, 2>(p, s);
+        case 1: return launch_typed<false, 1, 8, 2, true, false, true, false, 64, 2>(p, s);
+        case 2: return launch_typed<false, 1, 8, 2, true, false, false, true, 64, 2>(p, s);
+        default: return launch_typed<false, 1, 8, 2, true, false, true, true, 64, 2>(p, s);
+      }
+    }
     switch (form) {
-      case 0: return launch_typed<false, 1, 8, 2, false, false, false, false, 64>(p, s);
-      case 1: return launch_typed<false, 1, 8, 2, true, false, false, false, 64>(p, s);
-      case 2: return launch_typed<false, 1, 8, 2, false, false, true, false, 64>(p, s);
-      case 3: return launch_typed<false, 1, 8, 2, true, false, true, false, 64>(p, s);
-      case 4: return launch_typed<false, 1, 8, 2, false, false, false, true, 64>(p, s);
-      case 5: return launch_typed<false, 1, 8, 2, true, false, false, true, 64>(p, s);
-      case 6: return launch_typed<false, 1, 8, 2, false, false, true, true, 64>(p, s);
+      case 0: return launch_typed<false, 1, 8, 2, true, false, false, false, 64>(p, s);
+      case 1: return launch_typed<false, 1, 8, 2, true, false, true, false, 64>(p, s);
+      case 2: return launch_typed<false, 1, 8, 2, true, false, false, true, 64>(p, s);
       default: return launch_typed<false, 1, 8, 2, true, false, true, true, 64>(p, s);
     }
   }
