@@ -298,8 +298,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     Two kernels stand behind it.  Short query runs -- speculative verify: T * (Hq / Hkv) <=
     VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query rows
     (HBM-bound: the context is read once per kv head); everything else through the tiled
-    matrix-core prefill kernel (head_dim 128, and 64 with an even number of kv heads;
-    other long query runs at head_dim 64 go through the verify kernel 64 tokens at a time).
+    matrix-core prefill kernel (head_dim 128, and 64 with two or more kv heads; long query runs
+    at head_dim 64 over a single kv head go through the verify kernel 64 tokens at a time).
     `route` = "verify" or "tiled" forces one.  fp8 pools
     (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both.  sinks and sliding_window are
     as in `decode`, the window counted back from each query token; so is q_transform, the position of
