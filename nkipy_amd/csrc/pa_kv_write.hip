@@ -115,7 +115,9 @@ __device__ __forceinline__ uint32_t pack_fp8x2(float a, float b, uint32_t old, b
 
 // ESZ: bytes per stored element (4 fp32 copy, 2 bf16 copy, 1 fp8 quantise from bf16 rows)
 template <int ESZ, int XCPR>      // XCPR: D / 8 of a transforming write, 0 for a plain one
-__global__ __launch_bounds__(WG) void kv_write_kernel(KvWriteParams p) {
+// (eight waves per SIMD: the workgroups are short chains of dependent loads, and more of them resident measured 2-3 % faster
+// than the 96 registers the compiler takes when left alone)
+__global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void kv_write_kernel(KvWriteParams p) {
   constexpr bool XFORM = XCPR != 0;
   __shared__ float red[WG / 64];
   const int which = blockIdx.x & 1;            // 0: K, 1: V
