@@ -42,8 +42,7 @@ template <int CPR>
 __device__ __forceinline__ void norm_rope_chunk(float (&x)[8], int c, const uint16_t* w, float eps,
                                                 const uint16_t* cos_row, const uint16_t* sin_row) {
   constexpr int D = 8 * CPR;
-  // round to bf16 with the conversion instruction (round to nearest even)
-  auto r16 = [](float f) __attribute__((always_inline)) { return __uint_as_float(pack_bf16x2(f, 0.f) << 16); };
+  // (roundings to bf16 go through the conversion instruction, round to nearest even, two values at a time)
   if (w) {
     float ss = 0.f;
 #pragma unroll
@@ -56,13 +55,26 @@ __device__ __forceinline__ void norm_rope_chunk(float (&x)[8], int c, const uint
     // x / sqrt(mean + eps) as x * rsq(...): within 2 float32 ulp of the divided form, far below
     // the bf16 rounding that follows
     const float inv = __builtin_amdgcn_rsqf(__fdiv_rn(ss, (float)D) + eps);
+    const uint4 ww = *(const uint4*)(w + 8 * c);
+    const uint32_t wv[4] = {ww.x, ww.y, ww.z, ww.w};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] = r16((x[j] * inv) * bf16_bits_to_float(w[8 * c + j]));
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t r = pack_bf16x2((x[2 * j] * inv) * bf16_bits_to_float(wv[j] & 0xffffu), (x[2 * j + 1] * inv) * bf16_bits_to_float(wv[j] >> 16));
+      x[2 * j] = __uint_as_float(r << 16);
+      x[2 * j + 1] = __uint_as_float(r & 0xffff0000u);
+    }
   }
   constexpr int hc = CPR / 2;
   const bool first = c < hc;
   const int fi = 8 * (first ? c : c - hc);
-  const uint4 cw = *(const uint4*)(cos_row + fi), sw = *(const uint4*)(sin_row + fi);
+  const uint4 cw = *(const uint4*)(cos_row + fi);
+  uint4 sw = *(const uint4*)(sin_row + fi);
+  // first half: x0 c - x1 s with x0 = own; second half: x0 s + x1 c with x1 = own.  Both are
+  // round(round(own c) + round(other s')) with s' = -s in the first half: rounding to nearest even is
+  // symmetric in sign and the sum commutes, so the bits are those of the two written-out forms.  The sign
+  // goes into the packed sine words, two elements per instruction.
+  const uint32_t flip = first ? 0x80008000u : 0u;
+  sw.x ^= flip; sw.y ^= flip; sw.z ^= flip; sw.w ^= flip;
   float cs[8], sn[8];
   {
     const uint32_t a[4] = {cw.x, cw.y, cw.z, cw.w}, b[4] = {sw.x, sw.y, sw.z, sw.w};
@@ -72,11 +84,21 @@ __device__ __forceinline__ void norm_rope_chunk(float (&x)[8], int c, const uint
       sn[2 * j] = bf16_bits_to_float(b[j] & 0xffffu); sn[2 * j + 1] = bf16_bits_to_float(b[j] >> 16);
     }
   }
+  // two roundings per conversion instruction
+  auto r16x2 = [](float& f0, float& f1) __attribute__((always_inline)) {
+    const uint32_t w = pack_bf16x2(f0, f1);
+    f0 = __uint_as_float(w << 16);
+    f1 = __uint_as_float(w & 0xffff0000u);
+  };
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float other = lane_xor<hc>(x[j]);
-    // first half: x0 c - x1 s with x0 = own; second half: x0 s + x1 c with x1 = own
-    x[j] = first ? r16(r16(x[j] * cs[j]) - r16(other * sn[j])) : r16(r16(other * sn[j]) + r16(x[j] * cs[j]));
+  for (int j = 0; j < 8; j += 2) {
+    float a0 = x[j] * cs[j], a1 = x[j + 1] * cs[j + 1];
+    float b0 = lane_xor<hc>(x[j]) * sn[j], b1 = lane_xor<hc>(x[j + 1]) * sn[j + 1];
+    r16x2(a0, a1);
+    r16x2(b0, b1);
+    float s0 = a0 + b0, s1 = a1 + b1;
+    r16x2(s0, s1);
+    x[j] = s0; x[j + 1] = s1;
   }
 }
 
