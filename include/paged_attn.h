@@ -289,7 +289,9 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
  * the same tile (1 = on, the default); key 5: query rows per wavefront of pa_verify (0 =
  * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never);
- * key 7: query tokens from which pa_prefill at head dim 64 takes the tiled kernel (0 = the default, 65). */
+ * key 7: query tokens from which pa_prefill at head dim 64 takes the tiled kernel (0 = the default, 65);
+ * key 3 value 6: one q head per wave at head dim 64; key 8: pa_o_proj takes 256 x 256 tiles
+ * also where it would take 128 x 128 ones (1 = on). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

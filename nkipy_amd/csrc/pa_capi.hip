@@ -113,6 +113,7 @@ int pa_debug_set(int key, int value) {
   if (key == 5) { g_verify_rows = value; return 0; }
   if (key == 6) { g_prefill_split = value; return 0; }
   if (key == 7) { g_d64_tiled_from = value > 0 ? value : PA_VERIFY_MAX_TOKENS + 1; return 0; }
+  if (key == 8) { o_proj_debug_force_large(value); return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 

@@ -259,6 +259,7 @@ struct OProjParams {
   int M, K, N;
 };
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s);
+void o_proj_debug_force_large(int on);      // debug: 256 x 256 tiles also where the 128 x 128 form would be taken
 
 // matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats
 hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s);

@@ -212,6 +212,164 @@ void o_proj_kernel(OProjParams p) {
   }
 }
 
+// Between the two: a few hundred to a few thousand rows (a prefill chunk of a small batch) give fewer 256 x 256 tiles
+// than the device has CUs.  Same product, operand layouts and copy scheme on 128 x 128 tiles: a workgroup of 4
+// wavefronts, wavefront (wm, wn) owning rows 64 wm .. +63 and columns 64 wn .. +63 (two 32-row blocks x two
+// 32-column chunks), stages of 32 KB (x tile [128 m][128 B] + w tile [64 k][256 B]), two workgroups per CU.
+constexpr int MBM = 128, MBN = 128;
+constexpr int MXT_B = MBM * BK * 2;        // 16 KB
+constexpr int MWT_B = BK * MBN * 2;        // 16 KB
+constexpr int MSTAGE_B = MXT_B + MWT_B;
+
+// MNST: ring stages.  2 (64 KB: two workgroups per CU) when there are more tiles than CUs; 4 (128 KB, copies three
+// k-steps ahead) when every CU holds at most one workgroup anyway and nothing else hides the copies' latency.
+template <bool BIAS, int MNST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void o_proj_mid_kernel(OProjParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int wm = wave & 1, wn = wave >> 1;
+
+  // tile order as in the large form: an XCD owns row tiles xcd, xcd + 8, ... and walks them in groups of 4 column tiles
+  const int MT = (p.M + MBM - 1) / MBM, NT = (p.N + MBN - 1) / MBN;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int mtx = (MT + 7) / 8;
+  const int grp = slot / (4 * mtx), rem = slot % (4 * mtx);
+  const int mt = xcd + 8 * (rem >> 2), nt = 4 * grp + (rem & 3);
+  if (mt >= MT || nt >= NT) return;
+  const int m0 = mt * MBM, n0 = nt * MBN;
+
+  // copy maps: x tile = 16 units of 8 rows x 128 B, w tile = 16 units of 4 rows x 256 B; wave w issues units w, w + 4,
+  // w + 8, w + 12 of each; swizzles as in the large form
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
+  const long x_row_b = (long)p.K * 2, w_row_b = (long)p.N * 2;
+  uint32_t xoff[4], woff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int lrow = 8 * (wave + 4 * j) + (lane >> 3);
+    const int r = min(lrow, p.M - 1 - m0);
+    xoff[j] = (uint32_t)(r * x_row_b) + (uint32_t)(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);
+    const int wr = 4 * (wave + 4 * j) + (lane >> 4);
+    const int chunk = (lane & 15) ^ (4 * ((lane >> 4) & 3));
+    const int col = min(n0 + 8 * chunk, p.N - 8);
+    woff[j] = (uint32_t)(wr * w_row_b) + (uint32_t)(col * 2);
+  }
+  const char* xbase = (const char*)p.x + (long)m0 * x_row_b;
+  const char* wbase = (const char*)p.w;
+  const int ktiles = p.K / BK;
+  int kt_req = 0, stage_req = 0;
+  auto request = [&]() __attribute__((always_inline)) {
+    // (requests past the end repeat the last step into a stage nobody reads any more: the wait counts stay exact)
+    const uint32_t sb = smem_base + stage_req * MSTAGE_B;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma16(xbase, xoff[j], sb + (wave + 4 * j) * 1024);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma16(wbase, woff[j], sb + MXT_B + (wave + 4 * j) * 1024);
+    if (++kt_req < ktiles) {
+      xbase += BK * 2;
+      wbase += (long)BK * w_row_b;
+    }
+    stage_req = stage_req + 1 == MNST ? 0 : stage_req + 1;
+  };
+
+  int x_off[4], w_off[2];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) x_off[s] = (64 * wm + n) * 128 + (((2 * s + h) ^ ((n >> 1) & 7)) << 4);
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int row = 8 * h + (sl >> 2);
+    const int y = 2 * (g & 1) + ((sl & 3) >> 1);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) w_off[c] = MXT_B + row * 256 + (((4 * (2 * wn + c) + y) ^ (4 * (row & 3))) << 4) + (sl & 1) * 8;
+  }
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mb][c][i] = 0.f;
+
+  auto load_x = [&](bf16x8_t (&xf)[2], int stage, int s) __attribute__((always_inline)) {
+    const char* b = smem + stage * MSTAGE_B + x_off[s];
+    xf[0] = *(const bf16x8_t*)b;
+    xf[1] = *(const bf16x8_t*)(b + 32 * 128);
+  };
+  auto load_w = [&](bf16x8_t (&wf)[2], int stage, int s) __attribute__((always_inline)) {
+    const char* b = smem + stage * MSTAGE_B + 16 * s * 256;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const lds_char* src = (const lds_char*)(b + w_off[c]);
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 4 * 256));
+      struct { s16x4_t a, b; } pair = {lo, hi};
+      wf[c] = __builtin_bit_cast(bf16x8_t, pair);
+    }
+  };
+  auto mma = [&](const bf16x8_t (&wf)[2], const bf16x8_t (&xf)[2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        acc[mb][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[c], xf[mb], acc[mb][c], 0, 0, 0);
+  };
+
+#pragma unroll
+  for (int s = 0; s < MNST - 1; ++s) request();
+  int stage = 0;
+  for (int kt = 0; kt < ktiles; ++kt) {
+    wait_vmcnt<(MNST - 2) * 8>();          // this wave's part of step kt has landed (8 copies per wave and step)
+    __builtin_amdgcn_s_barrier();          // ... and everyone's; all waves are done with step kt - 1
+    request();
+    bf16x8_t wa[2], wb[2], xa[2], xb[2];
+    load_w(wa, stage, 0); load_x(xa, stage, 0);
+    load_w(wb, stage, 1); load_x(xb, stage, 1);
+    mma(wa, xa);
+    load_w(wa, stage, 2); load_x(xa, stage, 2);
+    mma(wb, xb);
+    load_w(wb, stage, 3); load_x(xb, stage, 3);
+    mma(wa, xa);
+    mma(wb, xb);
+    stage = stage + 1 == MNST ? 0 : stage + 1;
+  }
+  wait_vmcnt<0>();                         // nothing may still be landing in LDS
+
+  __builtin_amdgcn_s_barrier();            // every wave is done reading the ring
+  uint16_t* out = (uint16_t*)p.out;
+  constexpr int PROW_B = 128 + 8;
+  char* patch = smem + wave * (32 * PROW_B);
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int col = 32 * c + 8 * i4 + 4 * h;           // column inside the wave's 64
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (BIAS) {
+          const int gc = min(n0 + 64 * wn + col, p.N - 4);
+          const uint2 bw = *(const uint2*)((const uint16_t*)p.bias + gc);
+          b0 = bf16_bits_to_float(bw.x & 0xffffu); b1 = bf16_bits_to_float(bw.x >> 16);
+          b2 = bf16_bits_to_float(bw.y & 0xffffu); b3 = bf16_bits_to_float(bw.y >> 16);
+        }
+        const uint32_t w0 = pack_bf16x2(acc[mb][c][4 * i4] + b0, acc[mb][c][4 * i4 + 1] + b1);
+        const uint32_t w1 = pack_bf16x2(acc[mb][c][4 * i4 + 2] + b2, acc[mb][c][4 * i4 + 3] + b3);
+        *(uint2*)(patch + n * PROW_B + 2 * col) = make_uint2(w0, w1);
+      }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = 8 * j + (lane >> 3), ch = lane & 7;
+      const uint2 lo = *(const uint2*)(patch + r * PROW_B + 16 * ch), hi = *(const uint2*)(patch + r * PROW_B + 16 * ch + 8);
+      const int m = m0 + 64 * wm + 32 * mb + r, col = n0 + 64 * wn + 8 * ch;
+      if (m < p.M && col < p.N) *(uint4*)(out + (long)m * p.N + col) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+  }
+}
+
 // Few rows (decode: M = batch, or a verify step): the work is w's bytes, once.  One workgroup of 4 waves per
 // 64 output columns owns ALL rows (BM = 32 MBT of them) and streams its 128-byte-wide column slab of w through
 // a deep ring of small stages (K step 64: w tile [64 k][128 B] + x tile [BM][128 B]), so that N / 64
@@ -343,11 +501,42 @@ hipError_t launch_skinny(const OProjParams& p, hipStream_t s) {
 
 }  // namespace
 
+static std::atomic<int> g_o_proj_force_large{0};
+void o_proj_debug_force_large(int on) { g_o_proj_force_large = on; }
+
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
   // up to 256 rows: one workgroup per 64 columns owns every row (the call is bound by w's bytes)
   if (p.M <= 64) return launch_skinny<2>(p, s);
   if (p.M <= 128) return launch_skinny<4>(p, s);
   if (p.M <= 256) return launch_skinny<8>(p, s);
+  {
+    // fewer large tiles than CUs (256 on this part): the 128 x 128 form fills the device better
+    const long big_tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    if (big_tiles < 224 && !g_o_proj_force_large) {
+      const long MTm = (p.M + MBM - 1) / MBM, NTm = (p.N + MBN - 1) / MBN;
+      const long total_m = 8 * ((MTm + 7) / 8) * 4 * ((NTm + 3) / 4);
+      if (total_m > 0x7fffffffL) return hipErrorInvalidValue;
+      const bool deep = MTm * NTm <= 256;
+      static std::atomic<int> configured_mid{0};
+      if (!configured_mid.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute((const void*)o_proj_mid_kernel<false, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * MSTAGE_B);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_mid_kernel<true, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * MSTAGE_B);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_mid_kernel<false, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 4 * MSTAGE_B);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_mid_kernel<true, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 4 * MSTAGE_B);
+        if (e != hipSuccess) return e;
+        configured_mid.store(1, std::memory_order_release);
+      }
+      const dim3 grid((unsigned)total_m), wg(256);
+      if (deep) {
+        if (p.bias) hipLaunchKernelGGL((o_proj_mid_kernel<true, 4>), grid, wg, 4 * MSTAGE_B, s, p);
+        else hipLaunchKernelGGL((o_proj_mid_kernel<false, 4>), grid, wg, 4 * MSTAGE_B, s, p);
+      } else {
+        if (p.bias) hipLaunchKernelGGL((o_proj_mid_kernel<true, 2>), grid, wg, 2 * MSTAGE_B, s, p);
+        else hipLaunchKernelGGL((o_proj_mid_kernel<false, 2>), grid, wg, 2 * MSTAGE_B, s, p);
+      }
+      return hipGetLastError();
+    }
+  }
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute((const void*)o_proj_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_B);

@@ -44,6 +44,30 @@ def test_o_proj_vs_oracle(pa, M, K, N, bias):
     _close(dev_to_f32(got), want)
 
 
+@pytest.mark.parametrize("M,K,N,bias,force_large", [(1100, 256, 4096, True, False),   # 128 x 128 tiles, more tiles than CUs (two-stage ring)
+                                                    (700, 320, 1032, False, False),    # 128 x 128 tiles, deep ring, ragged edges
+                                                    (700, 320, 1032, True, True),      # the same through the 256 x 256 tiles
+                                                    (3900, 128, 4096, False, False)])  # enough 256 x 256 tiles by itself
+def test_o_proj_tile_forms(pa, M, K, N, bias, force_large):
+    """The row counts between the few-rows form and a device full of 256 x 256 tiles take 128 x 128 tiles; debug
+    switch 8 sends them through the large tiles instead.  Both against the oracle."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(M + N + int(force_large))
+    x = O.round_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = O.round_to_bf16((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32))
+    b = O.round_to_bf16(rng.standard_normal(N).astype(np.float32)) if bias else None
+    want = O.o_proj(x, w, b)
+    print(f"o_proj tile forms M={M} K={K} N={N} bias={bias} force_large={force_large}", flush=True)
+    lib.pa_debug_set(8, 1 if force_large else 0)
+    try:
+        got = pa.o_proj(bf16_to_dev(x), bf16_to_dev(w), None if b is None else bf16_to_dev(b))
+        torch.cuda.synchronize()
+    finally:
+        lib.pa_debug_set(8, 0)
+    _close(dev_to_f32(got), want)
+
+
 def test_identity_and_permutation_weights_move_bits(pa, rng):
     """Exact cases: an identity weight returns x bit for bit (which also pins the [.., Hq, D] -> [.., Hq*D]
     view), a column permutation permutes it, a zero x returns the bias in every row."""
