@@ -388,6 +388,7 @@ __global__ __launch_bounds__(256) void o_proj_skinny_kernel(OProjParams p) {
   const int n = lane & 31, h = lane >> 5;
   const int nb = wave & 1, mpar = wave >> 1;
   const int n0 = blockIdx.x * 64;
+  const int m0 = blockIdx.y * SBM;         // (more rows than one workgroup owns: a second grid dimension of row blocks)
 
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
   const long x_row_b = (long)p.K * 2, w_row_b = (long)p.N * 2;
@@ -397,7 +398,7 @@ __global__ __launch_bounds__(256) void o_proj_skinny_kernel(OProjParams p) {
 #pragma unroll
   for (int j = 0; j < XU / 4; ++j) {
     const int lrow = 8 * (wave + 4 * j) + (lane >> 3);
-    xoff[j] = (uint32_t)(min(lrow, p.M - 1) * x_row_b) + (uint32_t)(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);
+    xoff[j] = (uint32_t)(min(m0 + lrow, p.M - 1) * x_row_b) + (uint32_t)(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);
   }
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -465,7 +466,7 @@ __global__ __launch_bounds__(256) void o_proj_skinny_kernel(OProjParams p) {
   uint16_t* out = (uint16_t*)p.out;
 #pragma unroll
   for (int i = 0; i < MBT / 2; ++i) {
-    const int m = 32 * (2 * i + mpar) + n;
+    const int m = m0 + 32 * (2 * i + mpar) + n;
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
       const int col = n0 + 32 * nb + 8 * i4 + 4 * h;
@@ -493,9 +494,9 @@ hipError_t launch_skinny(const OProjParams& p, hipStream_t s) {
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
   }
-  const unsigned grid = (unsigned)((p.N + 63) / 64);
-  if (p.bias) hipLaunchKernelGGL((o_proj_skinny_kernel<MBT, true>), dim3(grid), dim3(256), lds, s, p);
-  else hipLaunchKernelGGL((o_proj_skinny_kernel<MBT, false>), dim3(grid), dim3(256), lds, s, p);
+  const dim3 grid((unsigned)((p.N + 63) / 64), (unsigned)((p.M + 32 * MBT - 1) / (32 * MBT)));
+  if (p.bias) hipLaunchKernelGGL((o_proj_skinny_kernel<MBT, true>), grid, dim3(256), lds, s, p);
+  else hipLaunchKernelGGL((o_proj_skinny_kernel<MBT, false>), grid, dim3(256), lds, s, p);
   return hipGetLastError();
 }
 
@@ -508,6 +509,10 @@ hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
   // up to 256 rows: one workgroup per 64 columns owns every row (the call is bound by w's bytes)
   if (p.M <= 64) return launch_skinny<2>(p, s);
   if (p.M <= 128) return launch_skinny<4>(p, s);
+  // a few hundred rows: the 128-row form over several row blocks as long as its workgroups (N / 64 per block) fit
+  // the device in one go; measured against the other forms at K = N = 4096
+  if (!g_o_proj_force_large && (long)((p.M + 127) / 128) * ((p.N + 63) / 64) <= 256 && (long)p.M * p.K * 2 < 0x7fffffffL)
+    return launch_skinny<4>(p, s);
   if (p.M <= 256) return launch_skinny<8>(p, s);
   {
     // fewer large tiles than CUs (256 on this part): the 128 x 128 form fills the device better
