@@ -45,12 +45,14 @@ def test_o_proj_vs_oracle(pa, M, K, N, bias):
 
 
 @pytest.mark.parametrize("M,K,N,bias,force_large", [(1100, 256, 4096, True, False),   # 128 x 128 tiles, more tiles than CUs (two-stage ring)
-                                                    (700, 320, 1032, False, False),    # 128 x 128 tiles, deep ring, ragged edges
+                                                    (900, 320, 2880, False, False),    # 128 x 128 tiles, deep ring, ragged edges
+                                                    (700, 320, 1032, True, False),     # the 128-row few-rows form over 6 row blocks
                                                     (700, 320, 1032, True, True),      # the same through the 256 x 256 tiles
                                                     (3900, 128, 4096, False, False)])  # enough 256 x 256 tiles by itself
 def test_o_proj_tile_forms(pa, M, K, N, bias, force_large):
-    """The row counts between the few-rows form and a device full of 256 x 256 tiles take 128 x 128 tiles; debug
-    switch 8 sends them through the large tiles instead.  Both against the oracle."""
+    """A few hundred rows take the 128-row few-rows form over several row blocks, the row counts between those and a
+    device full of 256 x 256 tiles take 128 x 128 tiles; debug switch 8 sends them through the large tiles instead.
+    All against the oracle."""
     from nkipy_amd import _lib
     lib = _lib.load()
     rng = np.random.default_rng(M + N + int(force_large))
