@@ -20,85 +20,122 @@
 // they are stored, and a second kernel does the same to Q in place.  A row of D elements is
 // held by D/8 consecutive lanes, 8 elements each; the mean of squares is a butterfly over
 // those lanes and the rotation partner (element i <-> i + D/2) sits D/16 lanes away.
+#include <type_traits>
+
 #include "pa_common.h"
+
+#define PA_HD __device__ __forceinline__
+#include "pa_div.h"
 
 namespace pa {
 namespace {
 
 constexpr int WG = 256;
+#ifndef QWG_
+#define QWG_ 256
+#define QUNR_ 2
+#endif
+constexpr int QWG = QWG_, QUNR = QUNR_;
 
-// RMSNorm (if w) and RoPE of one 8-element chunk c of a row held by `cpr` consecutive lanes.
-// x: the chunk's values; all lanes of the row call this together.  Arithmetic as the
-// reference's bf16 tensors give it: the norm in float32 rounded once to bf16, every product
-// and sum of the rotation rounded to bf16.
+// RMSNorm (if w) and RoPE of 8-element chunks of rows held by `cpr` consecutive lanes each.
+// Arithmetic as the reference's bf16 tensors give it: the norm in float32 rounded once to bf16,
+// every product and sum of the rotation rounded to bf16.
+
 // value of lane ^ MASK (MASK a power of two below 32) without a trip through LDS memory
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float v) {
   if (MASK == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128 /* row_ror:8 */, 0xf, 0xf, true));
   return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (MASK << 10) | 0x1f));   // bit mode: and 0x1f, or 0, xor MASK
 }
-// CPR: lanes (8-element chunks) per row = D / 8, a compile-time power of two
+// Step MASK of a butterfly sum over aligned groups of lanes, steps taken in the order 1, 2, 4, ...: v + the value
+// of a lane of the other half of the 2 MASK group.  Before step MASK all lanes of a MASK group hold the same
+// partial sum, so any lane of the other half serves, and the data-parallel-primitive forms of the adds reach one:
+// the quad permutations for 1 and 2, the mirror of 8 lanes for 4, of 16 lanes for 8.
+template <int MASK>
+__device__ __forceinline__ float butterfly_add(float v) {
+  constexpr int ctrl = MASK == 1 ? 0xB1 /* quad_perm [1,0,3,2] */ : MASK == 2 ? 0x4E /* quad_perm [2,3,0,1] */
+                     : MASK == 4 ? 0x141 /* row_half_mirror */ : 0x140 /* row_mirror */;
+  if (MASK <= 8) return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xf, 0xf, true));
+  return v + lane_xor<MASK>(v);
+}
+// two float32 -> two bf16 (round to nearest even) in one instruction, as one opaque operation: written as two
+// scalar conversions the compiler takes the pair apart again where the halves are used separately
+__device__ __forceinline__ uint32_t round2_bf16(float lo, float hi) {
+  uint32_t w;
+  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(lo), "v"(hi));
+  return w;
+}
+__device__ __forceinline__ void unpack_bf16x8(const uint4& v, float (&x)[8]) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    x[2 * j] = __uint_as_float(w[j] << 16);
+    x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+  }
+}
+
+// What chunk c of a row needs of the position's cos / sin rows: 8 cosines and 8 sines as float32, the sines
+// negated in the first half of the row.  First half: x0 c - x1 s with x0 = own; second half: x0 s + x1 c with
+// x1 = own.  Both are round(round(own c) + round(other s')) with s' = -s in the first half: rounding to nearest
+// even is symmetric in sign and the sum commutes, so the bits are those of the two written-out forms.
 template <int CPR>
-__device__ __forceinline__ void norm_rope_chunk(float (&x)[8], int c, const uint16_t* w, float eps,
-                                                const uint16_t* cos_row, const uint16_t* sin_row) {
+struct RopeCoeffs {
+  float cs[8], sn[8];
+  __device__ __forceinline__ void load(int c, const uint16_t* cos_row, const uint16_t* sin_row) {
+    constexpr int hc = CPR / 2;
+    const bool first = c < hc;
+    const int fi = 8 * (first ? c : c - hc);
+    const uint4 cw = *(const uint4*)(cos_row + fi);
+    uint4 sw = *(const uint4*)(sin_row + fi);
+    const uint32_t flip = first ? 0x80008000u : 0u;      // the sign, two elements per instruction
+    sw.x ^= flip; sw.y ^= flip; sw.z ^= flip; sw.w ^= flip;
+    unpack_bf16x8(cw, cs);
+    unpack_bf16x8(sw, sn);
+  }
+};
+
+// CPR: lanes (8-element chunks) per row = D / 8, a compile-time power of two.  x: the chunk's values; all
+// lanes of the row call this together.  wf: the chunk's norm weights (used if `norm`).  Returns the chunk
+// as it is stored.
+template <int CPR>
+__device__ __forceinline__ uint4 norm_rope_chunk(float (&x)[8], bool norm, const float (&wf)[8], float eps, const RopeCoeffs<CPR>& rc) {
   constexpr int D = 8 * CPR;
-  // (roundings to bf16 go through the conversion instruction, round to nearest even, two values at a time)
-  if (w) {
+  if (norm) {
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
-    if (CPR > 1) ss += lane_xor<1>(ss);
-    if (CPR > 2) ss += lane_xor<2>(ss);
-    if (CPR > 4) ss += lane_xor<4>(ss);
-    if (CPR > 8) ss += lane_xor<8>(ss);
-    if (CPR > 16) ss += lane_xor<16>(ss);
+    if (CPR > 1) ss = butterfly_add<1>(ss);
+    if (CPR > 2) ss = butterfly_add<2>(ss);
+    if (CPR > 4) ss = butterfly_add<4>(ss);
+    if (CPR > 8) ss = butterfly_add<8>(ss);
+    if (CPR > 16) ss = butterfly_add<16>(ss);
     // x / sqrt(mean + eps) as x * rsq(...): within 2 float32 ulp of the divided form, far below
     // the bf16 rounding that follows
     const float inv = __builtin_amdgcn_rsqf(__fdiv_rn(ss, (float)D) + eps);
-    const uint4 ww = *(const uint4*)(w + 8 * c);
-    const uint32_t wv[4] = {ww.x, ww.y, ww.z, ww.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t r = pack_bf16x2((x[2 * j] * inv) * bf16_bits_to_float(wv[j] & 0xffffu), (x[2 * j + 1] * inv) * bf16_bits_to_float(wv[j] >> 16));
+      const uint32_t r = round2_bf16((x[2 * j] * inv) * wf[2 * j], (x[2 * j + 1] * inv) * wf[2 * j + 1]);
       x[2 * j] = __uint_as_float(r << 16);
       x[2 * j + 1] = __uint_as_float(r & 0xffff0000u);
     }
   }
   constexpr int hc = CPR / 2;
-  const bool first = c < hc;
-  const int fi = 8 * (first ? c : c - hc);
-  const uint4 cw = *(const uint4*)(cos_row + fi);
-  uint4 sw = *(const uint4*)(sin_row + fi);
-  // first half: x0 c - x1 s with x0 = own; second half: x0 s + x1 c with x1 = own.  Both are
-  // round(round(own c) + round(other s')) with s' = -s in the first half: rounding to nearest even is
-  // symmetric in sign and the sum commutes, so the bits are those of the two written-out forms.  The sign
-  // goes into the packed sine words, two elements per instruction.
-  const uint32_t flip = first ? 0x80008000u : 0u;
-  sw.x ^= flip; sw.y ^= flip; sw.z ^= flip; sw.w ^= flip;
-  float cs[8], sn[8];
-  {
-    const uint32_t a[4] = {cw.x, cw.y, cw.z, cw.w}, b[4] = {sw.x, sw.y, sw.z, sw.w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      cs[2 * j] = bf16_bits_to_float(a[j] & 0xffffu); cs[2 * j + 1] = bf16_bits_to_float(a[j] >> 16);
-      sn[2 * j] = bf16_bits_to_float(b[j] & 0xffffu); sn[2 * j + 1] = bf16_bits_to_float(b[j] >> 16);
-    }
-  }
-  // two roundings per conversion instruction
-  auto r16x2 = [](float& f0, float& f1) __attribute__((always_inline)) {
-    const uint32_t w = pack_bf16x2(f0, f1);
-    f0 = __uint_as_float(w << 16);
-    f1 = __uint_as_float(w & 0xffff0000u);
-  };
+  uint32_t o[4];
 #pragma unroll
   for (int j = 0; j < 8; j += 2) {
-    float a0 = x[j] * cs[j], a1 = x[j + 1] * cs[j + 1];
-    float b0 = lane_xor<hc>(x[j]) * sn[j], b1 = lane_xor<hc>(x[j + 1]) * sn[j + 1];
-    r16x2(a0, a1);
-    r16x2(b0, b1);
-    float s0 = a0 + b0, s1 = a1 + b1;
-    r16x2(s0, s1);
-    x[j] = s0; x[j + 1] = s1;
+    const uint32_t a = round2_bf16(x[j] * rc.cs[j], x[j + 1] * rc.cs[j + 1]);
+    const uint32_t b = round2_bf16(lane_xor<hc>(x[j]) * rc.sn[j], lane_xor<hc>(x[j + 1]) * rc.sn[j + 1]);
+    o[j / 2] = round2_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
+                           __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+__device__ __forceinline__ void load_norm_weights(const uint16_t* w, int c, float (&wf)[8]) {
+  if (w) {
+    unpack_bf16x8(*(const uint4*)(w + 8 * c), wf);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) wf[j] = 1.f;
   }
 }
 
@@ -110,10 +147,6 @@ __device__ __forceinline__ void unpack8(const uint4& v, float (&x)[8]) {
     x[2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
   }
 }
-__device__ __forceinline__ uint4 pack8(const float (&x)[8]) {   // values already bf16-representable or to be rounded
-  return make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));
-}
-
 __device__ __forceinline__ float block_max(float v, float* red) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
@@ -167,27 +200,39 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
 
   // K rows of a transforming write: RMSNorm + RoPE at the row's absolute position
   const bool xf = XFORM && which == 0;
-  auto load_row_chunk = [&](const uint16_t* s0, int r, int c, int cpr) __attribute__((always_inline)) -> uint4 {
+  auto load_row_chunk = [&](const uint16_t* s0, int r, int c) __attribute__((always_inline)) -> uint4 {
     uint4 v = *(const uint4*)(s0 + (long)r * row_elems + c * 8);
     if (xf) {
       const int pos = min(jb * bs + lo + r, p.rope_max_pos - 1);
-      float x[8];
+      float x[8], wf[8];
       unpack8(v, x);
-      norm_rope_chunk<XFORM ? XCPR : 2>(x, c, p.k_norm_weight, p.norm_eps, p.rope_cos + (long)pos * (D / 2), p.rope_sin + (long)pos * (D / 2));
-      v = pack8(x);
+      RopeCoeffs<XFORM ? XCPR : 2> rc;
+      rc.load(c, p.rope_cos + (long)pos * (D / 2), p.rope_sin + (long)pos * (D / 2));
+      load_norm_weights(p.k_norm_weight, c, wf);
+      v = norm_rope_chunk<XFORM ? XCPR : 2>(x, p.k_norm_weight != nullptr, wf, p.norm_eps, rc);
     }
     return v;
   };
 
+  // Chunk i = threadIdx.x + k WG of the slab is chunk c of row r; (r, c) walk along with i without divisions
+  // (`cpr` is a run-time number for the plain kernels).
+  const int cpr = XFORM ? XCPR : D * ESZ / (ESZ == 1 ? 8 : 16);   // chunks per row
+  const int total = n * cpr;
+  const int r_first = threadIdx.x / cpr, c_first = threadIdx.x - r_first * cpr;
+  const int dr = WG / cpr, dc = WG - dr * cpr;
+  auto advance = [&](int& r, int& c) __attribute__((always_inline)) {
+    r += dr; c += dc;
+    if (c >= cpr) { c -= cpr; ++r; }
+  };
+
   if (ESZ != 1) {
     // ---- copy: 16 bytes per thread and step
-    const int cpr = D * ESZ / 16;               // chunks per row
     const char* s0 = src + (((long)b * p.T + t0) * row_elems + (long)h * D) * ESZ;
     char* d0 = dst + (((long)blk * bs + lo) * row_elems + (long)h * D) * ESZ;
-    for (int i = threadIdx.x; i < n * cpr; i += WG) {
-      const int r = i / cpr, c = i - r * cpr;
+    int r = r_first, c = c_first;
+    for (int i = threadIdx.x; i < total; i += WG, advance(r, c)) {
       uint4 v;
-      if (ESZ == 2 && XFORM) v = load_row_chunk((const uint16_t*)s0, r, c, cpr);
+      if (ESZ == 2 && XFORM) v = load_row_chunk((const uint16_t*)s0, r, c);
       else v = *(const uint4*)(s0 + (long)r * row_elems * ESZ + c * 16);
       *(uint4*)(d0 + (long)r * row_elems * ESZ + c * 16) = v;
     }
@@ -196,7 +241,6 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
 
   // ---- fp8: source rows are bf16, 8 elements (16 B in, 8 B out) per thread and step
   float* scale_tbl = which ? p.v_scale : p.k_scale;
-  const int cpr = D / 8;
   const uint16_t* s0 = (const uint16_t*)src + ((long)b * p.T + t0) * row_elems + (long)h * D;
   uint8_t* d_blk = (uint8_t*)dst + (long)blk * bs * row_elems + (long)h * D;
   const float s_old = lo > 0 ? scale_tbl[(long)blk * p.Hkv + h] : 0.f;   // read before anyone rewrites it
@@ -214,19 +258,15 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
       amax = fmaxf(amax, fabsf(bf16_bits_to_float(w[j] >> 16)));
     }
   };
+  {
+    int r = r_first, c = c_first, i = threadIdx.x;
 #pragma unroll
-  for (int k = 0; k < HOLD; ++k) {
-    const int i = threadIdx.x + k * WG;
-    held[k] = make_uint4(0, 0, 0, 0);
-    if (i < n * cpr) {
-      const int r = i / cpr, c = i - r * cpr;
-      held[k] = load_row_chunk(s0, r, c, cpr);
+    for (int k = 0; k < HOLD; ++k, i += WG, advance(r, c)) {
+      held[k] = make_uint4(0, 0, 0, 0);
+      if (i < total) held[k] = load_row_chunk(s0, r, c);
+      chunk_absmax(held[k]);
     }
-    chunk_absmax(held[k]);
-  }
-  for (int i = threadIdx.x + HOLD * WG; i < n * cpr; i += WG) {
-    const int r = i / cpr, c = i - r * cpr;
-    chunk_absmax(load_row_chunk(s0, r, c, cpr));
+    for (; i < total; i += WG, advance(r, c)) chunk_absmax(load_row_chunk(s0, r, c));
   }
   amax = block_max(amax, red);
   float s_new = fmaxf(s_old, __fdiv_rn(amax, 448.f));
@@ -249,63 +289,90 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
       *q = o;
     }
   }
-  auto encode_store = [&](const uint4& v, int i) __attribute__((always_inline)) {
-    const int r = i / cpr, c = i - r * cpr;
+  // x / s_new of the bf16 values x: the same bits from a product with the reciprocal and one correction
+  // (pa_div.h) wherever s_new allows it, which is everywhere but at the far ends of the float32 range
+  const float r_new = pa_refine_rcp(s_new, __builtin_amdgcn_rcpf(s_new));
+  auto encode_store = [&](auto fast, const uint4& v, int r, int c) __attribute__((always_inline)) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     float f[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      f[2 * j] = __fdiv_rn(bf16_bits_to_float(w[j] & 0xffffu), s_new);
-      f[2 * j + 1] = __fdiv_rn(bf16_bits_to_float(w[j] >> 16), s_new);
+      const float x0 = bf16_bits_to_float(w[j] & 0xffffu), x1 = bf16_bits_to_float(w[j] >> 16);
+      f[2 * j] = decltype(fast)::value ? pa_div_by(x0, s_new, r_new) : __fdiv_rn(x0, s_new);
+      f[2 * j + 1] = decltype(fast)::value ? pa_div_by(x1, s_new, r_new) : __fdiv_rn(x1, s_new);
     }
     uint2 o;
     o.x = pack_fp8x2(f[0], f[1], 0u, false); o.x = pack_fp8x2(f[2], f[3], o.x, true);
     o.y = pack_fp8x2(f[4], f[5], 0u, false); o.y = pack_fp8x2(f[6], f[7], o.y, true);
     *(uint2*)(d_blk + (long)(lo + r) * row_elems + c * 8) = o;
   };
+  auto encode_all = [&](auto fast) __attribute__((always_inline)) {
+    int r = r_first, c = c_first, i = threadIdx.x;
 #pragma unroll
-  for (int k = 0; k < HOLD; ++k) {
-    const int i = threadIdx.x + k * WG;
-    if (i < n * cpr) encode_store(held[k], i);
-  }
-  for (int i = threadIdx.x + HOLD * WG; i < n * cpr; i += WG) {
-    const int r = i / cpr, c = i - r * cpr;
-    encode_store(load_row_chunk(s0, r, c, cpr), i);
-  }
+    for (int k = 0; k < HOLD; ++k, i += WG, advance(r, c))
+      if (i < total) encode_store(fast, held[k], r, c);
+    for (; i < total; i += WG, advance(r, c)) encode_store(fast, load_row_chunk(s0, r, c), r, c);
+  };
+  if (pa_div_by_ok(s_new, __float_as_uint(s_new))) encode_all(std::true_type{});
+  else encode_all(std::false_type{});
   if (threadIdx.x == 0) scale_tbl[(long)blk * p.Hkv + h] = s_new;
 }
 
 // Q rows: RMSNorm + RoPE in place (or into q_out); rows t >= query_lens[b] become zeros.
 // One workgroup per token (b, t): its Hq rows share the position, so no index arithmetic
-// beyond the head stride is done per row.
-template <int CPR>
-__global__ __launch_bounds__(WG) void q_norm_rope_kernel(KvWriteParams p) {
-  constexpr int D = 8 * CPR, cpr = CPR;
+// beyond the head stride is done per row.  A thread asks for UNR of its rows before it looks
+// at the lengths (q_in holds all B * T tokens, so the addresses are valid for dead tokens too):
+// the row loads do not wait behind the lengths -> position -> table-row chain, and UNR of them
+// are in flight per lane.
+template <int CPR, int WGQ, int UNR>
+__global__ __launch_bounds__(WGQ) void q_norm_rope_kernel(KvWriteParams p) {
+  constexpr int D = 8 * CPR, cpr = CPR, hstep = WGQ / cpr;
   const int t = blockIdx.x, b = blockIdx.y;
-  const int c = threadIdx.x % cpr, h0 = threadIdx.x / cpr, hstep = WG / cpr;
+  const int c = threadIdx.x % cpr, h0 = threadIdx.x / cpr;
+  const long tok = ((long)b * p.T + t) * p.Hq;
+  if (h0 >= p.Hq) return;
+  uint4 v[UNR];
+  auto load_rows = [&](int hb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      v[u] = make_uint4(0, 0, 0, 0);
+      if (hb + u * hstep < p.Hq) v[u] = *(const uint4*)((const uint16_t*)p.q_in + (tok + hb + u * hstep) * D + c * 8);
+    }
+  };
+  load_rows(h0);
   int tq = p.query_lens[b];
   tq = min(max(tq, 0), p.T);
   const int start = p.seq_lens[b] - tq;
   const bool live = t < tq && start >= 0;
   const int pos = min(max(start + t, 0), p.rope_max_pos - 1);
-  const long tok = ((long)b * p.T + t) * p.Hq;
-  for (int hq = h0; hq < p.Hq; hq += hstep) {
-    const long off = (tok + hq) * D + c * 8;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (live) {
-      v = *(const uint4*)((const uint16_t*)p.q_in + off);
-      float x[8];
-      unpack8(v, x);
-      norm_rope_chunk<CPR>(x, c, p.q_norm_weight, p.norm_eps, p.rope_cos + (long)pos * (D / 2), p.rope_sin + (long)pos * (D / 2));
-      v = pack8(x);
+  RopeCoeffs<CPR> rc;      // the token's position and the lane's chunk are the same for all its rows
+  float wf[8];
+  if (live) {
+    rc.load(c, p.rope_cos + (long)pos * (D / 2), p.rope_sin + (long)pos * (D / 2));
+    load_norm_weights(p.q_norm_weight, c, wf);
+  }
+  for (int hb = h0;;) {
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      if (hb + u * hstep >= p.Hq) break;
+      if (live) {
+        float x[8];
+        unpack8(v[u], x);
+        v[u] = norm_rope_chunk<CPR>(x, p.q_norm_weight != nullptr, wf, p.norm_eps, rc);
+      } else {
+        v[u] = make_uint4(0, 0, 0, 0);
+      }
+      *(uint4*)((uint16_t*)p.q_out + (tok + hb + u * hstep) * D + c * 8) = v[u];
     }
-    *(uint4*)((uint16_t*)p.q_out + off) = v;
+    hb += UNR * hstep;
+    if (hb >= p.Hq) break;
+    load_rows(hb);
   }
 }
 
 template <int CPR>
 void launch_xform(const KvWriteParams& p, dim3 grid, hipStream_t s) {
-  if (p.q_in) hipLaunchKernelGGL(q_norm_rope_kernel<CPR>, dim3(p.T, p.B), dim3(WG), 0, s, p);
+  if (p.q_in) hipLaunchKernelGGL((q_norm_rope_kernel<CPR, QWG, QUNR>), dim3(p.T, p.B), dim3(QWG), 0, s, p);
   if (p.kv_dtype == PA_FP8_E4M3FN) hipLaunchKernelGGL((kv_write_kernel<1, CPR>), grid, dim3(WG), 0, s, p);
   else hipLaunchKernelGGL((kv_write_kernel<2, CPR>), grid, dim3(WG), 0, s, p);
 }
