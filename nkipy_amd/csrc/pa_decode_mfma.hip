@@ -503,23 +503,37 @@ struct DecodeWave {
       }
     }
   }
-  // Split-K partials of this wave's rows: slot(row) = (hbase + row) * slots_per_head + piece
-  __device__ __forceinline__ void store_partial(long slots_per_head, long piece) const {
+  // Split-K partials of this wave's rows for piece slot `piece`.  The workspace holds, per piece slot, the
+  // rows (virtual q heads) in order; the floats of a 16-row group are laid out as the lanes hold them, not row
+  // by row: float4 number ((j * 4 + g) * nh + r) of the group is what lane (g, r) stores with its j-th
+  // instruction (nh = rows of the group, j = i * VEC / 4 + e / 4, covering d = VEC (4 g + i) + e .. + 3).  An
+  // instruction then writes one contiguous run of 64 nh bytes instead of 16-byte pieces 128 bytes apart, and
+  // the merge kernel, whose threads walk the float4s of a group in order, reads contiguously as well.  The
+  // multi-token form, with four times decode's partial bytes, stores them as streaming writes (nothing in
+  // this kernel reads them back and most are issued as the kernel ends); for decode's few megabytes the
+  // merge kernel finding them in the cache is worth more.
+  __device__ __forceinline__ void store_partial(long piece) const {
+    typedef float f4_t __attribute__((ext_vector_type(4)));
+    const long rows_total = (long)p.Hq * (MULTI ? p.T : 1);
 #pragma unroll
     for (int rg = 0; rg < R; ++rg) {
       const float l = total_l(rg);
       if (16 * rg + r >= nheads) continue;
-      const long slot = (long)(hbase + 16 * rg + r) * slots_per_head + piece;
+      const int nh = min(16, nheads - 16 * rg);
+      const long row0 = piece * rows_total + hbase + 16 * rg;
       const float inv = (MULTI && l == 0.f) ? 0.f : 1.f / l;
-      float* dst = p.ws_out + slot * D;
+      f4_t* dst = (f4_t*)(p.ws_out + row0 * D);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int e = 0; e < VEC; e += 4)
-          *(float4*)(dst + VEC * (4 * g + i) + e) =
-              make_float4(oacc[rg][e][i] * inv, oacc[rg][e + 1][i] * inv, oacc[rg][e + 2][i] * inv, oacc[rg][e + 3][i] * inv);
+        for (int e = 0; e < VEC; e += 4) {
+          const f4_t val = {oacc[rg][e][i] * inv, oacc[rg][e + 1][i] * inv, oacc[rg][e + 2][i] * inv, oacc[rg][e + 3][i] * inv};
+          f4_t* at = dst + ((i * (VEC / 4) + e / 4) * 4 + g) * nh + r;
+          if (MULTI) __builtin_nontemporal_store(val, at);
+          else *at = val;
+        }
       }
-      if (g == 0) { p.ws_ml[slot * 2] = m_run[rg]; p.ws_ml[slot * 2 + 1] = l; }
+      if (g == 0) *(float2*)(p.ws_ml + (row0 + r) * 2) = make_float2(m_run[rg], l);
     }
   }
 };
@@ -761,7 +775,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
     w.stream(ti << 5, 32, n, ctx, p.bal_lockstep != 0);
     const int c_first = start / L, c_last = (start + T - 1) / L;
     if (c_first == c_last) w.store_final(b);
-    else w.store_partial(p.B + gv, b + cv);
+    else w.store_partial(b + cv);
     f += n;
     start += T;
     ++b;
@@ -781,18 +795,28 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int start = p.ws_start[b];                   // tiles before this sequence, written by the streaming kernel
   const int T = p.ws_start[b + 1] - start;
   const int N = p.ws_start[p.B];
-  constexpr int QUADS = D / 4;
+  constexpr int QUADS = D / 4, VEC = D / 16;
   const int item = blockIdx.y * (256 / G) + threadIdx.x / G;
   const int g = threadIdx.x % G;
-  const bool mine = item < p.Hq * p.T * QUADS;
-  const int hq = item / QUADS, q4 = item % QUADS;     // hq: virtual head when p.T > 1
-  uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hq) * D + 4 * q4;
+  const int rows_total = p.Hq * p.T;                  // virtual heads (p.T = 1 for decode)
+  const bool mine = item < rows_total * QUADS;
+  // item = number of a float4 within a piece slot, in the order the streaming kernel lays them out
+  // (store_partial): which row and which four d's it is
+  const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
+  const int row_f = min(item / QUADS, rows_total - 1);
+  const int hk = row_f / n_rows, grp = (row_f - hk * n_rows) & ~15;      // kv head, first row of the 16-row group
+  const int nh = min(16, n_rows - grp);
+  const int within = item - (hk * n_rows + grp) * QUADS;                // float4 number inside the group
+  const int jg = within / nh, r = within - jg * nh;
+  const int gq = jg & 3, j = jg >> 2;
+  const int d0 = VEC * (4 * gq + j / (VEC / 4)) + 4 * (j % (VEC / 4));
+  const int hq = hk * n_rows + grp + r;               // virtual head
+  uint16_t* dst = (uint16_t*)p.out + ((long)b * p.Hq + hq) * D + d0;
   int head = hq;                                      // the real q head of this item
   if (p.query_lens) {
-    const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
-    const int hk = hq / n_rows, j = hq % n_rows, t = j / n_rep;
-    head = hk * n_rep + (j - t * n_rep);
-    dst = (uint16_t*)p.out + (((long)b * p.T_stride + p.t0 + t) * p.Hq + head) * D + 4 * q4;
+    const int jrow = grp + r, t = jrow / n_rep;
+    head = hk * n_rep + (jrow - t * n_rep);
+    dst = (uint16_t*)p.out + (((long)b * p.T_stride + p.t0 + t) * p.Hq + head) * D + d0;
   }
   if (T == 0) {
     if (mine && g == 0) *(uint2*)dst = make_uint2(0u, 0u);
@@ -802,13 +826,13 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int L = (N + gv - 1) / gv;
   const int c_first = start / L, c_last = (start + T - 1) / L;
   if (c_first == c_last || !mine) return;   // single piece: written by the streaming kernel
-  const long base_slot = (long)hq * (p.B + gv) + b;
   float m = -INFINITY, l = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
   for (int c = c_first + g; c <= c_last; c += G) {
-    const float2 ml = *(const float2*)(p.ws_ml + (base_slot + c) * 2);
-    const float4 o = *(const float4*)(p.ws_out + (base_slot + c) * D + 4 * q4);
+    const long slot = (long)(b + c) * rows_total;
+    const float2 ml = *(const float2*)(p.ws_ml + (slot + hq) * 2);
+    const float4 o = *((const float4*)(p.ws_out + slot * D) + item);
     const float m_new = fmaxf(m, ml.x);
     const float m_ref = m_new == -INFINITY ? 0.f : m_new;   // pieces in which a row saw no key carry m = -inf, l = 0
     const float a = exp2f(m - m_ref);
@@ -892,7 +916,7 @@ void plan_decode_balanced(DecodeParams& p, int num_cus) {
 }
 
 size_t decode_balanced_workspace_bytes(int B, int Hq, int D, int gv) {
-  // partials [Hq][B + gv][D + 2] floats, then B + 1 tile prefix sums
+  // partials [B + gv piece slots][Hq rows][D + 2] floats, then B + 1 tile prefix sums
   return (size_t)Hq * ((size_t)B + gv) * ((size_t)D + 2) * sizeof(float) + ((size_t)B + 1) * sizeof(int32_t);
 }
 
