@@ -31,11 +31,14 @@ namespace pa {
 namespace {
 
 constexpr int WG = 256;
-#ifndef QWG_
-#define QWG_ 256
-#define QUNR_ 2
-#endif
-constexpr int QWG = QWG_, QUNR = QUNR_;
+// Waves per SIMD the write kernels are compiled for: their workgroups are short chains of dependent loads, so
+// residency counts, but a register budget that makes the compiler spill costs more (a reload from scratch waits
+// for every outstanding store as well).  6 (70 registers) for the plain forms, 4 (109) for the transforming fp8
+// form, which holds four fetched chunks with their cos / sin pieces.  Measured on the KV-write and pre-attention
+// workloads: (8, 8) 25.9 / 118.8 us per step, (6, 4) 20.0 / 85.6, (4, 4) 21.1 / 85.1.
+constexpr int KVW_MIN_WAVES = 6, KVW_MIN_WAVES_XFORM = 4;
+// The Q kernel: threads per workgroup and rows a thread has in flight (128 x 4 and 64 x 8 measured the same).
+constexpr int QWG = 256, QUNR = 2;
 
 // RMSNorm (if w) and RoPE of 8-element chunks of rows held by `cpr` consecutive lanes each.
 // Arithmetic as the reference's bf16 tensors give it: the norm in float32 rounded once to bf16,
@@ -81,16 +84,23 @@ __device__ __forceinline__ void unpack_bf16x8(const uint4& v, float (&x)[8]) {
 template <int CPR>
 struct RopeCoeffs {
   float cs[8], sn[8];
-  __device__ __forceinline__ void load(int c, const uint16_t* cos_row, const uint16_t* sin_row) {
+  // the 16 bytes of each table row that chunk c needs, as they lie in memory
+  static __device__ __forceinline__ void fetch(int c, const uint16_t* cos_row, const uint16_t* sin_row, uint4& cw, uint4& sw) {
     constexpr int hc = CPR / 2;
-    const bool first = c < hc;
-    const int fi = 8 * (first ? c : c - hc);
-    const uint4 cw = *(const uint4*)(cos_row + fi);
-    uint4 sw = *(const uint4*)(sin_row + fi);
-    const uint32_t flip = first ? 0x80008000u : 0u;      // the sign, two elements per instruction
+    const int fi = 8 * (c < hc ? c : c - hc);
+    cw = *(const uint4*)(cos_row + fi);
+    sw = *(const uint4*)(sin_row + fi);
+  }
+  __device__ __forceinline__ void set(int c, const uint4& cw, uint4 sw) {
+    const uint32_t flip = c < CPR / 2 ? 0x80008000u : 0u;      // the sign, two elements per instruction
     sw.x ^= flip; sw.y ^= flip; sw.z ^= flip; sw.w ^= flip;
     unpack_bf16x8(cw, cs);
     unpack_bf16x8(sw, sn);
+  }
+  __device__ __forceinline__ void load(int c, const uint16_t* cos_row, const uint16_t* sin_row) {
+    uint4 cw, sw;
+    fetch(c, cos_row, sin_row, cw, sw);
+    set(c, cw, sw);
   }
 };
 
@@ -170,9 +180,7 @@ __device__ __forceinline__ uint32_t pack_fp8x2(float a, float b, uint32_t old, b
 
 // ESZ: bytes per stored element (4 fp32 copy, 2 bf16 copy, 1 fp8 quantise from bf16 rows)
 template <int ESZ, int XCPR>      // XCPR: D / 8 of a transforming write, 0 for a plain one
-// (eight waves per SIMD: the workgroups are short chains of dependent loads, and more of them resident measured 2-3 % faster
-// than the 96 registers the compiler takes when left alone)
-__global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void kv_write_kernel(KvWriteParams p) {
+__global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(XCPR != 0 && ESZ == 1 ? KVW_MIN_WAVES_XFORM : KVW_MIN_WAVES, 8))) void kv_write_kernel(KvWriteParams p) {
   constexpr bool XFORM = XCPR != 0;
   __shared__ float red[WG / 64];
   const int which = blockIdx.x & 1;            // 0: K, 1: V
@@ -200,18 +208,30 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
 
   // K rows of a transforming write: RMSNorm + RoPE at the row's absolute position
   const bool xf = XFORM && which == 0;
-  auto load_row_chunk = [&](const uint16_t* s0, int r, int c) __attribute__((always_inline)) -> uint4 {
-    uint4 v = *(const uint4*)(s0 + (long)r * row_elems + c * 8);
+  // A chunk is fetched (the row's 16 bytes and, for a transforming write, the 16 bytes of the position's
+  // cos and sin rows) and then finished (transformed): callers with several chunks fetch them all first.
+  using Rope = RopeCoeffs<XFORM ? XCPR : 2>;
+  struct RawChunk { uint4 v, cw, sw; };
+  float k_wf[8];                                  // the lane's norm weights: its chunk index is the same for all its rows
+  auto fetch_chunk = [&](const uint16_t* s0, int r, int c) __attribute__((always_inline)) -> RawChunk {
+    RawChunk raw;
+    raw.v = *(const uint4*)(s0 + (long)r * row_elems + c * 8);
     if (xf) {
       const int pos = min(jb * bs + lo + r, p.rope_max_pos - 1);
-      float x[8], wf[8];
-      unpack8(v, x);
-      RopeCoeffs<XFORM ? XCPR : 2> rc;
-      rc.load(c, p.rope_cos + (long)pos * (D / 2), p.rope_sin + (long)pos * (D / 2));
-      load_norm_weights(p.k_norm_weight, c, wf);
-      v = norm_rope_chunk<XFORM ? XCPR : 2>(x, p.k_norm_weight != nullptr, wf, p.norm_eps, rc);
+      Rope::fetch(c, p.rope_cos + (long)pos * (D / 2), p.rope_sin + (long)pos * (D / 2), raw.cw, raw.sw);
     }
-    return v;
+    return raw;
+  };
+  auto finish_chunk = [&](const RawChunk& raw, int c) __attribute__((always_inline)) -> uint4 {
+    if (!xf) return raw.v;
+    float x[8];
+    unpack8(raw.v, x);
+    Rope rc;
+    rc.set(c, raw.cw, raw.sw);
+    return norm_rope_chunk<XFORM ? XCPR : 2>(x, p.k_norm_weight != nullptr, k_wf, p.norm_eps, rc);
+  };
+  auto load_row_chunk = [&](const uint16_t* s0, int r, int c) __attribute__((always_inline)) -> uint4 {
+    return finish_chunk(fetch_chunk(s0, r, c), c);
   };
 
   // Chunk i = threadIdx.x + k WG of the slab is chunk c of row r; (r, c) walk along with i without divisions
@@ -224,6 +244,7 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
     r += dr; c += dc;
     if (c >= cpr) { c -= cpr; ++r; }
   };
+  if (xf) load_norm_weights(p.k_norm_weight, c_first, k_wf);   // (XCPR divides WG: c stays c_first)
 
   if (ESZ != 1) {
     // ---- copy: 16 bytes per thread and step
@@ -259,11 +280,20 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(8, 8))) void
     }
   };
   {
+    // all HOLD fetches go out before the first is used; a chunk past the slab's end reads row 0 instead (the
+    // slab has one) and counts as zeros
     int r = r_first, c = c_first, i = threadIdx.x;
+    RawChunk raw[HOLD];
+    int ck[HOLD];
 #pragma unroll
     for (int k = 0; k < HOLD; ++k, i += WG, advance(r, c)) {
-      held[k] = make_uint4(0, 0, 0, 0);
-      if (i < total) held[k] = load_row_chunk(s0, r, c);
+      ck[k] = c;
+      raw[k] = fetch_chunk(s0, i < total ? r : 0, c);
+    }
+#pragma unroll
+    for (int k = 0; k < HOLD; ++k) {
+      const uint4 v = finish_chunk(raw[k], ck[k]);
+      held[k] = threadIdx.x + k * WG < total ? v : make_uint4(0, 0, 0, 0);
       chunk_absmax(held[k]);
     }
     for (; i < total; i += WG, advance(r, c)) chunk_absmax(load_row_chunk(s0, r, c));
