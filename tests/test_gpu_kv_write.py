@@ -36,7 +36,7 @@ def _case(rng, B, T, Hkv, D, bs, seqs, qlens, extra=2):
     return nb, tables, seqs, qlens, xk, xv
 
 
-@pytest.mark.parametrize("bs,D", [(16, 128), (32, 64), (48, 128), (64, 256)])
+@pytest.mark.parametrize("bs,D", [(16, 128), (32, 64), (48, 128), (64, 256), (16, 80), (32, 96), (16, 8)])
 def test_bf16_pool_rows_bit_exact(pa, rng, bs, D):
     B, T, Hkv = 3, 40, 2
     nb, tables, seqs, qlens, xk, xv = _case(rng, B, T, Hkv, D, bs, seqs=[40, 97, 5], qlens=[40, 33, 0])
@@ -73,7 +73,7 @@ def _to_fp8_dev(codes):
     return torch.from_numpy(codes.copy()).cuda().view(torch.float8_e4m3fn)
 
 
-@pytest.mark.parametrize("bs,D", [(16, 128), (64, 128), (32, 64)])
+@pytest.mark.parametrize("bs,D", [(16, 128), (64, 128), (32, 64), (16, 80), (32, 160), (64, 256)])
 def test_fp8_pool_codes_and_scales_bit_exact(pa, rng, bs, D):
     """Chunks that start inside a block (stale scale kept or raised, earlier rows recoded),
     whole fresh blocks, single tokens, an empty and an all-zero chunk."""
@@ -103,6 +103,40 @@ def test_fp8_extreme_values_saturate_like_the_oracle(pa, rng):
     pa.kv_write(bf16_to_dev(xk), bf16_to_dev(xv), dk, dv, _i32(tables), _i32(seqs), _i32(qlens), k_scale=dks, v_scale=dvs)
     O.kv_write(O.f32_to_bf16_bits(xk), O.f32_to_bf16_bits(xv), pk, pv, tables, seqs, qlens, k_scale=ks, v_scale=vs)
     assert np.array_equal(dks.cpu().numpy(), ks)
+    assert np.array_equal(dev_bits(dk), pk) and np.array_equal(dev_bits(dv), pv)
+
+
+@pytest.mark.parametrize("scale_bits,why", [
+    (0x3cffffff, "mantissa all ones: the reciprocal form would turn x = 2^-15 into a tie and round it to code 0"),
+    (0x3cfffffe, "its neighbour, which the reciprocal form takes"),
+    (0x2b000000, "2^-41, below the range the reciprocal form is used in"),
+    (0x2b800000, "2^-40, its lower end"),
+    (0x53800000, "2^40, its upper end"),
+    (0x54000000, "2^41, above it"),
+])
+def test_fp8_quotient_at_the_edges_of_the_reciprocal_form(pa, rng, scale_bits, why):
+    """The encode forms x / scale from a refined reciprocal where that is proven to give the division's bits and
+    divides elsewhere.  A block that already holds tokens under a stale scale larger than the new rows need keeps
+    that scale, so any float32 can be made the divisor: the edges of the proven range, and the one mantissa it
+    excludes together with the value that tells the two forms apart."""
+    B, T, Hkv, D, bs = 1, 8, 1, 128, 16
+    nb, tables, seqs, qlens, xk, xv = _case(rng, B, T, Hkv, D, bs, seqs=[12], qlens=[8])    # 4 earlier rows in block 0
+    s = np.array([scale_bits], np.uint32).view(np.float32)[0]
+    mags = np.float32(2.0) ** rng.integers(-14, 9, size=xk.shape).astype(np.float32)           # quotients 2^-14 .. 2^8
+    xk = (rng.standard_normal(xk.shape).astype(np.float32) * mags * s).astype(np.float32)
+    xk[0, 0, 0, :6] = np.array([2.0 ** -10, -2.0 ** -10, 3 * 2.0 ** -10, 447.0, 2.0 ** -9, 0.0], np.float32) * s
+    xk[0, 1, 0, :2] = [-0.0, 0.0]
+    xk = O.round_to_bf16(np.clip(xk, -400 * s, 400 * s).astype(np.float32))                    # stay under the stale scale
+    xv = xk[:, ::-1].copy()
+    pk, pv, ks, vs = _fp8_state(rng, nb, bs, Hkv, D)
+    ks[:] = s
+    vs[:] = s
+    dk, dv = _to_fp8_dev(pk), _to_fp8_dev(pv)
+    dks, dvs = torch.from_numpy(ks.copy()).cuda(), torch.from_numpy(vs.copy()).cuda()
+    print(f"scale {s!r} ({why})", flush=True)
+    pa.kv_write(bf16_to_dev(xk), bf16_to_dev(xv), dk, dv, _i32(tables), _i32(seqs), _i32(qlens), k_scale=dks, v_scale=dvs)
+    O.kv_write(O.f32_to_bf16_bits(xk), O.f32_to_bf16_bits(xv), pk, pv, tables, seqs, qlens, k_scale=ks, v_scale=vs)
+    assert np.array_equal(dks.cpu().numpy(), ks) and np.all(ks[tables[0, 0]] == s)              # the stale scale stayed
     assert np.array_equal(dev_bits(dk), pk) and np.array_equal(dev_bits(dv), pv)
 
 
