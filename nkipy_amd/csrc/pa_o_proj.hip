@@ -159,15 +159,50 @@ void o_proj_kernel(OProjParams p) {
         acc[mb][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[c], xf[mb], acc[mb][c], 0, 0, 0);
   };
 
+  // The loop is rotated by one k16-step: the products of a k-step's last k16-step are issued behind the barrier
+  // that opens the next k-step, between that step's copy requests, so that the matrix pipeline has work while
+  // the requests and the first fragment reads of the new stage are issued.
+  auto request_part = [&](int stage, int part) __attribute__((always_inline)) {     // a quarter of request()
+    const uint32_t sb = smem_base + stage * STAGE_B;
+    dma16(xbase, xoff[part], sb + (wave + 8 * part) * 1024);
+    dma16(wbase, woff[part >> 1][part & 1], sb + XT_B + (part >> 1) * WH_B + (wave + 8 * (part & 1)) * 1024);
+  };
   const int ktiles = p.K / BK;
+  bf16x8_t wa[4], wb[4], xa[2], xb[2];
   request(0);
-  for (int kt = 0; kt < ktiles; ++kt) {
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  if (ktiles > 1) request(1);
+  load_w(wa, 0, 0); load_x(xa, 0, 0);
+  for (int kt = 0; kt + 1 < ktiles; ++kt) {
     const int stage = kt & 1;
-    wait_vmcnt<0>();                       // this wave's part of step kt has landed
-    __builtin_amdgcn_s_barrier();          // ... and everyone's; all waves are done with step kt - 1
-    if (kt + 1 < ktiles) request(stage ^ 1);
-    bf16x8_t wa[4], wb[4], xa[2], xb[2];
-    load_w(wa, stage, 0); load_x(xa, stage, 0);
+    load_w(wb, stage, 1); load_x(xb, stage, 1);
+    mma(wa, xa);
+    load_w(wa, stage, 2); load_x(xa, stage, 2);
+    mma(wb, xb);
+    load_w(wb, stage, 3); load_x(xb, stage, 3);
+    mma(wa, xa);
+    wait_vmcnt<0>();                       // this wave's part of step kt + 1 has landed
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its reads of this stage are done
+    __builtin_amdgcn_s_barrier();          // everyone's; the stage of step kt is free
+    load_w(wa, stage ^ 1, 0); load_x(xa, stage ^ 1, 0);
+    const bool more = kt + 2 < ktiles;
+#define OPROJ_TAIL_PART(part, mb)                                                                              \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+    acc[mb][2 * ((part) & 1)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[2 * ((part) & 1)], xb[mb], acc[mb][2 * ((part) & 1)], 0, 0, 0);             \
+    acc[mb][2 * ((part) & 1) + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[2 * ((part) & 1) + 1], xb[mb], acc[mb][2 * ((part) & 1) + 1], 0, 0, 0); \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+    if (more) request_part(stage, part);
+    OPROJ_TAIL_PART(0, 0)
+    OPROJ_TAIL_PART(1, 0)
+    OPROJ_TAIL_PART(2, 1)
+    OPROJ_TAIL_PART(3, 1)
+#undef OPROJ_TAIL_PART
+    xbase += BK * 2;
+    wbase += (long)BK * w_row_b;
+  }
+  {
+    const int stage = (ktiles - 1) & 1;
     load_w(wb, stage, 1); load_x(xb, stage, 1);
     mma(wa, xa);
     load_w(wa, stage, 2); load_x(xa, stage, 2);
