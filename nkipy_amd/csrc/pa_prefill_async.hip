@@ -507,6 +507,26 @@ void prefill_async_kernel(PrefillParams p) {
       mma_pv(v1, pw[g >> 1], 1, j);
     }
   };
+  // The same with the products of the last two groups left for later: their V^T fragments end up in dv0 / dv1
+  // and the probabilities they multiply in dpw.  The tile loop issues them behind the next tile's barrier,
+  // where the matrix pipeline would otherwise wait for the copy requests and the first K fragments.
+  auto accumulate_but_last = [&](const uint32_t (&pw)[TT][8], int stage, bf16x8_t (&v0)[VC], bf16x8_t (&dv0)[VC],
+                                 bf16x8_t (&dv1)[VC], uint32_t (&dpw)[8], int j) __attribute__((always_inline)) {
+#pragma unroll
+    for (int g = 0; g + 2 < 2 * TT; g += 2) {
+      load_v(dv1, stage, g + 1);
+      mma_pv(v0, pw[g >> 1], 0, j);
+      load_v(g + 4 < 2 * TT ? v0 : dv0, stage, g + 2);
+      mma_pv(dv1, pw[g >> 1], 1, j);
+    }
+    if (TT == 1) {
+#pragma unroll
+      for (int c = 0; c < VC; ++c) dv0[c] = v0[c];
+    }
+    load_v(dv1, stage, 2 * TT - 1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dpw[i] = pw[TT - 1][i];
+  };
 
   // online softmax on this lane's column: scores -> packed bf16 probabilities, state update
   // (sacc: NS 32-key sub-tiles that start at key key0; j: which head of the wave)
@@ -675,16 +695,32 @@ void prefill_async_kernel(PrefillParams p) {
     Walk w_c = w_first;
     int stage_c = 0;
     int rs_n = 1;                                  // FP8: raw stage of the tile after the current one
+    // one q head per wave: the last two groups of a tile's O^T += V^T P^T wait here for the next barrier
+    constexpr bool DEFER = QH == 1;
+    bf16x8_t dv0[DEFER ? VC : 1], dv1[DEFER ? VC : 1];
+    uint32_t dpw[8];
+    bool pending = false;
+    auto flush_pending = [&]() __attribute__((always_inline)) {
+      if constexpr (DEFER) {
+        if (pending) {
+          mma_pv(dv0, dpw, 0, 0);
+          mma_pv(dv1, dpw, 1, 0);
+          pending = false;
+        }
+      }
+    };
     while (w_c.kt < ntiles) {
       if (FP8) {
         wait_vmcnt<2 * UPW>();                     // this wave's raw rows of the next tile have landed
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its bf16 rows of the current one are written
       } else {
         wait_vmcnt<(NST - 2) * UPW>();             // this wave's part of the current tile has landed
+        if (DEFER) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its reads of the previous one are done
       }
       __builtin_amdgcn_s_barrier();                // ... and everyone's; all waves are done with the previous tile
       if (FP8) shift_scales();
       request_next();
+      flush_pending();       // (behind the requests: issued in front of them it measured 0.3 % slower)
       if (FP8) {
         if (w_c.kt + 1 < ntiles) expand(w_c.kt + 1, rs_n, stage_c ^ 1);
         rs_n = (rs_n + 1) & 3;
@@ -697,7 +733,8 @@ void prefill_async_kernel(PrefillParams p) {
           scores(sacc, stage_c, v0, stage_c, 0);
           prefetch_next();
           softmax(sacc, pw, w_c.kt * BN, 0);
-          accumulate(pw, stage_c, v0, 0);
+          accumulate_but_last(pw, stage_c, v0, dv0, dv1, dpw, 0);
+          pending = true;
         } else {
           // two heads, one 32-key sub-tile at a time: its K fragments and its two groups of V^T fragments are
           // read once and serve both heads; scores, probabilities and fragments of one sub-tile are all the
@@ -734,6 +771,7 @@ void prefill_async_kernel(PrefillParams p) {
       walk_step(w_c);
       stage_c = stage_c + 1 == BFS ? 0 : stage_c + 1;
     }
+    flush_pending();
   }
   wait_vmcnt<0>();     // nothing may still be landing in LDS when the workgroup retires
 
