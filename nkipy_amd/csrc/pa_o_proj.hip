@@ -550,10 +550,12 @@ hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
     return launch_skinny<4>(p, s);
   if (p.M <= 256) return launch_skinny<8>(p, s);
   {
-    // fewer large tiles than CUs (256 on this part): the 128 x 128 form fills the device better
+    // fewer large tiles than CUs (256 on this part): the 128 x 128 form fills the device better, as long as its
+    // workgroups are all resident at once (two per CU); a third of them on some CUs costs a whole further round
+    // (K = N = 4096, us: M = 2 304 107 against 92 with the large tiles, M = 3 328 125 against 109; M = 2 048 72 against 82)
     const long big_tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-    if (big_tiles < 224 && !g_o_proj_force_large) {
-      const long MTm = (p.M + MBM - 1) / MBM, NTm = (p.N + MBN - 1) / MBN;
+    const long MTm = (p.M + MBM - 1) / MBM, NTm = (p.N + MBN - 1) / MBN;
+    if (big_tiles < 224 && MTm * NTm <= 512 && !g_o_proj_force_large) {
       const long total_m = 8 * ((MTm + 7) / 8) * 4 * ((NTm + 3) / 4);
       if (total_m > 0x7fffffffL) return hipErrorInvalidValue;
       const bool deep = MTm * NTm <= 256;
