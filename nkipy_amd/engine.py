@@ -218,6 +218,11 @@ class PagedAttention:
     into the layer's pool and runs the prefill / verify kernel (T > 1) or the decode kernel
     (T == 1).  Returns [max_seqs, T, Hq, D] (a preallocated buffer, overwritten by the next step of
     the same T), or, when the layer was given `o_weight`, the output projection of it, [max_seqs, T, hidden].
+
+    `attend` makes no host synchronisation and, after the first call of a given T, no allocation, so the
+    launch-bound decode step of a stack of layers can be captured into one HIP graph (`torch.cuda.graph`) with
+    xq / xk / xv as static buffers and replayed every step: `begin_step` stays outside the graph (it publishes
+    the step's table rows and lengths, which the replayed kernels read from the same device tensors).
     """
 
     def __init__(self, cache: PagedKVCache, n_heads: int, *, layer: int = 0, scale: Optional[float] = None,
@@ -294,9 +299,13 @@ class PagedAttention:
             paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq
         if T == 1:
+            # the host-known bound on the contexts sizes the launch and clamps the lengths the kernel reads; a
+            # launch that is being captured into a HIP graph will be replayed on longer contexts, so it gets the
+            # table capacity instead
+            capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
             paged_attn.decode(q[:, 0], kc, vc, c.block_tables, c.seq_lens, self.scale,
                               k_scale=ks, v_scale=vs, partition_size=self.partition_size,
-                              max_seq_len=max(c.max_seq_len, 1), out=out[:, 0],
+                              max_seq_len=None if capturing else max(c.max_seq_len, 1), out=out[:, 0],
                               sinks=self.sinks, sliding_window=self.sliding_window, q_transform=qt)
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:

@@ -299,3 +299,67 @@ def test_layer_with_output_projection(rng, bias):
                 assert_close_abs(got[s, :qlens[s]], want[s, :qlens[s]], 4e-2)
     with pytest.raises(ValueError):
         PagedAttention(cache, Hq, o_weight=bf16_to_dev(_rand(rng, (Hq * D - 64, hidden))))
+
+
+def test_decode_steps_replayed_from_one_graph_while_the_contexts_grow(rng):
+    """The launch-bound part of serving: the decode step of a stack of layers (K norm + RoPE + KV write, decode
+    attention with the Q transform on its load, output projection) captured once into a HIP graph and replayed
+    every step with new inputs, while begin_step outside the graph extends the sequences across block borders
+    and past the lengths they had at capture time.  Every replay is checked, bit for bit, against the same
+    layers run eagerly on a twin cache, with eager work between the replays."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    from tests.pa_testlib import dev_bits
+    S, L, Hq, Hkv, D, bs, hidden = 3, 2, 8, 2, 128, 16, 256
+    wq = bf16_to_dev(1.0 + 0.1 * rng.standard_normal(D).astype(np.float32))
+    wk = bf16_to_dev(1.0 + 0.1 * rng.standard_normal(D).astype(np.float32))
+    ow = [bf16_to_dev((rng.standard_normal((Hq * D, hidden)) / 32).astype(np.float32)) for _ in range(L)]
+
+    def stack():
+        cache = PagedKVCache(num_blocks=64, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=10,
+                             num_layers=L)
+        layers = [PagedAttention(cache, Hq, layer=l, rope_base=10000.0, max_positions=10 * bs, q_norm_weight=wq,
+                                 k_norm_weight=wk, o_weight=ow[l]) for l in range(L)]
+        return cache, layers
+
+    (ca, la), (cb, lb) = stack(), stack()
+    T0 = 40
+    prompt = [[_rand(rng, (S, T0, h, D)) for h in (Hq, Hkv, Hkv)] for _ in range(L)]
+    plens = [40, 7, 23]
+    for cache, layers in ((ca, la), (cb, lb)):
+        cache.begin_step(plens, T0)
+        for l in range(L):
+            layers[l].attend(*[bf16_to_dev(t) for t in prompt[l]])
+    # static inputs of the captured step, one set per layer
+    xs = [[torch.zeros((S, 1, h, D), dtype=torch.bfloat16, device="cuda") for h in (Hq, Hkv, Hkv)] for _ in range(L)]
+
+    def fill():
+        for l in range(L):
+            for t in xs[l]:
+                t.copy_(bf16_to_dev(_rand(rng, tuple(t.shape))))
+
+    def eager(cache, layers):
+        cache.begin_step([1] * S, 1)
+        return [layers[l].attend(*xs[l]) for l in range(L)]
+
+    fill()
+    want = [o.clone() for o in eager(cb, lb)]
+    got = eager(ca, la)                      # one eager decode step first: buffers and workspaces exist before the capture
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert np.array_equal(dev_bits(got[l]), dev_bits(want[l]))
+    fill()
+    ca.begin_step([1] * S, 1)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        outs = [la[l].attend(*xs[l]) for l in range(L)]
+    for step in range(45):                   # 41 -> 86 tokens in slot 0: five more blocks, twice the captured length
+        if step:
+            fill()
+            ca.begin_step([1] * S, 1)
+        print(f"replay {step}: lens {ca.lens}", flush=True)
+        g.replay()
+        want = eager(cb, lb)
+        torch.cuda.synchronize()
+        for l in range(L):
+            assert np.array_equal(dev_bits(outs[l]), dev_bits(want[l])), (step, l)
+    assert ca.lens == cb.lens == [86, 53, 69]
