@@ -446,6 +446,7 @@ static void fill_prefill_shape(PrefillParams& p, int B, int T, int Hq, int Hkv, 
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.impl = g_prefill_impl.load();
+  p.num_cus = current_num_cus();
 }
 
 static size_t prefill_split_bytes(const PrefillParams& p, int splits) {

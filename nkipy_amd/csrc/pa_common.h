@@ -215,6 +215,7 @@ struct PrefillParams {
   float* ws_o;              // splits > 1: [B * T * Hq, splits, D] partial outputs
   float* ws_ml;             // splits > 1: [B * T * Hq, splits, 2] partial (max, sum)
   QTransform qt;            // asynchronous kernel only: Q rows are normed and rotated as they are loaded
+  int num_cus;              // CUs of the device the call runs on (0: unknown, taken as 256); steers the workgroup shape
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);

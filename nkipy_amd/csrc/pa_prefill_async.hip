@@ -921,11 +921,17 @@ static int prefill_waves(const PrefillParams& p, int waves) {
   const bool sparse = p.sparse_stride > 0;
   // waves: 4 (two workgroups of 128 query rows per CU, 2-stage ring) or 8 (one workgroup of
   // 256 rows, 4-stage ring: half the copy requests per FLOP).  Measured within a few per cent of
-  // each other; automatic choice: 8 for dense chunks of more than 128 rows, 4 for short chunks
-  // and for the sparse form.
+  // each other; automatic choice: 8 for dense chunks of more than 128 rows that fill the device, 4 for short
+  // chunks, small grids and the sparse form.
   if (p.kv_fp8 || p.D == 64) return 8; // fp8 pools and head dim 64: the 8-wave form only
   if (prefill_packs(p)) return 4;
-  if (waves == 0) waves = (!sparse && p.T > 128) ? 8 : 4;
+  if (waves == 0) {
+    waves = (!sparse && p.T > 128) ? 8 : 4;
+    // fewer 256-row workgroups than CUs (one request's chunk of up to a few thousand tokens): the call is bound by
+    // its longest workgroup, and twice as many of half the size, two per CU, finish sooner (B = 1: T = 512 behind
+    // a 4 K prefix 66 -> 55 us, T = 1 024 37.5 -> 33.5 us; with the device full the 8-wave form is ~7 % ahead)
+    if (waves == 8 && p.block_tables && (long)p.B * p.Hq * ((p.T + 255) / 256) < (p.num_cus > 0 ? p.num_cus : 256)) waves = 4;
+  }
   return waves;
 }
 
