@@ -42,20 +42,31 @@
 namespace pa {
 namespace {
 
-template <int N> struct VecLoad;
-template <> struct VecLoad<1> {
+// N dwords per lane; NT: a streaming (non-temporal) load, for bytes that are read once
+template <int N, bool NT = false> struct VecLoad;
+template <bool NT> struct VecLoad<1, NT> {
   static __device__ __forceinline__ void get(const void* p, uint32_t* r) { r[0] = *(const uint32_t*)p; }
 };
-template <> struct VecLoad<2> {
+template <bool NT> struct VecLoad<2, NT> {
   static __device__ __forceinline__ void get(const void* p, uint32_t* r) {
-    uint2 v = *(const uint2*)p; r[0] = v.x; r[1] = v.y;
+    typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+    const u2_t v = NT ? __builtin_nontemporal_load((const u2_t*)p) : *(const u2_t*)p;
+    r[0] = v.x; r[1] = v.y;
   }
 };
-template <> struct VecLoad<4> {
+template <bool NT> struct VecLoad<4, NT> {
   static __device__ __forceinline__ void get(const void* p, uint32_t* r) {
-    uint4 v = *(const uint4*)p; r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+    typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+    const u4_t v = NT ? __builtin_nontemporal_load((const u4_t*)p) : *(const u4_t*)p;
+    r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
   }
 };
+// V rows are read whole by one instruction and never again: streamed, they stop displacing what is reused.  K is
+// fetched in 64-byte pieces, two instructions per 128-byte line: streaming it as well (or instead) measured slower.
+// Paged decode (64 sequences, 512-8192 tokens), kernel us, K / V plain-plain, streamed-streamed, streamed-plain,
+// plain-streamed: bf16 187.2, 175.9, 181.1, 169.2; fp8 (twice the sequences) 403.2, 415.4, 425.9, 384.4; the
+// four-token verify 197.4, 190.2, 193.6, 179.8.
+constexpr bool kStreamK = false, kStreamV = true;
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   uint4 v = make_uint4(a, b, c, d);
@@ -248,7 +259,7 @@ struct DecodeWave {
       const long row = (tl_ < 16) ? tr.row0 + tl_ : tr.row1 + (tl_ - 16);
       const char* rowp = kbase + row * row_stride;
 #pragma unroll
-      for (int s = 0; s < KLD; ++s) VecLoad<4>::get(rowp + (4 * s + g) * 16, tl.k[u][s]);
+      for (int s = 0; s < KLD; ++s) VecLoad<4, kStreamK>::get(rowp + (4 * s + g) * 16, tl.k[u][s]);
     }
   }
   __device__ __forceinline__ void load_v(VT& tl, int t0) const {
@@ -262,7 +273,7 @@ struct DecodeWave {
       const int tl_ = min(4 * j + g, tr.lmax);
       const long row = (tl_ < 16) ? tr.row0 + tl_ : tr.row1 + (tl_ - 16);
       const char* rowp = vbase + row * row_stride;
-      VecLoad<VW>::get(rowp + r * (VEC * ESZ), tl.v[j]);
+      VecLoad<VW, kStreamV>::get(rowp + r * (VEC * ESZ), tl.v[j]);
     }
   }
 
