@@ -30,6 +30,10 @@
 namespace pa {
 namespace {
 
+// What these kernels write (pool rows, transformed Q rows) goes out through streaming stores (pre-attention workload
+// 0.085 -> 0.074 ms, plain write 21.9 -> 20.9 us); streaming the loads as well measured slower: the new rows come out
+// of the kernel before this one.
+
 constexpr int WG = 256;
 // Waves per SIMD the write kernels are compiled for: their workgroups are short chains of dependent loads, so
 // residency counts, but a register budget that makes the compiler spill costs more (a reload from scratch waits
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(XCPR != 0 &&
       uint4 v;
       if (ESZ == 2 && XFORM) v = load_row_chunk((const uint16_t*)s0, r, c);
       else v = *(const uint4*)(s0 + (long)r * row_elems * ESZ + c * 16);
-      *(uint4*)(d0 + (long)r * row_elems * ESZ + c * 16) = v;
+      store_stream(d0 + (long)r * row_elems * ESZ + c * 16, v);
     }
     return;
   }
@@ -334,7 +338,7 @@ __global__ __launch_bounds__(WG) __attribute__((amdgpu_waves_per_eu(XCPR != 0 &&
     uint2 o;
     o.x = pack_fp8x2(f[0], f[1], 0u, false); o.x = pack_fp8x2(f[2], f[3], o.x, true);
     o.y = pack_fp8x2(f[4], f[5], 0u, false); o.y = pack_fp8x2(f[6], f[7], o.y, true);
-    *(uint2*)(d_blk + (long)(lo + r) * row_elems + c * 8) = o;
+    store_stream(d_blk + (long)(lo + r) * row_elems + c * 8, o);
   };
   auto encode_all = [&](auto fast) __attribute__((always_inline)) {
     int r = r_first, c = c_first, i = threadIdx.x;
@@ -392,7 +396,7 @@ __global__ __launch_bounds__(WGQ) void q_norm_rope_kernel(KvWriteParams p) {
       } else {
         v[u] = make_uint4(0, 0, 0, 0);
       }
-      *(uint4*)((uint16_t*)p.q_out + (tok + hb + u * hstep) * D + c * 8) = v[u];
+      store_stream((uint16_t*)p.q_out + (tok + hb + u * hstep) * D + c * 8, v[u]);
     }
     hb += UNR * hstep;
     if (hb >= p.Hq) break;

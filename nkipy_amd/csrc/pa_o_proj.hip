@@ -242,7 +242,7 @@ void o_proj_kernel(OProjParams p) {
       const int r = 4 * j + (lane >> 4), ch = lane & 15;
       const uint2 lo = *(const uint2*)(patch + r * PROW_B + 16 * ch), hi = *(const uint2*)(patch + r * PROW_B + 16 * ch + 8);
       const int m = m0 + 64 * wm + 32 * mb + r, col = n0 + 128 * wn + 8 * ch;
-      if (m < p.M && col < p.N) *(uint4*)(out + (long)m * p.N + col) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      if (m < p.M && col < p.N) store_stream(out + (long)m * p.N + col, make_uint4(lo.x, lo.y, hi.x, hi.y));
     }
   }
 }
@@ -400,7 +400,7 @@ void o_proj_mid_kernel(OProjParams p) {
       const int r = 8 * j + (lane >> 3), ch = lane & 7;
       const uint2 lo = *(const uint2*)(patch + r * PROW_B + 16 * ch), hi = *(const uint2*)(patch + r * PROW_B + 16 * ch + 8);
       const int m = m0 + 64 * wm + 32 * mb + r, col = n0 + 64 * wn + 8 * ch;
-      if (m < p.M && col < p.N) *(uint4*)(out + (long)m * p.N + col) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      if (m < p.M && col < p.N) store_stream(out + (long)m * p.N + col, make_uint4(lo.x, lo.y, hi.x, hi.y));
     }
   }
 }

@@ -828,8 +828,8 @@ void prefill_async_kernel(PrefillParams p) {
       const uint2 lo = *(const uint2*)(patch + r * OROW_B + 16 * ch), hi = *(const uint2*)(patch + r * OROW_B + 16 * ch + 8);
       const int tok = row_token(wave * 32 + r);
       if (tok < p.T && !idle_half)
-        *(uint4*)(out + ((long)b * p.T + tok) * q_row_stride + (long)(row_head(wave * 32 + r) + hj) * DH + 8 * ch) =
-            make_uint4(lo.x, lo.y, hi.x, hi.y);
+        store_stream(out + ((long)b * p.T + tok) * q_row_stride + (long)(row_head(wave * 32 + r) + hj) * DH + 8 * ch,
+                     make_uint4(lo.x, lo.y, hi.x, hi.y));
     }
   }
 }
