@@ -66,7 +66,11 @@ template <bool NT> struct VecLoad<4, NT> {
 // Paged decode (64 sequences, 512-8192 tokens), kernel us, K / V plain-plain, streamed-streamed, streamed-plain,
 // plain-streamed: bf16 187.2, 175.9, 181.1, 169.2; fp8 (twice the sequences) 403.2, 415.4, 425.9, 384.4; the
 // four-token verify 197.4, 190.2, 193.6, 179.8.
-constexpr bool kStreamK = false, kStreamV = true;
+// V is streamed only by the wave that is the rows' one reader: with more than one 16 R-row group per kv head the
+// other groups' waves read the same rows again and should find them in the cache (verify with 32 rows per kv head on
+// two waves: 229 us cached, 257 us streamed), hence the SV template argument, chosen per launch.  (A run-time choice
+// puts the loads into a conditional, which costs the decode kernel 4 %.)
+constexpr bool kStreamK = false;
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   uint4 v = make_uint4(a, b, c, d);
@@ -117,7 +121,7 @@ struct QOperandLayout {
   static constexpr int lane_xor(int bit) { return FP8 ? (bit == 2 ? 16 : bit == 4 ? 32 : 0) : (bit == 1 ? 16 : bit == 2 ? 32 : 0); }
 };
 
-template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false>
+template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false, bool SV = false>
 struct DecodeWave {
   using KT = KTile<D, FP8>;
   using VT = VTile<D, FP8>;
@@ -273,7 +277,7 @@ struct DecodeWave {
       const int tl_ = min(4 * j + g, tr.lmax);
       const long row = (tl_ < 16) ? tr.row0 + tl_ : tr.row1 + (tl_ - 16);
       const char* rowp = vbase + row * row_stride;
-      VecLoad<VW, kStreamV>::get(rowp + r * (VEC * ESZ), tl.v[j]);
+      VecLoad<VW, SV>::get(rowp + r * (VEC * ESZ), tl.v[j]);
     }
   }
 
@@ -695,10 +699,10 @@ __device__ __forceinline__ int scan_tiles(const DecodeParams& p, int lane, int f
   return base;
 }
 
-template <int D, bool FP8, bool MULTI, int R>
+template <int D, bool FP8, bool MULTI, int R, bool SV>
 __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p) {
   constexpr bool LEAN = R == 2 && D == 128;
-  using W = DecodeWave<D, FP8, MULTI, R, LEAN>;
+  using W = DecodeWave<D, FP8, MULTI, R, LEAN, SV>;
   __shared__ uint4 q_store[LEAN ? 8 * R * W::KSTEPS * 64 : 1];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -889,12 +893,18 @@ template <int D, bool FP8>
 hipError_t launch_balanced_typed(const DecodeParams& p, hipStream_t s) {
   const int head_slots = head_slots_of(p);
   dim3 grid(p.bal_gv / p.bal_ns, (head_slots + p.bal_hsw - 1) / p.bal_hsw);
-  if (p.query_lens && p.rows_per_wave == 32)
-    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 2>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
-  else if (p.query_lens)
-    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 1>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
-  else
-    hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, false, 1>), grid, dim3(64 * p.bal_hsw * p.bal_ns), 0, s, p);
+  const dim3 wg(64 * p.bal_hsw * p.bal_ns);
+  const bool one_reader = head_slots == p.Hkv;         // one wave per kv head: it alone reads that head's V rows
+  if (p.query_lens && p.rows_per_wave == 32) {
+    if (one_reader) hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 2, true>), grid, wg, 0, s, p);
+    else hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 2, false>), grid, wg, 0, s, p);
+  } else if (p.query_lens) {
+    if (one_reader) hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 1, true>), grid, wg, 0, s, p);
+    else hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 1, false>), grid, wg, 0, s, p);
+  } else {
+    if (one_reader) hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, false, 1, true>), grid, wg, 0, s, p);
+    else hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, false, 1, false>), grid, wg, 0, s, p);
+  }
   return hipGetLastError();
 }
 
