@@ -40,6 +40,15 @@ static std::atomic<int> g_decode_waves{0};
 static std::atomic<int> g_head_major{1};
 static std::atomic<int> g_prefill_impl{0};
 static std::atomic<int> g_lockstep{1};
+// The per-tile barrier that keeps the kv-head waves of a balanced decode workgroup on the same tile: debug switch 4,
+// 1 = automatic (the default), 0 = never, 2 = always.  Automatic: on for bf16 pools (the heads' rows of a token are one
+// contiguous piece of DRAM; config 2 80.4 % of HBM peak with it, 77.5 % without), off for fp8 pools (the waves' expansion
+// work makes them arrive apart, and waiting for the last costs more than the drift: config 5 77.6 % with, 79.3 % without).
+static int lockstep_for(int kv_dtype, int bal_ns) {
+  const int mode = g_lockstep.load();
+  if (bal_ns != 1 || mode == 0) return 0;
+  return mode == 2 || kv_dtype != PA_FP8_E4M3FN ? 1 : 0;
+}
 static std::atomic<int> g_verify_rows{0};
 static std::atomic<int> g_prefill_split{1};
 static std::atomic<int> g_d64_tiled_from{PA_VERIFY_MAX_TOKENS + 1};   // query tokens from which head dim 64 takes the tiled kernel
@@ -268,7 +277,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
   if (kind == 3) {
     plan_decode_balanced(p, current_num_cus());
-    p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
+    p.bal_lockstep = lockstep_for(kv_dtype, p.bal_ns);
     const size_t need = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
     if (!workspace || workspace_bytes < need)
       return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -392,7 +401,7 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     return fail_arg("%s: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", who, D, block_size);
   if (take_q_transform(who, q_transform, true, p.qt)) return -1;
   plan_decode_balanced(p, current_num_cus());
-  p.bal_lockstep = (g_lockstep.load() && p.bal_ns == 1) ? 1 : 0;
+  p.bal_lockstep = lockstep_for(kv_dtype, p.bal_ns);
   const size_t need = decode_balanced_workspace_bytes(B, Hq * Tc, D, p.bal_gv);
   if (!workspace || workspace_bytes < need)
     return fail_arg("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
