@@ -61,8 +61,9 @@ template <bool NT> struct VecLoad<4, NT> {
     r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
   }
 };
-// V rows are read whole by one instruction and never again: streamed, they stop displacing what is reused.  K is
-// fetched in 64-byte pieces, two instructions per 128-byte line: streaming it as well (or instead) measured slower.
+// V rows are read whole by one instruction and never again: streamed, they stop displacing what is reused.  K in
+// its operand order is fetched in 64-byte pieces, two instructions per 128-byte line: streaming that as well (or
+// instead) measured slower; DecodeWave::load_k has a second form that fetches whole lines and can be streamed.
 // Paged decode (64 sequences, 512-8192 tokens), kernel us, K / V plain-plain, streamed-streamed, streamed-plain,
 // plain-streamed: bf16 187.2, 175.9, 181.1, 169.2; fp8 (twice the sequences) 403.2, 415.4, 425.9, 384.4; the
 // four-token verify 197.4, 190.2, 193.6, 179.8.
@@ -128,6 +129,9 @@ struct DecodeWave {
   static constexpr int VEC = VT::VEC, KLD = KT::KLD, VW = VT::VW;
   static constexpr int KSTEPS = D / 32;
   static constexpr int ESZ = FP8 ? 1 : 2;
+  // K streamed too (with V), for bf16 pools: config 2 kernel 169.3 -> 166.4 us, verify 180.0 -> 178.0; on the fp8
+  // pool, whose expansion already costs vector instructions, the rearrangement costs more than it brings (375.5 -> 379.5)
+  static constexpr bool SK = SV && !FP8 && D * ESZ >= 128;
 
   const DecodeParams& p;
   int hk, hbase, nheads;     // kv head, first (virtual) q head, valid rows of this wave
@@ -138,6 +142,10 @@ struct DecodeWave {
   long row_stride;           // bytes between consecutive tokens of a block
   int last;                  // ctx - 1 of the current sequence
   int jbase;                 // first row of this wave inside its kv group
+  // SK: K travels as whole 128-byte lines (see load_k); where this lane's chunk of steps with even / odd s sits
+  // after the load (byte address of the source lane for ds_bpermute), and in which of the two loads of a line
+  int kperm_addr[2];
+  bool k_first_half;
   int row_end[R];            // MULTI: keys [0, row_end) are visible to this lane's row (0: padding row)
   bf16x8_t qf[LEAN ? 1 : R][LEAN ? 1 : KSTEPS];
   uint4* qlds;               // LEAN: this wave's [R][KSTEPS][64] fragment store in LDS
@@ -157,6 +165,9 @@ struct DecodeWave {
     r = lane & 15;
     g = lane >> 4;
     krow = 4 * (r & 3) + (r >> 2);
+    k_first_half = krow < 8;
+    kperm_addr[0] = 4 * (8 * (krow & 7) + g);
+    kperm_addr[1] = 4 * (8 * (krow & 7) + 4 + g);
     row_stride = (long)p.Hkv * D * ESZ;
     kbase = (const char*)p.k_cache + (long)hk * D * ESZ;
     vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
@@ -257,6 +268,23 @@ struct DecodeWave {
       tl.ksc[0] = p.k_scale[(long)tr.blk0 * p.Hkv + hk];
       tl.ksc[1] = p.k_scale[(long)tr.blk1 * p.Hkv + hk];
     }
+    if (SK) {
+      // One instruction = 8 rows x one whole 128-byte line (lane: row 8 hf + lane / 8 of the sub-tile in tile
+      // order, 16-byte chunk lane % 8), so that a streamed line is used up by the instruction that fetches it; slot
+      // [2 ln + hf] holds line ln of rows 8 hf .. 8 hf + 7.  k_chunk() below hands the matrix instructions their
+      // operand order back.
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const int tl_ = min(16 * u + 8 * hf + 2 * g + (r >> 3), tr.lmax);
+          const long row = (tl_ < 16) ? tr.row0 + tl_ : tr.row1 + (tl_ - 16);
+          const char* rowp = kbase + row * row_stride + (r & 7) * 16;
+#pragma unroll
+          for (int ln = 0; ln < KLD / 2; ++ln) VecLoad<4, true>::get(rowp + ln * 128, tl.k[u][2 * ln + hf]);
+        }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int tl_ = min(16 * u + krow, tr.lmax);
@@ -264,6 +292,23 @@ struct DecodeWave {
       const char* rowp = kbase + row * row_stride;
 #pragma unroll
       for (int s = 0; s < KLD; ++s) VecLoad<4, kStreamK>::get(rowp + (4 * s + g) * 16, tl.k[u][s]);
+    }
+  }
+  // The 16 bytes lane (g, r) feeds to the matrix instruction in step s of sub-tile u: chunk 4 s + g of tile row
+  // krow(r).  As loaded by the plain form they are tl.k[u][s]; as loaded by the streamed form they sit in line
+  // s / 2, in the load of the row's half, in lane 8 (krow % 8) + (4 s + g) % 8: one cross-lane read (LDS pipeline,
+  // no LDS memory) from each half's registers and a select.
+  __device__ __forceinline__ void k_chunk(const KT& tl, int u, int s, uint32_t (&out)[4]) const {
+    if (!SK) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d) out[d] = tl.k[u][s][d];
+      return;
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t a = (uint32_t)__builtin_amdgcn_ds_bpermute(kperm_addr[s & 1], (int)tl.k[u][2 * (s >> 1)][d]);
+      const uint32_t b = (uint32_t)__builtin_amdgcn_ds_bpermute(kperm_addr[s & 1], (int)tl.k[u][2 * (s >> 1) + 1][d]);
+      out[d] = k_first_half ? a : b;
     }
   }
   __device__ __forceinline__ void load_v(VT& tl, int t0) const {
@@ -301,9 +346,11 @@ struct DecodeWave {
         for (int rg = 0; rg < R; ++rg) {
           const bf16x8_t q = q_frag(rg, s);
 #pragma unroll
-          for (int u = 0; u < 2; ++u)
-            sacc[rg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                as_bf16x8(tl.k[u][s][0], tl.k[u][s][1], tl.k[u][s][2], tl.k[u][s][3]), q, sacc[rg][u], 0, 0, 0);
+          for (int u = 0; u < 2; ++u) {
+            uint32_t kc[4];
+            k_chunk(tl, u, s, kc);
+            sacc[rg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kc[0], kc[1], kc[2], kc[3]), q, sacc[rg][u], 0, 0, 0);
+          }
         }
       }
     } else {
@@ -312,10 +359,12 @@ struct DecodeWave {
         uint32_t w[2][8];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
+          uint32_t kc[4];
+          k_chunk(tl, u, s, kc);
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             float f[4];
-            fp8x4_to_float(tl.k[u][s][d], f);
+            fp8x4_to_float(kc[d], f);
             w[u][2 * d] = pack_hi16(f[0], f[1]);
             w[u][2 * d + 1] = pack_hi16(f[2], f[3]);
           }
