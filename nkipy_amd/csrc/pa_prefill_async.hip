@@ -76,6 +76,16 @@ __device__ __forceinline__ void dma16_lane(const char* addr, uint32_t lds_base) 
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :: "v"(addr), "s"(lds_base) : "memory", "m0");
 }
+// The same as streaming (non-temporal) copies, for tiles that no other workgroup reads: a line that is read once
+// and not kept in the caches comes from HBM at a higher rate.
+__device__ __forceinline__ void dma16_uniform_stream(const char* base, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+               :: "v"(lane_off), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_lane_stream(const char* addr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+               :: "v"(addr), "s"(lds_base) : "memory", "m0");
+}
 
 // Block-table reads go through the constant address space: wave-uniform indices then
 // become scalar loads (their own counter), not vector loads that would have to be
@@ -147,6 +157,8 @@ void prefill_async_kernel(PrefillParams p) {
   const int kvg = PAIR ? (p.Hkv + 1) / 2 : p.Hkv;    // K/V row groups: kv heads, or pairs of them
   const int hpg = n_rep / QH;                  // workgroups (per query tile) that cover the q heads of a kv head
   const int per_group = PACK ? nqt : nqt * hpg;
+  // PACK with one row tile per kv head: this workgroup is the only reader of its keys and values
+  const bool stream_kv = PACK && nqt == 1;
   const int groups = p.B * kvg;
   const int xcd = blockIdx.x & 7;
   const int part = SPLIT ? (int)(blockIdx.x >> 3) % p.splits : 0;      // which share of the key tiles
@@ -295,8 +307,13 @@ void prefill_async_kernel(PrefillParams p) {
           const uint32_t blk = (uint32_t)min(max(blk_pf[j], 0), p.num_blocks - 1);
           off = (uint64_t)blk * block_bytes_u + (uint32_t)((key0 + 4 * u) & (p.block_size - 1)) * kv_row_bytes_u;
         }
-        dma16_uniform(kbase + off, dma_lane_off_k, sbase + u * 1024);
-        dma16_uniform(vbase + off, dma_lane_off_v, sbase + TILE_B + u * 1024);
+        if (PACK && stream_kv) {
+          dma16_uniform_stream(kbase + off, dma_lane_off_k, sbase + u * 1024);
+          dma16_uniform_stream(vbase + off, dma_lane_off_v, sbase + TILE_B + u * 1024);
+        } else {
+          dma16_uniform(kbase + off, dma_lane_off_k, sbase + u * 1024);
+          dma16_uniform(vbase + off, dma_lane_off_v, sbase + TILE_B + u * 1024);
+        }
       }
     } else {                                      // last tile of a context: rows past it re-read its last row
 #pragma unroll
@@ -304,7 +321,8 @@ void prefill_async_kernel(PrefillParams p) {
         const bool is_k = j < UPW / 2;
         const int u = (wave + NW * j) & (UK - 1);
         const char* src = (is_k ? kbase : vbase) + lane_row(key0 + 4 * u + dma_rr) * kv_row_bytes + (is_k ? dma_chunk_k : dma_chunk_v) * 16;
-        dma16_lane(src, sbase + (is_k ? 0 : TILE_B) + u * 1024);
+        if (PACK && stream_kv) dma16_lane_stream(src, sbase + (is_k ? 0 : TILE_B) + u * 1024);
+        else dma16_lane(src, sbase + (is_k ? 0 : TILE_B) + u * 1024);
       }
     }
   };
