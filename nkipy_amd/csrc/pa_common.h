@@ -66,6 +66,15 @@ __device__ __forceinline__ void fp8x4_to_float(uint32_t w, float* f) {
   f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
 }
 
+// two OCP e4m3fn bytes (the low or the high half of w) -> a bf16 pair, exact, in one instruction: the scaled
+// conversion takes its scale's exponent only, and 1.0 leaves the values as they are (every e4m3 value is a bf16 value)
+template <bool HIGH_HALF>
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w) {
+  typedef __bf16 bf16_pair_t __attribute__((ext_vector_type(2)));
+  const bf16_pair_t v = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w, 1.0f, HIGH_HALF);
+  return __builtin_bit_cast(uint32_t, v);
+}
+
 // high halves of two floats packed as a bf16 pair (exact when both values are
 // representable in bf16, as every e4m3 value is): lo = a, hi = b
 __device__ __forceinline__ uint32_t pack_hi16(float a, float b) {

@@ -363,10 +363,8 @@ struct DecodeWave {
           k_chunk(tl, u, s, kc);
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            float f[4];
-            fp8x4_to_float(kc[d], f);
-            w[u][2 * d] = pack_hi16(f[0], f[1]);
-            w[u][2 * d + 1] = pack_hi16(f[2], f[3]);
+            w[u][2 * d] = fp8x2_to_bf16x2<false>(kc[d]);
+            w[u][2 * d + 1] = fp8x2_to_bf16x2<true>(kc[d]);
           }
         }
 #pragma unroll
@@ -447,15 +445,20 @@ struct DecodeWave {
     } else {
 #pragma unroll
       for (int dw = 0; dw < VW; ++dw) {
-        float f[8][4];
+        // codes of token pairs side by side first (bytes a0 b0 a1 b1 | a2 b2 a3 b3 of rows a = 2 jp, b = 2 jp + 1),
+        // then one conversion per pair gives the operand's (token 2 jp, token 2 jp + 1) word for a column
+        uint32_t t[4][2];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) fp8x4_to_float(tl.v[j][dw], f[j]);
+        for (int jp = 0; jp < 4; ++jp) {
+          t[jp][0] = __builtin_amdgcn_perm(tl.v[2 * jp + 1][dw], tl.v[2 * jp][dw], 0x05010400u);
+          t[jp][1] = __builtin_amdgcn_perm(tl.v[2 * jp + 1][dw], tl.v[2 * jp][dw], 0x07030602u);
+        }
 #pragma unroll
         for (int eb = 0; eb < 4; ++eb) {
           const int e = 4 * dw + eb;
           uint32_t w[4];
 #pragma unroll
-          for (int jp = 0; jp < 4; ++jp) w[jp] = pack_hi16(f[2 * jp][eb], f[2 * jp + 1][eb]);
+          for (int jp = 0; jp < 4; ++jp) w[jp] = (eb & 1) ? fp8x2_to_bf16x2<true>(t[jp][eb >> 1]) : fp8x2_to_bf16x2<false>(t[jp][eb >> 1]);
 #pragma unroll
           for (int rg = 0; rg < R; ++rg)
             oacc[rg][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), pf[rg], oacc[rg][e], 0, 0, 0);
