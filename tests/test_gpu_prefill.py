@@ -236,10 +236,12 @@ def test_prefill_argument_errors(pa):
 
 
 @pytest.mark.parametrize("impl", [5, 4], ids=["packed", "one_head_per_workgroup"])
-@pytest.mark.parametrize("T,Hq,Hkv", [(20, 8, 2), (64, 32, 8), (100, 10, 2), (127, 4, 2), (33, 16, 1)])
+@pytest.mark.parametrize("T,Hq,Hkv", [(20, 8, 2), (32, 16, 4), (64, 32, 8), (100, 10, 2), (127, 4, 2), (33, 16, 1)])
 def test_prefill_short_chunks_packed_rows(pa, impl, T, Hq, Hkv):
     """Chunks shorter than a 128-row tile: by default the rows of a workgroup are (token, head) pairs of
-    one kv head (ratios 2, 4, 5 and 16: head groups that do and do not divide a wave's 32 rows)."""
+    one kv head (ratios 2, 4, 5 and 16: head groups that do and do not divide a wave's 32 rows).  Up to 128 rows
+    per kv head (the first two cases, the second exactly 128) one workgroup is the only reader of its keys and values
+    and copies them with the streaming policy; beyond, several workgroups share them through the cache."""
     from nkipy_amd import _lib
     lib = _lib.load()
     rng = np.random.default_rng(T + Hq)
