@@ -223,6 +223,21 @@ int pa_blocksparse_prefill(const void* q, const void* k, const void* v, void* ou
 int pa_o_proj(const void* x, const void* w, const void* bias, void* out, int M, int K, int N, int dtype, void* stream);
 
 /*
+ * The same product with scratch memory for calls of few rows (a decode or verify step: M <= 128).  Such a call
+ * is bound by streaming `w` once, and one workgroup per 64 output columns leaves most of the device idle; with a
+ * workspace, up to four workgroups per column slab take equal ranges of K, leave float32 partial products there,
+ * and a second kernel adds them in the order of the ranges, then the bias, and rounds once (results are the same
+ * from call to call; they can differ from pa_o_proj's in the last bf16 bit, the sums being taken in another order).
+ *   workspace  device memory of pa_o_proj_workspace_bytes(M, K, N) bytes (0: the shape would not use one),
+ *              16-byte aligned, owned by the caller, free again when the call's work on `stream` is done;
+ *              NULL or too small for two ranges: the call runs as pa_o_proj does.
+ * No counterpart in the reference (np.matmul, examples/models/qwen3/kernels/attention.py:147, has no scratch argument).
+ */
+size_t pa_o_proj_workspace_bytes(int M, int K, int N);
+int pa_o_proj_ws(const void* x, const void* w, const void* bias, void* out, void* workspace, size_t workspace_bytes,
+                 int M, int K, int N, int dtype, void* stream);
+
+/*
  * Test hook: materialise the block-table gather.  out [B, max_seq_len, Hkv, D]
  * (elem_bytes per element, bits copied verbatim); rows >= seq_lens[b] are zero.
  * Bit-exact counterpart of np.take(pool, table, axis=0)

@@ -665,7 +665,18 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
   return check_hip(e, "pa_qk_norm_rope_kv_write launch");
 }
 
+size_t pa_o_proj_workspace_bytes(int M, int K, int N) {
+  if (M <= 0 || K <= 0 || N <= 0 || K % 64 || N % 8) return 0;
+  const int s = o_proj_splits(M, K, N);
+  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+
 int pa_o_proj(const void* x, const void* w, const void* bias, void* out, int M, int K, int N, int dtype, void* stream) {
+  return pa_o_proj_ws(x, w, bias, out, nullptr, 0, M, K, N, dtype, stream);
+}
+
+int pa_o_proj_ws(const void* x, const void* w, const void* bias, void* out, void* workspace, size_t workspace_bytes,
+                 int M, int K, int N, int dtype, void* stream) {
   tl_error[0] = 0;
   if (M < 0 || K <= 0 || N <= 0) return fail_arg("pa_o_proj: bad sizes M=%d K=%d N=%d", M, K, N);
   if (dtype != PA_BF16) return fail_arg("pa_o_proj: only bf16 is supported (dtype=%d)", dtype);
@@ -680,6 +691,15 @@ int pa_o_proj(const void* x, const void* w, const void* bias, void* out, int M, 
   OProjParams p;
   memset(&p, 0, sizeof(p));
   p.x = x; p.w = w; p.bias = bias; p.out = out; p.M = M; p.K = K; p.N = N;
+  p.splits = 1;
+  if (workspace) {
+    if (!aligned16(workspace)) return fail_arg("pa_o_proj: workspace must be 16-byte aligned");
+    // as many K ranges as the workspace holds, up to what the shape asks for; too small for two: unsplit
+    const size_t per_split = (size_t)M * N * sizeof(float);
+    int want = o_proj_splits(M, K, N);
+    if ((size_t)want * per_split > workspace_bytes) want = (int)(workspace_bytes / per_split);
+    if (want > 1) { p.splits = want; p.ws = (float*)workspace; }
+  }
   hipStream_t s = (hipStream_t)stream;
   profile_begin(s);
   hipError_t e = launch_o_proj(p, s);

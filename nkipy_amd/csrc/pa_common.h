@@ -281,8 +281,11 @@ struct OProjParams {
   const void* bias;         // [N] bf16 or null
   void* out;                // [M, N] bf16
   int M, K, N;
+  float* ws;                // split form: [splits, M, N] float32 partial products, or null
+  int splits;               // K ranges summed by a second kernel (1: none); o_proj_splits() or less
 };
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s);
+int o_proj_splits(int M, int K, int N);     // K ranges the few-rows forms would like to spread over more workgroups
 void o_proj_debug_force_large(int on);      // debug: 256 x 256 tiles also where the 128 x 128 form would be taken
 
 // matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats

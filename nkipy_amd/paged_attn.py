@@ -584,7 +584,7 @@ def qk_norm_rope_kv_write(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, 
     return out
 
 
-def o_proj(x, o_weight, bias=None, *, out=None):
+def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
     """Output projection behind the attention call: `np.matmul(output, o_weight)` (+ `o_bias`) of
     examples/models/qwen3/kernels/attention.py:143-147 and examples/models/gpt_oss/kernels/attention.py:155-163.
 
@@ -592,7 +592,10 @@ def o_proj(x, o_weight, bias=None, *, out=None):
     [..., K]; o_weight [K, N] bfloat16 with K = Hq * D (the reference's transposed o_proj.weight; a
     tensor-parallel rank passes its own K rows and all-reduces the result itself); bias [N]
     bfloat16 or None.  Returns [..., N] bfloat16 (`out`, if given, is written in place).  Products
-    and sums are float32; the result is rounded to bfloat16 once.
+    and sums are float32; the result is rounded to bfloat16 once.  Calls of up to 128 rows (decode,
+    verify steps) spread K over several workgroups per column slab and need scratch memory for the
+    partial sums: a uint8 tensor `workspace` of at least `o_proj_workspace_bytes(M, K, N)` bytes, or,
+    by default, a buffer cached per (device, stream).
     """
     lib = _lib.load()
     for n, t in (("x", x), ("o_weight", o_weight)):
@@ -620,9 +623,23 @@ def o_proj(x, o_weight, bias=None, *, out=None):
         _need_device("out", out)
         _check(tuple(out.shape) == lead + (N,) and out.dtype == torch.bfloat16, f"out must be bfloat16 {lead + (N,)}")
     with _on(x.device):
-        rc = lib.pa_o_proj(_ptr(x), _ptr(o_weight), _ptr(bias), _ptr(out), M, K, N, BF16, _stream_ptr(x.device))
+        stream = _stream_ptr(x.device)
+        need = int(lib.pa_o_proj_workspace_bytes(M, K, N))
+        if workspace is not None:
+            _need_device("workspace", workspace)
+            _check(workspace.dtype == torch.uint8 and workspace.is_contiguous(), "workspace must be a contiguous uint8 tensor")
+            _same_device(x, workspace=workspace)
+        elif need:
+            workspace = _workspace(x.device, need, stream)
+        rc = lib.pa_o_proj_ws(_ptr(x), _ptr(o_weight), _ptr(bias), _ptr(out), _ptr(workspace),
+                              workspace.numel() if workspace is not None else 0, M, K, N, BF16, stream)
     _raise_on(rc, "pa_o_proj")
     return out
+
+
+def o_proj_workspace_bytes(M: int, K: int, N: int) -> int:
+    """Scratch bytes `o_proj` would use for a call of M rows (0 for shapes that take none)."""
+    return int(_lib.load().pa_o_proj_workspace_bytes(int(M), int(K), int(N)))
 
 
 def default_scale(head_dim: int) -> float:

@@ -112,6 +112,46 @@ def test_fed_by_the_attention_output_and_preallocated_out(pa, rng):
     assert np.abs(dev_to_f32(out) - want_all).max() <= 2e-2
 
 
+@pytest.mark.parametrize("M,K,N,bias", [(1, 4096, 4096, False), (16, 4096, 4096, True), (64, 4096, 2880, True),
+                                        (128, 2048, 4096, False), (33, 1088, 1024, True)])
+def test_few_rows_split_over_k(pa, M, K, N, bias):
+    """Up to 128 rows with a workspace: several workgroups per column slab take ranges of K (17 steps of 64 in the
+    last case: ranges of 8 and 9) and a second kernel sums their float32 partials.  Against the oracle; the same bits
+    from the cached and from a caller's workspace and from call to call; without a workspace, or with one too small for
+    two ranges, the call runs unsplit, as pa_o_proj does."""
+    from nkipy_amd import _lib
+    from nkipy_amd.paged_attn import BF16, _ptr, _stream_ptr
+    lib = _lib.load()
+    rng = np.random.default_rng(M + K + N)
+    x = O.round_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = O.round_to_bf16((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32))
+    b = O.round_to_bf16(rng.standard_normal(N).astype(np.float32)) if bias else None
+    want = O.o_proj(x, w, b)
+    xd, wd, bd = bf16_to_dev(x), bf16_to_dev(w), None if b is None else bf16_to_dev(b)
+    need = pa.o_proj_workspace_bytes(M, K, N)
+    print(f"o_proj split M={M} K={K} N={N} bias={bias} workspace={need}", flush=True)
+    assert need > 0 and need % (M * N * 4) == 0 and 2 <= need // (M * N * 4) <= 4
+    got = pa.o_proj(xd, wd, bd)
+    torch.cuda.synchronize()
+    _close(dev_to_f32(got), want)
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")      # stale bytes (NaN patterns) must not matter
+    got_ws = pa.o_proj(xd, wd, bd, workspace=ws)
+    again = pa.o_proj(xd, wd, bd)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev_bits(got_ws), dev_bits(got)) and np.array_equal(dev_bits(again), dev_bits(got))
+    # unsplit: the entry point without a workspace, and a workspace that holds less than two ranges
+    plain = torch.empty_like(got)
+    rc = lib.pa_o_proj(_ptr(xd), _ptr(wd), _ptr(bd), _ptr(plain), M, K, N, BF16, _stream_ptr(xd.device))
+    assert rc == 0
+    small = pa.o_proj(xd, wd, bd, workspace=ws[:2 * M * N * 4 - 16])
+    torch.cuda.synchronize()
+    _close(dev_to_f32(plain), want)
+    assert np.array_equal(dev_bits(small), dev_bits(plain))
+    # the two orders of summation agree to the last bf16 step
+    assert np.abs(dev_to_f32(plain) - dev_to_f32(got)).max() <= 2.0 ** -7 * np.abs(want).max()
+    assert pa.o_proj_workspace_bytes(300, K, N) == 0
+
+
 def test_argument_errors(pa):
     x = torch.zeros(4, 96, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError):
