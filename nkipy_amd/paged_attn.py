@@ -28,6 +28,7 @@ F32, BF16, FP8 = 0, 1, 2
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float8_e4m3fn: FP8}
 
 _workspaces = {}
+_o_proj_need = {}           # (M, K, N) -> scratch bytes of o_proj's few-rows form (a pure function of the shape)
 
 
 def _need_device(name, t):
@@ -624,12 +625,17 @@ def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
         _check(tuple(out.shape) == lead + (N,) and out.dtype == torch.bfloat16, f"out must be bfloat16 {lead + (N,)}")
     with _on(x.device):
         stream = _stream_ptr(x.device)
-        need = int(lib.pa_o_proj_workspace_bytes(M, K, N))
+        need = _o_proj_need.get((M, K, N))
+        if need is None:
+            need = _o_proj_need[(M, K, N)] = int(lib.pa_o_proj_workspace_bytes(M, K, N))
         if workspace is not None:
             _need_device("workspace", workspace)
             _check(workspace.dtype == torch.uint8 and workspace.is_contiguous(), "workspace must be a contiguous uint8 tensor")
             _same_device(x, workspace=workspace)
         elif need:
+            # (the split form is one more launch: where a step of a few rows is launched call by call and bound by the
+            # host it costs 5 us per layer, replayed from a HIP graph it saves 6; it is taken either way, so that the
+            # result does not depend on how the call was issued)
             workspace = _workspace(x.device, need, stream)
         rc = lib.pa_o_proj_ws(_ptr(x), _ptr(o_weight), _ptr(bias), _ptr(out), _ptr(workspace),
                               workspace.numel() if workspace is not None else 0, M, K, N, BF16, stream)
