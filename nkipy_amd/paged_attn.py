@@ -631,6 +631,7 @@ def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
         if workspace is not None:
             _need_device("workspace", workspace)
             _check(workspace.dtype == torch.uint8 and workspace.is_contiguous(), "workspace must be a contiguous uint8 tensor")
+            _check(workspace.data_ptr() % 16 == 0, "workspace must be 16-byte aligned")
             _same_device(x, workspace=workspace)
         elif need:
             # (the split form is one more launch: where a step of a few rows is launched call by call and bound by the

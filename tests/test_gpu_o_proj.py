@@ -166,3 +166,11 @@ def test_argument_errors(pa):
         pa.o_proj(x.float(), torch.zeros(128, 64, dtype=torch.float32, device="cuda"))
     with pytest.raises(NotImplementedError):
         pa.o_proj(np.zeros((4, 128), np.float32), np.zeros((128, 64), np.float32))
+    w = torch.zeros(1024, 256, dtype=torch.bfloat16, device="cuda")
+    x = torch.zeros(4, 1024, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(pa.o_proj_workspace_bytes(4, 1024, 256) + 16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(ValueError):
+        pa.o_proj(x, w, workspace=ws[1:])                                             # workspace not 16-byte aligned
+    with pytest.raises(ValueError):
+        pa.o_proj(x, w, workspace=ws.float())                                         # not a uint8 tensor
+    assert pa.o_proj_workspace_bytes(4, 100, 256) == 0 and pa.o_proj_workspace_bytes(0, 1024, 256) == 0
