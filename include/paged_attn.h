@@ -96,9 +96,12 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * partitions; the default MFMA kernel for bf16 / fp8 KV instead cuts the
  * flattened stream of all sequences' 32-token tiles into equal chunks, one per
  * resident wavefront group, so its partition length follows the batch and the
- * device, not partition_size.  The result does not depend on the split.
- * max_seq_len: upper bound of seq_lens (sizes the grid; 0 = max_blocks_per_seq *
- * block_size).  seq_lens[b] == 0 yields zeros.
+ * device, not partition_size.  Small calls without sinks or a window (at most
+ * four partitions per sequence and at most 288 MiB of K and V by max_seq_len)
+ * take the fixed-partition MFMA kernel, whose fixed cost is lower.  The result
+ * does not depend on the split beyond the order of float32 sums.
+ * max_seq_len: upper bound of seq_lens (sizes the grid and picks the kernel; 0 =
+ * max_blocks_per_seq * block_size).  seq_lens[b] == 0 yields zeros.
  * q_dtype / kv_dtype: (F32, F32), (BF16, BF16) or (BF16, FP8_E4M3FN).
  * sinks: NULL, or [Hq] float32 per-head logits that join every softmax as one more column and
  *   are dropped afterwards (examples/models/gpt_oss/kernels/attention.py:137-148): they only

@@ -200,11 +200,30 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
 
 // Which kernel pa_decode takes for a shape: 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced;
 // -1 when a forced kernel (debug switch 0) does not take the shape.
-static int decode_kind(const DecodeParams& p, int q_dtype, int kv_dtype) {
+// The balanced kernel pays a fixed price for its schedule (a scan of the lengths in every workgroup, partials and a
+// merge launch whatever the sizes: 11 us for the smallest call), the fixed-partition kernel merges a sequence's
+// waves inside the workgroup and needs the merge launch only past one partition, but leaves the device unevenly
+// filled at scale.  Per call replayed from a HIP graph (B x context, 32 / 8 heads of 128, bf16, us, fixed against
+// balanced): 1 x 256 5.7 / 11.4, 16 x 256 5.9 / 12.7, 16 x 1 K 16.6 / 20.7, 64 x 1 K 45.7 / 50.8, 4 x 8 K 30.7 /
+// 31.3; 16 x 8 K 114 / 92, 64 x 2 K 109 / 91.  So calls of at most four partitions per sequence that can touch at
+// most this many bytes of K and V, by the caller's bound on the lengths, take the fixed partitions when nothing
+// needs the balanced kernel (with more partitions per sequence the two are level at best: 8 x 4 K inside a layer
+// step 52.5 / 49.7).
+constexpr long kDecodeSmallCallBytes = 288L << 20;
+static bool decode_small_call(const DecodeParams& p, int kv_dtype) {
+  const long esz = kv_dtype == PA_FP8_E4M3FN ? 1 : (kv_dtype == PA_BF16 ? 2 : 4);
+  if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
+  if (num_partitions_for(p.max_seq_len, p.partition_size) > 4) return false;
+  const double bytes = 2.0 * p.B * (double)p.max_seq_len * p.Hkv * p.D * esz;
+  return bytes <= (double)kDecodeSmallCallBytes;
+}
+static int decode_kind(const DecodeParams& p, int q_dtype, int kv_dtype, bool needs_balanced = false) {
   const int impl = g_decode_impl.load();
   const bool mfma_ok = decode_mfma_supported(p, q_dtype, kv_dtype);
   if ((impl == 2 || impl == 3) && !mfma_ok) return -1;
-  return !mfma_ok || impl == 1 ? 1 : (impl == 2 ? 2 : 3);
+  if (!mfma_ok || impl == 1) return 1;
+  if (impl == 0) return !needs_balanced && decode_small_call(p, kv_dtype) ? 2 : 3;
+  return impl == 2 ? 2 : 3;
 }
 
 size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len,
@@ -214,13 +233,17 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
   memset(&p, 0, sizeof(p));
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = 1; p.rows_per_wave = 16;
   p.block_size = block_size; p.block_shift = ilog2_exact(block_size);
+  p.max_seq_len = max_seq_len; p.partition_size = partition_size;
   const int kind = decode_kind(p, q_dtype, kv_dtype);
-  if (kind == 3) {
-    plan_decode_balanced(p, current_num_cus());
-    return decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
-  }
   const int np = num_partitions_for(max_seq_len, partition_size);
-  return np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+  const size_t fixed = np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+  if (kind == 1 || kind < 0) return fixed;
+  plan_decode_balanced(p, current_num_cus());
+  const size_t balanced = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
+  if (kind == 3) return balanced;
+  // fixed partitions, by choice or by the size of the call: a call with sinks or a window takes the balanced
+  // kernel all the same, so the answer covers both
+  return fixed > balanced ? fixed : balanced;
 }
 
 int pa_decode(const void* q, const void* k_cache, const void* v_cache,
@@ -266,7 +289,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   if (p.num_partitions > 65535 || B > 65535) return fail_arg("pa_decode: grid too large (partitions=%d B=%d)", p.num_partitions, B);
   hipStream_t s = (hipStream_t)stream;
   // kernel choice: 0 automatic, 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced
-  const int kind = decode_kind(p, q_dtype, kv_dtype);
+  const int kind = decode_kind(p, q_dtype, kv_dtype, sinks != nullptr || sliding_window > 0);
   if (kind < 0) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
   if (kind == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
   if ((sinks || sliding_window > 0) && kind != 3)

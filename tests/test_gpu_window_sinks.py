@@ -75,17 +75,27 @@ def test_decode_window_fp8_long_single_sequence(pa):
 
 
 def test_neutral_options_change_nothing(pa):
-    """A window at least as long as every context and sinks of -inf give the plain result bit for bit."""
+    """A window at least as long as every context and sinks of -inf give the plain result bit for bit, in the
+    kernel that implements them (the balanced one).  A plain call this small is served by the fixed-partition
+    kernel by default, whose sums are taken in another order: equal to the tolerance there."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
     rng = np.random.default_rng(22)
     D, Hq, Hkv, bs = 128, 8, 2, 32
     ctxs = [5, 700, 2049]
     k, v, tables = make_paged(rng, len(ctxs), Hkv, D, bs, ctxs)
     q = rng.standard_normal((len(ctxs), Hq, D)).astype(np.float32)
     args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), 0.09)
-    plain = dev_bits(pa.decode(*args))
-    assert np.array_equal(dev_bits(pa.decode(*args, sliding_window=2049)), plain)
-    assert np.array_equal(dev_bits(pa.decode(*args, sinks=_f32(np.full(Hq, -np.inf)))), plain)
-    assert not np.array_equal(dev_bits(pa.decode(*args, sliding_window=2048)), plain)
+    lib.pa_debug_set(0, 3)
+    try:
+        plain = pa.decode(*args)
+        assert np.array_equal(dev_bits(pa.decode(*args, sliding_window=2049)), dev_bits(plain))
+        assert np.array_equal(dev_bits(pa.decode(*args, sinks=_f32(np.full(Hq, -np.inf)))), dev_bits(plain))
+        assert not np.array_equal(dev_bits(pa.decode(*args, sliding_window=2048)), dev_bits(plain))
+    finally:
+        lib.pa_debug_set(0, 0)
+    assert_close_abs(dev_to_f32(pa.decode(*args)), dev_to_f32(plain), BF16_TOL)
+    assert np.array_equal(dev_bits(pa.decode(*args, sliding_window=2049)), dev_bits(plain))    # options: the balanced kernel
 
 
 @pytest.fixture(params=[16, 32], ids=["rows16", "rows32"])
