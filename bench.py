@@ -10,7 +10,8 @@ carries, under "configs", one record each for config 3 (paged chunked prefill),
 config 4 (blocksparse prefill) and config 5 (fp8-KV long-context decode), timed in
 the same run with the same protocol: both halves of the headline metric and every
 benchmark-sized configuration, plus "o_proj", the output projection behind config 3's
-attention.  --config N prints that configuration alone.
+attention.  --config N prints that configuration alone (6-13: the kernels and steps around the
+attention call; their docstrings say what each one is).
 
 value      whole-step throughput: algorithmic HBM bytes / step time for the decode
            configs (GB/s), attention FLOPs / step time for the prefill configs
@@ -591,12 +592,63 @@ def bench_prefill_layer_step(steps, warmup, lib, pa, W):
     }
 
 
+def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
+    """config 13: a decode step of a small batch through the engine glue, per attention layer: QK RMSNorm + RoPE +
+    K/V row into the pool + paged decode + output projection (`PagedAttention.attend`), `layers` layers with a pool
+    and weights of their own, issued call by call and replayed from one HIP graph.  Launch-bound: the figure is
+    microseconds per layer; the bytes a layer has to move (its contexts' K and V, the projection weight) are given
+    for scale."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
+    nblk = (ctx + 64) // bs + 1
+    cache = PagedKVCache(B * nblk + 8, bs, Hkv, D, max_seqs=B, max_blocks_per_seq=nblk, num_layers=layers)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1313)
+    one = torch.ones(D, dtype=torch.bfloat16, device="cuda")
+    att = [PagedAttention(cache, Hq, layer=l, rope_base=1e6, max_positions=nblk * bs, q_norm_weight=one, k_norm_weight=one,
+                          o_weight=(torch.randn(Hq * D, N, generator=gen, device="cuda") / 64).to(torch.bfloat16))
+           for l in range(layers)]
+    for pool in cache.k_caches + cache.v_caches:
+        pool.copy_(torch.randn(pool.shape, generator=gen, device="cuda", dtype=torch.float32))
+    cache.extend(list(range(B)), [ctx] * B)      # contexts of `ctx` tokens (the pool holds whatever it holds)
+    q1 = torch.randn(B, 1, Hq, D, generator=gen, device="cuda").to(torch.bfloat16)
+    k1 = torch.randn(B, 1, Hkv, D, generator=gen, device="cuda").to(torch.bfloat16)
+
+    def step():
+        for a in att:
+            a.attend(q1, k1, k1)
+
+    cache.begin_step([1] * B, 1)
+    sec_eager = _time_steps(step, steps, warmup)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    sec = _time_steps(graph.replay, steps, 5)
+    kv_bytes = 2 * B * (ctx + 1) * Hkv * D * 2
+    byts = kv_bytes + Hq * D * N * 2 + B * (2 * Hq * D + 2 * Hkv * D + N) * 2
+    us = sec / layers * 1e6
+    return {
+        "metric": "decode layer step (QK-norm + RoPE + KV write + paged decode + o_proj), layers/s, HIP graph replay",
+        "value": round(1e6 / us, 1), "unit": "layer steps/s",
+        "ms_per_step": round(sec * 1e3, 5), "us_per_layer": round(us, 2),
+        "eager_us_per_layer": round(sec_eager / layers * 1e6, 2),
+        "dtype": "bf16, float32 norm, bf16 rotation, fp32 accumulate",
+        "config": {"workload": f"decode layer step: B={B}, context={ctx}, layers={layers}, Hq={Hq}, Hkv={Hkv}, D={D}, "
+                               f"block_size={bs}, hidden={N}; one step = {layers} layers", "algorithmic_bytes_per_layer": byts},
+        "roofline": {"bound": "hbm", "achieved": round(byts / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(byts / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "five launches per layer (KV write with K transform, decode + merge, projection + merge)",
+                     "kernel_avg_ms": round(us * 1e-3, 5), "launches_timed": steps * layers},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12],
+    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     ap.add_argument("--const-data", action="store_true",
@@ -643,6 +695,8 @@ def main():
             res = bench_prefill(args.steps, args.warmup, lib, pa, W, gpt_oss=True)
         elif cfg == 12:
             res = bench_o_proj(args.steps, args.warmup, lib, pa, W)
+        elif cfg == 13:
+            res = bench_decode_layer_step(args.steps, args.warmup, lib, pa, W)
         else:
             res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
         gc.collect()
