@@ -123,15 +123,41 @@ __global__ __launch_bounds__(kGenericThreads) void decode_generic_kernel(DecodeP
 template <typename QT>
 __global__ void decode_reduce_kernel(DecodeParams p) {
   const int hq = blockIdx.x, b = blockIdx.y;
+  const long base = ((long)b * p.Hq + hq) * p.num_partitions;
+  // The kernel is a chain of dependent loads (length -> partition count -> maxima -> partials), each a trip to
+  // memory, around a few additions.  The first PRE partitions' values are therefore requested at once and before the
+  // length is known (their slots exist whatever the length; what a partition past the context holds is not used).
+  constexpr int PRE = 4;
+  const int npre = min(PRE, p.num_partitions);
+  const int d0 = threadIdx.x;
+  float m_[PRE], l_[PRE], o_[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    m_[i] = -INFINITY; l_[i] = 0.f; o_[i] = 0.f;
+    if (i < npre) {
+      m_[i] = p.ws_ml[(base + i) * 2];
+      l_[i] = p.ws_ml[(base + i) * 2 + 1];
+      if (d0 < p.D) o_[i] = p.ws_out[(base + i) * p.D + d0];
+    }
+  }
   int ctx = p.seq_lens[b];
   ctx = min(max(ctx, 0), p.max_seq_len);
   const int np = (ctx + p.partition_size - 1) / p.partition_size;
-  const long base = ((long)b * p.Hq + hq) * p.num_partitions;
   float mt = -INFINITY;
-  for (int i = 0; i < np; ++i) mt = fmaxf(mt, p.ws_ml[(base + i) * 2]);
-  for (int d = threadIdx.x; d < p.D; d += blockDim.x) {
+#pragma unroll
+  for (int i = 0; i < PRE; ++i)
+    if (i < np) mt = fmaxf(mt, m_[i]);
+  for (int i = PRE; i < np; ++i) mt = fmaxf(mt, p.ws_ml[(base + i) * 2]);
+  for (int d = d0; d < p.D; d += blockDim.x) {
     float lt = 0.f, ot = 0.f;
-    for (int i = 0; i < np; ++i) {
+#pragma unroll
+    for (int i = 0; i < PRE; ++i)
+      if (i < np) {
+        const float w = l_[i] * exp2f(m_[i] - mt);
+        lt += w;
+        ot += w * (d == d0 ? o_[i] : p.ws_out[(base + i) * p.D + d]);
+      }
+    for (int i = PRE; i < np; ++i) {
       const float w = p.ws_ml[(base + i) * 2 + 1] * exp2f(p.ws_ml[(base + i) * 2] - mt);
       lt += w;
       ot += w * p.ws_out[(base + i) * p.D + d];

@@ -535,11 +535,14 @@ __global__ __launch_bounds__(256) void o_proj_split_reduce_kernel(OProjParams p)
   const long item = (long)blockIdx.x * 256 + threadIdx.x;
   if (item >= total) return;
   const float4* src = (const float4*)p.ws + item;
-  float4 a = src[0];
-  for (int z = 1; z < p.splits; ++z) {
-    const float4 b = src[(long)z * total];
-    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
-  }
+  // all ranges requested at once (at most four exist: o_proj_splits), added in their order
+  float4 part[4];
+#pragma unroll
+  for (int z = 0; z < 4; ++z) part[z] = z < p.splits ? src[(long)z * total] : make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 a = part[0];
+#pragma unroll
+  for (int z = 1; z < 4; ++z)
+    if (z < p.splits) { a.x += part[z].x; a.y += part[z].y; a.z += part[z].z; a.w += part[z].w; }
   if (BIAS) {
     const uint2 bw = *(const uint2*)((const uint16_t*)p.bias + (item * 4) % p.N);
     a.x += bf16_bits_to_float(bw.x & 0xffffu); a.y += bf16_bits_to_float(bw.x >> 16);
