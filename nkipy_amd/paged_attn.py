@@ -50,12 +50,21 @@ def _check(cond, msg):
 
 
 def _same_device(ref, **others):
+    idx = ref.get_device()                  # an int: comparing device objects costs several times as much per tensor
     for n, t in others.items():
-        if t is not None:
-            _check(t.device == ref.device, f"{n} is on {t.device}, expected {ref.device}")
+        if t is not None and t.get_device() != idx:
+            raise ValueError(f"{n} is on {t.device}, expected {ref.device}")
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream_ptr(device):
+    """The current stream of `device` as the C ABI takes it.  torch's raw-stream query when this build has it (a
+    fraction of a microsecond; the Stream object of the public call costs several, and a decode step of a small batch
+    is bound by the host), the public call otherwise."""
+    if _raw_stream is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
