@@ -32,6 +32,8 @@ _o_proj_need = {}           # (M, K, N) -> scratch bytes of o_proj's few-rows fo
 
 
 def _need_device(name, t):
+    if isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous():
+        return                               # the usual case first: these checks run some twenty times per layer call
     if isinstance(t, np.ndarray):
         raise NotImplementedError(
             f"{name} is a NumPy array: the paged attention ops run hand-written HIP kernels and have "
@@ -175,8 +177,18 @@ class QTransform:
 
     def __init__(self, rope_cos, rope_sin, norm_weight=None, eps=1e-6):
         self.rope_cos, self.rope_sin, self.norm_weight, self.eps = rope_cos, rope_sin, norm_weight, float(eps)
+        self._checked = None                 # (key, struct) of the last validated state
 
     def _struct(self, D, q):
+        # validated once per state: the same object is passed on every call of every step
+        key = (D, q.get_device(), q.dtype, id(self.rope_cos), id(self.rope_sin), id(self.norm_weight), self.eps)
+        if self._checked is not None and self._checked[0] == key:
+            return self._checked[1]
+        st = self._build(D, q)
+        self._checked = (key, st)
+        return st
+
+    def _build(self, D, q):
         for n, t in (("rope_cos", self.rope_cos), ("rope_sin", self.rope_sin)):
             _need_device(n, t)
             _check(t.dim() == 2 and t.shape[1] == D // 2 and t.dtype == torch.bfloat16 and t.shape[0] > 0,
