@@ -165,6 +165,41 @@ def test_partition_size_invariance(pa):
         assert np.max(np.abs(o - outs[0])) <= 2 ** -7 * max(1.0, np.abs(outs[0]).max())  # a bf16 ulp or so
 
 
+def test_small_calls_take_the_fixed_partition_kernel(pa):
+    """pa_decode's own choice: a call that can touch little of the pool by its max_seq_len (at most four
+    partitions per sequence) gives the fixed-partition kernel's bits, the same call with a bound of many partitions,
+    or with sinks, the balanced kernel's; all of them the oracle's values."""
+    rng = np.random.default_rng(77)
+    B, Hq, Hkv, D, bs = 5, 16, 4, 128, 32
+    ctxs = [1, 700, 1500, 33, 1024]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    wide = np.full((B, 4096 // bs), -1, np.int32)            # the same blocks under a capacity of 8 partitions
+    wide[:, :tables.shape[1]] = tables
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+    dq, dk, dv = bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v)
+    sinks = torch.full((Hq,), -float("inf"), device="cuda")
+    want = O.paged_decode(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32),
+                          0.09, q_dtype="bf16")
+
+    def run(impl, tab, **kw):
+        _set_impl(impl)
+        try:
+            o = pa.decode(dq, dk, dv, _i32(tab), _i32(ctxs), 0.09, **kw)
+            torch.cuda.synchronize()
+        finally:
+            _set_impl(0)
+        return o
+
+    fixed, balanced = run(2, tables, max_seq_len=1500), run(3, tables, max_seq_len=1500)
+    for o in (fixed, balanced):
+        assert_close_abs(dev_to_f32(o), want, BF16_TOL)
+    assert not np.array_equal(dev_bits(fixed), dev_bits(balanced))        # (else the test below shows nothing)
+    assert np.array_equal(dev_bits(run(0, tables, max_seq_len=1500)), dev_bits(fixed))
+    assert np.array_equal(dev_bits(run(0, wide)), dev_bits(run(3, wide)))                 # bound = 4 096 tokens
+    assert np.array_equal(dev_bits(run(0, tables, max_seq_len=1500, sinks=sinks)),
+                          dev_bits(run(3, tables, max_seq_len=1500, sinks=sinks)))
+
+
 def test_identity_table_equals_dense_cache(pa):
     """A dense (B, S, Hkv, D) cache viewed as a pool with an identity table."""
     rng = np.random.default_rng(5)
