@@ -301,7 +301,9 @@ class PagedAttention:
         if T == 1:
             # the host-known bound on the contexts sizes the launch and clamps the lengths the kernel reads; a
             # launch that is being captured into a HIP graph will be replayed on longer contexts, so it gets the
-            # table capacity instead
+            # table capacity instead (the bound also picks the decode kernel: with a capacity of more than four
+            # partitions a captured step takes the balanced kernel where the eager step of short contexts takes the
+            # fixed partitions, and the two agree to the order of their float32 sums, not bit for bit)
             capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
             paged_attn.decode(q[:, 0], kc, vc, c.block_tables, c.seq_lens, self.scale,
                               k_scale=ks, v_scale=vs, partition_size=self.partition_size,
