@@ -79,8 +79,13 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
 /* The same for a known shape and dtype pair: exactly what the kernel pa_decode picks for it
  * needs (the balanced schedule's [Hq][B + chunks][D + 2] floats for bf16 / fp8 pools at head
  * dim 64 or 128 and a power-of-two block size >= 16, whatever max_seq_len is; the fixed
- * partitions' B x Hq x ceil(max_seq_len / partition_size) slots otherwise).  Never more than
- * pa_decode_workspace_bytes.  Sizing helper next to the output allocation of
+ * partitions' B x Hq x ceil(max_seq_len / partition_size) slots otherwise, and where the bound
+ * makes the call small enough for the fixed-partition matrix-core kernel).  max_seq_len is the
+ * positive bound the pa_decode call will pass, already clamped to the table capacity; with
+ * max_seq_len <= 0 (pa_decode then uses the capacity, which this function is not told) the
+ * answer covers every matrix-core kernel that call can pick — the balanced schedule or up to
+ * four fixed partitions — and is 0 for shapes that take the scalar kernel, whose callers must
+ * give the bound.  With a positive bound never more than pa_decode_workspace_bytes.  Sizing helper next to the output allocation of
  * nkipy/src/nkipy/runtime/device_tensor.py:51-74. */
 size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len,
                                      int partition_size, int q_dtype, int kv_dtype);
@@ -296,7 +301,9 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
                              int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq,
                              int num_blocks, int kv_dtype, void* stream);
 
-/* Debug switches (process-wide; tests only).  key 0: decode kernel choice
+/* Debug switches (process-wide; tests only).  They work only when PA_ENABLE_DEBUG=1 was in the
+ * environment at the library's first use; otherwise every call is refused with an argument error
+ * and changes nothing, so a server that links the library cannot have its kernels rerouted.  key 0: decode kernel choice
  * (0 = automatic, 1 = scalar-ALU kernel, 2 = MFMA kernel with fixed partitions,
  * 3 = MFMA kernel with the balanced schedule); key 1: waves per workgroup of the
  * fixed-partition MFMA kernel (0 = default); key 2: its grid order (1 = kv head
@@ -320,16 +327,6 @@ int pa_debug_set(int key, int value);
  * spike/src/spike/spike_model.py:290-363. */
 int pa_profile_enable(int on);
 int pa_profile_collect(float* ms, int cap);
-
-/* Matrix-core ceiling probe for benchmarks (no counterpart in the reference): runs
- * `iters` x 16 back-to-back v_mfma_f32_32x32x16_bf16 per wavefront on `blocks`
- * workgroups of 8 wavefronts, operands taken once from `operands` (blocks * 65536
- * bytes of bf16 values, device memory), nothing else in the loop; `sink` receives
- * blocks * 512 floats.  Synchronous; *ms is the kernel time.  FLOP = blocks * 8 *
- * iters * 16 * 32768.  The rate depends on the operand data (the chip is power
- * limited): benchmarks quote it for their own data distribution beside the nominal
- * peak. */
-int pa_probe_mfma(const void* operands, void* sink, int blocks, int iters, float* ms, void* stream);
 
 #ifdef __cplusplus
 }

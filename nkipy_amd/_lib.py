@@ -48,7 +48,6 @@ SIGNATURES = {
     "pa_debug_set": (c_int, [c_int, c_int]),
     "pa_profile_enable": (c_int, [c_int]),
     "pa_profile_collect": (c_int, [ctypes.POINTER(c_float), c_int]),
-    "pa_probe_mfma": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(c_float), c_void_p]),
 }
 
 

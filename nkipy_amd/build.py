@@ -1,6 +1,7 @@
-"""Builds libpaged_attn.so (HIP kernels + C ABI) for gfx950 with hipcc.
+"""Builds libpaged_attn.so (HIP kernels + C ABI) for gfx950 with hipcc, and libpa_bench.so, the
+matrix-core ceiling probe that only the benchmark loads.
 
-The library has no Python or torch dependency; it links only the HIP runtime.
+Neither library has a Python or torch dependency; they link only the HIP runtime.
 Run `python -m nkipy_amd.build` or call `build()`.
 """
 from __future__ import annotations
@@ -15,7 +16,9 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpaged_attn.so")
 
-SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip", "pa_prefill_async.hip", "pa_kv_write.hip", "pa_o_proj.hip", "pa_probe.hip"]
+SOURCES = ["pa_capi.hip", "pa_decode_generic.hip", "pa_decode_mfma.hip", "pa_prefill.hip", "pa_prefill_async.hip", "pa_kv_write.hip", "pa_o_proj.hip"]
+BENCH_SOURCES = ["pa_probe.hip"]
+BENCH_LIB_PATH = os.path.join(LIB_DIR, "libpa_bench.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -43,11 +46,12 @@ def build(extra_flags=(), jobs: int = 4) -> str:
     """Compile every HIP source and link the shared library; returns its path."""
     os.makedirs(LIB_DIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"link failed:\n{r.stderr}")
+        objs = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES + BENCH_SOURCES))
+    for path, part in ((LIB_PATH, objs[:len(SOURCES)]), (BENCH_LIB_PATH, objs[len(SOURCES):])):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *part, "-o", path]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"link of {os.path.basename(path)} failed:\n{r.stderr}")
     return LIB_PATH
 
 

@@ -3,6 +3,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -54,25 +55,42 @@ static std::atomic<int> g_prefill_split{1};
 static std::atomic<int> g_d64_tiled_from{PA_VERIFY_MAX_TOKENS + 1};   // query tokens from which head dim 64 takes the tiled kernel
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
+// Events come from a free list that pa_profile_collect refills, so that a timed pass which follows a collected
+// pass of the same length creates none: the records are then all the profiling adds to a step.
 static std::atomic<int> g_profile{0};
 static std::mutex g_prof_mu;
 static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
+static std::vector<hipEvent_t> g_prof_free;
 static thread_local hipEvent_t tl_start = nullptr;
+
+static hipEvent_t profile_event() {
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    if (!g_prof_free.empty()) {
+      hipEvent_t e = g_prof_free.back();
+      g_prof_free.pop_back();
+      return e;
+    }
+  }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  return e;
+}
 
 void profile_begin(hipStream_t s) {
   if (!g_profile.load(std::memory_order_relaxed)) return;
-  hipEvent_t a = nullptr;
-  if (hipEventCreate(&a) != hipSuccess) return;
+  hipEvent_t a = profile_event();
+  if (!a) return;
   (void)hipEventRecord(a, s);
   tl_start = a;
 }
 
 void profile_end(hipStream_t s) {
   if (!tl_start) return;
-  hipEvent_t b = nullptr;
-  if (hipEventCreate(&b) != hipSuccess) { (void)hipEventDestroy(tl_start); tl_start = nullptr; return; }
-  (void)hipEventRecord(b, s);
+  hipEvent_t b = profile_event();
   std::lock_guard<std::mutex> lk(g_prof_mu);
+  if (!b) { g_prof_free.push_back(tl_start); tl_start = nullptr; return; }
+  (void)hipEventRecord(b, s);
   g_prof_events.emplace_back(tl_start, b);
   tl_start = nullptr;
 }
@@ -113,7 +131,22 @@ int pa_version(void) { return 100; }
 
 const char* pa_last_error(void) { return tl_error; }
 
+// The switches reroute kernels for every thread of the process, so a server that links the library cannot be
+// switched by accident or by another component: they work only when PA_ENABLE_DEBUG=1 was in the environment
+// when the first call looked (tests set it), and are refused otherwise.
+static bool debug_enabled() {
+  static const bool on = [] {
+    const char* v = getenv("PA_ENABLE_DEBUG");
+    return v && v[0] == '1' && v[1] == 0;
+  }();
+  return on;
+}
+
 int pa_debug_set(int key, int value) {
+  tl_error[0] = 0;
+  if (!debug_enabled())
+    return fail_arg("pa_debug_set: the debug switches are off (set PA_ENABLE_DEBUG=1 in the environment before the "
+                    "library's first use)");
   if (key == 0) { g_decode_impl = value; return 0; }
   if (key == 1) { g_decode_waves = value; return 0; }
   if (key == 2) { g_head_major = value; return 0; }
@@ -143,27 +176,15 @@ int pa_profile_collect(float* ms, int cap) {
     if (hipEventSynchronize(pr.second) == hipSuccess &&
         hipEventElapsedTime(&t, pr.first, pr.second) == hipSuccess && ms && n < cap)
       ms[n++] = t;
-    (void)hipEventDestroy(pr.first);
-    (void)hipEventDestroy(pr.second);
+  }
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    for (auto& pr : ev) {
+      g_prof_free.push_back(pr.first);
+      g_prof_free.push_back(pr.second);
+    }
   }
   return n;
-}
-
-int pa_probe_mfma(const void* operands, void* sink, int blocks, int iters, float* ms, void* stream) {
-  tl_error[0] = 0;
-  if (!operands || !sink || !ms || blocks <= 0 || iters <= 0) return fail_arg("pa_probe_mfma: bad arguments");
-  if (!aligned16(operands)) return fail_arg("pa_probe_mfma: operands must be 16-byte aligned");
-  hipStream_t s = (hipStream_t)stream;
-  hipEvent_t e0, e1;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return check_hip(hipGetLastError(), "pa_probe_mfma events");
-  (void)hipEventRecord(e0, s);
-  hipError_t e = launch_mfma_probe(operands, sink, blocks, iters, s);
-  (void)hipEventRecord(e1, s);
-  if (e == hipSuccess) e = hipEventSynchronize(e1);
-  if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  return check_hip(e, "pa_probe_mfma");
 }
 
 // Checks an optional Q transform and copies it into the kernel parameters; returns 0 or -1.
@@ -237,6 +258,16 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
   const int kind = decode_kind(p, q_dtype, kv_dtype);
   const int np = num_partitions_for(max_seq_len, partition_size);
   const size_t fixed = np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
+  if (max_seq_len <= 0) {
+    // no bound given: pa_decode then takes the table capacity, which this function is not told.  The answer covers
+    // every kernel that call can pick: the balanced one, or fixed partitions, which are chosen for at most four
+    // (the scalar kernel's partitions are not bounded that way: its callers give the bound)
+    if (kind == 1 || kind < 0) return 0;
+    plan_decode_balanced(p, current_num_cus());
+    const size_t balanced = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
+    const size_t four = (size_t)B * Hq * 4 * ((size_t)D + 2) * sizeof(float);
+    return four > balanced ? four : balanced;
+  }
   if (kind == 1 || kind < 0) return fixed;
   plan_decode_balanced(p, current_num_cus());
   const size_t balanced = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);

@@ -288,8 +288,6 @@ hipError_t launch_o_proj(const OProjParams& p, hipStream_t s);
 int o_proj_splits(int M, int K, int N);     // K ranges the few-rows forms would like to spread over more workgroups
 void o_proj_debug_force_large(int on);      // debug: 256 x 256 tiles also where the 128 x 128 form would be taken
 
-// matrix-core ceiling probe: `operands` holds blocks * 512 * 128 bytes of bf16 values, `sink` blocks * 512 floats
-hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s);
 hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,
                          int B, int row_bytes, int block_size, int max_blocks, int num_blocks,
                          int max_seq_len, hipStream_t s);

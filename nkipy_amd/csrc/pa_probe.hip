@@ -4,10 +4,12 @@
 // DATA (constant operands toggle few wires and run near the nominal clock, N(0,1) values
 // measured about 30 % lower), so benchmarks quote it for the same data distribution as
 // their inputs next to the nominal peak.
+//
+// Built into libpa_bench.so, a library of its own that only the benchmark loads: the
+// product library exports nothing that exists for measurements alone.
 #include "pa_common.h"
 
 namespace pa {
-namespace {
 
 __global__ __launch_bounds__(512) void mfma_probe_kernel(const uint4* operands, float* sink, int iters) {
   f32x16_t acc[4];
@@ -31,11 +33,25 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(const uint4* operands, 
   sink[(long)blockIdx.x * 512 + threadIdx.x] = s;
 }
 
-}  // namespace
-
-hipError_t launch_mfma_probe(const void* operands, void* sink, int blocks, int iters, hipStream_t s) {
-  hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(512), 0, s, (const uint4*)operands, (float*)sink, iters);
-  return hipGetLastError();
-}
-
 }  // namespace pa
+
+// Runs `iters` x 16 back-to-back v_mfma_f32_32x32x16_bf16 per wavefront on `blocks` workgroups of 8
+// wavefronts, operands taken once from `operands` (blocks * 65536 bytes of bf16 values, device memory),
+// nothing else in the loop; `sink` receives blocks * 512 floats.  Synchronous; *ms is the kernel time.
+// FLOP = blocks * 8 * iters * 16 * 32768.  Returns 0, -1 for bad arguments, or the hipError_t.
+extern "C" int pa_bench_probe_mfma(const void* operands, void* sink, int blocks, int iters, float* ms, void* stream) {
+  if (!operands || !sink || !ms || blocks <= 0 || iters <= 0 || ((uintptr_t)operands & 15u)) return -1;
+  hipStream_t s = (hipStream_t)stream;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return (int)hipGetLastError();
+  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return (int)hipGetLastError(); }
+  (void)hipEventRecord(e0, s);
+  hipLaunchKernelGGL(pa::mfma_probe_kernel, dim3(blocks), dim3(512), 0, s, (const uint4*)operands, (float*)sink, iters);
+  hipError_t e = hipGetLastError();
+  (void)hipEventRecord(e1, s);
+  if (e == hipSuccess) e = hipEventSynchronize(e1);
+  if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return (int)e;
+}

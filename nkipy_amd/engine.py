@@ -92,11 +92,18 @@ class PagedKVCache:
     """
 
     def __init__(self, num_blocks: int, block_size: int, n_kv_heads: int, head_dim: int, *, max_seqs: int,
-                 max_blocks_per_seq: int, dtype=torch.bfloat16, device="cuda", num_layers: int = 1):
+                 max_blocks_per_seq: int, dtype=torch.bfloat16, device="cuda", num_layers: int = 1,
+                 max_model_len: Optional[int] = None):
         if dtype not in (torch.bfloat16, torch.float8_e4m3fn):
             raise ValueError(f"unsupported pool dtype {dtype}")
         if num_layers < 1:
             raise ValueError("num_layers must be at least 1")
+        # the longest sequence a slot may grow to: the table capacity (whole blocks) unless the model's own limit is
+        # lower (a model of 1000 positions over blocks of 64 has a capacity of 1024 and a limit of 1000)
+        cap = max_blocks_per_seq * block_size
+        if max_model_len is not None and not 0 < max_model_len <= cap:
+            raise ValueError(f"max_model_len {max_model_len} outside (0, {cap}] (the table capacity)")
+        self.max_model_len = cap if max_model_len is None else int(max_model_len)
         self.block_size, self.n_kv_heads, self.head_dim = block_size, n_kv_heads, head_dim
         self.max_seqs, self.max_blocks_per_seq, self.num_layers = max_seqs, max_blocks_per_seq, num_layers
         self.device = torch.device(device)
@@ -139,8 +146,9 @@ class PagedKVCache:
         for s, n in zip(slots, n_new):
             if n < 0:
                 raise ValueError("n_new must be non-negative")
-            if (self.lens[s] + n + self.block_size - 1) // self.block_size > self.max_blocks_per_seq:
-                raise ValueError(f"slot {s}: {self.lens[s] + n} tokens exceed the table capacity")
+            if self.lens[s] + n > self.max_model_len:
+                raise ValueError(f"slot {s}: {self.lens[s] + n} tokens exceed the longest sequence the cache admits "
+                                 f"({self.max_model_len}: the table capacity, or max_model_len if that is lower)")
         if sum(max(x, 0) for x in need) > self.allocator.num_free:
             raise OutOfBlocks(f"{sum(need)} blocks requested, {self.allocator.num_free} free")
         for s, n, k in zip(slots, n_new, need):
@@ -222,7 +230,11 @@ class PagedAttention:
     `attend` makes no host synchronisation and, after the first call of a given T, no allocation, so the
     launch-bound decode step of a stack of layers can be captured into one HIP graph (`torch.cuda.graph`) with
     xq / xk / xv as static buffers and replayed every step: `begin_step` stays outside the graph (it publishes
-    the step's table rows and lengths, which the replayed kernels read from the same device tensors).
+    the step's table rows and lengths, which the replayed kernels read from the same device tensors).  A captured
+    decode step is sized by `max_seq_len`, the longest context it will be replayed on (default: the longest
+    sequence the cache admits).  The bound also picks the decode kernel: up to four partitions of
+    `partition_size` tokens take the fixed-partition kernel, which is what makes small steps cheap, longer
+    bounds the balanced one; the two agree to the order of their float32 sums, not bit for bit.
     """
 
     def __init__(self, cache: PagedKVCache, n_heads: int, *, layer: int = 0, scale: Optional[float] = None,
@@ -251,13 +263,13 @@ class PagedAttention:
         elif q_norm_weight is not None or k_norm_weight is not None:
             raise ValueError("the fused pre-attention kernel applies the norm together with RoPE: give rope_base")
         if self.rope is not None:
-            # the kernels clamp positions past the table to its last row: a table shorter than what the
-            # block tables can hold would silently rotate late tokens by the wrong angle
-            cap = cache.max_blocks_per_seq * cache.block_size
+            # the kernels clamp positions past the table to its last row: a table shorter than the longest
+            # sequence the cache admits would silently rotate late tokens by the wrong angle
+            cap = cache.max_model_len
             if self.rope[0].shape[0] < cap:
-                raise ValueError(f"RoPE tables cover {self.rope[0].shape[0]} positions, the cache holds sequences of up "
-                                 f"to {cap} tokens ({cache.max_blocks_per_seq} blocks of {cache.block_size}): give "
-                                 f"max_positions >= {cap}")
+                raise ValueError(f"RoPE tables cover {self.rope[0].shape[0]} positions, the cache admits sequences of up "
+                                 f"to {cap} tokens ({cache.max_blocks_per_seq} blocks of {cache.block_size}, max_model_len "
+                                 f"{cache.max_model_len}): give max_positions >= {cap} or the cache a lower max_model_len")
         # output projection behind the attention call (examples/models/qwen3/kernels/attention.py:143-147;
         # with the bias gpt_oss/kernels/attention.py:155-163): o_weight [n_heads * head_dim, hidden] bfloat16 as the
         # reference stores it, this rank's rows; `attend` then returns [max_seqs, T, hidden] for the caller to all-reduce
@@ -274,8 +286,11 @@ class PagedAttention:
         self.cache.begin_step(query_lens, xq.shape[1])
         return self.attend(xq, xk, xv)
 
-    def attend(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor) -> torch.Tensor:
+    def attend(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, *,
+               max_seq_len: Optional[int] = None) -> torch.Tensor:
         c, l = self.cache, self.layer
+        if max_seq_len is not None and not 0 < max_seq_len <= c.max_model_len:
+            raise ValueError(f"max_seq_len {max_seq_len} outside (0, {c.max_model_len}]")
         B, T = xq.shape[:2]
         if B != c.max_seqs or T != c.step_tokens:
             raise ValueError(f"expected [{c.max_seqs}, {c.step_tokens}, ...] as opened by begin_step, got [{B}, {T}, ...]")
@@ -299,15 +314,17 @@ class PagedAttention:
             paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq
         if T == 1:
-            # the host-known bound on the contexts sizes the launch and clamps the lengths the kernel reads; a
-            # launch that is being captured into a HIP graph will be replayed on longer contexts, so it gets the
-            # table capacity instead (the bound also picks the decode kernel: with a capacity of more than four
-            # partitions a captured step takes the balanced kernel where the eager step of short contexts takes the
-            # fixed partitions, and the two agree to the order of their float32 sums, not bit for bit)
+            # the bound on the contexts sizes the launch, clamps the lengths the kernel reads and picks the kernel.
+            # The caller's bound if given; else what the host knows of this step's contexts, unless the launch is
+            # being captured into a HIP graph: that will be replayed on longer contexts, so it gets the longest
+            # sequence the cache admits.
             capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
+            bound = max_seq_len if max_seq_len is not None else (c.max_model_len if capturing else max(c.max_seq_len, 1))
+            if bound < c.max_seq_len:
+                raise ValueError(f"max_seq_len {bound} is below a live context of {c.max_seq_len} tokens")
             paged_attn.decode(q[:, 0], kc, vc, c.block_tables, c.seq_lens, self.scale,
                               k_scale=ks, v_scale=vs, partition_size=self.partition_size,
-                              max_seq_len=None if capturing else max(c.max_seq_len, 1), out=out[:, 0],
+                              max_seq_len=bound, out=out[:, 0],
                               sinks=self.sinks, sliding_window=self.sliding_window, q_transform=qt)
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:

@@ -144,23 +144,37 @@ def decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size) -> int:
     return int(_lib.load().pa_decode_workspace_bytes(B, Hq, D, max_seq_len, partition_size))
 
 
-_WORKSPACE_SLOTS = 16     # (device, stream) pairs whose workspace is kept; the least recently used goes first
-_retired = []             # buffers a captured graph may still write to: kept until the process ends
+_WORKSPACE_SLOTS = 16     # (device, stream) pairs whose eager workspace is kept; the least recently used goes first
+_graph_workspaces = {}    # buffers handed out while a stream was being captured: a graph has their address baked in
+_graph_retired = []       # ... and those that a later capture outgrew; both are kept until the process ends
 
 
 def _workspace(device, nbytes, stream=None):
     """Scratch for split-K partials, cached per (device, stream) so that calls on one stream reuse one
-    buffer and calls on different streams never share one.  The cache holds at most _WORKSPACE_SLOTS
-    entries (a server that cycles streams does not accumulate device memory); dropping an entry returns
-    its memory to torch's allocator, which reuses it in stream order.  While the stream is being
-    captured into a HIP graph a buffer that is too small is retired, not dropped: graphs captured
-    earlier on that stream have its address baked in.  Callers that replay graphs should pass a
-    `workspace=` of their own, sized with the *_workspace_bytes functions, and keep it alive."""
+    buffer and calls on different streams never share one.
+
+    Eager calls: the cache holds at most _WORKSPACE_SLOTS entries (a server that cycles streams does not
+    accumulate device memory); dropping or outgrowing an entry returns its memory to torch's allocator,
+    which reuses it in stream order.
+
+    Calls issued while the stream is being captured into a HIP graph take their buffer from a second cache
+    that eager calls never touch and that is never evicted or freed: the graph has the address baked in, and
+    neither a larger eager call on the same stream after the capture nor the eviction of a stream's entry may
+    take that memory away from it.  A capture that needs more than the cached graph buffer retires it (kept
+    alive) and takes a new one.  All graphs captured on one capture stream share that one buffer, as all calls
+    on a stream do: replays of two of them that overlap on different streams race on it.  Callers that replay
+    graphs concurrently pass a `workspace=` of their own per graph, sized with the *_workspace_bytes functions,
+    and keep it alive."""
     key = (device, (stream or _stream_ptr(device)).value)
+    if torch.device(device).type == "cuda" and torch.cuda.is_current_stream_capturing():
+        buf = _graph_workspaces.get(key)
+        if buf is None or buf.numel() < nbytes:
+            if buf is not None:
+                _graph_retired.append(buf)
+            buf = _graph_workspaces[key] = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        return buf
     buf = _workspaces.pop(key, None)
     if buf is None or buf.numel() < nbytes:
-        if buf is not None and buf.is_cuda and torch.cuda.is_current_stream_capturing():
-            _retired.append(buf)
         buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
     _workspaces[key] = buf              # (re)inserted last: dict order is the LRU order
     while len(_workspaces) > _WORKSPACE_SLOTS:
@@ -611,7 +625,8 @@ def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
     examples/models/qwen3/kernels/attention.py:143-147 and examples/models/gpt_oss/kernels/attention.py:155-163.
 
     x: the attention output, bfloat16, [..., Hq, D] (as `decode` / `prefill` return it) or already
-    [..., K]; o_weight [K, N] bfloat16 with K = Hq * D (the reference's transposed o_proj.weight; a
+    [..., K] (with a single q head the two readings coincide: `out`'s rank decides, and without `out` x is
+    read as [..., K]); o_weight [K, N] bfloat16 with K = Hq * D (the reference's transposed o_proj.weight; a
     tensor-parallel rank passes its own K rows and all-reduces the result itself); bias [N]
     bfloat16 or None.  Returns [..., N] bfloat16 (`out`, if given, is written in place).  Products
     and sums are float32; the result is rounded to bfloat16 once.  Calls of up to 128 rows (decode,
@@ -625,10 +640,17 @@ def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
     _check(x.dtype == torch.bfloat16 and o_weight.dtype == torch.bfloat16, "o_proj supports bfloat16 only")
     _check(o_weight.dim() == 2, "o_weight must be [K, N]")
     K, N = o_weight.shape
-    if x.dim() >= 2 and x.shape[-1] != K and x.shape[-1] * x.shape[-2] == K:
-        lead = tuple(x.shape[:-2])            # [..., Hq, D] -> [..., Hq * D]
+    heads_form = x.dim() >= 2 and x.shape[-1] * x.shape[-2] == K      # [..., Hq, D] -> [..., Hq * D]
+    flat_form = x.dim() >= 1 and x.shape[-1] == K
+    if heads_form and flat_form:
+        # one q head (Hq = 1, D = K): both readings fit x.  `out`, when given, says which one the caller means (an engine
+        # layer with one q head passes x [B, T, 1, D] and out [B, T, N]); without it x is read as [..., K]
+        heads_form = isinstance(out, torch.Tensor) and out.dim() == x.dim() - 1
+        flat_form = not heads_form
+    if heads_form:
+        lead = tuple(x.shape[:-2])
     else:
-        _check(x.dim() >= 1 and x.shape[-1] == K, f"x's last dimension(s) {tuple(x.shape[-2:])} do not give K={K}")
+        _check(flat_form, f"x's last dimension(s) {tuple(x.shape[-2:])} do not give K={K}")
         lead = tuple(x.shape[:-1])
     M = 1
     for d in lead:

@@ -12,6 +12,12 @@ Every operator writes into buffers the caller passes (`out`, the caches) and ret
 the caller-allocates rule of nkipy/src/nkipy/runtime/device_tensor.py:51-74 carries over and a
 captured graph replays without allocations.  Optional tensors may be None; `sliding_window` 0 means
 none.
+
+`workspace` (paged_decode, paged_prefill, o_proj): optional uint8 scratch for split-K partials, sized with
+`paged_attn.decode_workspace_bytes` / `lib.pa_verify_workspace_bytes` / `pa_prefill_workspace_bytes` /
+`o_proj_workspace_bytes`.  Without it the ops use a buffer cached per (device, stream), which all graphs
+captured on one stream share.  A caller that replays several graphs at once gives each its own.  The
+scratch carries nothing from call to call, so it is not declared as a mutated argument.
 """
 from __future__ import annotations
 
@@ -38,10 +44,12 @@ def paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
                  max_seq_len: int = 0, sinks: Optional[torch.Tensor] = None, sliding_window: int = 0,
                  rope_cos: Optional[torch.Tensor] = None, rope_sin: Optional[torch.Tensor] = None,
-                 q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6) -> None:
+                 q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6,
+                 workspace: Optional[torch.Tensor] = None, partition_size: int = 512) -> None:
     paged_attn.decode(q, k_cache, v_cache, block_tables, seq_lens, scale, k_scale=k_scale, v_scale=v_scale,
                       max_seq_len=max_seq_len or None, out=out, sinks=sinks, sliding_window=_win(sliding_window),
-                      q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps))
+                      q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps), workspace=workspace,
+                      partition_size=partition_size)
 
 
 @torch.library.custom_op(f"{_NS}::paged_prefill", mutates_args=("out",), device_types="cuda")
@@ -50,10 +58,11 @@ def paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                   k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
                   sinks: Optional[torch.Tensor] = None, sliding_window: int = 0,
                   rope_cos: Optional[torch.Tensor] = None, rope_sin: Optional[torch.Tensor] = None,
-                  q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6) -> None:
+                  q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6,
+                  workspace: Optional[torch.Tensor] = None) -> None:
     paged_attn.prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, k_scale=k_scale,
                        v_scale=v_scale, out=out, sinks=sinks, sliding_window=_win(sliding_window),
-                       q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps))
+                       q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps), workspace=workspace)
 
 
 @torch.library.custom_op(f"{_NS}::blocksparse_prefill", mutates_args=("out",), device_types="cuda")
@@ -130,8 +139,9 @@ def k_norm_rope_kv_write_fp8(xk: torch.Tensor, xv: torch.Tensor, k_cache: torch.
 # the projection behind the attention call (examples/models/qwen3/kernels/attention.py:143-147; with the bias
 # examples/models/gpt_oss/kernels/attention.py:155-163); the tensor-parallel all-reduce stays with the caller
 @torch.library.custom_op(f"{_NS}::o_proj", mutates_args=("out",), device_types="cuda")
-def o_proj(x: torch.Tensor, o_weight: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
-    paged_attn.o_proj(x, o_weight, bias, out=out)
+def o_proj(x: torch.Tensor, o_weight: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           workspace: Optional[torch.Tensor] = None) -> None:
+    paged_attn.o_proj(x, o_weight, bias, out=out, workspace=workspace)
 
 
 def _no_cpu(name):

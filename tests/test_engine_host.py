@@ -103,9 +103,10 @@ def test_begin_step_is_all_or_nothing_and_layers_share_tables():
         _cache(num_layers=0)
 
 
-def test_rope_table_must_cover_the_cache_capacity():
-    """Positions past the RoPE table are clamped by the kernels, so the layer refuses a table that is
-    shorter than the longest sequence the block tables can hold."""
+def test_rope_table_must_cover_the_longest_admitted_sequence():
+    """Positions past the RoPE table are clamped by the kernels, so the layer refuses a table that is shorter
+    than the longest sequence the cache admits: the table capacity, or the cache's max_model_len when the
+    model's limit is lower (capacity is rounded up to whole blocks)."""
     import torch
     from nkipy_amd.engine import PagedAttention, PagedKVCache
     cache = PagedKVCache(num_blocks=8, block_size=16, n_kv_heads=2, head_dim=64, max_seqs=2, max_blocks_per_seq=4,
@@ -115,6 +116,17 @@ def test_rope_table_must_cover_the_cache_capacity():
         PagedAttention(cache, 4, rope_tables=short)
     exact = (torch.zeros(64, 32, dtype=torch.bfloat16), torch.zeros(64, 32, dtype=torch.bfloat16))
     PagedAttention(cache, 4, rope_tables=exact)
+    # a model of 60 positions over blocks of 16: capacity 64, limit 60; a 60-row table is enough, and the cache
+    # refuses to grow a sequence past the limit
+    limited = PagedKVCache(num_blocks=8, block_size=16, n_kv_heads=2, head_dim=64, max_seqs=2, max_blocks_per_seq=4,
+                           device="cpu", max_model_len=60)
+    PagedAttention(limited, 4, rope_tables=(torch.zeros(60, 32, dtype=torch.bfloat16), torch.zeros(60, 32, dtype=torch.bfloat16)))
+    limited.extend([0], [60])
+    with pytest.raises(ValueError, match="longest sequence"):
+        limited.extend([0], [1])
+    with pytest.raises(ValueError):
+        PagedKVCache(num_blocks=8, block_size=16, n_kv_heads=2, head_dim=64, max_seqs=2, max_blocks_per_seq=4,
+                     device="cpu", max_model_len=65)
 
 
 def test_workspace_cache_is_bounded():

@@ -70,6 +70,27 @@ def test_o_proj_tile_forms(pa, M, K, N, bias, force_large):
     _close(dev_to_f32(got), want)
 
 
+@pytest.mark.parametrize("M,K,N,bias", [(4352, 4096, 4096, True),      # 256 x 256 tiles: 17 row tiles (so row tiles 8.. of an XCD's walk), 64 k-steps
+                                        (1024, 4096, 4096, False),     # 128 x 128 tiles, deep ring (one workgroup per CU)
+                                        (2048, 4096, 2880, True)])     # 128 x 128 tiles, two-stage ring, ragged last column tile
+def test_o_proj_long_k_every_row_tile(pa, M, K, N, bias):
+    """The tiled forms at the projection's real depth (K = 4096: 64 steps through the ring, far more than the
+    ring is deep or the loop is rotated by), rows checked in every row tile: 16 per 128 rows, at in-tile
+    positions that change from block to block, against the oracle on those rows."""
+    rng = np.random.default_rng(M + K + N)
+    x = O.round_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = O.round_to_bf16((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32))
+    b = O.round_to_bf16(rng.standard_normal(N).astype(np.float32)) if bias else None
+    rows = np.unique(np.minimum(np.arange(0, M, 8) + (np.arange((M + 7) // 8) * 5) % 8, M - 1))
+    rows = np.union1d(rows, [0, M - 1])
+    want = O.o_proj(x[rows], w, b)
+    print(f"o_proj long K M={M} K={K} N={N} bias={bias}, {len(rows)} rows checked", flush=True)
+    got = pa.o_proj(bf16_to_dev(x), bf16_to_dev(w), None if b is None else bf16_to_dev(b))
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (M, N)
+    _close(dev_to_f32(got)[rows], want)
+
+
 def test_identity_and_permutation_weights_move_bits(pa, rng):
     """Exact cases: an identity weight returns x bit for bit (which also pins the [.., Hq, D] -> [.., Hq*D]
     view), a column permutation permutes it, a zero x returns the bias in every row."""
@@ -174,3 +195,25 @@ def test_argument_errors(pa):
     with pytest.raises(ValueError):
         pa.o_proj(x, w, workspace=ws.float())                                         # not a uint8 tensor
     assert pa.o_proj_workspace_bytes(4, 100, 256) == 0 and pa.o_proj_workspace_bytes(0, 1024, 256) == 0
+
+
+def test_single_q_head_layouts(pa, rng):
+    """With one q head [.., 1, D] and [.., K] both fit x (K = D): `out`'s rank says which is meant — an engine
+    layer of one q head per rank passes x [B, T, 1, D] and out [B, T, N] — and without `out` x is read as [.., K]."""
+    B, T, D, N = 3, 5, 128, 72
+    x = O.round_to_bf16(rng.standard_normal((B, T, 1, D)).astype(np.float32))
+    w = O.round_to_bf16((rng.standard_normal((D, N)) / np.sqrt(D)).astype(np.float32))
+    want = O.o_proj(x.reshape(B * T, D), w).reshape(B, T, N)
+    xd, wd = bf16_to_dev(x), bf16_to_dev(w)
+    out3 = torch.empty((B, T, N), dtype=torch.bfloat16, device="cuda")
+    assert pa.o_proj(xd, wd, out=out3) is out3
+    out4 = torch.empty((B, T, 1, N), dtype=torch.bfloat16, device="cuda")
+    pa.o_proj(xd, wd, out=out4)
+    plain = pa.o_proj(xd, wd)
+    torch.cuda.synchronize()
+    assert tuple(plain.shape) == (B, T, 1, N)
+    _close(dev_to_f32(out3), want)
+    assert np.array_equal(dev_bits(out4).reshape(B, T, N), dev_bits(out3))
+    assert np.array_equal(dev_bits(plain).reshape(B, T, N), dev_bits(out3))
+    with pytest.raises(ValueError):
+        pa.o_proj(xd, wd, out=torch.empty((B, N), dtype=torch.bfloat16, device="cuda"))

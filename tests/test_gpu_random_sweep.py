@@ -12,6 +12,9 @@ from tests.pa_testlib import assert_close_abs, bf16_to_dev, dev_to_f32, make_pag
 
 pytestmark = pytest.mark.gpu
 
+# elements whose error lay above the plain absolute bar and inside the allowance for large outputs, per case
+WIDENED = {}
+
 N_CASES = int(os.environ.get("PA_SWEEP_CASES", "60"))      # more cases for an occasional longer soak of the same generator
 FIRST_CASE = int(os.environ.get("PA_SWEEP_FIRST", "0"))
 
@@ -93,8 +96,23 @@ def test_random_case(case):
     # key hands a single V row through, and a rare row reaches |v| > 4, where one bf16 step is 2^-5: the device
     # rounds the output once and the oracle its probabilities once, so allow 2^-7 of the largest output (case
     # 4765 of this generator: 4.28 -> 0.031, reproduced by the device arithmetic written out in NumPy).
+    plain_tol = tol
     tol = max(tol, 2.0 ** -7 * float(np.abs(want).max()))
+    over = int((np.abs(got.astype(np.float64) - want) > plain_tol).sum())
+    WIDENED[case] = (over, int(want.size))
+    print(f"elements above the plain bar {plain_tol} (allowed up to {tol:.4f}): {over} of {want.size}", flush=True)
     assert_close_abs(got, want, tol)
     if c["kind"] != "decode":
         for b, n in enumerate(qlens):
             assert np.all(got[b, n:] == 0)
+
+
+def test_sweep_summary_of_the_widened_bar(capsys):
+    """Says how many elements of the cases above needed the allowance for large outputs (2^-7 of the largest
+    expected value) rather than the plain 2e-2 / 5e-2 absolute bar."""
+    cases = sum(1 for over, _ in WIDENED.values() if over)
+    elems = sum(over for over, _ in WIDENED.values())
+    total = sum(n for _, n in WIDENED.values())
+    with capsys.disabled():
+        print(f"\n[sweep] {len(WIDENED)} cases, {total} elements: {elems} elements in {cases} cases lay above the plain "
+              f"absolute bar and inside the 2^-7 max|want| allowance" + (f" (cases {sorted(c for c, (o, _) in WIDENED.items() if o)})" if cases else ""))

@@ -47,6 +47,13 @@ def test_decode_workspace_for_shape_and_noalloc_limit(lib):
     exact = lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 1, 1)     # bf16: balanced schedule
     assert 0 < exact <= upper and exact < 64 << 20          # no term that grows with max_seq_len
     assert lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 0, 0) == 64 * 32 * 2048 * 130 * 4   # fp32
+    # no bound (max_seq_len 0: pa_decode then uses the table capacity, unknown here): enough for the balanced schedule
+    # and for up to four fixed partitions, which a large batch of small capacity takes and which then needs more
+    for B in (4, 128, 600):
+        unbounded = lib.pa_decode_workspace_bytes_for(B, 32, 8, 128, 32, 0, 512, 1, 1)
+        assert unbounded >= B * 32 * 4 * 130 * 4
+        for msl in (100, 512, 2048, 1 << 20):
+            assert unbounded >= lib.pa_decode_workspace_bytes_for(B, 32, 8, 128, 32, msl, 512, 1, 1)
     z = ctypes.c_void_p(0)
     rc = lib.pa_decode_noalloc(z, z, z, z, z, z, z, z, 8192, 64, 8, 128, 32, 4, 64, 0, 1.0, 512, 1, 1, z, 0, z, z)
     assert rc == -1 and b"static" in lib.pa_last_error()
@@ -243,3 +250,33 @@ def test_device_kernel_o_proj_signature_without_gpu(lib):
     assert lib.pa_o_proj(z, z, z, z, 4, 128, 64, 0, z) == -1 and b"bf16" in lib.pa_last_error()
     assert lib.pa_o_proj(z, z, z, z, 0, 128, 64, 1, z) == 0
     assert lib.pa_o_proj(z, z, z, z, 4, 128, 64, 1, z) == -1 and b"null" in lib.pa_last_error()
+
+
+def test_debug_switches_are_refused_without_the_environment_variable():
+    """pa_debug_set reroutes kernels for the whole process, so it only works when PA_ENABLE_DEBUG=1 was set
+    before the library's first use (these tests set it); a process without it gets an argument error."""
+    import subprocess
+    import sys
+    from nkipy_amd import build
+    code = ("import ctypes, sys\n"
+            f"lib = ctypes.CDLL({build.LIB_PATH!r})\n"
+            "lib.pa_last_error.restype = ctypes.c_char_p\n"
+            "rc = lib.pa_debug_set(0, 1)\n"
+            "sys.exit(0 if rc == -1 and b'PA_ENABLE_DEBUG' in lib.pa_last_error() else 1)\n")
+    env = {k: v for k, v in os.environ.items() if k != "PA_ENABLE_DEBUG"}
+    assert subprocess.run([sys.executable, "-c", code], env=env).returncode == 0
+    env["PA_ENABLE_DEBUG"] = "1"
+    code_on = code.replace("rc == -1 and b'PA_ENABLE_DEBUG' in lib.pa_last_error()", "rc == 0 and lib.pa_debug_set(0, 0) == 0")
+    assert subprocess.run([sys.executable, "-c", code_on], env=env).returncode == 0
+
+
+def test_bench_probe_library_is_separate():
+    """The matrix-core ceiling probe is built into a library of its own; the product library exports no
+    pa_probe / pa_bench symbol."""
+    from nkipy_amd import _lib, build
+    if not os.path.exists(build.BENCH_LIB_PATH):
+        build.build()
+    probe = ctypes.CDLL(build.BENCH_LIB_PATH)
+    assert hasattr(probe, "pa_bench_probe_mfma")
+    lib = _lib.load()
+    assert not hasattr(lib, "pa_probe_mfma") and not hasattr(lib, "pa_bench_probe_mfma")

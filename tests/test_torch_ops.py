@@ -94,3 +94,64 @@ def test_ops_match_the_python_ops_and_replay_in_a_graph():
                                               k_norm_weight=wn), kd, vd, td, sd, qlens, 0.09)
     torch.cuda.synchronize()
     assert np.array_equal(dev_bits(o), dev_bits(two))
+
+
+@pytest.mark.gpu
+def test_graph_keeps_its_scratch_when_the_batch_grows_and_a_larger_eager_call_follows():
+    """A decode + projection step captured through the dispatcher, once with the ops' cached scratch and once
+    with the caller's `workspace`, is replayed after (i) more slots have gone live and contexts have grown (the
+    lengths and tables are device tensors the replay reads) and (ii) an eager call on the capture stream's
+    neighbour, the current stream, that needs a far larger scratch and a cache flush of every eager entry.
+    Each replay must equal the eager result on the same state."""
+    import nkipy_amd as pa
+    import nkipy_amd.torch_ops  # noqa: F401
+    from nkipy_amd import paged_attn
+    rng = np.random.default_rng(11)
+    B, Hq, Hkv, D, bs, N = 16, 8, 2, 128, 32, 512
+    cap_tokens = 4096
+    ctxs_small = [0] * B
+    ctxs_small[0], ctxs_small[1] = 37, 300
+    ctxs_big = [int(x) for x in rng.integers(500, cap_tokens, B)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, [cap_tokens] * B)
+    kd, vd, td = bf16_to_dev(k), bf16_to_dev(v), _i32(tables)
+    sd = _i32(ctxs_small)
+    q = bf16_to_dev(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    w = bf16_to_dev((rng.standard_normal((Hq * D, N)) / 32).astype(np.float32))
+    att, proj = torch.empty_like(q), torch.empty((B, N), dtype=torch.bfloat16, device="cuda")
+    need = max(paged_attn.decode_workspace_bytes(B, Hq, D, cap_tokens, 512), paged_attn.o_proj_workspace_bytes(B, Hq * D, N))
+    own = torch.empty(need, dtype=torch.uint8, device="cuda")
+
+    def step(ws):
+        torch.ops.nkipy_amd.paged_decode(q, kd, vd, td, sd, 0.09, att, max_seq_len=cap_tokens, workspace=ws, partition_size=512)
+        torch.ops.nkipy_amd.o_proj(att, w, proj, workspace=ws)
+
+    step(None)
+    torch.cuda.synchronize()
+    graphs = []
+    for ws in (None, own):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            step(ws)
+        graphs.append(g)
+    # between capture and replay: the batch grows, and an eager call that outgrows every cached scratch runs
+    sd.copy_(_i32(ctxs_big))
+    q.copy_(bf16_to_dev(rng.standard_normal((B, Hq, D)).astype(np.float32)))
+    big_B = 512
+    kb, vb, tb = make_paged(rng, big_B, Hkv, D, bs, [64] * big_B)
+    bigq = bf16_to_dev(rng.standard_normal((big_B, 4 * Hkv, D)).astype(np.float32))
+    pa.decode(bigq, bf16_to_dev(kb), bf16_to_dev(vb), _i32(tb), _i32([64] * big_B), 0.09)
+    paged_attn._workspaces.clear()                      # every eager entry gone: a graph's scratch must not have been one
+    torch.cuda.synchronize()
+    step(own)
+    torch.cuda.synchronize()
+    want_att, want_proj = dev_bits(att).copy(), dev_bits(proj).copy()
+    for g in graphs:
+        for _ in range(2):
+            att.zero_()
+            proj.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(dev_bits(att), want_att)
+            assert np.array_equal(dev_bits(proj), want_proj)
+            pa.decode(bigq, bf16_to_dev(kb), bf16_to_dev(vb), _i32(tb), _i32([64] * big_B), 0.09)   # eager work between replays
+            torch.cuda.synchronize()
