@@ -17,7 +17,8 @@ value      whole-step throughput: algorithmic HBM bytes / step time for the deco
            configs (GB/s), attention FLOPs / step time for the prefill configs
            (TFLOP/s); the step includes every kernel the op launches.
 roofline   the dominant kernel alone, timed with HIP events on its launch stream
-           inside the library (pa_profile_*), during the same K launches the step time is taken from.
+           inside the library (pa_profile_*), over the K launches right behind the K the step time is
+           taken from ("ms_per_step_with_events" is that second block's own step time).
 warm-up    --warmup is a minimum; blocks of K launches follow until two consecutive blocks agree within
            2 % (the clock ramps for tens of launches after the allocation phase); the last block is the
            measurement ("warmup_effective_steps", "warmup_converged" say what happened).
@@ -67,27 +68,30 @@ WARMUP_CAP_S = 1.5       # ... or the warm-up ends after this long (and says so)
 
 
 def _measure(step, steps, warmup, lib):
-    """Step time and the dominant kernel's time from ONE pass of `steps` launches.
+    """Step time and the dominant kernel's time from two adjacent blocks of `steps` launches in the steady state.
 
     `warmup` is a minimum: after it, blocks of `steps` launches are timed until two consecutive blocks agree
     within WARMUP_AGREE (the shader clock keeps ramping for some tens of launches after an allocation phase,
     however few warm-up steps the command line asked for), for at most WARMUP_CAP_S.  The block that agreed
-    with its predecessor is the measurement: its wall time between two synchronisations is the step time, and
-    the HIP events the library records around the dominant kernel during those same launches give the kernel
-    time.  Returns (seconds per step, kernel milliseconds per launch, info for the JSON record)."""
-    lib.pa_profile_enable(1)
+    with its predecessor gives the step time (wall clock between two synchronisations, nothing else on the
+    stream).  The block right behind it runs with the library's HIP events around the dominant kernel and gives
+    the kernel time; its own wall time is reported too (`ms_per_step_with_events`: two event records per step
+    cost a few microseconds, which is why the step time is not taken from that block), so that step >= kernel
+    can be read off one and the same block.  Returns (seconds per step, kernel milliseconds per launch, info)."""
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    _collect_kernel_ms(lib, 0)
-    prev, blocks, t_begin, converged = None, 0, time.perf_counter(), False
-    while True:
+
+    def block():
         t0 = time.perf_counter()
         for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        sec = (time.perf_counter() - t0) / steps
-        kms = _collect_kernel_ms(lib, 4 * steps)
+        return (time.perf_counter() - t0) / steps
+
+    prev, blocks, t_begin, converged = None, 0, time.perf_counter(), False
+    while True:
+        sec = block()
         blocks += 1
         if prev is not None and abs(sec - prev) <= WARMUP_AGREE * min(sec, prev):
             converged = True
@@ -95,8 +99,15 @@ def _measure(step, steps, warmup, lib):
         if time.perf_counter() - t_begin > WARMUP_CAP_S and blocks >= 2:
             break
         prev = sec
+    lib.pa_profile_enable(1)
+    step()                                   # creates the events the timed block reuses
+    torch.cuda.synchronize()
+    _collect_kernel_ms(lib, 0)
+    sec_ev = block()
     lib.pa_profile_enable(0)
-    info = {"warmup_effective_steps": warmup + (blocks - 1) * steps, "warmup_converged": converged}
+    kms = _collect_kernel_ms(lib, 4 * steps)
+    info = {"warmup_effective_steps": warmup + (blocks - 1) * steps, "warmup_converged": converged,
+            "ms_per_step_with_events": round(sec_ev * 1e3, 5)}
     return sec, kms, info
 
 
@@ -292,6 +303,9 @@ def _load_bench_lib():
         _bench_lib.pa_bench_probe_mfma.restype = ctypes.c_int
         _bench_lib.pa_bench_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                                    ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+        _bench_lib.pa_bench_probe_tile_loop.restype = ctypes.c_int
+        _bench_lib.pa_bench_probe_tile_loop.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                                        ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
     return _bench_lib
 
 
@@ -314,6 +328,54 @@ def _mfma_ceiling(lib, sample):
             raise RuntimeError(f"pa_bench_probe_mfma failed ({rc})")
         best = max(best, blocks * 8 * iters * 16 * 32768.0 / (ms.value * 1e-3) / 1e12)
     return round(best, 1)
+
+
+def bench_tile_loop_probe(steps, warmup):
+    """config 14 (a probe, not a benchmark of the product): the key loop of the tiled prefill kernel as a stand-alone
+    loop, in the shipped structure (8 waves x 32 query rows, two waves per SIMD) and as 4 waves x 64 rows with one wave
+    per SIMD, the whole register file and a software pipeline over 32-key x 32-row units; the same 256 rows x 64 keys
+    per workgroup and tile either way.  On N(0,1) and on constant operands: time per tile, shader cycles per tile
+    (2048 = matrix pipeline never idle) and the clock the chip ran at."""
+    probe = _load_bench_lib()
+    blocks, iters = 256, 2000
+    nbytes = 2 * 8 * 6144 * 2048 + (1 << 20)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1014)
+    src = torch.randn(nbytes // 2, generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    sink = torch.empty(blocks * 512, dtype=torch.float32, device="cuda")
+    stamps = torch.zeros(blocks * 2, dtype=torch.int64, device="cuda")
+    ms = ctypes.c_float(0.0)
+    forms = {0: "8 waves x 32 rows, two waves per SIMD (shipped structure)", 1: "4 waves x 64 rows, one wave per SIMD, pipelined units"}
+    out = {}
+    for data in ("N(0,1)", "constant"):
+        if data == "constant":
+            src.fill_(0.011)
+        for form, name in forms.items():
+            best = None
+            for _ in range(max(3, warmup // 10) + max(3, steps // 10)):
+                rc = probe.pa_bench_probe_tile_loop(form, src.data_ptr(), sink.data_ptr(), stamps.data_ptr(), blocks, iters,
+                                                    ctypes.byref(ms), torch.cuda.current_stream().cuda_stream)
+                if rc != 0:
+                    raise RuntimeError(f"pa_bench_probe_tile_loop failed ({rc})")
+                st = stamps.cpu().numpy().reshape(blocks, 2).astype(np.float64)
+                rec = {"ms": round(ms.value, 4), "ns_per_tile": round(ms.value * 1e6 / iters, 1),
+                       "tflops": round(blocks * iters * 256 * 32768.0 / (ms.value * 1e-3) / 1e12, 1),
+                       "shader_cycles_per_tile": round(float(st[:, 0].mean()) / iters, 1),
+                       "clock_mhz": round(float((st[:, 0] / (st[:, 1] * 10.0)).mean()) * 1000.0, 1)}
+                rec["matrix_pipe_busy"] = round(2048.0 / rec["shader_cycles_per_tile"], 4)
+                if best is None or rec["ms"] < best["ms"]:
+                    best = rec
+            out[f"{data}: {name}"] = best
+    ref = out["N(0,1): " + forms[0]]
+    return {
+        "metric": "tile-loop probe of the prefill key loop, TFLOP/s (shipped structure, N(0,1) operands)",
+        "value": ref["tflops"], "unit": "TFLOP/s", "ms_per_step": ref["ms"], "dtype": "bf16, fp32 accumulate",
+        "config": {"workload": f"stand-alone key loop: {blocks} workgroups x {iters} tiles of 256 query rows x 64 keys, head dim 128; "
+                               "no masks, tables or lengths"},
+        "roofline": {"bound": "mfma", "achieved": ref["tflops"], "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(ref["tflops"] / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "tile_loop_32rows_kernel"},
+        "forms": out, "cpu_baseline": None,
+    }
 
 
 def bench_prefill(steps, warmup, lib, pa, W, fp8=False, gpt_oss=False):
@@ -690,7 +752,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13],
+    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     ap.add_argument("--const-data", action="store_true",
@@ -739,6 +801,8 @@ def main():
             res = bench_o_proj(args.steps, args.warmup, lib, pa, W)
         elif cfg == 13:
             res = bench_decode_layer_step(args.steps, args.warmup, lib, pa, W)
+        elif cfg == 14:
+            res = bench_tile_loop_probe(args.steps, args.warmup)
         else:
             res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
         gc.collect()
