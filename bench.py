@@ -755,6 +755,10 @@ def main():
     ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
+    ap.add_argument("--prefill-impl", type=int, default=0,
+                    help="force a form of the tiled prefill kernel through the library's debug switch 3 (4 / 8: waves per "
+                         "workgroup; for config 4, 8 is the staggered 256-row form); 0: the library's own choice.  For "
+                         "comparisons of kernel forms; recorded in the line as prefill_impl")
     ap.add_argument("--const-data", action="store_true",
                     help="prefill configs 3 / 9 / 11 and the projection 12: every Q, K and V (x and w) element is the same value instead of N(0,1).  Same "
                          "kernel, same instruction stream, far fewer bit flips in the matrix cores' operands: the time "
@@ -769,10 +773,15 @@ def main():
         sys.exit(3)
     import gc
 
+    if args.prefill_impl:
+        os.environ["PA_ENABLE_DEBUG"] = "1"      # read by the library at its first use
     import nkipy_amd as pa
     from nkipy_amd import _lib, workloads as W
     lib = _lib.load()
     torch.cuda.set_device(0)
+    if args.prefill_impl and lib.pa_debug_set(3, args.prefill_impl) != 0:
+        print(f"bench.py: {lib.pa_last_error().decode()}", file=sys.stderr)
+        sys.exit(2)
     if args.no_cpu:
         global _NO_CPU
         _NO_CPU = True
@@ -832,6 +841,8 @@ def main():
         line["prefill_roofline_frac"] = subs["C3"]["roofline"]["frac"]
         par = [line.get("parity")] + [r.get("parity") for r in subs.values()]
         line["parity_all_pass"] = None if any(x is None for x in par) else all(x["pass"] for x in par)
+    if args.prefill_impl:
+        line["prefill_impl"] = args.prefill_impl
     if args.const_data:
         line["data"] = "synthetic CONSTANT operands (power probe: not a benchmark result)"
     line["device"] = torch.cuda.get_device_name(0)

@@ -135,7 +135,12 @@ void prefill_async_kernel(PrefillParams p) {
   constexpr int KS = DH / 16;                // k-steps of the score product
   constexpr int VC = DH / 32;                // 32-wide d chunks of the output
   constexpr int TOKW = PAIR ? BMW / 2 : BMW; // query tokens per workgroup (plain form)
-  constexpr int NST = NW == 8 ? 4 : 2;   // LDS stages the copies land in
+  // Blocksparse with 8 waves (STAG): the workgroup's four 64-row query blocks walk the vertical-stride tiles together
+  // and then the local band STAGGERED: at band step s the q block j works on key tile (its own block) - local + 1 + s,
+  // so all four are busy on four different resident tiles for exactly `local` steps and one new tile is requested per
+  // step (four resident stages + one in flight).
+  constexpr bool STAG = SPARSE && NW == 8;
+  constexpr int NST = STAG ? 5 : NW == 8 ? 4 : 2;   // LDS stages the copies land in
   constexpr int UPW = FP8 ? 2 : 2 * UK / NW; // copy units per wave per tile (FP8: 8 raw rows of K, 8 of V)
   static_assert(!FP8 || (NW == 8 && MODE == 1 && !SPARSE && !PACK && TT == 2), "fp8 pools: 8-wave paged dense form only");
   constexpr int EB = FP8 ? 1 : 2;            // bytes per pool element
@@ -421,7 +426,26 @@ void prefill_async_kernel(PrefillParams p) {
   typedef const __attribute__((address_space(4))) float* const_f32_ptr;
   float ksq[4] = {0.f, 0.f, 0.f, 0.f}, vsq[4] = {0.f, 0.f, 0.f, 0.f};
   float ksq2[4] = {0.f, 0.f, 0.f, 0.f}, vsq2[4] = {0.f, 0.f, 0.f, 0.f};      // PAIR: the odd kv head's
+  // STAG: request r is vertical tile number r (tiles stag_v0 + r * stride, those some q block of the workgroup sees
+  // below its local window) for r < stag_nv, then band tile stag_band0 + (r - stag_nv); requests that fall outside
+  // [0, ntiles) are clamped into it (they re-read a valid tile and are never consumed, but keep the wait counts exact)
+  constexpr int QB = BMW / 64;                  // q blocks per workgroup
+  const int stag_v0 = head_phase == 0 ? 0 : p.sparse_stride - head_phase;
+  const int stag_vmax = min(wg_blk_lo + QB - 1 - p.sparse_local, ntiles - 1);
+  const int stag_nv = STAG && stag_vmax >= stag_v0 ? (stag_vmax - stag_v0) / p.sparse_stride + 1 : 0;
+  // band steps in which every q block's tile would lie before tile 0 are left out (a local window longer than the
+  // sequence so far)
+  const int stag_skip = max(p.sparse_local - wg_blk_lo - QB, 0);
+  const int stag_band0 = wg_blk_lo - p.sparse_local + 1 + stag_skip;
+  int stag_req = 0;                             // next request
   auto request_next = [&]() __attribute__((always_inline)) {
+    if constexpr (STAG) {
+      const int t = stag_req < stag_nv ? stag_v0 + stag_req * p.sparse_stride : stag_band0 + (stag_req - stag_nv);
+      issue_tile(min(max(t, 0), ntiles - 1), stage_i);
+      ++stag_req;
+      stage_i = stage_i + 1 == NST ? 0 : stage_i + 1;
+      return;
+    }
     issue_tile(w_i.kt < ntiles ? w_i.kt : kt_first, stage_i);
     if (FP8) {
       const long si = (long)min(max(blk_pf[0], 0), p.num_blocks - 1) * p.Hkv + kv0;
@@ -727,7 +751,45 @@ void prefill_async_kernel(PrefillParams p) {
         }
       }
     };
-    while (w_c.kt < ntiles) {
+    if constexpr (STAG) {
+      const int n_steps = stag_nv + p.sparse_local - stag_skip;
+      const int jq = qblk - wg_blk_lo;             // this wave's q block within the workgroup
+      int stage_v = 0;                             // stage of the request with the step's number
+      for (int g = 0; g < n_steps; ++g) {
+        const bool band = g >= stag_nv;
+        // vertical steps consume request g (three younger ones may still be in flight); band steps consume
+        // requests g .. g + 3, the youngest of them issued one step ago
+        if (band) wait_vmcnt<0>(); else wait_vmcnt<(NST - 2) * UPW>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        request_next();                            // request g + 4, into the stage request g - 1 has left
+        flush_pending();
+        int tile, stage;
+        bool act = wave_has_rows;
+        if (!band) {
+          tile = stag_v0 + g * p.sparse_stride;
+          stage = stage_v;
+          act = act && tile <= qblk - p.sparse_local;          // strictly below this q block's window
+        } else {
+          const int sb = g - stag_nv;
+          tile = qblk - p.sparse_local + 1 + stag_skip + sb;
+          stage = stage_v + jq;
+          stage = stage >= NST ? stage - NST : stage;
+          act = act && tile >= 0;
+        }
+        if (act) {
+          f32x16_t sacc[TT];
+          uint32_t pw[TT][8];
+          bf16x8_t v0[VC];
+          scores(sacc, stage, v0, stage, 0);
+          softmax(sacc, pw, tile * BN, 0);
+          accumulate_but_last(pw, stage, v0, dv0, dv1, dpw, 0);
+          pending = true;
+        }
+        stage_v = stage_v + 1 == NST ? 0 : stage_v + 1;
+      }
+    }
+    while (!STAG && w_c.kt < ntiles) {
       if (FP8) {
         wait_vmcnt<2 * UPW>();                     // this wave's raw rows of the next tile have landed
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its bf16 rows of the current one are written
@@ -886,7 +948,7 @@ __global__ __launch_bounds__(256) void prefill_split_reduce_kernel(PrefillParams
 
 template <bool SPARSE, int MODE, int NW, int TT = 2, bool WIN = false, bool PACK = false, bool SPLIT = false, bool FP8 = false, int DH = HD, int QH = 1>
 hipError_t launch_typed(const PrefillParams& p, hipStream_t s) {
-  constexpr int lds = (NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
+  constexpr int lds = (SPARSE && NW == 8 ? 5 : NW == 8 ? 4 : 2) * 2 * 32 * TT * ROW_B;
   constexpr int TOKW = DH == 64 ? 16 * NW : 32 * NW;      // query tokens per workgroup (plain form)
   static std::atomic<int> configured{0};
   if (!configured.load(std::memory_order_acquire)) {

@@ -183,6 +183,36 @@ def test_config4_shape_shrunk(pa):
     assert_close_abs(dev_to_f32(got), want, BF16_TOL)
 
 
+@pytest.mark.parametrize("B,S,Hq,Hkv,local,stride", [(1, 640, 3, 3, 2, 4), (2, 1024, 4, 2, 4, 8), (1, 2048, 8, 8, 4, 8),
+                                                    (1, 700, 2, 1, 1, 3), (1, 1500, 2, 2, 6, 2), (1, 900, 2, 2, 1000, 8),
+                                                    (1, 512, 9, 9, 3, 1)])
+def test_blocksparse_staggered_256_row_form(pa, B, S, Hq, Hkv, local, stride):
+    """The 8-wave blocksparse form (debug switch 3 = 8): four q blocks per workgroup walk the vertical-stride tiles
+    together and the local band staggered, one key tile apart.  Windows shorter and longer than the four q blocks,
+    a window longer than the sequence, every tile vertical (stride 1), sequence lengths that are not multiples of
+    256 or 64, GQA: against the oracle, and bit for bit the 4-wave form's result."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(S + local + stride)
+    q = O.round_to_bf16(rng.standard_normal((B, S, Hq, 128)).astype(np.float32))
+    k = O.round_to_bf16(rng.standard_normal((B, S, Hkv, 128)).astype(np.float32))
+    v = O.round_to_bf16(rng.standard_normal((B, S, Hkv, 128)).astype(np.float32))
+    want = O.blocksparse_prefill(q, k, v, 0.09, block=64, local_blocks=local, vert_stride=stride)
+    got = {}
+    try:
+        for impl in (4, 8):
+            print(f"blocksparse B={B} S={S} Hq={Hq} Hkv={Hkv} local={local} stride={stride} impl={impl}", flush=True)
+            lib.pa_debug_set(3, impl)
+            out = pa.blocksparse_prefill(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), 0.09, block=64,
+                                         local_blocks=local, vert_stride=stride)
+            torch.cuda.synchronize()
+            got[impl] = out
+    finally:
+        lib.pa_debug_set(3, 0)
+    assert_close_abs(dev_to_f32(got[8]), want, BF16_TOL)
+    assert torch.equal(got[4], got[8])
+
+
 @pytest.mark.parametrize("impl", [1, 4, 8], ids=["staged", "async4", "async8"])
 def test_prefill_kernel_variants_agree(pa, impl):
     """Every prefill kernel variant (register-staged, asynchronous ring with 4 or 8 waves, the
