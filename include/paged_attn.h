@@ -159,6 +159,11 @@ int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
  *   kv_dtype     PA_BF16 or PA_FP8_E4M3FN (then k_scale / v_scale [num_blocks, Hkv] f32)
  *   workspace    pa_verify_workspace_bytes(B, T, Hq, D) bytes, 16-byte aligned
  *   sinks, sliding_window   as for pa_decode (the window counts back from each query token's own position)
+ *   max_seq_len  0, or a host-known upper bound of seq_lens (longer contexts are read up to the bound).  The table
+ *                capacity says nothing about the size of a call; with a bound, a small call -- at most four
+ *                512-token partitions per sequence and little K and V in all, no sinks, no window: the
+ *                reference's own use, one sequence and a handful of draft tokens -- runs on fixed partitions
+ *                as a small pa_decode call does, without the balanced schedule's fixed cost.  Same workspace.
  * D in {64, 128}; block_size a power of two >= 16; T <= PA_VERIFY_MAX_TOKENS.
  */
 #define PA_VERIFY_MAX_TOKENS 64
@@ -168,7 +173,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
               const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
               void* out, void* workspace, size_t workspace_bytes,
               int B, int T, int Hq, int Hkv, int D, int block_size,
-              int max_blocks_per_seq, int num_blocks,
+              int max_blocks_per_seq, int num_blocks, int max_seq_len,
               float scale, int kv_dtype, const float* sinks, int sliding_window,
               const pa_q_transform* q_transform, void* stream);
 
@@ -316,7 +321,8 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never);
  * key 7: query tokens from which pa_prefill at head dim 64 takes the tiled kernel (0 = the default, 65);
  * key 3 value 6: one q head per wave at head dim 64; key 8: pa_o_proj takes 256 x 256 tiles
- * also where it would take 128 x 128 ones (1 = on). */
+ * also where it would take 128 x 128 ones (1 = on); key 9: the longest length bound (tokens) up to which a small
+ * pa_decode call runs as one partition per sequence on eight wavefronts (default 1024; 0 = never). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

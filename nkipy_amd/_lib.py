@@ -35,7 +35,7 @@ SIGNATURES = {
     "pa_decode": (c_int, [c_void_p] * 9 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "pa_decode_noalloc": (c_int, [c_void_p] * 8 + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "pa_verify_workspace_bytes": (c_size_t, [c_int] * 4),
-    "pa_verify": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 8 + [c_float, c_int, c_void_p, c_int, c_void_p, c_void_p]),
+    "pa_verify": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 9 + [c_float, c_int, c_void_p, c_int, c_void_p, c_void_p]),
     "pa_prefill_workspace_bytes": (c_size_t, [c_int] * 7),
     "pa_prefill": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p, c_void_p]),
     "pa_blocksparse_prefill": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_float, c_int, c_void_p]),

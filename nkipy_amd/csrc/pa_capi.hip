@@ -53,6 +53,9 @@ static int lockstep_for(int kv_dtype, int bal_ns) {
 static std::atomic<int> g_verify_rows{0};
 static std::atomic<int> g_prefill_split{1};
 static std::atomic<int> g_d64_tiled_from{PA_VERIFY_MAX_TOKENS + 1};   // query tokens from which head dim 64 takes the tiled kernel
+// Small decode calls whose length bound is at most this many tokens run as ONE partition per sequence on eight waves
+// (the waves merge through LDS, so there is no split-K workspace and no merge launch): debug switch 9, 0 = never.
+static std::atomic<int> g_decode_single_max{1024};
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 // Events come from a free list that pa_profile_collect refills, so that a timed pass which follows a collected
@@ -156,6 +159,7 @@ int pa_debug_set(int key, int value) {
   if (key == 6) { g_prefill_split = value; return 0; }
   if (key == 7) { g_d64_tiled_from = value > 0 ? value : PA_VERIFY_MAX_TOKENS + 1; return 0; }
   if (key == 8) { o_proj_debug_force_large(value); return 0; }
+  if (key == 9) { g_decode_single_max = value < 0 ? 0 : value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -323,6 +327,19 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   const int kind = decode_kind(p, q_dtype, kv_dtype, sinks != nullptr || sliding_window > 0);
   if (kind < 0) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
   if (kind == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
+  // a small call of short contexts: the whole context as one partition on eight waves, which merge through LDS, so
+  // that there is no merge launch.  Per call replayed from a HIP graph (32 / 8 heads of 128, bf16, us, two partitions of
+  // 512 + merge against one partition): contexts of 350-700 tokens B = 1 10.1 / 9.7, B = 16 12.3 / 11.1, B = 64
+  // 31.3 / 26.6; 512-1024 tokens B = 8 10.4 / 12.0 (the longer chain per wave costs more than the launch), B = 64
+  // 36.7 / 34.7.  So: bounds up to three quarters of the limit always, up to the limit when the grid is large anyway.
+  int waves = g_decode_waves.load();
+  const int single_max = g_decode_single_max.load();
+  if (kind == 2 && waves == 0 && g_decode_impl.load() == 0 && p.num_partitions > 1 && Hq / Hkv <= 8 &&
+      (max_seq_len <= single_max - single_max / 4 || (max_seq_len <= single_max && (long)B * Hkv >= 256))) {
+    p.partition_size = (max_seq_len + 31) & ~31;
+    p.num_partitions = 1;
+    waves = 8;
+  }
   if ((sinks || sliding_window > 0) && kind != 3)
     return fail_arg("pa_decode: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
                     "head_dim 64 or 128, block_size a power of two >= 16)");
@@ -353,7 +370,7 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
     p.ws_ml = p.ws_out + (size_t)B * Hq * p.num_partitions * D;
   }
   profile_begin(s);
-  hipError_t e = kind == 2 ? launch_decode_mfma(p, kv_dtype, g_decode_waves.load(), s)
+  hipError_t e = kind == 2 ? launch_decode_mfma(p, kv_dtype, waves, s)
                            : launch_decode_generic(p, q_dtype, kv_dtype, s);
   profile_end(s);
   if (e != hipSuccess) return check_hip(e, "pa_decode launch");
@@ -425,7 +442,7 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
                          const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
                          void* out, void* workspace, size_t workspace_bytes,
                          int B, int T, int t0, int Tc, int Hq, int Hkv, int D, int block_size,
-                         int max_blocks_per_seq, int num_blocks, float scale, int kv_dtype,
+                         int max_blocks_per_seq, int num_blocks, int max_seq_len, float scale, int kv_dtype,
                          const float* sinks, int sliding_window, const pa_q_transform* q_transform, hipStream_t s) {
   const long cap = (long)max_blocks_per_seq * block_size;
   DecodeParams p;
@@ -454,6 +471,29 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   if (!decode_mfma_supported(p, PA_BF16, kv_dtype))
     return fail_arg("%s: unsupported shape (D=%d must be 64 or 128, block_size=%d a power of two >= 16)", who, D, block_size);
   if (take_q_transform(who, q_transform, true, p.qt)) return -1;
+  if (max_seq_len > 0 && max_seq_len < p.max_seq_len) p.max_seq_len = max_seq_len;     // the caller's bound on the contexts
+  // Small calls (the reference's own use of this path: one sequence, a handful of draft tokens) take fixed partitions,
+  // as small pa_decode calls do and for the same reason: the balanced schedule costs what it costs whatever the sizes
+  // (256 chunks, each leaving partials of 16 rows; B = 1, T = 4 behind 1 K tokens: 13.7 us per call replayed from a
+  // graph).  It needs the caller's bound on the lengths (the table capacity says nothing about the sizes), 16 rows
+  // per wave, no sinks and no window, and a workspace that holds the partitions' partials.
+  if (max_seq_len > 0 && !sinks && sliding_window == 0 && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
+    DecodeParams f = p;
+    f.partition_size = 512;
+    f.num_partitions = num_partitions_for(f.max_seq_len, f.partition_size);
+    const size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
+    if (decode_small_call(f, kv_dtype) && (need_f == 0 || (workspace && workspace_bytes >= need_f))) {
+      f.head_major = g_head_major.load();
+      f.ws_out = (float*)workspace;
+      f.ws_ml = f.ws_out + (size_t)B * Hq * Tc * f.num_partitions * D;
+      profile_begin(s);
+      hipError_t e = launch_decode_mfma(f, kv_dtype, 0, s);
+      profile_end(s);
+      if (e != hipSuccess) return check_hip(e, "verify kernel launch");
+      if (f.num_partitions > 1) e = launch_decode_reduce(f, PA_BF16, s);
+      return check_hip(e, "verify merge launch");
+    }
+  }
   plan_decode_balanced(p, current_num_cus());
   p.bal_lockstep = lockstep_for(kv_dtype, p.bal_ns);
   const size_t need = decode_balanced_workspace_bytes(B, Hq * Tc, D, p.bal_gv);
@@ -480,7 +520,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
               const int32_t* block_tables, const int32_t* seq_lens, const int32_t* query_lens,
               void* out, void* workspace, size_t workspace_bytes,
               int B, int T, int Hq, int Hkv, int D, int block_size,
-              int max_blocks_per_seq, int num_blocks,
+              int max_blocks_per_seq, int num_blocks, int max_seq_len,
               float scale, int kv_dtype, const float* sinks, int sliding_window,
               const pa_q_transform* q_transform, void* stream) {
   tl_error[0] = 0;
@@ -500,7 +540,7 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
     return fail_arg("pa_verify: q, k_cache, v_cache, out and workspace must be 16-byte aligned");
   return verify_launch("pa_verify", q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens, out,
                        workspace, workspace_bytes, B, T, 0, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks,
-                       scale, kv_dtype, sinks, sliding_window, q_transform, (hipStream_t)stream);
+                       max_seq_len, scale, kv_dtype, sinks, sliding_window, q_transform, (hipStream_t)stream);
 }
 
 static void fill_prefill_shape(PrefillParams& p, int B, int T, int Hq, int Hkv, int D, int block_size,
@@ -579,7 +619,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
       const int tc = T - t0 < PA_VERIFY_MAX_TOKENS ? T - t0 : PA_VERIFY_MAX_TOKENS;
       const int rc = verify_launch("pa_prefill", q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens,
                                    out, workspace, workspace_bytes, B, T, t0, tc, Hq, Hkv, D, block_size,
-                                   max_blocks_per_seq, num_blocks, scale, kv_dtype, sinks, sliding_window, q_transform,
+                                   max_blocks_per_seq, num_blocks, 0, scale, kv_dtype, sinks, sliding_window, q_transform,
                                    (hipStream_t)stream);
       if (rc) return rc;
     }

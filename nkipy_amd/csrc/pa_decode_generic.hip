@@ -119,11 +119,15 @@ __global__ __launch_bounds__(kGenericThreads) void decode_generic_kernel(DecodeP
 }
 
 // Merge of split-K partials: m = max m_i, w_i = l_i 2^(m_i - m),
-// out = sum w_i o_i / sum w_i.   One workgroup per (q head, sequence).
+// out = sum w_i o_i / sum w_i.   One workgroup per (row, sequence); a row is a q head, or, for a
+// launch with several query tokens per sequence (p.query_lens), a (token, head) pair of a kv head, token-major:
+// such a row may have seen no key in a partition (m = -inf, l = 0) or be padding (zeros).
 template <typename QT>
 __global__ void decode_reduce_kernel(DecodeParams p) {
-  const int hq = blockIdx.x, b = blockIdx.y;
-  const long base = ((long)b * p.Hq + hq) * p.num_partitions;
+  const int vr = blockIdx.x, b = blockIdx.y;
+  const bool multi = p.query_lens != nullptr;
+  const int rows_total = p.Hq * (multi ? p.T : 1);
+  const long base = ((long)b * rows_total + vr) * p.num_partitions;
   // The kernel is a chain of dependent loads (length -> partition count -> maxima -> partials), each a trip to
   // memory, around a few additions.  The first PRE partitions' values are therefore requested at once and before the
   // length is known (their slots exist whatever the length; what a partition past the context holds is not used).
@@ -142,27 +146,38 @@ __global__ void decode_reduce_kernel(DecodeParams p) {
   }
   int ctx = p.seq_lens[b];
   ctx = min(max(ctx, 0), p.max_seq_len);
+  long out_at = ((long)b * p.Hq + vr) * p.D;
+  if (multi) {
+    // context and rows of this launch as the streaming kernel takes them (query tokens [t0, t0 + T) of T_stride)
+    const int qfull = min(min(max(p.query_lens[b], 0), p.T_stride), ctx);
+    const int tq = min(max(qfull - p.t0, 0), p.T);
+    ctx = tq > 0 ? ctx - qfull + p.t0 + tq : 0;
+    const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
+    const int hk = vr / n_rows, j = vr - hk * n_rows, t = j / n_rep;
+    out_at = (((long)b * p.T_stride + p.t0 + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * p.D;
+  }
   const int np = (ctx + p.partition_size - 1) / p.partition_size;
   float mt = -INFINITY;
 #pragma unroll
   for (int i = 0; i < PRE; ++i)
     if (i < np) mt = fmaxf(mt, m_[i]);
   for (int i = PRE; i < np; ++i) mt = fmaxf(mt, p.ws_ml[(base + i) * 2]);
+  const float m_ref = mt == -INFINITY ? 0.f : mt;
   for (int d = d0; d < p.D; d += blockDim.x) {
     float lt = 0.f, ot = 0.f;
 #pragma unroll
     for (int i = 0; i < PRE; ++i)
       if (i < np) {
-        const float w = l_[i] * exp2f(m_[i] - mt);
+        const float w = l_[i] * exp2f(m_[i] - m_ref);
         lt += w;
         ot += w * (d == d0 ? o_[i] : p.ws_out[(base + i) * p.D + d]);
       }
     for (int i = PRE; i < np; ++i) {
-      const float w = p.ws_ml[(base + i) * 2 + 1] * exp2f(p.ws_ml[(base + i) * 2] - mt);
+      const float w = p.ws_ml[(base + i) * 2 + 1] * exp2f(p.ws_ml[(base + i) * 2] - m_ref);
       lt += w;
       ot += w * p.ws_out[(base + i) * p.D + d];
     }
-    Store<QT>::put(p.out, ((long)b * p.Hq + hq) * p.D + d, np > 0 ? ot / lt : 0.f);
+    Store<QT>::put(p.out, out_at + d, lt > 0.f ? ot / lt : 0.f);
   }
 }
 
@@ -213,7 +228,7 @@ hipError_t launch_decode_generic(const DecodeParams& p, int q_dtype, int kv_dtyp
 }
 
 hipError_t launch_decode_reduce(const DecodeParams& p, int q_dtype, hipStream_t s) {
-  dim3 grid(p.Hq, p.B), block(p.D <= 64 ? 64 : 128);
+  dim3 grid(p.Hq * (p.query_lens ? p.T : 1), p.B), block(p.D <= 64 ? 64 : 128);
   if (q_dtype == PA_F32) hipLaunchKernelGGL(decode_reduce_kernel<float>, grid, block, 0, s, p);
   else hipLaunchKernelGGL(decode_reduce_kernel<uint16_t>, grid, block, 0, s, p);
   return hipGetLastError();

@@ -640,9 +640,12 @@ __host__ __device__ __forceinline__ int head_slots_of(const DecodeParams& p) {
 // Fixed partitions: one workgroup per (partition, head slot, sequence), NW waves
 // interleave the partition's tiles and merge through LDS.
 // ---------------------------------------------------------------------------
-template <int D, bool FP8, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void decode_mfma_kernel(DecodeParams p) {
-  using W = DecodeWave<D, FP8>;
+// MULTI (a few query tokens per sequence, small calls of pa_verify): the rows of a kv head are its (query token, q
+// head) pairs, token-major, 16 per wave as in the balanced kernel; a row may see no key in a partition (its causal
+// bound lies before it), which leaves an empty partial (m = -inf, l = 0); rows past the query length come out as zeros.
+template <int D, bool FP8, int NW, bool MULTI = false>
+__global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(DecodeParams p) {
+  using W = DecodeWave<D, FP8, MULTI>;
   constexpr int VEC = W::VEC;
   constexpr int OSTRIDE = D + 16;   // LDS row stride (floats) for the merge
 
@@ -652,24 +655,34 @@ __global__ __launch_bounds__(NW * 64, 2) void decode_mfma_kernel(DecodeParams p)
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   W w(p, hidx, lane);
-  const int ctx = clamp_ctx(p, b);
+  const SeqSpan sp = seq_span(p, b);
+  const int ctx = sp.ctx;
+  // where virtual row vr (q head, or (token, head) pair) of sequence b lies in out
+  const int n_rep = p.Hq / p.Hkv;
+  auto out_row = [&](int vr) __attribute__((always_inline)) -> uint16_t* {
+    if (!MULTI) return (uint16_t*)p.out + ((long)b * p.Hq + vr) * D;
+    const int n_rows = n_rep * p.T;
+    const int hk = vr / n_rows, j = vr - hk * n_rows, t = j / n_rep;
+    return (uint16_t*)p.out + (((long)b * p.T_stride + p.t0 + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D;
+  };
   const int t_begin = part * p.partition_size;
   if (t_begin >= ctx) {
     if (ctx == 0 && part == 0 && p.num_partitions == 1) {
-      for (int i = tid; i < w.nheads * D; i += NW * 64)
-        ((uint16_t*)p.out)[((long)b * p.Hq + w.hbase) * D + i] = 0;
+      for (int i = tid; i < w.nheads * D; i += NW * 64) out_row(w.hbase + i / D)[i % D] = 0;
     }
     return;
   }
   const int t_end = min(ctx, t_begin + p.partition_size);
   const int ntiles = (t_end - t_begin + 31) >> 5;
-  w.begin(b, ctx);
+  w.begin(b, ctx, sp.tq);
   w.stream(t_begin + 32 * wave, 32 * NW, (ntiles - wave + NW - 1) / NW, t_end);
 
   // ---- merge the NW wave states through LDS ----
+  // (eight waves keep rows for at most 8 q heads per kv head: 16 rows of 8 waves would not fit the static 64 KB)
+  constexpr int MROWS = NW > 4 ? 8 : 16;
   __shared__ float sm_m[NW][16];
   __shared__ float sm_l[NW][16];
-  __shared__ __attribute__((aligned(16))) float sm_o[NW][16][OSTRIDE];
+  __shared__ __attribute__((aligned(16))) float sm_o[NW][MROWS][OSTRIDE];
   const float l_tot = w.total_l();
   const int r = w.r, g = w.g, nheads = w.nheads;
   if (g == 0) { sm_m[wave][r] = w.m_run[0]; sm_l[wave][r] = l_tot; }
@@ -679,25 +692,27 @@ __global__ __launch_bounds__(NW * 64, 2) void decode_mfma_kernel(DecodeParams p)
       *(f32x4_t*)&sm_o[wave][r][e * 16 + 4 * g] = w.oacc[0][e];
   }
   __syncthreads();
+  const long rows_total = (long)p.Hq * (MULTI ? p.T : 1);
   for (int idx = tid; idx < nheads * D; idx += NW * 64) {
     const int h = idx / D, d = idx % D;
     const int pos = (d % VEC) * 16 + d / VEC;
     float mt = -INFINITY;
 #pragma unroll
     for (int x = 0; x < NW; ++x) mt = fmaxf(mt, sm_m[x][h]);
+    const float m_ref = (MULTI && mt == -INFINITY) ? 0.f : mt;      // a row that saw no key here: every weight 0
     float lt = 0.f, ot = 0.f;
 #pragma unroll
     for (int x = 0; x < NW; ++x) {
-      const float wt = __builtin_amdgcn_exp2f(sm_m[x][h] - mt);   // idle waves: 2^-inf = 0
+      const float wt = __builtin_amdgcn_exp2f(sm_m[x][h] - m_ref);   // idle waves: 2^-inf = 0
       lt += sm_l[x][h] * wt;
       ot += sm_o[x][h][pos] * wt;
     }
-    const float o = ot / lt;
-    const int hq = w.hbase + h;
+    const float o = (MULTI && lt == 0.f) ? 0.f : ot / lt;
+    const int vr = w.hbase + h;
     if (p.num_partitions == 1) {
-      ((uint16_t*)p.out)[((long)b * p.Hq + hq) * D + d] = float_to_bf16_bits(o);
+      out_row(vr)[d] = float_to_bf16_bits(o);
     } else {
-      const long slot = ((long)b * p.Hq + hq) * p.num_partitions + part;
+      const long slot = ((long)b * rows_total + vr) * p.num_partitions + part;
       p.ws_out[slot * D + d] = o;
       if (d == 0) { p.ws_ml[slot * 2] = mt; p.ws_ml[slot * 2 + 1] = lt; }
     }
@@ -931,11 +946,21 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
 template <int D, bool FP8>
 hipError_t launch_typed(const DecodeParams& p, int waves, hipStream_t s) {
   const int n_rep = p.Hq / p.Hkv;
-  dim3 grid(p.num_partitions, p.Hkv * ((n_rep + 15) / 16), p.B);
-  if (p.head_major) grid = dim3(p.Hkv * ((n_rep + 15) / 16), p.num_partitions, p.B);
+  const int slots = head_slots_of(p);                  // Hkv x 16-row groups of a kv head's rows
+  dim3 grid(p.num_partitions, slots, p.B);
+  if (p.head_major) grid = dim3(slots, p.num_partitions, p.B);
+  if (p.query_lens) {      // multi-token rows: the four-wave form
+    if (p.rows_per_wave != 16) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 4, true>), grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+  }
   switch (waves) {
     case 1: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 1>), grid, dim3(64), 0, s, p); break;
     case 2: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 2>), grid, dim3(128), 0, s, p); break;
+    case 8:
+      if (n_rep > 8) return hipErrorInvalidValue;      // its merge area holds 8 rows per wave
+      hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 8>), grid, dim3(512), 0, s, p);
+      break;
     default: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 4>), grid, dim3(256), 0, s, p); break;
   }
   return hipGetLastError();

@@ -313,15 +313,15 @@ class PagedAttention:
         else:
             paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq
+        capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
+        bound = max_seq_len if max_seq_len is not None else (c.max_model_len if capturing else max(c.max_seq_len, 1))
+        if bound < c.max_seq_len:
+            raise ValueError(f"max_seq_len {bound} is below a live context of {c.max_seq_len} tokens")
         if T == 1:
             # the bound on the contexts sizes the launch, clamps the lengths the kernel reads and picks the kernel.
             # The caller's bound if given; else what the host knows of this step's contexts, unless the launch is
             # being captured into a HIP graph: that will be replayed on longer contexts, so it gets the longest
             # sequence the cache admits.
-            capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
-            bound = max_seq_len if max_seq_len is not None else (c.max_model_len if capturing else max(c.max_seq_len, 1))
-            if bound < c.max_seq_len:
-                raise ValueError(f"max_seq_len {bound} is below a live context of {c.max_seq_len} tokens")
             paged_attn.decode(q[:, 0], kc, vc, c.block_tables, c.seq_lens, self.scale,
                               k_scale=ks, v_scale=vs, partition_size=self.partition_size,
                               max_seq_len=bound, out=out[:, 0],
@@ -329,7 +329,7 @@ class PagedAttention:
             # the decode kernel treats every slot as live; idle slots (seq_len 0) come back as zeros
         else:
             paged_attn.prefill(q, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
-                               k_scale=ks, v_scale=vs, out=out,
+                               k_scale=ks, v_scale=vs, out=out, max_seq_len=bound,
                                sinks=self.sinks, sliding_window=self.sliding_window, q_transform=qt)
         if self.o_weight is None:
             return out

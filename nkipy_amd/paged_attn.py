@@ -323,7 +323,7 @@ def verify_supported(T, D, block_size) -> bool:
 
 def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
             out=None, workspace=None, route=None, validate_tables=False, sinks=None, sliding_window=None,
-            q_transform=None):
+            q_transform=None, max_seq_len=None):
     """Chunked prefill against a cached prefix (causal).
 
     q [B, T, Hq, D] bfloat16 holds the last query_lens[b] tokens of each sequence
@@ -340,6 +340,9 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     (float8_e4m3fn / uint8 codes with k_scale, v_scale) work on both.  sinks and sliding_window are
     as in `decode`, the window counted back from each query token; so is q_transform, the position of
     row t being seq_lens[b] - query_lens[b] + t.
+    max_seq_len: host-known upper bound of seq_lens, as in `decode`; with it a small verify call (a few
+    short sequences, no sinks, no window) takes fixed partitions instead of the balanced schedule, whose
+    fixed cost dominates at that size.  The tiled kernel does not use it.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -391,6 +394,9 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
         _check(out.shape == q.shape and out.dtype == q.dtype, "out must match q in shape and dtype")
     qt_keep, qt_ptr = _qt_arg(q_transform, D, q)
     stream = _stream_ptr(q.device)
+    cap = block_tables.shape[1] * block_size
+    msl = 0 if max_seq_len is None else int(max_seq_len)
+    _check(max_seq_len is None or 0 < msl <= cap, f"max_seq_len {msl} outside (0, {cap}]")
     if route == "verify":
         need = int(lib.pa_verify_workspace_bytes(B, T, Hq, D))
         if workspace is None:
@@ -403,7 +409,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
             rc = lib.pa_verify(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                                _ptr(block_tables), _ptr(seq_lens), _ptr(query_lens), _ptr(out),
                                _ptr(workspace), ws_bytes, B, T, Hq, Hkv, D, block_size,
-                               block_tables.shape[1], num_blocks, float(scale), kv_code, _ptr(sinks), win,
+                               block_tables.shape[1], num_blocks, msl, float(scale), kv_code, _ptr(sinks), win,
                                qt_ptr, stream)
         _raise_on(rc, "pa_verify")
         return out

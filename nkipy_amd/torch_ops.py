@@ -59,10 +59,11 @@ def paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                   sinks: Optional[torch.Tensor] = None, sliding_window: int = 0,
                   rope_cos: Optional[torch.Tensor] = None, rope_sin: Optional[torch.Tensor] = None,
                   q_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6,
-                  workspace: Optional[torch.Tensor] = None) -> None:
+                  workspace: Optional[torch.Tensor] = None, max_seq_len: int = 0) -> None:
     paged_attn.prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, k_scale=k_scale,
                        v_scale=v_scale, out=out, sinks=sinks, sliding_window=_win(sliding_window),
-                       q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps), workspace=workspace)
+                       q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps), workspace=workspace,
+                       max_seq_len=max_seq_len or None)
 
 
 @torch.library.custom_op(f"{_NS}::blocksparse_prefill", mutates_args=("out",), device_types="cuda")

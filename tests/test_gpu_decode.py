@@ -395,3 +395,39 @@ def test_device_kernel_convention(pa):
     ret = kern(inputs=ins)                      # outputs=None: result returned by value
     torch.cuda.synchronize()
     assert np.array_equal(ret.numpy(), out.numpy())
+
+
+@pytest.mark.parametrize("B,ctx_hi,fp8", [(3, 700, False), (70, 1000, False), (5, 768, True), (2, 520, False)])
+def test_small_calls_as_one_partition_on_eight_waves(B, ctx_hi, fp8):
+    """Small calls whose length bound is short take one partition per sequence on eight waves (no merge launch):
+    against the oracle, and against the same call with that route switched off (two partitions and the merge)."""
+    import nkipy_amd as pa
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(B + ctx_hi)
+    Hq, Hkv, D, bs = 32, 8, 128, 32
+    ctxs = [int(x) for x in rng.integers(1, ctx_hi + 1, B)]
+    ctxs[0] = ctx_hi
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    q = O.round_to_bf16(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    scale = pa.default_scale(D)
+    i32 = lambda x: torch.from_numpy(np.asarray(x, np.int32)).cuda()  # noqa: E731
+    if fp8:
+        kq, ks = O.quantize_kv_fp8(k)
+        vq, vs = O.quantize_kv_fp8(v)
+        want = O.paged_decode(q, kq, vq, tables, np.asarray(ctxs, np.int32), scale, k_scale=ks, v_scale=vs, q_dtype="bf16")
+        kd, vd = (torch.from_numpy(x).cuda().view(torch.float8_e4m3fn) for x in (kq, vq))
+        kw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda())
+    else:
+        want = O.paged_decode(q, O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32), scale, q_dtype="bf16")
+        kd, vd, kw = bf16_to_dev(k), bf16_to_dev(v), {}
+    print(f"decode one partition B={B} ctx<={ctx_hi} fp8={fp8}", flush=True)
+    got = pa.decode(bf16_to_dev(q), kd, vd, i32(tables), i32(ctxs), scale, max_seq_len=ctx_hi, **kw)
+    lib.pa_debug_set(9, 0)
+    try:
+        two = pa.decode(bf16_to_dev(q), kd, vd, i32(tables), i32(ctxs), scale, max_seq_len=ctx_hi, **kw)
+        torch.cuda.synchronize()
+    finally:
+        lib.pa_debug_set(9, 1024)
+    assert np.abs(dev_to_f32(got) - want).max() <= (5e-2 if fp8 else 2e-2)
+    assert np.abs(dev_to_f32(got) - dev_to_f32(two)).max() <= 2.0 ** -7 * max(np.abs(want).max(), 1.0)

@@ -289,3 +289,51 @@ def test_head_dim_64_many_rows_of_a_short_run_take_the_tiled_kernel(pa):
     assert not np.array_equal(got, via_verify)          # two kernels: different summation orders
     for b, n in enumerate(qlens):
         assert np.all(got[b, n:] == 0)
+
+
+@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
+@pytest.mark.parametrize("T,Hq,Hkv,D,bs", [(4, 32, 8, 128, 32), (8, 8, 2, 128, 16), (3, 40, 2, 64, 16), (5, 6, 2, 64, 64),
+                                           (16, 16, 4, 128, 32), (7, 1, 1, 128, 32)])
+def test_verify_small_calls_with_a_length_bound(pa, T, Hq, Hkv, D, bs, fp8):
+    """With the caller's bound on the contexts a small call takes fixed partitions (one to four of 512 tokens): a
+    single sequence behind about 1 K tokens (the reference's own use), a ragged batch with an idle slot and a
+    one-token sequence, contexts a few tokens past a partition boundary (the early query rows then see no key in
+    the last partition and leave an empty partial), a bound far above the contexts (partitions with no tokens),
+    bf16 and fp8 pools.  Against the oracle; rows past the query length are zeros."""
+    rng = np.random.default_rng(77 * T + Hq + D)
+    for qlens, prefixes, bound in [([T], [1020], 1100), ([T, max(T - 1, 1), 1, T, 0, T], [0, 300, 65, 1533, 40, 512 - 2], 1600),
+                                   ([T, T], [512 - 1, 1024 + 1 - T], 2048), ([T, 2], [3, 40], 70), ([T], [100], 2000)]:
+        q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+        bound = min(bound, tables.shape[1] * bs)        # never above the table capacity
+        assert ctxs.max() <= bound
+        scale = 1.0 / np.sqrt(D)
+        if fp8:
+            kq, ks = O.quantize_kv_fp8(k)
+            vq, vs = O.quantize_kv_fp8(v)
+            want = O.paged_prefill(q, kq, vq, tables, ctxs, ql, scale, q_dtype="bf16", k_scale=ks, v_scale=vs)
+            kd, vd = (torch.from_numpy(x).cuda().view(torch.float8_e4m3fn) for x in (kq, vq))
+            kw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda())
+        else:
+            want = O.paged_prefill(q, k, v, tables, ctxs, ql, scale, q_dtype="bf16")
+            kd, vd, kw = bf16_to_dev(k), bf16_to_dev(v), {}
+        print(f"verify small call T={T} Hq={Hq} Hkv={Hkv} D={D} bs={bs} fp8={fp8} qlens={qlens} bound={bound}", flush=True)
+        got = pa.verify(bf16_to_dev(q), kd, vd, _i32(tables), _i32(ctxs), _i32(ql), scale, max_seq_len=bound, **kw)
+        plain = pa.verify(bf16_to_dev(q), kd, vd, _i32(tables), _i32(ctxs), _i32(ql), scale, **kw)
+        torch.cuda.synchronize()
+        got = dev_to_f32(got)
+        assert_close_abs(got, want, FP8_TOL if fp8 else BF16_TOL)
+        assert np.abs(got - dev_to_f32(plain)).max() <= 2.0 ** -7 * max(np.abs(want).max(), 1.0)      # the balanced route, to a bf16 step
+        for b, n in enumerate(qlens):
+            assert np.all(got[b, n:] == 0)
+
+
+def test_verify_length_bound_clamps_like_decode(pa):
+    """A bound below a context: the kernels read the context up to the bound, as pa_decode does with its max_seq_len."""
+    rng = np.random.default_rng(5)
+    T, Hq, Hkv, D, bs = 4, 8, 2, 128, 32
+    q, k, v, tables, ctxs, ql = _case(rng, T, [T, T], [900, 200], Hq, Hkv, bs, D)
+    bound = 600
+    want = O.paged_prefill(q, k, v, tables, np.minimum(ctxs, bound).astype(np.int32), ql, 0.09, q_dtype="bf16")
+    got = pa.verify(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.09, max_seq_len=bound)
+    torch.cuda.synchronize()
+    assert_close_abs(dev_to_f32(got), want, BF16_TOL)

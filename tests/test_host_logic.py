@@ -103,7 +103,7 @@ def test_c_abi_argument_errors_without_gpu(lib):
         a = dict(B=2, T=4, Hq=8, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1)
         a.update(kw)
         return lib.pa_verify(z, z, z, z, z, z, z, z, z, z, 0, a["B"], a["T"], a["Hq"], a["Hkv"], a["D"], a["bs"],
-                             a["mb"], a["nb"], 1.0, a["kd"], z, a.get("win", 0), z, z)
+                             a["mb"], a["nb"], a.get("msl", 0), 1.0, a["kd"], z, a.get("win", 0), z, z)
     assert ver(Hq=7) == -1 and b"multiple" in lib.pa_last_error()
     assert ver(kd=0) == -1 and b"kv_dtype" in lib.pa_last_error()
     assert ver(T=65) == -1 and b"pa_prefill" in lib.pa_last_error()
