@@ -468,27 +468,31 @@ void prefill_async_kernel(PrefillParams p) {
   };
   // FP8: codes of tile kt in raw stage rs -> bf16 values in stage bs, this wave's 8 rows; rows past the
   // context get the scale 0 (their codes are a copy of the last valid row, their block may not exist)
+  // A lane expands one 16-byte chunk (8 codes) of two rows, rows lane / 16 and lane / 16 + 4 of the wave's eight,
+  // chunk lane % 16: a store instruction then writes whole rows, 16 consecutive lanes the 16 different chunk
+  // positions of one row, and no two of them share a bank.  (With a lane expanding 16 codes of one row into two
+  // chunks, the lanes of a row wrote every other chunk position per instruction and collided pairwise.)
   auto expand = [&](int kt, int rs, int bs) __attribute__((always_inline)) {
-    const char* raw = smem + BFS * STAGE_B + rs * RAW_STAGE_B + wave * 1024 + lane * 16;
-    const int row = 8 * wave + (lane >> 3), c16 = lane & 7;
-    const bool live = kt * BN + row < ctx;
+    const char* raw = smem + BFS * STAGE_B + rs * RAW_STAGE_B + wave * 1024;
+    const int ch = lane & 15;
     // PAIR: the first 64 codes of a raw row belong to the even kv head, the others to the odd one
-    const float ks = PAIR && c16 >= 4 ? ksq2[0] : ksq[0], vs = PAIR && c16 >= 4 ? vsq2[0] : vsq[0];
-    const float sk = live ? ks : 0.f, sv = live ? vs : 0.f;
-    const uint4 rk = *(const uint4*)raw, rv = *(const uint4*)(raw + RAW_TILE_B);
-    auto half = [&](uint32_t a, uint32_t b2, float scl) __attribute__((always_inline)) -> uint4 {
+    const float ks = PAIR && ch >= 8 ? ksq2[0] : ksq[0], vs = PAIR && ch >= 8 ? vsq2[0] : vsq[0];
+    auto widen = [&](uint2 c, float scl) __attribute__((always_inline)) -> uint4 {
       float f[8];
-      fp8x4_to_float(a, f);
-      fp8x4_to_float(b2, f + 4);
+      fp8x4_to_float(c.x, f);
+      fp8x4_to_float(c.y, f + 4);
       return make_uint4(pack_bf16x2(f[0] * scl, f[1] * scl), pack_bf16x2(f[2] * scl, f[3] * scl),
                         pack_bf16x2(f[4] * scl, f[5] * scl), pack_bf16x2(f[6] * scl, f[7] * scl));
     };
-    char* kd = smem + bs * STAGE_B + row * ROW_B;
-    *(uint4*)(kd + (((2 * c16) ^ (row & 15)) << 4)) = half(rk.x, rk.y, sk);
-    *(uint4*)(kd + (((2 * c16 + 1) ^ (row & 15)) << 4)) = half(rk.z, rk.w, sk);
-    char* vd = kd + TILE_B;
-    *(uint4*)(vd + (((2 * c16) ^ (4 * (row & 3))) << 4)) = half(rv.x, rv.y, sv);
-    *(uint4*)(vd + (((2 * c16 + 1) ^ (4 * (row & 3))) << 4)) = half(rv.z, rv.w, sv);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int lrow = (lane >> 4) + 4 * u, row = 8 * wave + lrow;
+      const bool live = kt * BN + row < ctx;
+      const uint2 rk = *(const uint2*)(raw + lrow * HD + ch * 8), rv = *(const uint2*)(raw + RAW_TILE_B + lrow * HD + ch * 8);
+      char* kd = smem + bs * STAGE_B + row * ROW_B;
+      *(uint4*)(kd + ((ch ^ (row & 15)) << 4)) = widen(rk, live ? ks : 0.f);
+      *(uint4*)(kd + TILE_B + ((ch ^ (4 * (row & 3))) << 4)) = widen(rv, live ? vs : 0.f);
+    }
   };
 
   // ---- fragment loads and matrix steps, one "group" at a time -------------------------
