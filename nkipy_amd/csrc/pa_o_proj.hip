@@ -527,6 +527,113 @@ __global__ __launch_bounds__(256) void o_proj_skinny_kernel(OProjParams p) {
   }
 }
 
+// Very few rows (M <= 32: a decode step of a small batch, a verify step of one sequence).  The call is w's bytes
+// and a handful of latencies, so nothing is recycled: a workgroup of 4 waves owns 128 output columns and a range
+// of at most 8 k-steps of 64, requests ALL of its operands at once -- per k-step the x tile [32 rows][128 B] and the
+// w tile [64 k][256 B], 20 KB, up to 160 KB -- and multiplies as the steps land: one memory round trip for the whole
+// workgroup instead of a ring that is filled, drained and refilled (the ring form spends a third of its life filling,
+// and copies 64 x rows where 8 are live).  (N / 128) x (K / 512) workgroups: 256 at K = N = 4096.  Wave w takes
+// the 32-column chunk w; operand layouts, swizzles and the product are those of the kernels above.  The K ranges
+// leave float32 partial tiles for o_proj_split_reduce_kernel (one range: bf16 output and bias directly).
+constexpr int RS_X = 32 * 128, RS_W = 64 * 256, RS_STAGE = RS_X + RS_W;      // 4 KB + 16 KB per k-step
+constexpr int RS_MAX_STEPS = 8;
+template <bool BIAS>
+__global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * 128;
+  const int kt_total = p.K / BK;
+  const int kt_begin = (int)((long)kt_total * blockIdx.y / gridDim.y);
+  const int ktiles = (int)((long)kt_total * (blockIdx.y + 1) / gridDim.y) - kt_begin;      // <= RS_MAX_STEPS (host)
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_char*)smem;
+  const long x_row_b = (long)p.K * 2, w_row_b = (long)p.N * 2;
+  // copy maps.  x: 4 units of 8 rows x 128 B, wave w issues unit w; lane i fills (row 8w + i/8, position i%8) with
+  // chunk (i%8) ^ ((row >> 1) & 7).  w: 16 units of 4 rows x 256 B, wave w issues units w, w+4, w+8, w+12; lane i
+  // fills (row 4u + i/16, position i%16) with chunk (i%16) ^ 4 (row & 3).  Rows past M and columns past N are clamped.
+  uint32_t xoff, woff[4];
+  {
+    const int lrow = 8 * wave + (lane >> 3);
+    xoff = (uint32_t)(min(lrow, p.M - 1) * x_row_b) + (uint32_t)(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = 4 * (wave + 4 * j) + (lane >> 4);
+    const int chunk = (lane & 15) ^ (4 * ((lane >> 4) & 3));
+    woff[j] = (uint32_t)(r * w_row_b) + (uint32_t)(min(n0 + 8 * chunk, p.N - 8) * 2);
+  }
+  {
+    const char* xb = (const char*)p.x + (long)kt_begin * (BK * 2);
+    const char* wb = (const char*)p.w + (long)kt_begin * BK * w_row_b;
+    for (int kt = 0; kt < ktiles; ++kt) {
+      const uint32_t sb = smem_base + kt * RS_STAGE;
+      dma16(xb, xoff, sb + wave * 1024);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dma16(wb, woff[j], sb + RS_X + (wave + 4 * j) * 1024);
+      xb += BK * 2;
+      wb += (long)BK * w_row_b;
+    }
+  }
+  int x_off[4], w_off;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) x_off[s] = n * 128 + (((2 * s + h) ^ ((n >> 1) & 7)) << 4);
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int row = 8 * h + (sl >> 2);
+    const int y = 2 * (g & 1) + ((sl & 3) >> 1);
+    w_off = RS_X + row * 256 + (((4 * wave + y) ^ (4 * (row & 3))) << 4) + (sl & 1) * 8;
+  }
+  f32x16_t acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  auto step = [&](int kt) __attribute__((always_inline)) {
+    const char* sb = smem + kt * RS_STAGE;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const lds_char* src = (const lds_char*)(sb + 16 * s * 256 + w_off);
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)src);
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(src + 4 * 256));
+      struct { s16x4_t a, b; } pair = {lo, hi};
+      const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, pair);
+      const bf16x8_t xf = *(const bf16x8_t*)(sb + x_off[s]);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc, 0, 0, 0);
+    }
+  };
+  if (ktiles == RS_MAX_STEPS) {
+    // a full range: the steps are multiplied as they land (5 copy instructions per wave and step)
+#define RS_STEP(kt) wait_vmcnt<5 * (RS_MAX_STEPS - 1 - (kt))>(); __builtin_amdgcn_s_barrier(); step(kt);
+    RS_STEP(0) RS_STEP(1) RS_STEP(2) RS_STEP(3) RS_STEP(4) RS_STEP(5) RS_STEP(6) RS_STEP(7)
+#undef RS_STEP
+  } else {
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    for (int kt = 0; kt < ktiles; ++kt) step(kt);
+  }
+  // a lane holds, for its row, 4 consecutive columns at 4 places
+  const int m = n;
+#pragma unroll
+  for (int i4 = 0; i4 < 4; ++i4) {
+    const int col = n0 + 32 * wave + 8 * i4 + 4 * h;
+    if (m < p.M && col < p.N) {
+      if (p.splits > 1) {
+        *(float4*)(p.ws + ((long)blockIdx.y * p.M + m) * p.N + col) =
+            make_float4(acc[4 * i4], acc[4 * i4 + 1], acc[4 * i4 + 2], acc[4 * i4 + 3]);
+      } else {
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (BIAS) {
+          const uint2 bw = *(const uint2*)((const uint16_t*)p.bias + col);
+          b0 = bf16_bits_to_float(bw.x & 0xffffu); b1 = bf16_bits_to_float(bw.x >> 16);
+          b2 = bf16_bits_to_float(bw.y & 0xffffu); b3 = bf16_bits_to_float(bw.y >> 16);
+        }
+        *(uint2*)((uint16_t*)p.out + (long)m * p.N + col) = make_uint2(pack_bf16x2(acc[4 * i4] + b0, acc[4 * i4 + 1] + b1),
+                                                                        pack_bf16x2(acc[4 * i4 + 2] + b2, acc[4 * i4 + 3] + b3));
+      }
+    }
+  }
+}
+
 // Sum of the split form's partial tiles, always in the order of the K ranges, plus the bias; one rounding to bf16.
 // A thread owns four consecutive columns of a row (N is a multiple of 8, so they never straddle rows).
 template <bool BIAS>
@@ -535,13 +642,13 @@ __global__ __launch_bounds__(256) void o_proj_split_reduce_kernel(OProjParams p)
   const long item = (long)blockIdx.x * 256 + threadIdx.x;
   if (item >= total) return;
   const float4* src = (const float4*)p.ws + item;
-  // all ranges requested at once (at most four exist: o_proj_splits), added in their order
-  float4 part[4];
+  // all ranges requested at once (at most eight exist: o_proj_splits), added in their order
+  float4 part[8];
 #pragma unroll
-  for (int z = 0; z < 4; ++z) part[z] = z < p.splits ? src[(long)z * total] : make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int z = 0; z < 8; ++z) part[z] = z < p.splits ? src[(long)z * total] : make_float4(0.f, 0.f, 0.f, 0.f);
   float4 a = part[0];
 #pragma unroll
-  for (int z = 1; z < 4; ++z)
+  for (int z = 1; z < 8; ++z)
     if (z < p.splits) { a.x += part[z].x; a.y += part[z].y; a.z += part[z].z; a.w += part[z].w; }
   if (BIAS) {
     const uint2 bw = *(const uint2*)((const uint16_t*)p.bias + (item * 4) % p.N);
@@ -581,8 +688,38 @@ hipError_t launch_skinny(const OProjParams& p, hipStream_t s) {
 // Up to 128 rows the call streams w once through N / 64 workgroups; with a workspace up to four K ranges per column
 // slab bring that towards the CU count (K = N = 4096, kernel time without the merge: 16.9 -> 9.9 us at 64 rows with
 // four ranges, 12.4 with eight), each at least 8 steps of 64 long.
+// M <= 32: the resident form, ranges of at most 8 k-steps (then K / 512 of them, up to eight); 0 when K is longer
+static int o_proj_resident_splits(int M, int K) {
+  if (M <= 0 || M > 32) return 0;
+  const int s = (K / BK + RS_MAX_STEPS - 1) / RS_MAX_STEPS;
+  return s <= 8 ? s : 0;
+}
+
+static hipError_t launch_resident(const OProjParams& p, hipStream_t s) {
+  static std::atomic<int> configured{0};
+  constexpr int lds = RS_MAX_STEPS * RS_STAGE;
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute((const void*)o_proj_resident_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_resident_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    configured.store(1, std::memory_order_release);
+  }
+  const int ktiles = (p.K / BK + p.splits - 1) / p.splits;
+  const dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)p.splits);
+  const int bytes = ktiles * RS_STAGE;
+  if (p.bias && p.splits == 1) hipLaunchKernelGGL((o_proj_resident_kernel<true>), grid, dim3(256), bytes, s, p);
+  else hipLaunchKernelGGL((o_proj_resident_kernel<false>), grid, dim3(256), bytes, s, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || p.splits == 1) return e;
+  const unsigned blocks = (unsigned)(((long)p.M * p.N / 4 + 255) / 256);
+  if (p.bias) hipLaunchKernelGGL((o_proj_split_reduce_kernel<true>), dim3(blocks), dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((o_proj_split_reduce_kernel<false>), dim3(blocks), dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
 int o_proj_splits(int M, int K, int N) {
   if (M <= 0 || M > 128) return 1;
+  if (const int r = o_proj_resident_splits(M, K)) return r;
   const long slabs = (N + 63) / 64;
   long s = 256 / slabs;
   if (s > 4) s = 4;
@@ -594,6 +731,8 @@ static std::atomic<int> g_o_proj_force_large{0};
 void o_proj_debug_force_large(int on) { g_o_proj_force_large = on; }
 
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
+  // up to 32 rows with the workspace for its K ranges (or K <= 512): everything resident, one round trip
+  if (const int r = o_proj_resident_splits(p.M, p.K); r > 0 && p.splits == r && (r == 1 || p.ws)) return launch_resident(p, s);
   // up to 256 rows: one workgroup per 64 columns owns every row (the call is bound by w's bytes)
   if (p.M <= 64) return launch_skinny<2>(p, s);
   if (p.M <= 128) return launch_skinny<4>(p, s);
