@@ -181,11 +181,11 @@ def _cpu_prefill_baseline(run_fn, flops, desc):
 # this file on the seeded workloads (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00: the factors a plain copy
 # of known size shows); the summaries with the commands are under profiles/.  Not re-measured at run time.
 MEASURED_TRAFFIC_BYTES = {
-    2: {"bytes": 1_098_900_000, "source": "profiles/decode_balanced_kernel_C2.md"},
-    3: {"bytes": 385_200_000, "source": "profiles/prefill_async_kernel_C3.md"},
-    4: {"bytes": 743_900_000, "source": "profiles/prefill_async_kernel_C4.md"},
-    5: {"bytes": 2_402_400_000, "source": "profiles/decode_balanced_kernel_C5.md"},
-    8: {"bytes": 1_123_600_000, "source": "profiles/decode_balanced_kernel_verify_T4.md"},
+    2: {"bytes": 1_099_100_000, "source": "profiles/decode_balanced_kernel_C2.md"},
+    3: {"bytes": 380_800_000, "source": "profiles/prefill_async_kernel_C3.md"},
+    4: {"bytes": 709_500_000, "source": "profiles/prefill_async_kernel_C4.md"},
+    5: {"bytes": 2_404_500_000, "source": "profiles/decode_balanced_kernel_C5.md"},
+    8: {"bytes": 1_125_700_000, "source": "profiles/decode_balanced_kernel_verify_T4.md"},
 }
 
 
@@ -696,15 +696,13 @@ def bench_prefill_layer_step(steps, warmup, lib, pa, W):
     }
 
 
-def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
-    """config 13: a decode step of a small batch through the engine glue, per attention layer: QK RMSNorm + RoPE +
-    K/V row into the pool + paged decode + output projection (`PagedAttention.attend`), `layers` layers with a pool
-    and weights of their own, issued call by call and replayed from one HIP graph.  Launch-bound: the figure is
-    microseconds per layer; the bytes a layer has to move (its contexts' K and V, the projection weight) are given
-    for scale."""
+def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound):
+    """Seconds per step of `layers` attention layers, issued call by call and replayed from one HIP graph, on a cache
+    whose tables hold `capacity` tokens per sequence; `bound` is the length bound given to `attend` (None: the
+    engine's own choice, which under capture is the longest context the cache admits)."""
     from nkipy_amd.engine import PagedAttention, PagedKVCache
     Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
-    nblk = (ctx + 64) // bs + 1
+    nblk = (capacity + bs - 1) // bs
     cache = PagedKVCache(B * nblk + 8, bs, Hkv, D, max_seqs=B, max_blocks_per_seq=nblk, num_layers=layers)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1313)
@@ -720,7 +718,7 @@ def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
 
     def step():
         for a in att:
-            a.attend(q1, k1, k1)
+            a.attend(q1, k1, k1, max_seq_len=bound)
 
     cache.begin_step([1] * B, 1)
     sec_eager = _time_steps(step, steps, warmup)
@@ -728,6 +726,23 @@ def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
     with torch.cuda.graph(graph):
         step()
     sec = _time_steps(graph.replay, steps, 5)
+    del graph
+    return sec, sec_eager, nblk * bs
+
+
+def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
+    """config 13: a decode step of a small batch through the engine glue, per attention layer: QK RMSNorm + RoPE +
+    K/V row into the pool + paged decode + output projection (`PagedAttention.attend`), `layers` layers with a pool
+    and weights of their own, issued call by call and replayed from one HIP graph.  Launch-bound: the figure is
+    microseconds per layer; the bytes a layer has to move (its contexts' K and V, the projection weight) are given
+    for scale.  The length bound a captured step carries picks its decode kernel, so the figure depends on what the
+    caller can promise: the headline is a cache whose tables end just above the contexts (the bound is then the
+    table capacity); `capacity_8k` repeats it on tables of 8 192 tokens per sequence, once with no promise (the
+    captured step must serve any length: the balanced kernel) and once with `attend(max_seq_len=1088)`."""
+    Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
+    sec, sec_eager, cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, ctx + 96, None)
+    big_free, _, big_cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, 8192, None)
+    big_bound, _, _ = _decode_layer_step_times(steps, warmup, B, ctx, layers, 8192, ctx + 64)
     kv_bytes = 2 * B * (ctx + 1) * Hkv * D * 2
     byts = kv_bytes + Hq * D * N * 2 + B * (2 * Hq * D + 2 * Hkv * D + N) * 2
     us = sec / layers * 1e6
@@ -736,9 +751,13 @@ def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
         "value": round(1e6 / us, 1), "unit": "layer steps/s",
         "ms_per_step": round(sec * 1e3, 5), "us_per_layer": round(us, 2),
         "eager_us_per_layer": round(sec_eager / layers * 1e6, 2),
+        "capacity_8k": {"table_capacity_tokens": big_cap,
+                        "us_per_layer_no_bound": round(big_free / layers * 1e6, 2),
+                        f"us_per_layer_max_seq_len_{ctx + 64}": round(big_bound / layers * 1e6, 2)},
         "dtype": "bf16, float32 norm, bf16 rotation, fp32 accumulate",
-        "config": {"workload": f"decode layer step: B={B}, context={ctx}, layers={layers}, Hq={Hq}, Hkv={Hkv}, D={D}, "
-                               f"block_size={bs}, hidden={N}; one step = {layers} layers", "algorithmic_bytes_per_layer": byts},
+        "config": {"workload": f"decode layer step: B={B}, context={ctx}, table capacity={cap} tokens per sequence, "
+                               f"layers={layers}, Hq={Hq}, Hkv={Hkv}, D={D}, block_size={bs}, hidden={N}; "
+                               f"one step = {layers} layers", "algorithmic_bytes_per_layer": byts},
         "roofline": {"bound": "hbm", "achieved": round(byts / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(byts / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": "five launches per layer (KV write with K transform, decode + merge, projection + merge)",

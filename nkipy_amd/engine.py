@@ -294,6 +294,10 @@ class PagedAttention:
         B, T = xq.shape[:2]
         if B != c.max_seqs or T != c.step_tokens:
             raise ValueError(f"expected [{c.max_seqs}, {c.step_tokens}, ...] as opened by begin_step, got [{B}, {T}, ...]")
+        capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
+        bound = max_seq_len if max_seq_len is not None else (c.max_model_len if capturing else max(c.max_seq_len, 1))
+        if bound < c.max_seq_len:
+            raise ValueError(f"max_seq_len {bound} is below a live context of {c.max_seq_len} tokens")
         kc, vc, ks, vs = c.k_caches[l], c.v_caches[l], c.k_scales[l], c.v_scales[l]
         out = self._out.get(T)
         if out is None:
@@ -313,10 +317,6 @@ class PagedAttention:
         else:
             paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq
-        capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
-        bound = max_seq_len if max_seq_len is not None else (c.max_model_len if capturing else max(c.max_seq_len, 1))
-        if bound < c.max_seq_len:
-            raise ValueError(f"max_seq_len {bound} is below a live context of {c.max_seq_len} tokens")
         if T == 1:
             # the bound on the contexts sizes the launch, clamps the lengths the kernel reads and picks the kernel.
             # The caller's bound if given; else what the host knows of this step's contexts, unless the launch is

@@ -363,3 +363,69 @@ def test_decode_steps_replayed_from_one_graph_while_the_contexts_grow(rng):
         for l in range(L):
             assert np.array_equal(dev_bits(outs[l]), dev_bits(want[l])), (step, l)
     assert ca.lens == cb.lens == [86, 53, 69]
+
+
+@pytest.mark.parametrize("bound", [None, 256])
+def test_graph_replay_on_tables_longer_than_four_partitions(rng, bound):
+    """Tables of 3 072 tokens per sequence: a decode step captured without a promise about the lengths must serve any
+    of them and takes the balanced kernel, while the eager twin, which knows its contexts are short, takes the
+    fixed-partition one; the two agree to the order of their float32 sums (tolerance, not bits).  With the same
+    `max_seq_len` given to both, the captured step takes the small-call kernel too and every replay equals the eager
+    step bit for bit; a context that would outgrow the promise is refused on the host."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    from tests.pa_testlib import dev_bits
+    S, L, Hq, Hkv, D, bs, hidden = 3, 2, 8, 2, 128, 16, 256
+    ow = [bf16_to_dev((rng.standard_normal((Hq * D, hidden)) / 32).astype(np.float32)) for _ in range(L)]
+
+    def stack():
+        cache = PagedKVCache(num_blocks=96, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S,
+                             max_blocks_per_seq=192, num_layers=L)
+        layers = [PagedAttention(cache, Hq, layer=l, rope_base=10000.0, max_positions=192 * bs, o_weight=ow[l])
+                  for l in range(L)]
+        return cache, layers
+
+    (ca, la), (cb, lb) = stack(), stack()
+    T0 = 40
+    prompt = [[_rand(rng, (S, T0, h, D)) for h in (Hq, Hkv, Hkv)] for _ in range(L)]
+    for cache, layers in ((ca, la), (cb, lb)):
+        cache.begin_step([40, 7, 23], T0)
+        for l in range(L):
+            layers[l].attend(*[bf16_to_dev(t) for t in prompt[l]])
+    xs = [[torch.zeros((S, 1, h, D), dtype=torch.bfloat16, device="cuda") for h in (Hq, Hkv, Hkv)] for _ in range(L)]
+
+    def fill():
+        for l in range(L):
+            for t in xs[l]:
+                t.copy_(bf16_to_dev(_rand(rng, tuple(t.shape))))
+
+    def eager(cache, layers):
+        cache.begin_step([1] * S, 1)
+        return [layers[l].attend(*xs[l], max_seq_len=bound) for l in range(L)]
+
+    fill()
+    eager(ca, la), eager(cb, lb)             # buffers and workspaces exist before the capture
+    torch.cuda.synchronize()
+    fill()
+    ca.begin_step([1] * S, 1)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        outs = [la[l].attend(*xs[l], max_seq_len=bound) for l in range(L)]
+    for step in range(12):
+        if step:
+            fill()
+            ca.begin_step([1] * S, 1)
+        print(f"bound {bound} replay {step}: lens {ca.lens}", flush=True)
+        g.replay()
+        want = eager(cb, lb)
+        torch.cuda.synchronize()
+        for l in range(L):
+            if bound is None:
+                a, b = outs[l].float().cpu().numpy(), want[l].float().cpu().numpy()
+                assert np.abs(a - b).max() <= 2e-2 + 2 ** -7 * np.abs(b).max(), (step, l)
+            else:
+                assert np.array_equal(dev_bits(outs[l]), dev_bits(want[l])), (step, l)
+    if bound is not None:
+        ca.begin_step([bound] * S, bound)    # contexts beyond the promise
+        with pytest.raises(ValueError):
+            la[0].attend(*[torch.zeros((S, bound, h, D), dtype=torch.bfloat16, device="cuda") for h in (Hq, Hkv, Hkv)],
+                         max_seq_len=bound)
