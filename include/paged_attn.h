@@ -251,6 +251,53 @@ int pa_o_proj_ws(const void* x, const void* w, const void* bias, void* out, void
                  int M, int K, int N, int dtype, void* stream);
 
 /*
+ * One decode step of an attention layer in one call: the cache update, the attention and (optionally) the output
+ * projection -- the decode branch of the reference's attention_kernel as a whole
+ * (examples/models/qwen3/kernels/attention.py:78-147: QK norm and RoPE, `cache_k[:, query_pos] = xk`, scores,
+ * softmax, P V, `np.matmul(output, o_weight)`; with sinks, window and bias the gpt-oss form,
+ * examples/models/gpt_oss/kernels/attention.py:85-163), called once per layer and step by the decode loop of
+ * examples/models/qwen3/qwen3.py:310-336,372-396.  The result is, bit for bit, that of
+ *     pa_qk_norm_rope_kv_write(NULL, xk, xv, NULL, ...)   (pa_kv_write without q_transform)
+ *     pa_decode(q, ..., q_transform)
+ *     pa_o_proj_ws(attention output, o_weight, o_bias, out, ...)
+ * on the same arguments; what the one call adds is that a small step (the fixed-partition decode kernels, bf16 pool)
+ * runs as three launches instead of five: the kernel that reaches a sequence's newest token takes its K / V rows
+ * from xk / xv (K transformed on the way) and stores them in the pool itself, and the projection merges the
+ * sequence's split-K partials while it forms its rows.  Calls that those kernels do not take (fp8 or fp32 pools,
+ * large batches or long contexts, sinks, a window) run the separate launches inside.
+ *   new_kv    the step's new token per sequence: xk, xv [B, Hkv, D] of the pool's source type (bf16; float32 for
+ *             an fp32 pool); query_lens [B]: 1 for a sequence that takes a token this step, 0 for one that does
+ *             not (its row of xk / xv is ignored); seq_lens counts the new token, as for pa_kv_write;
+ *             k_norm_weight [D] bf16 or NULL: K's RMSNorm weight, used with q_transform's tables and eps (K is
+ *             normed and rotated exactly when Q is: q_transform NULL = both go in as given)
+ *   k_cache, v_cache, k_scale, v_scale   as for pa_kv_write: updated in place
+ *   attn_out  [B, Hq, D] like q, or NULL when out_proj is given and the attention output itself is not wanted
+ *   out_proj  NULL (attention only), or o_weight [Hq * D, N] bf16 row-major, o_bias [N] bf16 or NULL, out [B, N]
+ *             bf16, N a multiple of 8 (pa_o_proj's conventions)
+ *   workspace pa_decode_step_workspace_bytes(...) bytes, 16-byte aligned; the other arguments as for pa_decode
+ */
+typedef struct pa_new_kv {
+  const void* xk;
+  const void* xv;
+  const void* k_norm_weight;
+  const int32_t* query_lens;
+} pa_new_kv;
+typedef struct pa_out_proj {
+  const void* o_weight;
+  const void* o_bias;
+  void* out;
+  int N;
+} pa_out_proj;
+size_t pa_decode_step_workspace_bytes(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len, int partition_size,
+                                      int N, int q_dtype, int kv_dtype);
+int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* v_cache, float* k_scale, float* v_scale,
+                   const int32_t* block_tables, const int32_t* seq_lens, void* attn_out, const pa_out_proj* out_proj,
+                   void* workspace, size_t workspace_bytes,
+                   int B, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks, int max_seq_len,
+                   float scale, int partition_size, int q_dtype, int kv_dtype,
+                   const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream);
+
+/*
  * Test hook: materialise the block-table gather.  out [B, max_seq_len, Hkv, D]
  * (elem_bytes per element, bits copied verbatim); rows >= seq_lens[b] are zero.
  * Bit-exact counterpart of np.take(pool, table, axis=0)
@@ -322,7 +369,10 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * key 7: query tokens from which pa_prefill at head dim 64 takes the tiled kernel (0 = the default, 65);
  * key 3 value 6: one q head per wave at head dim 64; key 8: pa_o_proj takes 256 x 256 tiles
  * also where it would take 128 x 128 ones (1 = on); key 9: the longest length bound (tokens) up to which a small
- * pa_decode call runs as one partition per sequence on eight wavefronts (default 1024; 0 = never). */
+ * pa_decode call runs as one partition per sequence on eight wavefronts (default 1024; 0 = never); key 10: what
+ * pa_decode_step lets ride on its decode and projection launches (0 = the new row and the merge, the default; 1 = neither:
+ * the separate launches; 2 = the new row only; 3 = the merge only); key 11: tokens per partition that the smallest
+ * fixed-partition decode calls take instead of the caller's larger ones (default 256; 0 = the caller's always). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

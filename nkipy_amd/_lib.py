@@ -27,6 +27,16 @@ class QTransformStruct(ctypes.Structure):
                 ("rope_max_pos", c_int), ("norm_eps", c_float)]
 
 
+class NewKvStruct(ctypes.Structure):
+    """`pa_new_kv` of include/paged_attn.h."""
+    _fields_ = [("xk", c_void_p), ("xv", c_void_p), ("k_norm_weight", c_void_p), ("query_lens", c_void_p)]
+
+
+class OutProjStruct(ctypes.Structure):
+    """`pa_out_proj` of include/paged_attn.h."""
+    _fields_ = [("o_weight", c_void_p), ("o_bias", c_void_p), ("out", c_void_p), ("N", c_int)]
+
+
 SIGNATURES = {
     "pa_version": (c_int, []),
     "pa_last_error": (ctypes.c_char_p, []),
@@ -42,6 +52,8 @@ SIGNATURES = {
     "pa_o_proj": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
     "pa_o_proj_ws": (c_int, [c_void_p] * 5 + [c_size_t] + [c_int] * 4 + [c_void_p]),
     "pa_o_proj_workspace_bytes": (c_size_t, [c_int] * 3),
+    "pa_decode_step_workspace_bytes": (c_size_t, [c_int] * 10),
+    "pa_decode_step": (c_int, [c_void_p] * 11 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "pa_gather_kv": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_void_p]),
     "pa_kv_write": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_void_p]),
     "pa_qk_norm_rope_kv_write": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 2 + [c_int] + [c_void_p] * 7 + [c_int] * 9 + [c_void_p]),

@@ -1,5 +1,6 @@
 // extern "C" surface of libpaged_attn.so: argument validation on the host,
 // kernel selection, launch.  See include/paged_attn.h for the contract.
+#include <algorithm>
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
@@ -56,6 +57,8 @@ static std::atomic<int> g_d64_tiled_from{PA_VERIFY_MAX_TOKENS + 1};   // query t
 // Small decode calls whose length bound is at most this many tokens run as ONE partition per sequence on eight waves
 // (the waves merge through LDS, so there is no split-K workspace and no merge launch): debug switch 9, 0 = never.
 static std::atomic<int> g_decode_single_max{1024};
+static std::atomic<int> g_decode_fine{256};     // tokens per partition of the smallest fixed-partition calls (0: the caller's always)
+static std::atomic<int> g_step_fusion{0};       // pa_decode_step, debug switch 10
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 // Events come from a free list that pa_profile_collect refills, so that a timed pass which follows a collected
@@ -160,6 +163,8 @@ int pa_debug_set(int key, int value) {
   if (key == 7) { g_d64_tiled_from = value > 0 ? value : PA_VERIFY_MAX_TOKENS + 1; return 0; }
   if (key == 8) { o_proj_debug_force_large(value); return 0; }
   if (key == 9) { g_decode_single_max = value < 0 ? 0 : value; return 0; }
+  if (key == 10) { g_step_fusion = value; return 0; }
+  if (key == 11) { g_decode_fine = value < 0 ? 0 : value & ~31; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -228,19 +233,37 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
 // The balanced kernel pays a fixed price for its schedule (a scan of the lengths in every workgroup, partials and a
 // merge launch whatever the sizes: 11 us for the smallest call), the fixed-partition kernel merges a sequence's
 // waves inside the workgroup and needs the merge launch only past one partition, but leaves the device unevenly
-// filled at scale.  Per call replayed from a HIP graph (B x context, 32 / 8 heads of 128, bf16, us, fixed against
-// balanced): 1 x 256 5.7 / 11.4, 16 x 256 5.9 / 12.7, 16 x 1 K 16.6 / 20.7, 64 x 1 K 45.7 / 50.8, 4 x 8 K 30.7 /
-// 31.3; 16 x 8 K 114 / 92, 64 x 2 K 109 / 91.  So calls of at most four partitions per sequence that can touch at
+// filled at scale.  Measured where it matters, inside a decode step of eight attention layers with a pool each (so
+// that every layer's K and V come from HBM, not from a cache the previous call warmed), us per layer with fixed
+// partitions of 512 / balanced (B x context, 32 / 8 heads of 128, bf16): 1 x 1 K 25.8 / 29.2, 1 x 4 K 28.3 / 31.7,
+// 4 x 2 K 28.5 / 35.9, 8 x 1 K 29.6 / 36.0, 4 x 4 K 33.1 / 38.4, 8 x 2 K 40.1 / 39.6, 8 x 4 K 47.4 / 49.8,
+// 16 x 2 K 59.3 / 49.1, 32 x 1 K 61.8 / 49.6, 16 x 4 K 78.6 / 77.6.  (Timed call by call on one pool, which then sits
+// in the last-level cache, the fixed partitions stay ahead up to four times these sizes; a serving step is not that.)
+// 16 x 1 K 41.2 / 38.8, 8 x 600 29.1 / 30.6, 32 x 600 47.4 / 42.8: what decides is the number of sequences, not the
+// bytes.  So calls of at most 80 (sequence, kv head) pairs and at most eight partitions per sequence that can touch at
 // most this many bytes of K and V, by the caller's bound on the lengths, take the fixed partitions when nothing
-// needs the balanced kernel (with more partitions per sequence the two are level at best: 8 x 4 K inside a layer
-// step 52.5 / 49.7).
-constexpr long kDecodeSmallCallBytes = 288L << 20;
-static bool decode_small_call(const DecodeParams& p, int kv_dtype) {
+// needs the balanced kernel.
+constexpr long kDecodeSmallCallBytes = 160L << 20;
+constexpr int kDecodeSmallCallPartitions = 8;
+constexpr long kDecodeSmallCallPairs = 80;
+static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts = kDecodeSmallCallPartitions) {
   const long esz = kv_dtype == PA_FP8_E4M3FN ? 1 : (kv_dtype == PA_BF16 ? 2 : 4);
   if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
-  if (num_partitions_for(p.max_seq_len, p.partition_size) > 4) return false;
+  if (num_partitions_for(p.max_seq_len, p.partition_size) > max_parts) return false;
+  if ((long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16) > kDecodeSmallCallPairs) return false;
   const double bytes = 2.0 * p.B * (double)p.max_seq_len * p.Hkv * p.D * esz;
   return bytes <= (double)kDecodeSmallCallBytes;
+}
+// Partitions of 256 tokens instead of the caller's (larger) ones when those would give the device very few
+// workgroups (a single sequence, mostly): same units, partitions of 512 / of 256: 1 x 1 K 25.8 / 22.9, 1 x 4 K
+// 28.3 / 27.9; with more workgroups to begin with the finer ones cost more than they bring (8 x 1 K 29.6 / 32.4).
+static int decode_fine_partition(const DecodeParams& p) {
+  const int kFine = g_decode_fine.load();
+  if (kFine <= 0 || p.partition_size <= kFine || p.max_seq_len <= kFine) return p.partition_size;
+  const long slots = (long)p.Hkv * ((p.Hq / p.Hkv + 15) / 16);      // workgroups per sequence and partition
+  if (p.B * slots * num_partitions_for(p.max_seq_len, p.partition_size) > 64) return p.partition_size;
+  if (num_partitions_for(p.max_seq_len, kFine) > 16) return p.partition_size;
+  return kFine;
 }
 static int decode_kind(const DecodeParams& p, int q_dtype, int kv_dtype, bool needs_balanced = false) {
   const int impl = g_decode_impl.load();
@@ -260,17 +283,18 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
   p.block_size = block_size; p.block_shift = ilog2_exact(block_size);
   p.max_seq_len = max_seq_len; p.partition_size = partition_size;
   const int kind = decode_kind(p, q_dtype, kv_dtype);
-  const int np = num_partitions_for(max_seq_len, partition_size);
+  int np = num_partitions_for(max_seq_len, partition_size);
+  if (kind == 2 && max_seq_len > 0) np = std::max(np, num_partitions_for(max_seq_len, decode_fine_partition(p)));
   const size_t fixed = np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
   if (max_seq_len <= 0) {
     // no bound given: pa_decode then takes the table capacity, which this function is not told.  The answer covers
-    // every kernel that call can pick: the balanced one, or fixed partitions, which are chosen for at most four
+    // every kernel that call can pick: the balanced one, or fixed partitions, which are chosen for at most eight
     // (the scalar kernel's partitions are not bounded that way: its callers give the bound)
     if (kind == 1 || kind < 0) return 0;
     plan_decode_balanced(p, current_num_cus());
     const size_t balanced = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
-    const size_t four = (size_t)B * Hq * 4 * ((size_t)D + 2) * sizeof(float);
-    return four > balanced ? four : balanced;
+    const size_t most = (size_t)B * Hq * 16 * ((size_t)D + 2) * sizeof(float);      // (up to sixteen of the finer partitions)
+    return most > balanced ? most : balanced;
   }
   if (kind == 1 || kind < 0) return fixed;
   plan_decode_balanced(p, current_num_cus());
@@ -281,35 +305,43 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
   return fixed > balanced ? fixed : balanced;
 }
 
-int pa_decode(const void* q, const void* k_cache, const void* v_cache,
-              const float* k_scale, const float* v_scale,
-              const int32_t* block_tables, const int32_t* seq_lens,
-              void* out, void* workspace, size_t workspace_bytes,
-              int B, int Hq, int Hkv, int D, int block_size,
-              int max_blocks_per_seq, int num_blocks, int max_seq_len,
-              float scale, int partition_size, int q_dtype, int kv_dtype,
-              const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream) {
-  tl_error[0] = 0;
-  if (sliding_window < 0) return fail_arg("pa_decode: sliding_window=%d must be >= 0 (0 = none)", sliding_window);
-  if (B < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("pa_decode: bad sizes B=%d Hq=%d Hkv=%d D=%d", B, Hq, Hkv, D);
-  if (Hq % Hkv) return fail_arg("pa_decode: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+// pa_decode in two halves, so that pa_decode_step can decide between them what rides on the decode launch:
+// plan_decode validates and picks the kernel, run_decode sizes the workspace and launches.
+struct DecodePlan {
+  DecodeParams p;
+  int kind;                 // 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced
+  int waves;                // fixed partitions: waves per workgroup (0: the kernel's default)
+  int caller_partition;     // the caller's partition size (p.partition_size may be a finer one)
+  int q_dtype, kv_dtype;
+};
+
+static int plan_decode(const char* who, DecodePlan& pl, const void* q, const void* k_cache, const void* v_cache,
+                       const float* k_scale, const float* v_scale, const int32_t* block_tables, const int32_t* seq_lens,
+                       void* out, bool out_required, int B, int Hq, int Hkv, int D, int block_size,
+                       int max_blocks_per_seq, int num_blocks, int max_seq_len, float scale, int partition_size,
+                       int q_dtype, int kv_dtype, const float* sinks, int sliding_window,
+                       const pa_q_transform* q_transform) {
+  if (sliding_window < 0) return fail_arg("%s: sliding_window=%d must be >= 0 (0 = none)", who, sliding_window);
+  if (B < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("%s: bad sizes B=%d Hq=%d Hkv=%d D=%d", who, B, Hq, Hkv, D);
+  if (Hq % Hkv) return fail_arg("%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0)
-    return fail_arg("pa_decode: bad paging sizes block_size=%d max_blocks_per_seq=%d num_blocks=%d",
+    return fail_arg("%s: bad paging sizes block_size=%d max_blocks_per_seq=%d num_blocks=%d", who,
                     block_size, max_blocks_per_seq, num_blocks);
-  if (partition_size <= 0) return fail_arg("pa_decode: partition_size=%d must be positive", partition_size);
+  if (partition_size <= 0) return fail_arg("%s: partition_size=%d must be positive", who, partition_size);
   if (!(q_dtype == PA_F32 && kv_dtype == PA_F32) && !(q_dtype == PA_BF16 && kv_dtype == PA_BF16) &&
       !(q_dtype == PA_BF16 && kv_dtype == PA_FP8_E4M3FN))
-    return fail_arg("pa_decode: unsupported dtype pair q=%d kv=%d", q_dtype, kv_dtype);
-  if (D != 32 && D != 64 && D != 128 && D != 256) return fail_arg("pa_decode: head_dim %d not in {32,64,128,256}", D);
+    return fail_arg("%s: unsupported dtype pair q=%d kv=%d", who, q_dtype, kv_dtype);
+  if (D != 32 && D != 64 && D != 128 && D != 256) return fail_arg("%s: head_dim %d not in {32,64,128,256}", who, D);
   if (B == 0) return 0;
-  if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || !out) return fail_arg("pa_decode: null pointer argument");
-  if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("pa_decode: fp8 KV needs k_scale and v_scale");
+  if (!q || !k_cache || !v_cache || !block_tables || !seq_lens || (out_required && !out))
+    return fail_arg("%s: null pointer argument", who);
+  if (kv_dtype == PA_FP8_E4M3FN && (!k_scale || !v_scale)) return fail_arg("%s: fp8 KV needs k_scale and v_scale", who);
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
-    return fail_arg("pa_decode: q, k_cache, v_cache and out must be 16-byte aligned");
+    return fail_arg("%s: q, k_cache, v_cache and out must be 16-byte aligned", who);
   const long cap = (long)max_blocks_per_seq * block_size;
   if (max_seq_len <= 0 || max_seq_len > cap) max_seq_len = (int)(cap > 0x7fffffffL ? 0x7fffffffL : cap);
 
-  DecodeParams p;
+  DecodeParams& p = pl.p;
   memset(&p, 0, sizeof(p));
   p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
   p.block_tables = block_tables; p.seq_lens = seq_lens; p.out = out;
@@ -321,64 +353,108 @@ int pa_decode(const void* q, const void* k_cache, const void* v_cache,
   p.max_seq_len = max_seq_len;
   p.scale_log2e = scale * kLog2e;
   p.head_major = g_head_major.load();
-  if (p.num_partitions > 65535 || B > 65535) return fail_arg("pa_decode: grid too large (partitions=%d B=%d)", p.num_partitions, B);
-  hipStream_t s = (hipStream_t)stream;
+  pl.caller_partition = partition_size;
+  pl.q_dtype = q_dtype; pl.kv_dtype = kv_dtype;
+  if (p.num_partitions > 65535 || B > 65535) return fail_arg("%s: grid too large (partitions=%d B=%d)", who, p.num_partitions, B);
   // kernel choice: 0 automatic, 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced
-  const int kind = decode_kind(p, q_dtype, kv_dtype, sinks != nullptr || sliding_window > 0);
-  if (kind < 0) return fail_arg("pa_decode: MFMA kernel forced but shape unsupported");
-  if (kind == 2 && partition_size % 32) return fail_arg("pa_decode: the fixed-partition MFMA kernel needs partition_size %% 32 == 0");
+  const int kind = pl.kind = decode_kind(p, q_dtype, kv_dtype, sinks != nullptr || sliding_window > 0);
+  if (kind < 0) return fail_arg("%s: MFMA kernel forced but shape unsupported", who);
+  if (kind == 2 && partition_size % 32) return fail_arg("%s: the fixed-partition MFMA kernel needs partition_size %% 32 == 0", who);
   // a small call of short contexts: the whole context as one partition on eight waves, which merge through LDS, so
   // that there is no merge launch.  Per call replayed from a HIP graph (32 / 8 heads of 128, bf16, us, two partitions of
   // 512 + merge against one partition): contexts of 350-700 tokens B = 1 10.1 / 9.7, B = 16 12.3 / 11.1, B = 64
   // 31.3 / 26.6; 512-1024 tokens B = 8 10.4 / 12.0 (the longer chain per wave costs more than the launch), B = 64
   // 36.7 / 34.7.  So: bounds up to three quarters of the limit always, up to the limit when the grid is large anyway.
-  int waves = g_decode_waves.load();
+  pl.waves = g_decode_waves.load();
   const int single_max = g_decode_single_max.load();
-  if (kind == 2 && waves == 0 && g_decode_impl.load() == 0 && p.num_partitions > 1 && Hq / Hkv <= 8 &&
-      (max_seq_len <= single_max - single_max / 4 || (max_seq_len <= single_max && (long)B * Hkv >= 256))) {
-    p.partition_size = (max_seq_len + 31) & ~31;
-    p.num_partitions = 1;
-    waves = 8;
+  if (kind == 2 && pl.waves == 0 && g_decode_impl.load() == 0 && p.num_partitions > 1) {
+    if (Hq / Hkv <= 8 &&
+        (max_seq_len <= single_max - single_max / 4 || (max_seq_len <= single_max && (long)B * Hkv >= 256))) {
+      p.partition_size = (max_seq_len + 31) & ~31;
+      p.num_partitions = 1;
+      pl.waves = 8;
+    } else {
+      p.partition_size = decode_fine_partition(p);
+      p.num_partitions = num_partitions_for(max_seq_len, p.partition_size);
+    }
   }
   if ((sinks || sliding_window > 0) && kind != 3)
-    return fail_arg("pa_decode: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
-                    "head_dim 64 or 128, block_size a power of two >= 16)");
+    return fail_arg("%s: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
+                    "head_dim 64 or 128, block_size a power of two >= 16)", who);
   p.sinks = sinks; p.window = sliding_window;
-  if (take_q_transform("pa_decode", q_transform, kind != 1, p.qt)) return -1;
-  if (!aligned16(workspace)) return fail_arg("pa_decode: workspace must be 16-byte aligned");
-  if (kind == 3) {
+  if (take_q_transform(who, q_transform, kind != 1, p.qt)) return -1;
+  return 0;
+}
+
+// Launches the planned decode.  leave_partials (fixed partitions with more than one partition only): the merge
+// launch is left out, the caller's consumer reads p.ws_out / p.ws_ml.  Returns the bytes of workspace used in *used.
+static int run_decode(const char* who, DecodePlan& pl, void* workspace, size_t workspace_bytes, bool leave_partials,
+                      size_t* used, hipStream_t s) {
+  DecodeParams& p = pl.p;
+  const int B = p.B, Hq = p.Hq, D = p.D;
+  if (used) *used = 0;
+  if (!aligned16(workspace)) return fail_arg("%s: workspace must be 16-byte aligned", who);
+  if (pl.kind == 3) {
     plan_decode_balanced(p, current_num_cus());
-    p.bal_lockstep = lockstep_for(kv_dtype, p.bal_ns);
+    p.bal_lockstep = lockstep_for(pl.kv_dtype, p.bal_ns);
     const size_t need = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
     if (!workspace || workspace_bytes < need)
-      return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+      return fail_arg("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+    if (used) *used = need;
     p.ws_out = (float*)workspace;
     p.ws_ml = p.ws_out + (size_t)Hq * ((size_t)B + p.bal_gv) * D;
     p.ws_start = (int32_t*)(p.ws_ml + (size_t)Hq * ((size_t)B + p.bal_gv) * 2);
     profile_begin(s);
-    hipError_t e = launch_decode_balanced(p, kv_dtype, s);
+    hipError_t e = launch_decode_balanced(p, pl.kv_dtype, s);
     profile_end(s);
-    if (e != hipSuccess) return check_hip(e, "pa_decode launch");
+    if (e != hipSuccess) return check_hip(e, "decode launch");
     e = launch_decode_balanced_reduce(p, s);
-    return check_hip(e, "pa_decode reduce launch");
+    return check_hip(e, "decode reduce launch");
   }
   if (p.num_partitions > 1) {
-    const size_t need = (size_t)B * Hq * p.num_partitions * ((size_t)D + 2) * sizeof(float);
-    if (!workspace || workspace_bytes < need)
-      return fail_arg("pa_decode: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    p.ws_out = (float*)workspace;
-    p.ws_ml = p.ws_out + (size_t)B * Hq * p.num_partitions * D;
+    size_t need = (size_t)B * Hq * p.num_partitions * ((size_t)D + 2) * sizeof(float);
+    if ((!workspace || workspace_bytes < need) && p.partition_size != pl.caller_partition) {
+      // a workspace sized for the caller's partitions only: those, then
+      p.partition_size = pl.caller_partition;
+      p.num_partitions = num_partitions_for(p.max_seq_len, p.partition_size);
+      need = (size_t)B * Hq * p.num_partitions * ((size_t)D + 2) * sizeof(float);
+    }
+    if (p.num_partitions > 1) {
+      if (!workspace || workspace_bytes < need)
+        return fail_arg("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+      if (used) *used = need;
+      p.ws_out = (float*)workspace;
+      p.ws_ml = p.ws_out + (size_t)B * Hq * p.num_partitions * D;
+    }
   }
   profile_begin(s);
-  hipError_t e = kind == 2 ? launch_decode_mfma(p, kv_dtype, waves, s)
-                           : launch_decode_generic(p, q_dtype, kv_dtype, s);
+  hipError_t e = pl.kind == 2 ? launch_decode_mfma(p, pl.kv_dtype, pl.waves, s)
+                              : launch_decode_generic(p, pl.q_dtype, pl.kv_dtype, s);
   profile_end(s);
-  if (e != hipSuccess) return check_hip(e, "pa_decode launch");
-  if (p.num_partitions > 1) {
-    e = launch_decode_reduce(p, q_dtype, s);
-    if (e != hipSuccess) return check_hip(e, "pa_decode reduce launch");
+  if (e != hipSuccess) return check_hip(e, "decode launch");
+  if (p.num_partitions > 1 && !leave_partials) {
+    e = launch_decode_reduce(p, pl.q_dtype, s);
+    if (e != hipSuccess) return check_hip(e, "decode reduce launch");
   }
   return 0;
+}
+
+int pa_decode(const void* q, const void* k_cache, const void* v_cache,
+              const float* k_scale, const float* v_scale,
+              const int32_t* block_tables, const int32_t* seq_lens,
+              void* out, void* workspace, size_t workspace_bytes,
+              int B, int Hq, int Hkv, int D, int block_size,
+              int max_blocks_per_seq, int num_blocks, int max_seq_len,
+              float scale, int partition_size, int q_dtype, int kv_dtype,
+              const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream) {
+  tl_error[0] = 0;
+  DecodePlan pl;
+  if (int rc = plan_decode("pa_decode", pl, q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, out, true, B, Hq,
+                           Hkv, D, block_size, max_blocks_per_seq, num_blocks, max_seq_len, scale, partition_size, q_dtype,
+                           kv_dtype, sinks, sliding_window, q_transform))
+    return rc;
+  if (B == 0) return 0;
+  return run_decode("pa_decode", pl, workspace, workspace_bytes, false, nullptr, (hipStream_t)stream);
 }
 
 // ---- pa_decode for callers that cannot allocate ------------------------------------------------
@@ -482,7 +558,7 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     f.partition_size = 512;
     f.num_partitions = num_partitions_for(f.max_seq_len, f.partition_size);
     const size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
-    if (decode_small_call(f, kv_dtype) && (need_f == 0 || (workspace && workspace_bytes >= need_f))) {
+    if (decode_small_call(f, kv_dtype, 4) && (need_f == 0 || (workspace && workspace_bytes >= need_f))) {
       f.head_major = g_head_major.load();
       f.ws_out = (float*)workspace;
       f.ws_ml = f.ws_out + (size_t)B * Hq * Tc * f.num_partitions * D;
@@ -799,6 +875,125 @@ int pa_o_proj_ws(const void* x, const void* w, const void* bias, void* out, void
   hipError_t e = launch_o_proj(p, s);
   profile_end(s);
   return check_hip(e, "pa_o_proj launch");
+}
+
+// ---- one decode step of an attention layer in one call -------------------------------------------
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+size_t pa_decode_step_workspace_bytes(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len, int partition_size,
+                                      int N, int q_dtype, int kv_dtype) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0 || partition_size <= 0 || N < 0) return 0;
+  const size_t dec = pa_decode_workspace_bytes_for(B, Hq, Hkv, D, block_size, max_seq_len, partition_size, q_dtype, kv_dtype);
+  const size_t proj = N > 0 ? pa_o_proj_workspace_bytes(B, Hq * D, N) : 0;
+  return align256(dec) + align256(proj) + align256((size_t)B * Hq * D * 4) + 256;
+}
+
+int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* v_cache, float* k_scale, float* v_scale,
+                   const int32_t* block_tables, const int32_t* seq_lens, void* attn_out, const pa_out_proj* proj,
+                   void* workspace, size_t workspace_bytes,
+                   int B, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks, int max_seq_len,
+                   float scale, int partition_size, int q_dtype, int kv_dtype,
+                   const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream) {
+  tl_error[0] = 0;
+  const char* who = "pa_decode_step";
+  DecodePlan pl;
+  if (int rc = plan_decode(who, pl, q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, attn_out, proj == nullptr,
+                           B, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks, max_seq_len, scale, partition_size,
+                           q_dtype, kv_dtype, sinks, sliding_window, q_transform))
+    return rc;
+  if (!new_kv) return fail_arg("%s: new_kv is required (pa_decode is the call without a cache update)", who);
+  if (B == 0) return 0;
+  if (!new_kv->xk || !new_kv->xv || !new_kv->query_lens) return fail_arg("%s: new_kv needs xk, xv and query_lens", who);
+  if (!aligned16(new_kv->xk) || !aligned16(new_kv->xv) || !aligned16(new_kv->k_norm_weight))
+    return fail_arg("%s: xk, xv and k_norm_weight must be 16-byte aligned", who);
+  if (new_kv->k_norm_weight && !q_transform)
+    return fail_arg("%s: k_norm_weight comes with q_transform (the norm and rotation are applied to Q and K alike)", who);
+  const int K = Hq * D;
+  int N = 0;
+  if (proj) {
+    N = proj->N;
+    if (!proj->o_weight || !proj->out) return fail_arg("%s: out_proj needs o_weight and out", who);
+    if (q_dtype != PA_BF16) return fail_arg("%s: the output projection is bf16 only", who);
+    if (N <= 0 || N % 8) return fail_arg("%s: N=%d must be a positive multiple of 8", who, N);
+    if (K % 64) return fail_arg("%s: Hq * head_dim = %d must be a multiple of 64", who, K);
+    if ((long)N * 2 * 64 > 0xffffffffL || (long)K * 2 * 256 > 0xffffffffL)
+      return fail_arg("%s: row of %d (K) or %d (N) elements too long for 32-bit tile offsets", who, K, N);
+    if (!aligned16(proj->o_weight) || !aligned16(proj->o_bias) || !aligned16(proj->out))
+      return fail_arg("%s: o_weight, o_bias and out must be 16-byte aligned", who);
+  }
+  if (!aligned16(workspace)) return fail_arg("%s: workspace must be 16-byte aligned", who);
+  hipStream_t s = (hipStream_t)stream;
+  DecodeParams& p = pl.p;
+  const int fusion = g_step_fusion.load();
+
+  // the cache update: on the decode launch where its kernel takes the row, else a launch of its own in front
+  const bool fused_row = pl.kind == 2 && decode_new_row_supported(p, q_dtype, kv_dtype) && fusion != 1 && fusion != 3;
+  if (fused_row) {
+    p.new_k = new_kv->xk; p.new_v = new_kv->xv; p.new_lens = new_kv->query_lens;
+    if (q_transform) {
+      p.new_kt = p.qt;
+      p.new_kt.norm_weight = (const uint16_t*)new_kv->k_norm_weight;
+    }
+  }
+  if (!fused_row) {
+    int rc;
+    if (q_transform)
+      rc = pa_qk_norm_rope_kv_write(nullptr, new_kv->xk, new_kv->xv, nullptr, nullptr, new_kv->k_norm_weight,
+                                    q_transform->norm_eps, q_transform->rope_cos, q_transform->rope_sin,
+                                    q_transform->rope_max_pos, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens,
+                                    new_kv->query_lens, B, 1, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks,
+                                    kv_dtype, stream);
+    else
+      rc = pa_kv_write(new_kv->xk, new_kv->xv, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens,
+                       new_kv->query_lens, B, 1, Hkv, D, block_size, max_blocks_per_seq, num_blocks, kv_dtype, stream);
+    if (rc) return rc;
+  }
+
+  // workspace, from its end: the attention output when the caller wants none, the projection's K-range partials;
+  // the decode launch gets what is in front of them
+  char* ws = (char*)workspace;
+  size_t avail = workspace ? workspace_bytes & ~(size_t)255 : 0;
+  const size_t esz = q_dtype == PA_F32 ? 4 : 2;
+  void* attn = attn_out;
+  if (!attn) {
+    const size_t need = align256((size_t)B * Hq * D * esz);
+    if (avail < need) return fail_arg("%s: workspace of %zu bytes too small (pa_decode_step_workspace_bytes)", who, workspace_bytes);
+    avail -= need;
+    attn = ws + avail;
+    p.out = attn;
+  }
+  int splits = 1;
+  float* proj_ws = nullptr;
+  if (proj) {
+    const size_t per_split = (size_t)B * N * sizeof(float);
+    int want = o_proj_splits(B, K, N);
+    if (align256((size_t)want * per_split) > avail) want = (int)(avail / per_split);
+    if (want > 1) {
+      splits = want;
+      avail -= align256((size_t)splits * per_split);
+      proj_ws = (float*)(ws + avail);
+    }
+  }
+  // the merge of the decode partitions on the projection's load of its rows, where both kernels are the small-call ones
+  const bool merge_on_load = proj && !attn_out && pl.kind == 2 && p.num_partitions > 1 && fusion != 1 && fusion != 2 &&
+                             q_dtype == PA_BF16 && o_proj_takes_partials(B, K, D, splits, proj_ws != nullptr);
+  if (int rc = run_decode(who, pl, ws, avail, merge_on_load, nullptr, s)) return rc;
+  if (!proj) return 0;
+
+  OProjParams o;
+  memset(&o, 0, sizeof(o));
+  o.w = proj->o_weight; o.bias = proj->o_bias; o.out = proj->out; o.M = B; o.K = K; o.N = N;
+  o.splits = splits; o.ws = proj_ws;
+  if (merge_on_load && p.num_partitions > 1) {
+    o.part_o = p.ws_out; o.part_ml = p.ws_ml; o.part_seq_lens = seq_lens;
+    o.part_np = p.num_partitions; o.part_size = p.partition_size; o.part_max_seq_len = p.max_seq_len; o.part_D = D;
+  } else {
+    o.x = attn;
+  }
+  profile_begin(s);
+  hipError_t e = launch_o_proj(o, s);
+  profile_end(s);
+  return check_hip(e, "pa_decode_step projection launch");
 }
 
 int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,

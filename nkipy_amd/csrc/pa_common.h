@@ -201,10 +201,21 @@ struct DecodeParams {
   int bal_hsw, bal_ns, bal_gv;  // balanced schedule: head slots and chunks per workgroup, total chunks
   int bal_lockstep;         // keep the head waves of a workgroup on the same tile with a barrier
   QTransform qt;            // balanced schedule only: Q rows are normed and rotated as they are loaded
+  // Fixed-partition kernels, bf16 pools: the step's new token handed over with the call instead of written to the
+  // pool by a launch of its own.  Row (b, kv head) of new_k / new_v [B, Hkv, D] bf16 is token seq_lens[b] - 1 of
+  // sequence b (the reference's cache update, examples/models/qwen3/kernels/attention.py:100-106): the wave that
+  // reaches that token attends to it from registers, and one wave per (sequence, kv head) stores it in the pool.
+  // new_kt is the K half of the pre-attention transform (its norm weight is K's; cos null: rows go in as given).
+  // Sequences with new_lens[b] == 0 take no new token (null: every sequence takes one).
+  const void* new_k;
+  const void* new_v;
+  const int32_t* new_lens;
+  QTransform new_kt;
 };
 
 hipError_t launch_decode_generic(const DecodeParams& p, int q_dtype, int kv_dtype, hipStream_t s);
 hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hipStream_t s);
+bool decode_new_row_supported(const DecodeParams& p, int q_dtype, int kv_dtype);   // shapes whose fixed-partition kernels take p.new_k
 bool decode_mfma_supported(const DecodeParams& p, int q_dtype, int kv_dtype);
 hipError_t launch_decode_reduce(const DecodeParams& p, int q_dtype, hipStream_t s);
 void plan_decode_balanced(DecodeParams& p, int num_cus);
@@ -283,9 +294,17 @@ struct OProjParams {
   int M, K, N;
   float* ws;                // split form: [splits, M, N] float32 partial products, or null
   int splits;               // K ranges summed by a second kernel (1: none); o_proj_splits() or less
+  // The resident few-rows form can take its x rows from the split-K partials of a fixed-partition decode launch
+  // instead of from memory (x null): row b of x is sequence b's attention output [Hq * D], merged from the
+  // sequence's partitions while the tile is formed, with the arithmetic of decode_reduce_kernel.
+  const float* part_o;      // [M, Hq, np, D] normalised partial outputs
+  const float* part_ml;     // [M, Hq, np, 2] (max, sum) of each partial
+  const int32_t* part_seq_lens;   // [M] context lengths (clamped to part_max_seq_len as the decode launch did)
+  int part_np, part_size, part_max_seq_len, part_D;
 };
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s);
 int o_proj_splits(int M, int K, int N);     // K ranges the few-rows forms would like to spread over more workgroups
+bool o_proj_takes_partials(int M, int K, int D, int splits, bool have_ws);   // launch_o_proj can merge decode partials on its x load
 void o_proj_debug_force_large(int on);      // debug: 256 x 256 tiles also where the 128 x 128 form would be taken
 
 hipError_t launch_gather(const void* cache, const int32_t* tables, const int32_t* seq_lens, void* out,

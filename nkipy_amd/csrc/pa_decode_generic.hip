@@ -124,6 +124,9 @@ __global__ __launch_bounds__(kGenericThreads) void decode_generic_kernel(DecodeP
 // such a row may have seen no key in a partition (m = -inf, l = 0) or be padding (zeros).
 template <typename QT>
 __global__ void decode_reduce_kernel(DecodeParams p) {
+  // no contraction of the sums below into multiply-adds of the compiler's choosing: the projection's merge-on-load
+  // (o_proj_resident_kernel) repeats this arithmetic and must round where this kernel rounds
+#pragma clang fp contract(off)
   const int vr = blockIdx.x, b = blockIdx.y;
   const bool multi = p.query_lens != nullptr;
   const int rows_total = p.Hq * (multi ? p.T : 1);
@@ -170,12 +173,12 @@ __global__ void decode_reduce_kernel(DecodeParams p) {
       if (i < np) {
         const float w = l_[i] * exp2f(m_[i] - m_ref);
         lt += w;
-        ot += w * (d == d0 ? o_[i] : p.ws_out[(base + i) * p.D + d]);
+        ot = __builtin_fmaf(w, d == d0 ? o_[i] : p.ws_out[(base + i) * p.D + d], ot);
       }
     for (int i = PRE; i < np; ++i) {
       const float w = p.ws_ml[(base + i) * 2 + 1] * exp2f(p.ws_ml[(base + i) * 2] - m_ref);
       lt += w;
-      ot += w * p.ws_out[(base + i) * p.D + d];
+      ot = __builtin_fmaf(w, p.ws_out[(base + i) * p.D + d], ot);    // (the projection's merge-on-load repeats this arithmetic)
     }
     Store<QT>::put(p.out, out_at + d, lt > 0.f ? ot / lt : 0.f);
   }

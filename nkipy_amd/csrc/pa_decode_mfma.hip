@@ -122,8 +122,14 @@ struct QOperandLayout {
   static constexpr int lane_xor(int bit) { return FP8 ? (bit == 2 ? 16 : bit == 4 ? 32 : 0) : (bit == 1 ? 16 : bit == 2 ? 32 : 0); }
 };
 
-template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false, bool SV = false>
+// NEWROW (decode, bf16 pools, fixed partitions): the sequence's newest token is not in the pool yet but comes with
+// the call (p.new_k / p.new_v).  The wave whose tile holds it (`take_new_row`) keeps the lane's pieces of the row in
+// registers and puts them in the place of what the tile loads brought for that token (and for the rows behind it,
+// which the loads redirect to it), so the scores and the output are those of a pool that already held the row; the
+// same wave stores the row in the pool for the steps to come.
+template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false, bool SV = false, bool NEWROW = false>
 struct DecodeWave {
+  static_assert(!NEWROW || (!FP8 && !MULTI && R == 1 && !LEAN && !SV), "the new-row form is plain bf16 decode");
   using KT = KTile<D, FP8>;
   using VT = VTile<D, FP8>;
   static constexpr int VEC = VT::VEC, KLD = KT::KLD, VW = VT::VW;
@@ -153,6 +159,12 @@ struct DecodeWave {
   bf16x8_t pf[R];            // P^T fragments of the current tile
   f32x4_t oacc[R][VEC];
   float m_run[R], l_run[R];
+  // NEWROW: chunk 4 s + g of the new K row (the lane's operand piece in k-step s, as transformed), the lane's
+  // VEC elements of the new V row, the tile that holds the token (-1: none for this wave) and, while that tile is
+  // worked on, the token's index in it (tile rows from there on are the new row)
+  uint4 knew[NEWROW ? KSTEPS : 1];
+  uint32_t vnew[NEWROW ? VW : 1];
+  int new_t0, new_from;
 
   __device__ __forceinline__ DecodeWave(const DecodeParams& p_, int head_slot, int lane, uint4* qlds_ = nullptr)
       : p(p_), qlds(qlds_), qlane(lane) {
@@ -171,6 +183,42 @@ struct DecodeWave {
     row_stride = (long)p.Hkv * D * ESZ;
     kbase = (const char*)p.k_cache + (long)hk * D * ESZ;
     vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
+    new_t0 = -1;
+    new_from = 64;
+  }
+
+  // NEWROW: this wave is the one whose tiles include token `pos` (= ctx - 1, the step's new token, whose rows begin()
+  // has put into knew / vnew): from now on the tile that holds it is patched.  The same wave, if it is the first
+  // of the kv head's rows, stores both rows in the pool when its tiles are done (store_new_row: K by the lanes
+  // r = 0, chunks 4 s + g; V by the lanes g = 0, elements VEC r ..) -- not before: on this target loads and stores
+  // share one counter and may complete out of order, so with a store pending the compiler waits for every load in
+  // flight wherever it waits for one, and the tile loop would lose its prefetch.
+  __device__ __forceinline__ void adopt_new_row(int pos) { new_t0 = pos & ~31; }
+  __device__ __forceinline__ void store_new_row(int b, int pos) {
+    if (jbase != 0) return;
+    const int blk = p.block_tables[(long)b * p.max_blocks + (pos >> p.block_shift)];
+    if (blk < 0 || blk >= p.num_blocks) return;      // a bad table entry must not redirect the write
+    const long row = (long)blk * p.block_size + (pos & (p.block_size - 1));
+    char* kdst = const_cast<char*>(kbase) + row * row_stride;
+    char* vdst = const_cast<char*>(vbase) + row * row_stride;
+    if (r == 0) {
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) *(uint4*)(kdst + (4 * s + g) * 16) = knew[NEWROW ? s : 0];
+    }
+    if (g == 0) {
+      constexpr int NV = NEWROW ? VW : 1;
+      if (VW == 4) *(uint4*)(vdst + r * (VEC * ESZ)) = make_uint4(vnew[0], vnew[1 % NV], vnew[2 % NV], vnew[3 % NV]);
+      else *(uint2*)(vdst + r * (VEC * ESZ)) = make_uint2(vnew[0], vnew[1 % NV]);
+    }
+  }
+  // NEWROW, a context clamped below its new token (the length bound of the call is shorter than the sequence): the
+  // token is not attended to, only stored, with K transformed at its own position
+  __device__ __forceinline__ void retransform_new_k(int b, int pos) {
+    const uint16_t* krow = (const uint16_t*)p.new_k + ((long)b * p.Hkv + hk) * D;
+    uint4 kraw[NEWROW ? KSTEPS : 1];
+#pragma unroll
+    for (int s = 0; s < (NEWROW ? KSTEPS : 1); ++s) kraw[s] = *(const uint4*)(krow + (4 * s + g) * 8);
+    transform_new_k(kraw, pos);
   }
 
   // MULTI: element offset in q / out of row group rg's row of this lane, its query token and q head
@@ -189,6 +237,16 @@ struct DecodeWave {
   __device__ __forceinline__ void begin(int b, int ctx, int tq = 1) {
     table = p.block_tables + (long)b * p.max_blocks;
     last = ctx - 1;
+    // NEWROW: the new token's rows are requested here, with the Q rows, by every wave (one round trip for all of
+    // them; the wave that turns out to hold the token adopts them, see adopt_new_row), and K is transformed behind Q
+    uint4 kraw[NEWROW ? KSTEPS : 1];
+    if constexpr (NEWROW) {
+      const uint16_t* krow = (const uint16_t*)p.new_k + ((long)b * p.Hkv + hk) * D;
+      const uint16_t* vrow = (const uint16_t*)p.new_v + ((long)b * p.Hkv + hk) * D;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) kraw[s] = *(const uint4*)(krow + (4 * s + g) * 8);
+      VecLoad<VW>::get(vrow + r * VEC, vnew);
+    }
 #pragma unroll
     for (int rg = 0; rg < R; ++rg) {
       bool row_valid = 16 * rg + r < nheads;
@@ -239,6 +297,33 @@ struct DecodeWave {
       for (int e = 0; e < VEC; ++e) oacc[rg][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       m_run[rg] = -INFINITY;
       l_run[rg] = 0.f;
+    }
+    if constexpr (NEWROW) transform_new_k(kraw, last);
+  }
+
+  // NEWROW: the raw K row -> knew, normed and rotated at position pos as the write kernel would (same arithmetic,
+  // same bits; new_kt.cos null: stored as given)
+  __device__ __forceinline__ void transform_new_k(uint4 (&kraw)[NEWROW ? KSTEPS : 1], int pos) {
+    if constexpr (NEWROW) {
+      if (p.new_kt.cos) {
+        float x[KSTEPS][8];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          const uint32_t w[4] = {kraw[s].x, kraw[s].y, kraw[s].z, kraw[s].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[s][2 * j] = bf16_bits_to_float(w[j] & 0xffffu);
+            x[s][2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+          }
+        }
+        q_norm_rope_lane<D / 8, KSTEPS, QOperandLayout<false>>(x, p.new_kt, min(max(pos, 0), p.new_kt.max_pos - 1), g);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+          kraw[s] = make_uint4(pack_bf16x2(x[s][0], x[s][1]), pack_bf16x2(x[s][2], x[s][3]),
+                               pack_bf16x2(x[s][4], x[s][5]), pack_bf16x2(x[s][6], x[s][7]));
+      }
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) knew[s] = kraw[s];
     }
   }
 
@@ -302,6 +387,12 @@ struct DecodeWave {
     if (!SK) {
 #pragma unroll
       for (int d = 0; d < 4; ++d) out[d] = tl.k[u][s][d];
+      if (NEWROW) {
+        const bool nw = 16 * u + krow >= new_from;     // the new token's row, or one redirected to it
+        const uint32_t kn[4] = {knew[NEWROW ? s : 0].x, knew[NEWROW ? s : 0].y, knew[NEWROW ? s : 0].z, knew[NEWROW ? s : 0].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) out[d] = nw ? kn[d] : out[d];
+      }
       return;
     }
 #pragma unroll
@@ -336,6 +427,7 @@ struct DecodeWave {
   __device__ __forceinline__ void scores_softmax(const KT& tl, const VT& vt, int t0, int t_end) {
     f32x4_t sacc[R][2];
     if (LEAN) asm volatile("" : "+v"(qlane));
+    if (NEWROW) new_from = t0 == new_t0 ? last - t0 : 64;
 #pragma unroll
     for (int rg = 0; rg < R; ++rg) sacc[rg][0] = sacc[rg][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     // each Q fragment is fetched once and used for both 16-token halves
@@ -436,8 +528,14 @@ struct DecodeWave {
         const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
         uint32_t w[4];
 #pragma unroll
-        for (int jp = 0; jp < 4; ++jp)
-          w[jp] = __builtin_amdgcn_perm(tl.v[2 * jp + 1][e >> 1], tl.v[2 * jp][e >> 1], sel);
+        for (int jp = 0; jp < 4; ++jp) {
+          uint32_t hi = tl.v[2 * jp + 1][e >> 1], lo = tl.v[2 * jp][e >> 1];
+          if (NEWROW) {      // tile rows 4 j + g from the new token's on are the new row
+            hi = 4 * (2 * jp + 1) + g >= new_from ? vnew[NEWROW ? e >> 1 : 0] : hi;
+            lo = 4 * (2 * jp) + g >= new_from ? vnew[NEWROW ? e >> 1 : 0] : lo;
+          }
+          w[jp] = __builtin_amdgcn_perm(hi, lo, sel);
+        }
 #pragma unroll
         for (int rg = 0; rg < R; ++rg)
           oacc[rg][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w[0], w[1], w[2], w[3]), pf[rg], oacc[rg][e], 0, 0, 0);
@@ -643,9 +741,11 @@ __host__ __device__ __forceinline__ int head_slots_of(const DecodeParams& p) {
 // MULTI (a few query tokens per sequence, small calls of pa_verify): the rows of a kv head are its (query token, q
 // head) pairs, token-major, 16 per wave as in the balanced kernel; a row may see no key in a partition (its causal
 // bound lies before it), which leaves an empty partial (m = -inf, l = 0); rows past the query length come out as zeros.
-template <int D, bool FP8, int NW, bool MULTI = false>
+// NEWROW: the step's new K / V row comes with the call (see DecodeWave); the workgroup of the partition that holds
+// token ctx - 1 attends to it from registers and stores it.
+template <int D, bool FP8, int NW, bool MULTI = false, bool NEWROW = false>
 __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(DecodeParams p) {
-  using W = DecodeWave<D, FP8, MULTI>;
+  using W = DecodeWave<D, FP8, MULTI, 1, false, false, NEWROW>;
   constexpr int VEC = W::VEC;
   constexpr int OSTRIDE = D + 16;   // LDS row stride (floats) for the merge
 
@@ -657,6 +757,12 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
   W w(p, hidx, lane);
   const SeqSpan sp = seq_span(p, b);
   const int ctx = sp.ctx;
+  int new_len = 0;
+  bool takes_new = false;
+  if constexpr (NEWROW) {
+    new_len = min(p.seq_lens[b], p.max_blocks * p.block_size);
+    takes_new = new_len >= 1 && (!p.new_lens || p.new_lens[b] >= 1);
+  }
   // where virtual row vr (q head, or (token, head) pair) of sequence b lies in out
   const int n_rep = p.Hq / p.Hkv;
   auto out_row = [&](int vr) __attribute__((always_inline)) -> uint16_t* {
@@ -675,7 +781,30 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
   const int t_end = min(ctx, t_begin + p.partition_size);
   const int ntiles = (t_end - t_begin + 31) >> 5;
   w.begin(b, ctx, sp.tq);
+  int store_pos = -1;       // NEWROW: this wave stores the new token's rows at this position when its tiles are done
+  if constexpr (NEWROW) {
+    // the new token is number seq_lens[b] - 1, as the write kernel places it (lengths beyond the table count as
+    // its capacity); a sequence that takes none this step (new_lens[b] == 0) or is empty is streamed as it is
+    if (takes_new) {
+      const int pos = new_len - 1;
+      if (pos == ctx - 1) {
+        // seen by this call: the wave that streams its tile patches that tile and stores the row
+        if (pos >= t_begin && pos < t_end && ((pos - t_begin) >> 5) % NW == wave) {
+          w.adopt_new_row(pos);
+          store_pos = pos;
+        }
+      } else if (part == 0 && wave == 0) {
+        store_pos = pos;                    // a length bound below the new token: stored, not attended to
+      }
+    }
+  }
   w.stream(t_begin + 32 * wave, 32 * NW, (ntiles - wave + NW - 1) / NW, t_end);
+  if constexpr (NEWROW) {
+    if (store_pos >= 0) {
+      if (store_pos != ctx - 1) w.retransform_new_k(b, store_pos);     // K was rotated for position ctx - 1
+      w.store_new_row(b, store_pos);
+    }
+  }
 
   // ---- merge the NW wave states through LDS ----
   // (eight waves keep rows for at most 8 q heads per kv head: 16 rows of 8 waves would not fit the static 64 KB)
@@ -954,6 +1083,19 @@ hipError_t launch_typed(const DecodeParams& p, int waves, hipStream_t s) {
     hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 4, true>), grid, dim3(256), 0, s, p);
     return hipGetLastError();
   }
+  if (p.new_k) {
+    if constexpr (FP8) {
+      return hipErrorInvalidValue;
+    } else {
+      if (waves == 8) {
+        if (n_rep > 8) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((decode_mfma_kernel<D, false, 8, false, true>), grid, dim3(512), 0, s, p);
+      } else {
+        hipLaunchKernelGGL((decode_mfma_kernel<D, false, 4, false, true>), grid, dim3(256), 0, s, p);
+      }
+      return hipGetLastError();
+    }
+  }
   switch (waves) {
     case 1: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 1>), grid, dim3(64), 0, s, p); break;
     case 2: hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 2>), grid, dim3(128), 0, s, p); break;
@@ -993,6 +1135,10 @@ bool decode_mfma_supported(const DecodeParams& p, int q_dtype, int kv_dtype) {
   if (p.D != 64 && p.D != 128) return false;
   if (p.block_shift < 4) return false;   // power-of-two block size >= 16
   return true;
+}
+
+bool decode_new_row_supported(const DecodeParams& p, int q_dtype, int kv_dtype) {
+  return decode_mfma_supported(p, q_dtype, kv_dtype) && kv_dtype == PA_BF16 && p.T == 1 && !p.query_lens;
 }
 
 hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hipStream_t s) {

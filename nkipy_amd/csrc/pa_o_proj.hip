@@ -537,7 +537,13 @@ __global__ __launch_bounds__(256) void o_proj_skinny_kernel(OProjParams p) {
 // leave float32 partial tiles for o_proj_split_reduce_kernel (one range: bf16 output and bias directly).
 constexpr int RS_X = 32 * 128, RS_W = 64 * 256, RS_STAGE = RS_X + RS_W;      // 4 KB + 16 KB per k-step
 constexpr int RS_MAX_STEPS = 8;
-template <bool BIAS>
+// MERGE: the x rows are not in memory: row b is the attention output of sequence b, still in the form of the
+// per-partition partials a fixed-partition decode launch left (p.part_o, p.part_ml).  The workgroup merges what its
+// K range needs (a 16-byte chunk of a row is 8 elements of one q head: the partitions' weights
+// l_i 2^(m_i - max m), the weighted sum, one division, one rounding to bf16: decode_reduce_kernel's arithmetic
+// in its order, so the bits are those that kernel would have written) and stores the chunks where the copies
+// would have put them, while its w tiles are on their way.
+template <bool BIAS, bool MERGE = false>
 __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x;
@@ -569,11 +575,67 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     const char* wb = (const char*)p.w + (long)kt_begin * BK * w_row_b;
     for (int kt = 0; kt < ktiles; ++kt) {
       const uint32_t sb = smem_base + kt * RS_STAGE;
-      dma16(xb, xoff, sb + wave * 1024);
+      if (!MERGE) dma16(xb, xoff, sb + wave * 1024);
 #pragma unroll
       for (int j = 0; j < 4; ++j) dma16(wb, woff[j], sb + RS_X + (wave + 4 * j) * 1024);
       xb += BK * 2;
       wb += (long)BK * w_row_b;
+    }
+  }
+  if (MERGE) {
+#pragma clang fp contract(off)      // round where decode_reduce_kernel rounds: products and sums as written
+    // item = (k-step kt, row m < M, chunk c): elements k0 .. k0 + 7 of x row m, k0 = (kt_begin + kt) * 64 + 8 c, all of
+    // one q head.  Up to NPRE partitions' values are requested before any is used (slots past a sequence's own
+    // partition count exist and are loaded, not used), two items at a time: the merge is a chain of trips to memory.
+    constexpr int NPRE = 4;
+    const int Dh = p.part_D, Hq = p.K / Dh, np_max = p.part_np;
+    const int per_step = 8 * p.M, items = ktiles * per_step;
+#pragma unroll 2
+    for (int item = tid; item < items; item += 256) {
+      const int kt = item / per_step, rem = item - kt * per_step;
+      const int m = rem >> 3, c = rem & 7;
+      const int k0 = (kt_begin + kt) * BK + 8 * c;
+      const int head = k0 / Dh, d = k0 - head * Dh;
+      const long base = ((long)m * Hq + head) * np_max;
+      float2 ml[NPRE];
+      float4 oa[NPRE], ob[NPRE];
+#pragma unroll
+      for (int i = 0; i < NPRE; ++i) {
+        const long at = base + min(i, np_max - 1);
+        ml[i] = *(const float2*)(p.part_ml + at * 2);
+        oa[i] = *(const float4*)(p.part_o + at * Dh + d);
+        ob[i] = *(const float4*)(p.part_o + at * Dh + d + 4);
+      }
+      const int ctx = min(max(p.part_seq_lens[m], 0), p.part_max_seq_len);
+      const int np = min((ctx + p.part_size - 1) / p.part_size, np_max);
+      float mt = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < NPRE; ++i)
+        if (i < np) mt = fmaxf(mt, ml[i].x);
+      for (int i = NPRE; i < np; ++i) mt = fmaxf(mt, p.part_ml[(base + i) * 2]);
+      const float m_ref = mt == -INFINITY ? 0.f : mt;
+      float lt = 0.f, ot[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ot[j] = 0.f;
+      auto add = [&](float2 mli, const float4& a, const float4& b) __attribute__((always_inline)) {
+        const float wgt = mli.y * exp2f(mli.x - m_ref);
+        lt += wgt;
+        ot[0] = __builtin_fmaf(wgt, a.x, ot[0]); ot[1] = __builtin_fmaf(wgt, a.y, ot[1]);
+        ot[2] = __builtin_fmaf(wgt, a.z, ot[2]); ot[3] = __builtin_fmaf(wgt, a.w, ot[3]);
+        ot[4] = __builtin_fmaf(wgt, b.x, ot[4]); ot[5] = __builtin_fmaf(wgt, b.y, ot[5]);
+        ot[6] = __builtin_fmaf(wgt, b.z, ot[6]); ot[7] = __builtin_fmaf(wgt, b.w, ot[7]);
+      };
+#pragma unroll
+      for (int i = 0; i < NPRE; ++i)
+        if (i < np) add(ml[i], oa[i], ob[i]);
+      for (int i = NPRE; i < np; ++i)
+        add(*(const float2*)(p.part_ml + (base + i) * 2), *(const float4*)(p.part_o + (base + i) * Dh + d),
+            *(const float4*)(p.part_o + (base + i) * Dh + d + 4));
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = lt > 0.f ? ot[j] / lt : 0.f;
+      *(uint4*)(smem + kt * RS_STAGE + m * 128 + ((c ^ ((m >> 1) & 7)) << 4)) =
+          make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
     }
   }
   int x_off[4], w_off;
@@ -601,14 +663,15 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc, 0, 0, 0);
     }
   };
-  if (ktiles == RS_MAX_STEPS) {
+  if (!MERGE && ktiles == RS_MAX_STEPS) {
     // a full range: the steps are multiplied as they land (5 copy instructions per wave and step)
 #define RS_STEP(kt) wait_vmcnt<5 * (RS_MAX_STEPS - 1 - (kt))>(); __builtin_amdgcn_s_barrier(); step(kt);
     RS_STEP(0) RS_STEP(1) RS_STEP(2) RS_STEP(3) RS_STEP(4) RS_STEP(5) RS_STEP(6) RS_STEP(7)
 #undef RS_STEP
   } else {
     wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
+    if (MERGE) __syncthreads();          // the merged x chunks are ordinary LDS stores of other waves
+    else __builtin_amdgcn_s_barrier();
     for (int kt = 0; kt < ktiles; ++kt) step(kt);
   }
   // a lane holds, for its row, 4 consecutive columns at 4 places
@@ -701,13 +764,18 @@ static hipError_t launch_resident(const OProjParams& p, hipStream_t s) {
   if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute((const void*)o_proj_resident_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_resident_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_resident_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void*)o_proj_resident_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured.store(1, std::memory_order_release);
   }
   const int ktiles = (p.K / BK + p.splits - 1) / p.splits;
   const dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)p.splits);
   const int bytes = ktiles * RS_STAGE;
-  if (p.bias && p.splits == 1) hipLaunchKernelGGL((o_proj_resident_kernel<true>), grid, dim3(256), bytes, s, p);
+  if (p.part_o) {
+    if (p.bias && p.splits == 1) hipLaunchKernelGGL((o_proj_resident_kernel<true, true>), grid, dim3(256), bytes, s, p);
+    else hipLaunchKernelGGL((o_proj_resident_kernel<false, true>), grid, dim3(256), bytes, s, p);
+  } else if (p.bias && p.splits == 1) hipLaunchKernelGGL((o_proj_resident_kernel<true>), grid, dim3(256), bytes, s, p);
   else hipLaunchKernelGGL((o_proj_resident_kernel<false>), grid, dim3(256), bytes, s, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.splits == 1) return e;
@@ -727,12 +795,18 @@ int o_proj_splits(int M, int K, int N) {
   return s < 2 ? 1 : (int)s;
 }
 
+bool o_proj_takes_partials(int M, int K, int D, int splits, bool have_ws) {
+  const int r = o_proj_resident_splits(M, K);
+  return r > 0 && splits == r && (r == 1 || have_ws) && (D == 64 || D == 128) && K % D == 0;
+}
+
 static std::atomic<int> g_o_proj_force_large{0};
 void o_proj_debug_force_large(int on) { g_o_proj_force_large = on; }
 
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
   // up to 32 rows with the workspace for its K ranges (or K <= 512): everything resident, one round trip
   if (const int r = o_proj_resident_splits(p.M, p.K); r > 0 && p.splits == r && (r == 1 || p.ws)) return launch_resident(p, s);
+  if (p.part_o) return hipErrorInvalidValue;      // only the resident form merges partials (o_proj_takes_partials)
   // up to 256 rows: one workgroup per 64 columns owns every row (the call is bound by w's bytes)
   if (p.M <= 64) return launch_skinny<2>(p, s);
   if (p.M <= 128) return launch_skinny<4>(p, s);

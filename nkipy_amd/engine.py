@@ -286,6 +286,15 @@ class PagedAttention:
         self.cache.begin_step(query_lens, xq.shape[1])
         return self.attend(xq, xk, xv)
 
+    def _q_transform(self):
+        """The layer's Q transform for the attention kernels (one object, validated once), None without RoPE."""
+        if self.rope is None:
+            return None
+        qt = getattr(self, "_qt", None)
+        if qt is None:
+            qt = self._qt = paged_attn.QTransform(self.rope[0], self.rope[1], self.q_norm_weight, self.norm_eps)
+        return qt
+
     def attend(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, *,
                max_seq_len: Optional[int] = None) -> torch.Tensor:
         c, l = self.cache, self.layer
@@ -302,6 +311,32 @@ class PagedAttention:
         out = self._out.get(T)
         if out is None:
             out = self._out[T] = torch.empty((B, T, self.n_heads, c.head_dim), dtype=torch.bfloat16, device=c.device)
+        if T == 1 and (self.rope is None or paged_attn.q_transform_supported(1, c.head_dim, c.block_size)):
+            # a decode step: one call for the cache update, the attention and the projection (a small step then runs
+            # as three launches: the new row rides on the decode launch, the split-K merge on the projection's load).
+            # The bound on the contexts sizes the launch, clamps the lengths the kernel reads and picks the kernel:
+            # the caller's bound if given; else what the host knows of this step's contexts, unless the launch is
+            # being captured into a HIP graph, which will be replayed on longer contexts and so gets the longest
+            # sequence the cache admits.  The decode kernels treat every slot as live; idle slots (seq_len 0) come
+            # back as zeros (projected: the bias).
+            qt = self._q_transform()
+            if self.o_weight is None:
+                paged_attn.decode_step(xq[:, 0], xk[:, 0], xv[:, 0], kc, vc, c.block_tables, c.seq_lens, c.query_lens,
+                                       self.scale, k_scale=ks, v_scale=vs, partition_size=self.partition_size,
+                                       max_seq_len=bound, q_transform=qt,
+                                       k_norm_weight=None if self.rope is None else self.k_norm_weight, out=out[:, 0],
+                                       sinks=self.sinks, sliding_window=self.sliding_window)
+                return out
+            proj = self._proj.get(T)
+            if proj is None:
+                proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
+            paged_attn.decode_step(xq[:, 0], xk[:, 0], xv[:, 0], kc, vc, c.block_tables, c.seq_lens, c.query_lens,
+                                   self.scale, k_scale=ks, v_scale=vs, partition_size=self.partition_size,
+                                   max_seq_len=bound, q_transform=qt,
+                                   k_norm_weight=None if self.rope is None else self.k_norm_weight,
+                                   o_weight=self.o_weight, o_bias=self.o_bias, out=proj[:, 0],
+                                   sinks=self.sinks, sliding_window=self.sliding_window)
+            return proj
         qt = None
         if self.rope is not None:
             # the Q half of the norm and rotation rides on the attention kernel's Q load where that
@@ -313,7 +348,7 @@ class PagedAttention:
                                                  k_norm_weight=self.k_norm_weight, eps=self.norm_eps,
                                                  k_scale=ks, v_scale=vs, out=None if fused else xq)
             if fused:
-                q, qt = xq, paged_attn.QTransform(self.rope[0], self.rope[1], self.q_norm_weight, self.norm_eps)
+                q, qt = xq, self._q_transform()
         else:
             paged_attn.kv_write(xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, k_scale=ks, v_scale=vs)
             q = xq

@@ -693,6 +693,117 @@ def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
     return out
 
 
+def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
+                partition_size=512, max_seq_len=None, q_transform=None, k_norm_weight=None, o_weight=None, o_bias=None,
+                out=None, attn_out=None, workspace=None, sinks=None, sliding_window=None):
+    """One decode step of an attention layer in one call: the cache update, the attention and, with `o_weight`, the
+    output projection -- the decode branch of the reference's attention_kernel as a whole
+    (examples/models/qwen3/kernels/attention.py:78-147; examples/models/gpt_oss/kernels/attention.py:85-163).
+
+    Bit for bit the result of `qk_norm_rope_kv_write(None, xk, xv, ...)` (`kv_write` without `q_transform`), then
+    `decode(xq, ..., q_transform=...)`, then `o_proj(...)`; a small step over a bfloat16 pool runs as three launches
+    instead of five (the new row rides on the decode launch, the split-K merge on the projection's load).
+
+    xq [B, Hq, D], xk / xv [B, Hkv, D]: the step's new token per sequence, before norm and rotation when `q_transform`
+    (a `QTransform`: Q's norm weight and the RoPE tables) is given; `k_norm_weight` [D] is K's norm weight (None: K is
+    rotated only).  seq_lens counts the new token; query_lens [B] int32 is 1 for the sequences that take one and 0 for
+    those that do not.  The pools (and the scales of a float8 pool) are updated in place.
+    Returns the projected rows [B, N] when `o_weight` [Hq * D, N] is given (written to `out` if passed; `attn_out`
+    [B, Hq, D], if passed, also receives the attention output), else the attention output [B, Hq, D] (`out`).
+    """
+    lib = _lib.load()
+    for n, t in (("xq", xq), ("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
+                 ("block_tables", block_tables), ("seq_lens", seq_lens), ("query_lens", query_lens)):
+        _need_device(n, t)
+    _check(xq.dim() == 3, "xq must be [B, Hq, D]")
+    B, Hq, D = xq.shape
+    _check(xq.dtype in (torch.float32, torch.bfloat16), f"unsupported xq dtype {xq.dtype}")
+    _check_paging(k_cache, v_cache, block_tables, seq_lens, B)
+    num_blocks, block_size, Hkv, Dk = k_cache.shape
+    _check(Dk == D, f"head_dim mismatch: xq has {D}, cache has {Dk}")
+    _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    _check(D in (32, 64, 128, 256), f"head_dim {D} not in (32, 64, 128, 256)")
+    _check(tuple(xk.shape) == (B, Hkv, D) and xv.shape == xk.shape and xk.dtype == xq.dtype and xv.dtype == xq.dtype,
+           f"xk and xv must be {xq.dtype} [B, Hkv, D] = {(B, Hkv, D)}")
+    _check(query_lens.shape == (B,) and query_lens.dtype == torch.int32, "query_lens must be int32 [B]")
+    scaled = k_scale is not None or v_scale is not None
+    kv_code = _kv_code(k_cache, scaled)
+    q_code = _DTYPE_CODE[xq.dtype]
+    if kv_code == FP8:
+        _check(q_code == BF16, "fp8 KV needs bfloat16 rows")
+        _check(k_scale is not None and v_scale is not None, "fp8 KV needs both k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _need_device(n, t)
+            _check(t.dtype == torch.float32 and t.shape == (num_blocks, Hkv), f"{n} must be float32 [num_blocks, Hkv]")
+    else:
+        _check(kv_code == q_code, f"KV dtype {k_cache.dtype} does not match the rows' dtype {xq.dtype}")
+        _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
+    sinks, win = _check_variant(sinks, sliding_window, Hq, xq)
+    _check(isinstance(partition_size, int) and partition_size > 0, "partition_size must be a positive int")
+    cap = block_tables.shape[1] * block_size
+    msl = cap if max_seq_len is None else int(max_seq_len)
+    _check(0 < msl <= cap, f"max_seq_len {msl} outside (0, {cap}]")
+    if k_norm_weight is not None:
+        _need_device("k_norm_weight", k_norm_weight)
+        _check(q_transform is not None, "k_norm_weight comes with q_transform")
+        _check(tuple(k_norm_weight.shape) == (D,) and k_norm_weight.dtype == torch.bfloat16, "k_norm_weight must be bfloat16 [D]")
+    N = 0
+    if o_weight is not None:
+        _need_device("o_weight", o_weight)
+        _check(xq.dtype == torch.bfloat16 and o_weight.dtype == torch.bfloat16, "the output projection supports bfloat16 only")
+        _check(o_weight.dim() == 2 and o_weight.shape[0] == Hq * D, f"o_weight must be [Hq * D = {Hq * D}, N]")
+        N = o_weight.shape[1]
+        _check((Hq * D) % 64 == 0 and N % 8 == 0, f"Hq * D = {Hq * D} must be a multiple of 64 and N = {N} of 8")
+        if o_bias is not None:
+            _need_device("o_bias", o_bias)
+            _check(o_bias.dtype == torch.bfloat16 and tuple(o_bias.shape) == (N,), "o_bias must be bfloat16 [N]")
+        if out is None:
+            out = torch.empty((B, N), dtype=torch.bfloat16, device=xq.device)
+        else:
+            _need_device("out", out)
+            _check(tuple(out.shape) == (B, N) and out.dtype == torch.bfloat16, f"out must be bfloat16 {(B, N)}")
+        if attn_out is not None:
+            _need_device("attn_out", attn_out)
+            _check(attn_out.shape == xq.shape and attn_out.dtype == xq.dtype, "attn_out must match xq in shape and dtype")
+    else:
+        _check(o_bias is None and attn_out is None, "o_bias and attn_out come with o_weight (without it `out` is the attention output)")
+        if out is None:
+            out = torch.empty_like(xq)
+        else:
+            _need_device("out", out)
+            _check(out.shape == xq.shape and out.dtype == xq.dtype, "out must match xq in shape and dtype")
+        attn_out = out
+    _same_device(xq, xk=xk, xv=xv, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
+                 query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out, attn_out=attn_out, o_weight=o_weight,
+                 o_bias=o_bias, k_norm_weight=k_norm_weight)
+    key = (B, Hq, Hkv, D, block_size, msl, partition_size, N, q_code, kv_code)
+    need = _decode_step_need.get(key)
+    if need is None:
+        with _on(xq.device):
+            need = _decode_step_need[key] = int(lib.pa_decode_step_workspace_bytes(*key))
+    stream = _stream_ptr(xq.device)
+    if workspace is None:
+        workspace = _workspace(xq.device, need, stream)
+    else:
+        _need_device("workspace", workspace)
+        _check(workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.data_ptr() % 16 == 0,
+               "workspace must be a contiguous, 16-byte aligned uint8 tensor")
+        _check(workspace.numel() >= need, f"workspace needs {need} bytes")
+    qt_keep, qt_ptr = _qt_arg(q_transform, D, xq)
+    addr = lambda t: None if t is None else t.data_ptr()
+    nkv = _lib.NewKvStruct(addr(xk), addr(xv), addr(k_norm_weight), addr(query_lens))
+    proj = None if o_weight is None else _lib.OutProjStruct(addr(o_weight), addr(o_bias), addr(out), N)
+    with _on(xq.device):
+        rc = lib.pa_decode_step(_ptr(xq), ctypes.addressof(nkv), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+                                _ptr(block_tables), _ptr(seq_lens), _ptr(attn_out),
+                                None if proj is None else ctypes.addressof(proj), _ptr(workspace), workspace.numel(),
+                                B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
+                                float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, qt_ptr, stream)
+    _raise_on(rc, "pa_decode_step")
+    return out
+
+
+_decode_step_need = {}
 def o_proj_workspace_bytes(M: int, K: int, N: int) -> int:
     """Scratch bytes `o_proj` would use for a call of M rows (0 for shapes that take none)."""
     return int(_lib.load().pa_o_proj_workspace_bytes(int(M), int(K), int(N)))

@@ -166,14 +166,15 @@ def test_partition_size_invariance(pa):
 
 
 def test_small_calls_take_the_fixed_partition_kernel(pa):
-    """pa_decode's own choice: a call that can touch little of the pool by its max_seq_len (at most four
-    partitions per sequence) gives the fixed-partition kernel's bits, the same call with a bound of many partitions,
-    or with sinks, the balanced kernel's; all of them the oracle's values."""
+    """pa_decode's own choice: a call that can touch little of the pool by its max_seq_len (at most eight
+    partitions per sequence) gives the fixed-partition kernel's bits (on partitions of 256 tokens when the call is
+    small enough for those), the same call with a bound of many partitions, or with sinks, the balanced kernel's;
+    all of them the oracle's values."""
     rng = np.random.default_rng(77)
     B, Hq, Hkv, D, bs = 5, 16, 4, 128, 32
     ctxs = [1, 700, 1500, 33, 1024]
     k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
-    wide = np.full((B, 4096 // bs), -1, np.int32)            # the same blocks under a capacity of 8 partitions
+    wide = np.full((B, 8192 // bs), -1, np.int32)            # the same blocks under a capacity of 16 partitions
     wide[:, :tables.shape[1]] = tables
     q = rng.standard_normal((B, Hq, D)).astype(np.float32)
     dq, dk, dv = bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v)
@@ -194,8 +195,8 @@ def test_small_calls_take_the_fixed_partition_kernel(pa):
     for o in (fixed, balanced):
         assert_close_abs(dev_to_f32(o), want, BF16_TOL)
     assert not np.array_equal(dev_bits(fixed), dev_bits(balanced))        # (else the test below shows nothing)
-    assert np.array_equal(dev_bits(run(0, tables, max_seq_len=1500)), dev_bits(fixed))
-    assert np.array_equal(dev_bits(run(0, wide)), dev_bits(run(3, wide)))                 # bound = 4 096 tokens
+    assert np.array_equal(dev_bits(run(0, tables, max_seq_len=1500)), dev_bits(run(2, tables, max_seq_len=1500, partition_size=256)))
+    assert np.array_equal(dev_bits(run(0, wide)), dev_bits(run(3, wide)))                 # bound = 8 192 tokens
     assert np.array_equal(dev_bits(run(0, tables, max_seq_len=1500, sinks=sinks)),
                           dev_bits(run(3, tables, max_seq_len=1500, sinks=sinks)))
 
