@@ -111,8 +111,30 @@ struct QTransform {
 // stand-alone transform kernel (mean of squares as a butterfly over the chunk index, norm in
 // float32 rounded once to bf16, every product and sum of the rotation rounded to bf16), so
 // the two give the same bits.
+// The transform comes in two halves so that a caller can put other memory requests between them: the loads of
+// what it needs from the tables (norm weights, the position's cos and sin rows), and the arithmetic.
+template <int NS>
+struct NormRopeCoeffs {
+  uint4 w[NS], cs[NS], sn[NS];
+};
 template <int CPR, int NS, class L>
-__device__ __forceinline__ void q_norm_rope_lane(float (&x)[NS][8], const QTransform& t, int pos, int part) {
+__device__ __forceinline__ void norm_rope_fetch(const QTransform& t, int pos, int part, NormRopeCoeffs<NS>& c) {
+  constexpr int D = 8 * CPR;
+  constexpr int hc = CPR / 2;
+  const uint16_t* cos_row = t.cos + (long)pos * (D / 2);
+  const uint16_t* sin_row = t.sin + (long)pos * (D / 2);
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int ch = L::chunk(s, part);
+    const int fi = 8 * (ch < hc ? ch : ch - hc);
+    c.cs[s] = *(const uint4*)(cos_row + fi);
+    c.sn[s] = *(const uint4*)(sin_row + fi);
+    c.w[s] = make_uint4(0, 0, 0, 0);
+    if (t.norm_weight) c.w[s] = *(const uint4*)(t.norm_weight + 8 * ch);
+  }
+}
+template <int CPR, int NS, class L>
+__device__ __forceinline__ void norm_rope_apply(float (&x)[NS][8], const QTransform& t, int part, const NormRopeCoeffs<NS>& c) {
   constexpr int D = 8 * CPR;
   auto r16 = [](float f) __attribute__((always_inline)) { return __uint_as_float(pack_bf16x2(f, 0.f) << 16); };
   auto unpack = [](const uint4& v, float (&f)[8]) __attribute__((always_inline)) {
@@ -144,23 +166,20 @@ __device__ __forceinline__ void q_norm_rope_lane(float (&x)[NS][8], const QTrans
     for (int s = 0; s < NS; ++s) {
       const float inv = __builtin_amdgcn_rsqf(__fdiv_rn(ss[s], (float)D) + t.eps);
       float w[8];
-      unpack(*(const uint4*)(t.norm_weight + 8 * L::chunk(s, part)), w);
+      unpack(c.w[s], w);
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[s][j] = r16((x[s][j] * inv) * w[j]);
     }
   }
   constexpr int hc = CPR / 2;
-  const uint16_t* cos_row = t.cos + (long)pos * (D / 2);
-  const uint16_t* sin_row = t.sin + (long)pos * (D / 2);
   float y[NS][8];
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
-    const int c = L::chunk(s, part);
-    const bool first = c < hc;
-    const int fi = 8 * (first ? c : c - hc);
+    const int ch = L::chunk(s, part);
+    const bool first = ch < hc;
     float cs[8], sn[8];
-    unpack(*(const uint4*)(cos_row + fi), cs);
-    unpack(*(const uint4*)(sin_row + fi), sn);
+    unpack(c.cs[s], cs);
+    unpack(c.sn[s], sn);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float other = L::slot_xor(hc) ? x[s ^ L::slot_xor(hc)][j] : __shfl_xor(x[s][j], L::lane_xor(hc));
@@ -171,6 +190,12 @@ __device__ __forceinline__ void q_norm_rope_lane(float (&x)[NS][8], const QTrans
   for (int s = 0; s < NS; ++s)
 #pragma unroll
     for (int j = 0; j < 8; ++j) x[s][j] = y[s][j];
+}
+template <int CPR, int NS, class L>
+__device__ __forceinline__ void q_norm_rope_lane(float (&x)[NS][8], const QTransform& t, int pos, int part) {
+  NormRopeCoeffs<NS> c;
+  norm_rope_fetch<CPR, NS, L>(t, pos, part, c);
+  norm_rope_apply<CPR, NS, L>(x, t, part, c);
 }
 
 // ---- decode ------------------------------------------------------------------------

@@ -233,19 +233,34 @@ struct DecodeWave {
 
   // Start on sequence b (context ctx >= 1, of which the last tq tokens are the
   // queries): load Q^T fragments (B operand, zero for padded columns) and reset
-  // the softmax state.
+  // the softmax state.  In two halves, so that a caller can request its first tile
+  // between them: issue_q sends every load the start needs (Q rows, what their
+  // transform takes from the tables, with NEWROW the new token's rows), finish_q does
+  // the arithmetic.  begin() is the two in a row.
+  struct QPending {
+    uint4 qraw[R][KSTEPS];
+    NormRopeCoeffs<KSTEPS> qc[R];
+    uint4 kraw[NEWROW ? KSTEPS : 1];
+    NormRopeCoeffs<KSTEPS> kc;
+  };
   __device__ __forceinline__ void begin(int b, int ctx, int tq = 1) {
+    QPending q;
+    issue_q(q, b, ctx, tq);
+    finish_q(q);
+  }
+  __device__ __forceinline__ void issue_q(QPending& q, int b, int ctx, int tq = 1) {
     table = p.block_tables + (long)b * p.max_blocks;
     last = ctx - 1;
     // NEWROW: the new token's rows are requested here, with the Q rows, by every wave (one round trip for all of
     // them; the wave that turns out to hold the token adopts them, see adopt_new_row), and K is transformed behind Q
-    uint4 kraw[NEWROW ? KSTEPS : 1];
     if constexpr (NEWROW) {
       const uint16_t* krow = (const uint16_t*)p.new_k + ((long)b * p.Hkv + hk) * D;
       const uint16_t* vrow = (const uint16_t*)p.new_v + ((long)b * p.Hkv + hk) * D;
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) kraw[s] = *(const uint4*)(krow + (4 * s + g) * 8);
+      for (int s = 0; s < KSTEPS; ++s) q.kraw[s] = *(const uint4*)(krow + (4 * s + g) * 8);
       VecLoad<VW>::get(vrow + r * VEC, vnew);
+      if (p.new_kt.cos)
+        norm_rope_fetch<D / 8, KSTEPS, QOperandLayout<false>>(p.new_kt, min(max(last, 0), p.new_kt.max_pos - 1), g, q.kc);
     }
 #pragma unroll
     for (int rg = 0; rg < R; ++rg) {
@@ -259,14 +274,23 @@ struct DecodeWave {
       } else {
         qrow = (const uint16_t*)p.q + ((long)b * p.Hq + hbase + r) * D;
       }
-      uint4 qraw[KSTEPS];
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
         // d range of k-slots 8g..8g+7 in step s (must mirror the K loads below)
         const int d0 = FP8 ? ((4 * (s >> 1) + g) * 16 + (s & 1) * 8) : ((4 * s + g) * 8);
-        qraw[s] = make_uint4(0, 0, 0, 0);
-        if (row_valid) qraw[s] = *(const uint4*)(qrow + d0);
+        q.qraw[rg][s] = make_uint4(0, 0, 0, 0);
+        if (row_valid) q.qraw[rg][s] = *(const uint4*)(qrow + d0);
       }
+      if (p.qt.cos) {
+        const int qpos = MULTI ? row_end[rg] - 1 : last;
+        norm_rope_fetch<D / 8, KSTEPS, QOperandLayout<FP8>>(p.qt, min(max(qpos, 0), p.qt.max_pos - 1), g, q.qc[rg]);
+      }
+    }
+  }
+  __device__ __forceinline__ void finish_q(QPending& q) {
+#pragma unroll
+    for (int rg = 0; rg < R; ++rg) {
+      uint4 (&qraw)[KSTEPS] = q.qraw[rg];
       if (p.qt.cos) {
         // norm and rotation of the row on the way in; every lane takes part (a row is spread
         // over the four lanes r, r + 16, r + 32, r + 48), padded rows carry zeros
@@ -280,8 +304,7 @@ struct DecodeWave {
             x[s][2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
           }
         }
-        const int qpos = MULTI ? row_end[rg] - 1 : last;
-        q_norm_rope_lane<D / 8, KSTEPS, QOperandLayout<FP8>>(x, p.qt, min(max(qpos, 0), p.qt.max_pos - 1), g);
+        norm_rope_apply<D / 8, KSTEPS, QOperandLayout<FP8>>(x, p.qt, g, q.qc[rg]);
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
           qraw[s].x = pack_bf16x2(x[s][0], x[s][1]); qraw[s].y = pack_bf16x2(x[s][2], x[s][3]);
@@ -298,11 +321,33 @@ struct DecodeWave {
       m_run[rg] = -INFINITY;
       l_run[rg] = 0.f;
     }
-    if constexpr (NEWROW) transform_new_k(kraw, last);
+    if constexpr (NEWROW) {
+      // the raw K row -> knew, normed and rotated at position ctx - 1 as the write kernel would (same arithmetic,
+      // same bits; new_kt.cos null: stored as given)
+      if (p.new_kt.cos) {
+        float x[KSTEPS][8];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          const uint32_t w[4] = {q.kraw[s].x, q.kraw[s].y, q.kraw[s].z, q.kraw[s].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[s][2 * j] = bf16_bits_to_float(w[j] & 0xffffu);
+            x[s][2 * j + 1] = bf16_bits_to_float(w[j] >> 16);
+          }
+        }
+        norm_rope_apply<D / 8, KSTEPS, QOperandLayout<false>>(x, p.new_kt, g, q.kc);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+          q.kraw[s] = make_uint4(pack_bf16x2(x[s][0], x[s][1]), pack_bf16x2(x[s][2], x[s][3]),
+                                 pack_bf16x2(x[s][4], x[s][5]), pack_bf16x2(x[s][6], x[s][7]));
+      }
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) knew[s] = q.kraw[s];
+    }
   }
 
-  // NEWROW: the raw K row -> knew, normed and rotated at position pos as the write kernel would (same arithmetic,
-  // same bits; new_kt.cos null: stored as given)
+  // NEWROW: the raw K row -> knew, normed and rotated at position pos (the slow path of a token the call's length
+  // bound hides: see retransform_new_k)
   __device__ __forceinline__ void transform_new_k(uint4 (&kraw)[NEWROW ? KSTEPS : 1], int pos) {
     if constexpr (NEWROW) {
       if (p.new_kt.cos) {
@@ -572,11 +617,17 @@ struct DecodeWave {
   // includes the loads of tile i+1.
   __device__ __forceinline__ void stream(int t_first, int t_step, int n, int t_end, bool lockstep = false) {
     if (n <= 0) return;
-    KT ka, kb;
+    KT ka;
     VT va;
+    load_k(ka, t_first);
+    load_v(va, t_first);
+    stream_from(ka, va, t_first, t_step, n, t_end, lockstep);
+  }
+  // ... with the first tile's loads (into ka, va) already requested by the caller
+  __device__ __forceinline__ void stream_from(KT& ka, VT& va, int t_first, int t_step, int n, int t_end, bool lockstep = false) {
+    if (n <= 0) return;
+    KT kb;
     int t = t_first;
-    load_k(ka, t);
-    load_v(va, t);
     int i = 0;
     if (LEAN) {
       while (i + 2 < n) {
@@ -780,7 +831,18 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
   }
   const int t_end = min(ctx, t_begin + p.partition_size);
   const int ntiles = (t_end - t_begin + 31) >> 5;
-  w.begin(b, ctx, sp.tq);
+  // every load the start needs, then this wave's first tile, then the arithmetic of the start: the first tile is on
+  // its way while Q is normed and rotated (one trip to memory less on the path of every workgroup)
+  const int t_first = t_begin + 32 * wave, n_mine = (ntiles - wave + NW - 1) / NW;
+  typename W::QPending qp;
+  typename W::KT k_first;
+  typename W::VT v_first;
+  w.issue_q(qp, b, ctx, sp.tq);
+  if (n_mine > 0) {
+    w.load_k(k_first, t_first);
+    w.load_v(v_first, t_first);
+  }
+  w.finish_q(qp);
   int store_pos = -1;       // NEWROW: this wave stores the new token's rows at this position when its tiles are done
   if constexpr (NEWROW) {
     // the new token is number seq_lens[b] - 1, as the write kernel places it (lengths beyond the table count as
@@ -798,7 +860,7 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
       }
     }
   }
-  w.stream(t_begin + 32 * wave, 32 * NW, (ntiles - wave + NW - 1) / NW, t_end);
+  w.stream_from(k_first, v_first, t_first, 32 * NW, n_mine, t_end);
   if constexpr (NEWROW) {
     if (store_pos >= 0) {
       if (store_pos != ctx - 1) w.retransform_new_k(b, store_pos);     // K was rotated for position ctx - 1
