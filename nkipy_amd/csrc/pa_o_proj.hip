@@ -570,6 +570,45 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     const int chunk = (lane & 15) ^ (4 * ((lane >> 4) & 3));
     woff[j] = (uint32_t)(r * w_row_b) + (uint32_t)(min(n0 + 8 * chunk, p.N - 8) * 2);
   }
+  // MERGE: what the first NE items of this thread need (an item = one 16-byte chunk of an x row, see below) is
+  // requested here, ahead of the w tiles, by hand-placed loads whose arrival is awaited by hand too: memory answers in
+  // the order of the requests, so these are back long before the tiles, and the merge arithmetic runs while the tiles
+  // stream in.  (Loads the compiler places itself would be waited for with everything in flight, tiles included.)
+  constexpr int NPRE = 4, NE = 2;
+  typedef float f2_t __attribute__((ext_vector_type(2)));
+  typedef float f4_t __attribute__((ext_vector_type(4)));
+  f2_t e_ml[NE][NPRE];
+  f4_t e_oa[NE][NPRE], e_ob[NE][NPRE];
+  int e_len[NE];
+  const int m_items = MERGE ? ktiles * 8 * p.M : 0;
+  auto item_place = [&](int item, int& kt, int& m, int& c, int& d, long& base) __attribute__((always_inline)) {
+    const int per_step = 8 * p.M;
+    kt = item / per_step;
+    const int rem = item - kt * per_step;
+    m = rem >> 3; c = rem & 7;
+    const int k0 = (kt_begin + kt) * BK + 8 * c;
+    const int head = k0 / p.part_D;
+    d = k0 - head * p.part_D;
+    base = ((long)m * (p.K / p.part_D) + head) * p.part_np;
+  };
+  if (MERGE) {
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      int kt, m, c, d; long base;
+      item_place(min(tid + 256 * e, m_items - 1), kt, m, c, d, base);
+      const int32_t* plen = p.part_seq_lens + m;
+      asm volatile("global_load_dword %0, %1, off" : "=&v"(e_len[e]) : "v"(plen) : "memory");
+#pragma unroll
+      for (int i = 0; i < NPRE; ++i) {
+        const long at = base + min(i, p.part_np - 1);
+        const float* pml = p.part_ml + at * 2;
+        const float* po = p.part_o + at * p.part_D + d;
+        asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(e_ml[e][i]) : "v"(pml) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(e_oa[e][i]) : "v"(po) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=&v"(e_ob[e][i]) : "v"(po) : "memory");
+      }
+    }
+  }
   {
     const char* xb = (const char*)p.x + (long)kt_begin * (BK * 2);
     const char* wb = (const char*)p.w + (long)kt_begin * BK * w_row_b;
@@ -586,27 +625,11 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
 #pragma clang fp contract(off)      // round where decode_reduce_kernel rounds: products and sums as written
     // item = (k-step kt, row m < M, chunk c): elements k0 .. k0 + 7 of x row m, k0 = (kt_begin + kt) * 64 + 8 c, all of
     // one q head.  Up to NPRE partitions' values are requested before any is used (slots past a sequence's own
-    // partition count exist and are loaded, not used), two items at a time: the merge is a chain of trips to memory.
-    constexpr int NPRE = 4;
-    const int Dh = p.part_D, Hq = p.K / Dh, np_max = p.part_np;
-    const int per_step = 8 * p.M, items = ktiles * per_step;
-#pragma unroll 2
-    for (int item = tid; item < items; item += 256) {
-      const int kt = item / per_step, rem = item - kt * per_step;
-      const int m = rem >> 3, c = rem & 7;
-      const int k0 = (kt_begin + kt) * BK + 8 * c;
-      const int head = k0 / Dh, d = k0 - head * Dh;
-      const long base = ((long)m * Hq + head) * np_max;
-      float2 ml[NPRE];
-      float4 oa[NPRE], ob[NPRE];
-#pragma unroll
-      for (int i = 0; i < NPRE; ++i) {
-        const long at = base + min(i, np_max - 1);
-        ml[i] = *(const float2*)(p.part_ml + at * 2);
-        oa[i] = *(const float4*)(p.part_o + at * Dh + d);
-        ob[i] = *(const float4*)(p.part_o + at * Dh + d + 4);
-      }
-      const int ctx = min(max(p.part_seq_lens[m], 0), p.part_max_seq_len);
+    // partition count exist and are loaded, not used).
+    const int Dh = p.part_D, np_max = p.part_np;
+    auto finish = [&](int kt, int m, int c, int d, long base, int len, const f2_t (&ml)[NPRE], const f4_t (&oa)[NPRE],
+                      const f4_t (&ob)[NPRE]) __attribute__((always_inline)) {
+      const int ctx = min(max(len, 0), p.part_max_seq_len);
       const int np = min((ctx + p.part_size - 1) / p.part_size, np_max);
       float mt = -INFINITY;
 #pragma unroll
@@ -617,8 +640,8 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
       float lt = 0.f, ot[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) ot[j] = 0.f;
-      auto add = [&](float2 mli, const float4& a, const float4& b) __attribute__((always_inline)) {
-        const float wgt = mli.y * exp2f(mli.x - m_ref);
+      auto add = [&](float mi, float li, const f4_t& a, const f4_t& b) __attribute__((always_inline)) {
+        const float wgt = li * exp2f(mi - m_ref);
         lt += wgt;
         ot[0] = __builtin_fmaf(wgt, a.x, ot[0]); ot[1] = __builtin_fmaf(wgt, a.y, ot[1]);
         ot[2] = __builtin_fmaf(wgt, a.z, ot[2]); ot[3] = __builtin_fmaf(wgt, a.w, ot[3]);
@@ -627,15 +650,46 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
       };
 #pragma unroll
       for (int i = 0; i < NPRE; ++i)
-        if (i < np) add(ml[i], oa[i], ob[i]);
-      for (int i = NPRE; i < np; ++i)
-        add(*(const float2*)(p.part_ml + (base + i) * 2), *(const float4*)(p.part_o + (base + i) * Dh + d),
-            *(const float4*)(p.part_o + (base + i) * Dh + d + 4));
+        if (i < np) add(ml[i].x, ml[i].y, oa[i], ob[i]);
+      for (int i = NPRE; i < np; ++i) {
+        const f4_t a = *(const f4_t*)(p.part_o + (base + i) * Dh + d), b = *(const f4_t*)(p.part_o + (base + i) * Dh + d + 4);
+        add(p.part_ml[(base + i) * 2], p.part_ml[(base + i) * 2 + 1], a, b);
+      }
       float o[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) o[j] = lt > 0.f ? ot[j] / lt : 0.f;
       *(uint4*)(smem + kt * RS_STAGE + m * 128 + ((c ^ ((m >> 1) & 7)) << 4)) =
           make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+    };
+    // the early requests: back when at most the wave's tile copies are still out (four per k-step)
+    if (ktiles == RS_MAX_STEPS) wait_vmcnt<4 * RS_MAX_STEPS>();
+    else wait_vmcnt<0>();
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+#pragma unroll
+      for (int i = 0; i < NPRE; ++i) asm volatile("" : "+v"(e_ml[e][i]), "+v"(e_oa[e][i]), "+v"(e_ob[e][i]));
+      asm volatile("" : "+v"(e_len[e]));
+      const int item = tid + 256 * e;
+      if (item < m_items) {
+        int kt, m, c, d; long base;
+        item_place(item, kt, m, c, d, base);
+        finish(kt, m, c, d, base, e_len[e], e_ml[e], e_oa[e], e_ob[e]);
+      }
+    }
+    // more than NE items per thread (more than 8 rows): the rest by ordinary loads
+    for (int item = tid + 256 * NE; item < m_items; item += 256) {
+      int kt, m, c, d; long base;
+      item_place(item, kt, m, c, d, base);
+      f2_t ml[NPRE];
+      f4_t oa[NPRE], ob[NPRE];
+#pragma unroll
+      for (int i = 0; i < NPRE; ++i) {
+        const long at = base + min(i, np_max - 1);
+        ml[i] = *(const f2_t*)(p.part_ml + at * 2);
+        oa[i] = *(const f4_t*)(p.part_o + at * Dh + d);
+        ob[i] = *(const f4_t*)(p.part_o + at * Dh + d + 4);
+      }
+      finish(kt, m, c, d, base, p.part_seq_lens[m], ml, oa, ob);
     }
   }
   int x_off[4], w_off;
@@ -663,10 +717,16 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc, 0, 0, 0);
     }
   };
-  if (!MERGE && ktiles == RS_MAX_STEPS) {
-    // a full range: the steps are multiplied as they land (5 copy instructions per wave and step)
-#define RS_STEP(kt) wait_vmcnt<5 * (RS_MAX_STEPS - 1 - (kt))>(); __builtin_amdgcn_s_barrier(); step(kt);
-    RS_STEP(0) RS_STEP(1) RS_STEP(2) RS_STEP(3) RS_STEP(4) RS_STEP(5) RS_STEP(6) RS_STEP(7)
+  if (ktiles == RS_MAX_STEPS) {
+    // a full range: the steps are multiplied as they land (5 copy instructions per wave and step; 4 when the x tile
+    // is merged here, and then the first barrier also publishes the merged chunks, ordinary LDS stores of other waves)
+    constexpr int CPS = MERGE ? 4 : 5;
+    wait_vmcnt<CPS * (RS_MAX_STEPS - 1)>();
+    if (MERGE) __syncthreads();
+    else __builtin_amdgcn_s_barrier();
+    step(0);
+#define RS_STEP(kt) wait_vmcnt<CPS * (RS_MAX_STEPS - 1 - (kt))>(); __builtin_amdgcn_s_barrier(); step(kt);
+    RS_STEP(1) RS_STEP(2) RS_STEP(3) RS_STEP(4) RS_STEP(5) RS_STEP(6) RS_STEP(7)
 #undef RS_STEP
   } else {
     wait_vmcnt<0>();

@@ -48,10 +48,10 @@ def test_decode_workspace_for_shape_and_noalloc_limit(lib):
     assert 0 < exact <= upper and exact < 64 << 20          # no term that grows with max_seq_len
     assert lib.pa_decode_workspace_bytes_for(64, 32, 8, 128, 32, 1 << 20, 512, 0, 0) == 64 * 32 * 2048 * 130 * 4   # fp32
     # no bound (max_seq_len 0: pa_decode then uses the table capacity, unknown here): enough for the balanced schedule
-    # and for up to four fixed partitions, which a large batch of small capacity takes and which then needs more
+    # and for the fixed partitions of a small call (up to eight of the caller's, up to sixteen of the finer ones)
     for B in (4, 128, 600):
         unbounded = lib.pa_decode_workspace_bytes_for(B, 32, 8, 128, 32, 0, 512, 1, 1)
-        assert unbounded >= B * 32 * 4 * 130 * 4
+        assert unbounded >= B * 32 * 16 * 130 * 4
         for msl in (100, 512, 2048, 1 << 20):
             assert unbounded >= lib.pa_decode_workspace_bytes_for(B, 32, 8, 128, 32, msl, 512, 1, 1)
     z = ctypes.c_void_p(0)
@@ -112,6 +112,24 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert ver(win=-1) == -1 and b"sliding_window" in lib.pa_last_error()
     assert dec(win=-2) == -1 and b"sliding_window" in lib.pa_last_error()
     assert lib.pa_verify_workspace_bytes(0, 4, 8, 128) == 0
+    from nkipy_amd._lib import NewKvStruct, OutProjStruct
+    nkv, proj = NewKvStruct(None, None, None, None), OutProjStruct(None, None, None, 256)
+    def step(new_kv=ctypes.addressof(nkv), out_proj=None, **kw):
+        a = dict(B=2, Hq=8, Hkv=2, D=128, bs=16, mb=4, nb=8, msl=0, scale=1.0, part=512, qd=1, kd=1)
+        a.update(kw)
+        return lib.pa_decode_step(z, new_kv, z, z, z, z, z, z, z, out_proj, z, 0, a["B"], a["Hq"], a["Hkv"], a["D"], a["bs"],
+                                  a["mb"], a["nb"], a["msl"], a["scale"], a["part"], a["qd"], a["kd"], z, a.get("win", 0), z, z)
+    assert step(Hq=7) == -1 and b"multiple" in lib.pa_last_error()
+    assert step(D=96) == -1 and b"head_dim" in lib.pa_last_error()
+    assert step(win=-1) == -1 and b"sliding_window" in lib.pa_last_error()
+    assert step() == -1 and b"null" in lib.pa_last_error()
+    assert step(B=0, new_kv=None) == -1 and b"new_kv" in lib.pa_last_error()      # the call without a cache update is pa_decode
+    assert step(B=0) == 0
+    # what the one call needs covers what its three parts need
+    for B, msl in ((8, 1088), (1, 4096), (64, 8192)):
+        need = lib.pa_decode_step_workspace_bytes(B, 32, 8, 128, 32, msl, 512, 4096, 1, 1)
+        assert need >= lib.pa_decode_workspace_bytes_for(B, 32, 8, 128, 32, msl, 512, 1, 1) + lib.pa_o_proj_workspace_bytes(B, 4096, 4096) + B * 4096 * 2
+    assert lib.pa_decode_step_workspace_bytes(0, 32, 8, 128, 32, 100, 512, 4096, 1, 1) == 0
 
 
 def test_ops_refuse_host_arrays():

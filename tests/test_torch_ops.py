@@ -15,6 +15,8 @@ def test_ops_are_registered_with_mutation_schemas():
     assert "Tensor(a6!) out" in s and "-> ()" in s
     assert str(torch.ops.nkipy_amd.paged_kv_write.default._schema).count("!") == 2        # both caches
     assert str(torch.ops.nkipy_amd.paged_kv_write_fp8.default._schema).count("!") == 4    # ... and both scale tables
+    assert str(torch.ops.nkipy_amd.decode_step.default._schema).count("!") == 3           # both caches and out
+    assert str(torch.ops.nkipy_amd.decode_step_fp8.default._schema).count("!") == 5
 
 
 def test_ops_refuse_cpu_tensors_and_trace_with_fake_tensors():
@@ -25,6 +27,8 @@ def test_ops_refuse_cpu_tensors_and_trace_with_fake_tensors():
     sl = torch.ones(2, dtype=torch.int32)
     with pytest.raises(NotImplementedError):
         torch.ops.nkipy_amd.paged_decode(q, kc, kc, bt, sl, 0.1, torch.empty_like(q))
+    with pytest.raises(NotImplementedError):
+        torch.ops.nkipy_amd.decode_step(q, kc[:2, 0], kc[:2, 0], kc, kc, bt, sl, sl, 0.1, torch.empty_like(q))
     from torch._subclasses.fake_tensor import FakeTensorMode
     with FakeTensorMode():
         fq = torch.zeros(2, 4, 64, dtype=torch.bfloat16, device="cuda")
