@@ -101,9 +101,11 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * partitions; the default MFMA kernel for bf16 / fp8 KV instead cuts the
  * flattened stream of all sequences' 32-token tiles into equal chunks, one per
  * resident wavefront group, so its partition length follows the batch and the
- * device, not partition_size.  Small calls without sinks or a window (at most
- * four partitions per sequence and at most 288 MiB of K and V by max_seq_len)
- * take the fixed-partition MFMA kernel, whose fixed cost is lower.  The result
+ * device, not partition_size.  Small calls without sinks or a window (by max_seq_len:
+ * at most eight partitions per sequence, at most 80 (sequence, kv head) pairs and
+ * at most 160 MiB of K and V) take the fixed-partition MFMA kernel, whose fixed cost
+ * is lower, on partitions of 256 tokens when those of partition_size would give the
+ * device fewer than about 64 workgroups (a single sequence).  The result
  * does not depend on the split beyond the order of float32 sums.
  * max_seq_len: upper bound of seq_lens (sizes the grid and picks the kernel; 0 =
  * max_blocks_per_seq * block_size).  seq_lens[b] == 0 yields zeros.
@@ -160,8 +162,9 @@ int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
  *   workspace    pa_verify_workspace_bytes(B, T, Hq, D) bytes, 16-byte aligned
  *   sinks, sliding_window   as for pa_decode (the window counts back from each query token's own position)
  *   max_seq_len  0, or a host-known upper bound of seq_lens (longer contexts are read up to the bound).  The table
- *                capacity says nothing about the size of a call; with a bound, a small call -- at most four
- *                512-token partitions per sequence and little K and V in all, no sinks, no window: the
+ *                capacity says nothing about the size of a call; with a bound, a small call -- at most eight
+ *                512-token partitions per sequence, few sequences and little K and V in all (pa_decode's rule),
+ *                no sinks, no window: the
  *                reference's own use, one sequence and a handful of draft tokens -- runs on fixed partitions
  *                as a small pa_decode call does, without the balanced schedule's fixed cost.  Same workspace.
  * D in {64, 128}; block_size a power of two >= 16; T <= PA_VERIFY_MAX_TOKENS.

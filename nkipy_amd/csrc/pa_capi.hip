@@ -260,7 +260,7 @@ static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts
 static int decode_fine_partition(const DecodeParams& p) {
   const int kFine = g_decode_fine.load();
   if (kFine <= 0 || p.partition_size <= kFine || p.max_seq_len <= kFine) return p.partition_size;
-  const long slots = (long)p.Hkv * ((p.Hq / p.Hkv + 15) / 16);      // workgroups per sequence and partition
+  const long slots = (long)p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);      // workgroups per sequence and partition
   if (p.B * slots * num_partitions_for(p.max_seq_len, p.partition_size) > 64) return p.partition_size;
   if (num_partitions_for(p.max_seq_len, kFine) > 16) return p.partition_size;
   return kFine;
@@ -549,16 +549,26 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   if (take_q_transform(who, q_transform, true, p.qt)) return -1;
   if (max_seq_len > 0 && max_seq_len < p.max_seq_len) p.max_seq_len = max_seq_len;     // the caller's bound on the contexts
   // Small calls (the reference's own use of this path: one sequence, a handful of draft tokens) take fixed partitions,
-  // as small pa_decode calls do and for the same reason: the balanced schedule costs what it costs whatever the sizes
-  // (256 chunks, each leaving partials of 16 rows; B = 1, T = 4 behind 1 K tokens: 13.7 us per call replayed from a
-  // graph).  It needs the caller's bound on the lengths (the table capacity says nothing about the sizes), 16 rows
-  // per wave, no sinks and no window, and a workspace that holds the partitions' partials.
+  // as small pa_decode calls do, by the same rule and for the same reason: the balanced schedule costs what it costs
+  // whatever the sizes (256 chunks, each leaving partials of 16 rows).  Inside a verify step of eight attention layers
+  // (T = 4, 32 / 8 heads of 128, us per layer replayed from a graph, balanced / fixed partitions): B = 1 behind 4 K
+  // 36.0 / 32.9, B = 4 behind 2 K 41.4 / 34.4, B = 4 behind 4 K 47.6 / 38.1, B = 8 behind 2 K 46.8 / 44.0; a single
+  // sequence on the finer partitions, B = 1 behind 1 K: 30.5 -> 27.7.  It needs the caller's bound on the lengths (the
+  // table capacity says nothing about the sizes), 16 rows per wave, no sinks and no window, and a workspace that holds
+  // the partitions' partials.
   if (max_seq_len > 0 && !sinks && sliding_window == 0 && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
     DecodeParams f = p;
     f.partition_size = 512;
+    const bool small = decode_small_call(f, kv_dtype);
+    if (small) f.partition_size = decode_fine_partition(f);       // a single sequence: finer ones, as for pa_decode
     f.num_partitions = num_partitions_for(f.max_seq_len, f.partition_size);
-    const size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
-    if (decode_small_call(f, kv_dtype, 4) && (need_f == 0 || (workspace && workspace_bytes >= need_f))) {
+    size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
+    if (small && f.partition_size != 512 && need_f && !(workspace && workspace_bytes >= need_f)) {
+      f.partition_size = 512;
+      f.num_partitions = num_partitions_for(f.max_seq_len, f.partition_size);
+    }
+    need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
+    if (small && (need_f == 0 || (workspace && workspace_bytes >= need_f))) {
       f.head_major = g_head_major.load();
       f.ws_out = (float*)workspace;
       f.ws_ml = f.ws_out + (size_t)B * Hq * Tc * f.num_partitions * D;

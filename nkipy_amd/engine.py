@@ -232,9 +232,9 @@ class PagedAttention:
     xq / xk / xv as static buffers and replayed every step: `begin_step` stays outside the graph (it publishes
     the step's table rows and lengths, which the replayed kernels read from the same device tensors).  A captured
     decode step is sized by `max_seq_len`, the longest context it will be replayed on (default: the longest
-    sequence the cache admits).  The bound also picks the decode kernel: up to four partitions of
-    `partition_size` tokens take the fixed-partition kernel, which is what makes small steps cheap, longer
-    bounds the balanced one; the two agree to the order of their float32 sums, not bit for bit.
+    sequence the cache admits).  The bound also picks the decode kernel: a small batch with up to eight partitions
+    of `partition_size` tokens takes the fixed-partition kernel, which is what makes small steps cheap, longer
+    bounds and larger batches the balanced one; the two agree to the order of their float32 sums, not bit for bit.
     """
 
     def __init__(self, cache: PagedKVCache, n_heads: int, *, layer: int = 0, scale: Optional[float] = None,

@@ -295,7 +295,7 @@ def test_head_dim_64_many_rows_of_a_short_run_take_the_tiled_kernel(pa):
 @pytest.mark.parametrize("T,Hq,Hkv,D,bs", [(4, 32, 8, 128, 32), (8, 8, 2, 128, 16), (3, 40, 2, 64, 16), (5, 6, 2, 64, 64),
                                            (16, 16, 4, 128, 32), (7, 1, 1, 128, 32)])
 def test_verify_small_calls_with_a_length_bound(pa, T, Hq, Hkv, D, bs, fp8):
-    """With the caller's bound on the contexts a small call takes fixed partitions (one to four of 512 tokens): a
+    """With the caller's bound on the contexts a small call takes fixed partitions (one to eight of 512 tokens, or finer ones for a single sequence): a
     single sequence behind about 1 K tokens (the reference's own use), a ragged batch with an idle slot and a
     one-token sequence, contexts a few tokens past a partition boundary (the early query rows then see no key in
     the last partition and leave an empty partial), a bound far above the contexts (partitions with no tokens),
