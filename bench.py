@@ -104,10 +104,23 @@ def _measure(step, steps, warmup, lib):
     torch.cuda.synchronize()
     _collect_kernel_ms(lib, 0)
     sec_ev = block()
-    lib.pa_profile_enable(0)
     kms = _collect_kernel_ms(lib, 4 * steps)
+    # what the same pair of events reads around a kernel that does nothing, interleaved with real steps so that the
+    # device is in the state of the timed block: the share of `kms` that is not kernel time (a kernel trace, which
+    # stamps first wave to last, reads that much less than the events)
+    stream = torch.cuda.current_stream().cuda_stream
+    empty = []
+    for _ in range(10):
+        lib.pa_profile_enable(0)
+        step()
+        lib.pa_profile_enable(1)
+        lib.pa_profile_empty_launch(stream)
+        torch.cuda.synchronize()
+        empty += _collect_kernel_ms(lib, 4)
+    lib.pa_profile_enable(0)
     info = {"warmup_effective_steps": warmup + (blocks - 1) * steps, "warmup_converged": converged,
-            "ms_per_step_with_events": round(sec_ev * 1e3, 5)}
+            "ms_per_step_with_events": round(sec_ev * 1e3, 5),
+            "event_pair_around_empty_kernel_ms": round(float(np.median(empty)), 5) if empty else None}
     return sec, kms, info
 
 

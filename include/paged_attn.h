@@ -386,6 +386,10 @@ int pa_debug_set(int key, int value);
  * spike/src/spike/spike_model.py:290-363. */
 int pa_profile_enable(int on);
 int pa_profile_collect(float* ms, int cap);
+/* Launches a kernel that does nothing on `stream`, bracketed like the main kernels when timing is enabled: what
+ * pa_profile_collect then reports for it is the part of every such figure that is not kernel time (the events
+ * are stamped around the dispatch; a kernel trace reports first wave to last). */
+int pa_profile_empty_launch(void* stream);
 
 #ifdef __cplusplus
 }

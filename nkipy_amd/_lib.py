@@ -60,6 +60,7 @@ SIGNATURES = {
     "pa_debug_set": (c_int, [c_int, c_int]),
     "pa_profile_enable": (c_int, [c_int]),
     "pa_profile_collect": (c_int, [ctypes.POINTER(c_float), c_int]),
+    "pa_profile_empty_launch": (c_int, [c_void_p]),
 }
 
 

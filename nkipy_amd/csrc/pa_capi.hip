@@ -196,6 +196,19 @@ int pa_profile_collect(float* ms, int cap) {
   return n;
 }
 
+// What an event pair reads around a kernel that does nothing: the part of every pa_profile_collect figure that is
+// not the kernel (the events are stamped by the command processor around the dispatch, not by the kernel's first
+// and last wave, which is what a kernel trace reports).
+__global__ void profile_empty_kernel() {}
+int pa_profile_empty_launch(void* stream) {
+  hipStream_t s = (hipStream_t)stream;
+  profile_begin(s);
+  hipLaunchKernelGGL(profile_empty_kernel, dim3(1), dim3(64), 0, s);
+  hipError_t e = hipGetLastError();
+  profile_end(s);
+  return check_hip(e, "pa_profile_empty_launch");
+}
+
 // Checks an optional Q transform and copies it into the kernel parameters; returns 0 or -1.
 static int take_q_transform(const char* who, const pa_q_transform* qt, bool kernel_ok, QTransform& dst) {
   memset(&dst, 0, sizeof(dst));
