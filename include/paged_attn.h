@@ -293,6 +293,23 @@ typedef struct pa_out_proj {
 } pa_out_proj;
 size_t pa_decode_step_workspace_bytes(int B, int Hq, int Hkv, int D, int block_size, int max_seq_len, int partition_size,
                                       int N, int q_dtype, int kv_dtype);
+/*
+ * The same for a step of up to PA_VERIFY_MAX_TOKENS tokens per sequence: a speculative verify step of a layer
+ * (examples/models/gpt_oss/kernels/attention.py:80-163 with seq_len = K + 1, called from peagle/speculate.py:137-202)
+ * in one call, bit for bit pa_qk_norm_rope_kv_write (pa_kv_write without q_transform) + pa_verify + pa_o_proj_ws.
+ *   q [B, T, Hq, D] bf16; new_kv: xk, xv [B, T, Hkv, D], query_lens [B] (0 .. T new tokens per sequence; rows
+ *   t >= query_lens[b] are padding), k_norm_weight as for pa_decode_step; attn_out [B, T, Hq, D] or NULL;
+ *   out_proj->out [B, T, N]; workspace pa_verify_step_workspace_bytes(B, T, Hq, D, N) bytes; max_seq_len as for
+ *   pa_verify (with a bound, a small call merges its split-K partials on the projection's load: four launches
+ *   instead of five).
+ */
+size_t pa_verify_step_workspace_bytes(int B, int T, int Hq, int D, int N);
+int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* v_cache, float* k_scale, float* v_scale,
+                   const int32_t* block_tables, const int32_t* seq_lens, void* attn_out, const pa_out_proj* out_proj,
+                   void* workspace, size_t workspace_bytes,
+                   int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks,
+                   int max_seq_len, float scale, int kv_dtype,
+                   const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream);
 int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* v_cache, float* k_scale, float* v_scale,
                    const int32_t* block_tables, const int32_t* seq_lens, void* attn_out, const pa_out_proj* out_proj,
                    void* workspace, size_t workspace_bytes,

@@ -54,6 +54,8 @@ SIGNATURES = {
     "pa_o_proj_workspace_bytes": (c_size_t, [c_int] * 3),
     "pa_decode_step_workspace_bytes": (c_size_t, [c_int] * 10),
     "pa_decode_step": (c_int, [c_void_p] * 11 + [c_size_t] + [c_int] * 8 + [c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
+    "pa_verify_step_workspace_bytes": (c_size_t, [c_int] * 5),
+    "pa_verify_step": (c_int, [c_void_p] * 11 + [c_size_t] + [c_int] * 9 + [c_float, c_int, c_void_p, c_int, c_void_p, c_void_p]),
     "pa_gather_kv": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_void_p]),
     "pa_kv_write": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_void_p]),
     "pa_qk_norm_rope_kv_write": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 2 + [c_int] + [c_void_p] * 7 + [c_int] * 9 + [c_void_p]),

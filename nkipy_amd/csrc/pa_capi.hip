@@ -524,6 +524,15 @@ int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
                    max_seq_len, scale, partition_size, q_dtype, kv_dtype, sinks, sliding_window, q_transform, stream);
 }
 
+// A caller of verify_launch that can consume the fixed-partition route's split-K partials itself (the projection of
+// pa_verify_step) asks for them here: when the call takes that route with more than one partition, the merge launch
+// is left out and `f` says where the partials are.
+struct VerifyPartials {
+  bool want;
+  bool left;
+  DecodeParams f;
+};
+
 // Query tokens [t0, t0 + Tc) of the T tokens per sequence through the decode-shaped kernel (pa_verify: all
 // of them in one launch; pa_prefill for shapes the tiled kernel does not take: 64 at a time).
 static int verify_launch(const char* who, const void* q, const void* k_cache, const void* v_cache,
@@ -532,10 +541,12 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
                          void* out, void* workspace, size_t workspace_bytes,
                          int B, int T, int t0, int Tc, int Hq, int Hkv, int D, int block_size,
                          int max_blocks_per_seq, int num_blocks, int max_seq_len, float scale, int kv_dtype,
-                         const float* sinks, int sliding_window, const pa_q_transform* q_transform, hipStream_t s) {
+                         const float* sinks, int sliding_window, const pa_q_transform* q_transform, hipStream_t s,
+                         VerifyPartials* vp = nullptr) {
   const long cap = (long)max_blocks_per_seq * block_size;
   DecodeParams p;
   memset(&p, 0, sizeof(p));
+  if (vp) vp->left = false;
   p.q = q; p.k_cache = k_cache; p.v_cache = v_cache; p.k_scale = k_scale; p.v_scale = v_scale;
   p.block_tables = block_tables; p.seq_lens = seq_lens; p.query_lens = query_lens; p.out = out;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.D = D; p.T = Tc; p.T_stride = T; p.t0 = t0;
@@ -589,6 +600,11 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
       hipError_t e = launch_decode_mfma(f, kv_dtype, 0, s);
       profile_end(s);
       if (e != hipSuccess) return check_hip(e, "verify kernel launch");
+      if (vp && vp->want && f.num_partitions > 1) {
+        vp->left = true;
+        vp->f = f;
+        return 0;
+      }
       if (f.num_partitions > 1) e = launch_decode_reduce(f, PA_BF16, s);
       return check_hip(e, "verify merge launch");
     }
@@ -1012,6 +1028,7 @@ int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   if (merge_on_load && p.num_partitions > 1) {
     o.part_o = p.ws_out; o.part_ml = p.ws_ml; o.part_seq_lens = seq_lens;
     o.part_np = p.num_partitions; o.part_size = p.partition_size; o.part_max_seq_len = p.max_seq_len; o.part_D = D;
+    o.part_T = 1; o.part_n_rep = Hq / Hkv;
   } else {
     o.x = attn;
   }
@@ -1019,6 +1036,108 @@ int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   hipError_t e = launch_o_proj(o, s);
   profile_end(s);
   return check_hip(e, "pa_decode_step projection launch");
+}
+
+size_t pa_verify_step_workspace_bytes(int B, int T, int Hq, int D, int N) {
+  if (B <= 0 || T <= 0 || Hq <= 0 || D <= 0 || N < 0 || (long)B * T > 0x7fffffffL) return 0;
+  const size_t proj = N > 0 ? pa_o_proj_workspace_bytes(B * T, Hq * D, N) : 0;
+  return align256(pa_verify_workspace_bytes(B, T, Hq, D)) + align256(proj) + align256((size_t)B * T * Hq * D * 2) + 256;
+}
+
+int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* v_cache, float* k_scale, float* v_scale,
+                   const int32_t* block_tables, const int32_t* seq_lens, void* attn_out, const pa_out_proj* proj,
+                   void* workspace, size_t workspace_bytes,
+                   int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq, int num_blocks,
+                   int max_seq_len, float scale, int kv_dtype,
+                   const float* sinks, int sliding_window, const pa_q_transform* q_transform, void* stream) {
+  tl_error[0] = 0;
+  const char* who = "pa_verify_step";
+  if (!new_kv) return fail_arg("%s: new_kv is required (pa_verify is the call without a cache update)", who);
+  if (B < 0 || T < 0 || Hq <= 0 || Hkv <= 0 || D <= 0) return fail_arg("%s: bad sizes", who);
+  if (T > PA_VERIFY_MAX_TOKENS) return fail_arg("%s: T=%d exceeds %d query tokens per sequence", who, T, PA_VERIFY_MAX_TOKENS);
+  if (new_kv->k_norm_weight && !q_transform)
+    return fail_arg("%s: k_norm_weight comes with q_transform (the norm and rotation are applied to Q and K alike)", who);
+  if (!attn_out && !proj) return fail_arg("%s: neither attn_out nor out_proj given", who);
+  const int K = Hq * D;
+  int N = 0;
+  if (proj) {
+    N = proj->N;
+    if (!proj->o_weight || !proj->out) return fail_arg("%s: out_proj needs o_weight and out", who);
+    if (N <= 0 || N % 8) return fail_arg("%s: N=%d must be a positive multiple of 8", who, N);
+    if (K % 64) return fail_arg("%s: Hq * head_dim = %d must be a multiple of 64", who, K);
+    if ((long)N * 2 * 64 > 0xffffffffL || (long)K * 2 * 256 > 0xffffffffL)
+      return fail_arg("%s: row of %d (K) or %d (N) elements too long for 32-bit tile offsets", who, K, N);
+    if (!aligned16(proj->o_weight) || !aligned16(proj->o_bias) || !aligned16(proj->out))
+      return fail_arg("%s: o_weight, o_bias and out must be 16-byte aligned", who);
+  }
+  if (!aligned16(workspace) || !aligned16(attn_out)) return fail_arg("%s: workspace and attn_out must be 16-byte aligned", who);
+  // the cache update (argument checks of its own), then the attention, then the projection
+  int rc;
+  if (q_transform)
+    rc = pa_qk_norm_rope_kv_write(nullptr, new_kv->xk, new_kv->xv, nullptr, nullptr, new_kv->k_norm_weight,
+                                  q_transform->norm_eps, q_transform->rope_cos, q_transform->rope_sin,
+                                  q_transform->rope_max_pos, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens,
+                                  new_kv->query_lens, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks,
+                                  kv_dtype, stream);
+  else
+    rc = pa_kv_write(new_kv->xk, new_kv->xv, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens,
+                     new_kv->query_lens, B, T, Hkv, D, block_size, max_blocks_per_seq, num_blocks, kv_dtype, stream);
+  if (rc) return rc;
+  if (B == 0 || T == 0) return 0;
+  if (Hq % Hkv) return fail_arg("%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
+  if (kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN) return fail_arg("%s: kv_dtype must be bf16 or fp8-e4m3fn", who);
+  if (!q) return fail_arg("%s: null pointer argument", who);
+  const long M = (long)B * T;
+  hipStream_t s = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  size_t avail = workspace ? workspace_bytes & ~(size_t)255 : 0;
+  void* attn = attn_out;
+  if (!attn) {
+    const size_t need = align256((size_t)M * K * 2);
+    if (avail < need) return fail_arg("%s: workspace of %zu bytes too small (pa_verify_step_workspace_bytes)", who, workspace_bytes);
+    avail -= need;
+    attn = ws + avail;
+  }
+  int splits = 1;
+  float* proj_ws = nullptr;
+  if (proj) {
+    const size_t per_split = (size_t)M * N * sizeof(float);
+    int want = o_proj_splits((int)M, K, N);
+    if (align256((size_t)want * per_split) > avail) want = (int)(avail / per_split);
+    if (want > 1) {
+      splits = want;
+      avail -= align256((size_t)splits * per_split);
+      proj_ws = (float*)(ws + avail);
+    }
+  }
+  VerifyPartials vp;
+  vp.want = proj && !attn_out && g_step_fusion.load() != 1 && g_step_fusion.load() != 2 &&
+            o_proj_takes_partials((int)M, K, D, splits, proj_ws != nullptr);
+  rc = verify_launch(who, q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, new_kv->query_lens, attn, ws, avail,
+                     B, T, 0, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks, max_seq_len, scale, kv_dtype, sinks,
+                     sliding_window, q_transform, s, &vp);
+  if (rc || !proj) return rc;
+  if (vp.left && vp.f.num_partitions > 4) {
+    // the projection requests up to four partitions ahead of its weight tiles; more are merged by the launch after all
+    hipError_t e = launch_decode_reduce(vp.f, PA_BF16, s);
+    if (e != hipSuccess) return check_hip(e, "verify merge launch");
+    vp.left = false;
+  }
+  OProjParams o;
+  memset(&o, 0, sizeof(o));
+  o.w = proj->o_weight; o.bias = proj->o_bias; o.out = proj->out; o.M = (int)M; o.K = K; o.N = N;
+  o.splits = splits; o.ws = proj_ws;
+  if (vp.left) {
+    o.part_o = vp.f.ws_out; o.part_ml = vp.f.ws_ml; o.part_seq_lens = seq_lens; o.part_query_lens = new_kv->query_lens;
+    o.part_np = vp.f.num_partitions; o.part_size = vp.f.partition_size; o.part_max_seq_len = vp.f.max_seq_len; o.part_D = D;
+    o.part_T = T; o.part_n_rep = Hq / Hkv;
+  } else {
+    o.x = attn;
+  }
+  profile_begin(s);
+  hipError_t e = launch_o_proj(o, s);
+  profile_end(s);
+  return check_hip(e, "pa_verify_step projection launch");
 }
 
 int pa_gather_kv(const void* cache, const int32_t* block_tables, const int32_t* seq_lens,

@@ -320,12 +320,14 @@ struct OProjParams {
   float* ws;                // split form: [splits, M, N] float32 partial products, or null
   int splits;               // K ranges summed by a second kernel (1: none); o_proj_splits() or less
   // The resident few-rows form can take its x rows from the split-K partials of a fixed-partition decode launch
-  // instead of from memory (x null): row b of x is sequence b's attention output [Hq * D], merged from the
-  // sequence's partitions while the tile is formed, with the arithmetic of decode_reduce_kernel.
-  const float* part_o;      // [M, Hq, np, D] normalised partial outputs
-  const float* part_ml;     // [M, Hq, np, 2] (max, sum) of each partial
-  const int32_t* part_seq_lens;   // [M] context lengths (clamped to part_max_seq_len as the decode launch did)
+  // instead of from memory (x null): row m of x is the attention output [Hq * D] of one (sequence, query token),
+  // merged from the sequence's partitions while the tile is formed, with the arithmetic of decode_reduce_kernel.
+  const float* part_o;      // [B, Hq * T rows, np, D] normalised partial outputs (rows numbered as the decode kernels do)
+  const float* part_ml;     // [B, Hq * T rows, np, 2] (max, sum) of each partial
+  const int32_t* part_seq_lens;   // [B] context lengths (clamped to part_max_seq_len as the decode launch did)
+  const int32_t* part_query_lens; // multi-token launch: [B] query tokens per sequence; null for decode
   int part_np, part_size, part_max_seq_len, part_D;
+  int part_T, part_n_rep;         // tokens per sequence in the launch (x row m is token m % T of sequence m / T), q heads per kv head
 };
 hipError_t launch_o_proj(const OProjParams& p, hipStream_t s);
 int o_proj_splits(int M, int K, int N);     // K ranges the few-rows forms would like to spread over more workgroups

@@ -579,9 +579,11 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
   typedef float f4_t __attribute__((ext_vector_type(4)));
   f2_t e_ml[NE][NPRE];
   f4_t e_oa[NE][NPRE], e_ob[NE][NPRE];
-  int e_len[NE];
+  int e_len[NE], e_qlen[NE];
   const int m_items = MERGE ? ktiles * 8 * p.M : 0;
-  auto item_place = [&](int item, int& kt, int& m, int& c, int& d, long& base) __attribute__((always_inline)) {
+  // x row m is query token m % T of sequence m / T; its q head `head` is row hk n_rep T + t n_rep + j of the sequence's
+  // partials, the decode kernels' numbering of (token, head) pairs (T = 1: the q head itself)
+  auto item_place = [&](int item, int& kt, int& m, int& c, int& d, long& base, int& b) __attribute__((always_inline)) {
     const int per_step = 8 * p.M;
     kt = item / per_step;
     const int rem = item - kt * per_step;
@@ -589,15 +591,31 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     const int k0 = (kt_begin + kt) * BK + 8 * c;
     const int head = k0 / p.part_D;
     d = k0 - head * p.part_D;
-    base = ((long)m * (p.K / p.part_D) + head) * p.part_np;
+    const int T = p.part_T, n_rep = p.part_n_rep;
+    b = m / T;
+    const int t = m - b * T, hk = head / n_rep;
+    const int vr = hk * n_rep * T + t * n_rep + (head - hk * n_rep);
+    base = ((long)b * (p.K / p.part_D) * T + vr) * p.part_np;
+  };
+  // the keys the launch gave sequence b: its length, clamped as the launch clamped it; none when a multi-token launch
+  // finds no query token for it
+  auto context_of = [&](int len, int qlen) __attribute__((always_inline)) -> int {
+    int ctx = min(max(len, 0), p.part_max_seq_len);
+    if (p.part_query_lens && min(min(max(qlen, 0), p.part_T), ctx) <= 0) ctx = 0;
+    return ctx;
   };
   if (MERGE) {
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
-      int kt, m, c, d; long base;
-      item_place(min(tid + 256 * e, m_items - 1), kt, m, c, d, base);
-      const int32_t* plen = p.part_seq_lens + m;
+      int kt, m, c, d, b; long base;
+      item_place(min(tid + 256 * e, m_items - 1), kt, m, c, d, base, b);
+      const int32_t* plen = p.part_seq_lens + b;
       asm volatile("global_load_dword %0, %1, off" : "=&v"(e_len[e]) : "v"(plen) : "memory");
+      e_qlen[e] = 1;
+      if (p.part_query_lens) {
+        const int32_t* pq = p.part_query_lens + b;
+        asm volatile("global_load_dword %0, %1, off" : "=&v"(e_qlen[e]) : "v"(pq) : "memory");
+      }
 #pragma unroll
       for (int i = 0; i < NPRE; ++i) {
         const long at = base + min(i, p.part_np - 1);
@@ -627,9 +645,8 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     // one q head.  Up to NPRE partitions' values are requested before any is used (slots past a sequence's own
     // partition count exist and are loaded, not used).
     const int Dh = p.part_D, np_max = p.part_np;
-    auto finish = [&](int kt, int m, int c, int d, long base, int len, const f2_t (&ml)[NPRE], const f4_t (&oa)[NPRE],
+    auto finish = [&](int kt, int m, int c, int d, long base, int ctx, const f2_t (&ml)[NPRE], const f4_t (&oa)[NPRE],
                       const f4_t (&ob)[NPRE]) __attribute__((always_inline)) {
-      const int ctx = min(max(len, 0), p.part_max_seq_len);
       const int np = min((ctx + p.part_size - 1) / p.part_size, np_max);
       float mt = -INFINITY;
 #pragma unroll
@@ -668,18 +685,18 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     for (int e = 0; e < NE; ++e) {
 #pragma unroll
       for (int i = 0; i < NPRE; ++i) asm volatile("" : "+v"(e_ml[e][i]), "+v"(e_oa[e][i]), "+v"(e_ob[e][i]));
-      asm volatile("" : "+v"(e_len[e]));
+      asm volatile("" : "+v"(e_len[e]), "+v"(e_qlen[e]));
       const int item = tid + 256 * e;
       if (item < m_items) {
-        int kt, m, c, d; long base;
-        item_place(item, kt, m, c, d, base);
-        finish(kt, m, c, d, base, e_len[e], e_ml[e], e_oa[e], e_ob[e]);
+        int kt, m, c, d, b; long base;
+        item_place(item, kt, m, c, d, base, b);
+        finish(kt, m, c, d, base, context_of(e_len[e], e_qlen[e]), e_ml[e], e_oa[e], e_ob[e]);
       }
     }
     // more than NE items per thread (more than 8 rows): the rest by ordinary loads
     for (int item = tid + 256 * NE; item < m_items; item += 256) {
-      int kt, m, c, d; long base;
-      item_place(item, kt, m, c, d, base);
+      int kt, m, c, d, b; long base;
+      item_place(item, kt, m, c, d, base, b);
       f2_t ml[NPRE];
       f4_t oa[NPRE], ob[NPRE];
 #pragma unroll
@@ -689,7 +706,7 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
         oa[i] = *(const f4_t*)(p.part_o + at * Dh + d);
         ob[i] = *(const f4_t*)(p.part_o + at * Dh + d + 4);
       }
-      finish(kt, m, c, d, base, p.part_seq_lens[m], ml, oa, ob);
+      finish(kt, m, c, d, base, context_of(p.part_seq_lens[b], p.part_query_lens ? p.part_query_lens[b] : 1), ml, oa, ob);
     }
   }
   int x_off[4], w_off;
@@ -855,9 +872,13 @@ int o_proj_splits(int M, int K, int N) {
   return s < 2 ? 1 : (int)s;
 }
 
+// Worth it while a thread has at most the two items whose loads go out ahead of the weight tiles (8 rows at 8 k-steps
+// per range: a verify step of 32 rows took 41 us per layer with the merge here, 35 with the merge launch)
 bool o_proj_takes_partials(int M, int K, int D, int splits, bool have_ws) {
   const int r = o_proj_resident_splits(M, K);
-  return r > 0 && splits == r && (r == 1 || have_ws) && (D == 64 || D == 128) && K % D == 0;
+  if (!(r > 0 && splits == r && (r == 1 || have_ws) && (D == 64 || D == 128) && K % D == 0)) return false;
+  const int ktiles = (K / BK + r - 1) / r;
+  return (long)M * 8 * ktiles <= 512;
 }
 
 static std::atomic<int> g_o_proj_force_large{0};

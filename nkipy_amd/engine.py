@@ -337,6 +337,23 @@ class PagedAttention:
                                    o_weight=self.o_weight, o_bias=self.o_bias, out=proj[:, 0],
                                    sinks=self.sinks, sliding_window=self.sliding_window)
             return proj
+        if T > 1 and (self.rope is None or paged_attn.q_transform_supported(T, c.head_dim, c.block_size)) and \
+                paged_attn.prefill_route(B, T, self.n_heads, c.n_kv_heads, c.head_dim, c.block_size, ks is not None,
+                                         self.sliding_window or 0) == "verify":
+            # a verify step (a few tokens per sequence through the decode-shaped kernel): one call as well
+            qt = self._q_transform()
+            kw = dict(k_scale=ks, v_scale=vs, max_seq_len=bound, q_transform=qt,
+                      k_norm_weight=None if self.rope is None else self.k_norm_weight, sinks=self.sinks,
+                      sliding_window=self.sliding_window)
+            if self.o_weight is None:
+                paged_attn.verify_step(xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale, out=out, **kw)
+                return out
+            proj = self._proj.get(T)
+            if proj is None:
+                proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
+            paged_attn.verify_step(xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
+                                   o_weight=self.o_weight, o_bias=self.o_bias, out=proj, **kw)
+            return proj
         qt = None
         if self.rope is not None:
             # the Q half of the norm and rotation rides on the attention kernel's Q load where that

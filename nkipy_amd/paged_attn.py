@@ -316,6 +316,19 @@ VERIFY_MAX_ROWS = 32
 VERIFY_MAX_ROWS_FP8 = 256     # fp8 pools: the tiled kernel has no packed-rows form for them (B = 64, 4 K prefix: T = 64 718 vs 810 us)
 
 
+def prefill_route(B, T, Hq, Hkv, D, block_size, fp8=False, window=0) -> str:
+    """Which kernel `prefill` takes for a shape: "verify" (the decode-shaped kernel) or "tiled"."""
+    can_verify = verify_supported(T, D, block_size)
+    # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
+    rows = T * (Hq // Hkv)
+    if D == 64:
+        # the tiled kernel takes head dim 64 two kv heads at a time (not a single kv head); below 320 rows per kv head, and for small
+        # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself)
+        return "tiled" if not can_verify or (Hkv >= 2 and B >= 8 and rows >= 320) else "verify"
+    return "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
+                                       or (fp8 and (window > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"
+
+
 def verify_supported(T, D, block_size) -> bool:
     """Shapes the verify kernel is built for."""
     return T <= 64 and D in (64, 128) and block_size >= 16 and block_size & (block_size - 1) == 0
@@ -371,15 +384,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     sinks, win = _check_variant(sinks, sliding_window, Hq, q)
     can_verify = verify_supported(T, D, block_size)
     if route is None:
-        # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
-        rows = T * (Hq // Hkv)
-        if D == 64:
-            # the tiled kernel takes head dim 64 two kv heads at a time (not a single kv head); below 320 rows per kv head, and for small
-            # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself)
-            route = "tiled" if not can_verify or (Hkv >= 2 and B >= 8 and rows >= 320) else "verify"
-        else:
-            route = "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
-                                                or (kv_code == FP8 and (win > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"
+        route = prefill_route(B, T, Hq, Hkv, D, block_size, kv_code == FP8, win)
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")
@@ -804,6 +809,106 @@ def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens
 
 
 _decode_step_need = {}
+
+
+def verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
+                max_seq_len=None, q_transform=None, k_norm_weight=None, o_weight=None, o_bias=None, out=None,
+                attn_out=None, workspace=None, sinks=None, sliding_window=None):
+    """A speculative verify step of an attention layer in one call: `decode_step` for up to 64 new tokens per sequence
+    (examples/models/gpt_oss/kernels/attention.py:80-163 with seq_len = K + 1; peagle/speculate.py:137-202).
+
+    Bit for bit `qk_norm_rope_kv_write(None, xk, xv, ...)` (`kv_write` without `q_transform`), `verify(xq, ...)`,
+    `o_proj(...)`.  xq [B, T, Hq, D], xk / xv [B, T, Hkv, D] bfloat16; query_lens [B]: new tokens per sequence (rows
+    t >= query_lens[b] are padding: zero attention output, bias after the projection).  Returns [B, T, N] with
+    `o_weight`, else the attention output [B, T, Hq, D]."""
+    lib = _lib.load()
+    for n, t in (("xq", xq), ("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
+                 ("block_tables", block_tables), ("seq_lens", seq_lens), ("query_lens", query_lens)):
+        _need_device(n, t)
+    _check(xq.dim() == 4, "xq must be [B, T, Hq, D]")
+    B, T, Hq, D = xq.shape
+    _check(xq.dtype == torch.bfloat16, "verify_step supports bfloat16 rows only")
+    _check_paging(k_cache, v_cache, block_tables, seq_lens, B)
+    num_blocks, block_size, Hkv, Dk = k_cache.shape
+    _check(Dk == D, f"head_dim mismatch: xq has {D}, cache has {Dk}")
+    _check(Hq % Hkv == 0, f"Hq={Hq} is not a multiple of Hkv={Hkv}")
+    _check(verify_supported(T, D, block_size),
+           f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 (T={T}, D={D}, block_size={block_size})")
+    _check(tuple(xk.shape) == (B, T, Hkv, D) and xv.shape == xk.shape and xk.dtype == xq.dtype and xv.dtype == xq.dtype,
+           f"xk and xv must be bfloat16 [B, T, Hkv, D] = {(B, T, Hkv, D)}")
+    _check(query_lens.shape == (B,) and query_lens.dtype == torch.int32, "query_lens must be int32 [B]")
+    scaled = k_scale is not None or v_scale is not None
+    kv_code = _kv_code(k_cache, scaled)
+    _check(kv_code in (BF16, FP8), "verify_step needs a bfloat16 or fp8 KV cache")
+    if kv_code == FP8:
+        _check(k_scale is not None and v_scale is not None, "fp8 KV needs both k_scale and v_scale")
+        for n, t in (("k_scale", k_scale), ("v_scale", v_scale)):
+            _need_device(n, t)
+            _check(t.dtype == torch.float32 and t.shape == (num_blocks, Hkv), f"{n} must be float32 [num_blocks, Hkv]")
+    else:
+        _check(not scaled, "k_scale/v_scale are only valid with an fp8 KV cache")
+    sinks, win = _check_variant(sinks, sliding_window, Hq, xq)
+    cap = block_tables.shape[1] * block_size
+    msl = 0 if max_seq_len is None else int(max_seq_len)
+    _check(max_seq_len is None or 0 < msl <= cap, f"max_seq_len {msl} outside (0, {cap}]")
+    if k_norm_weight is not None:
+        _need_device("k_norm_weight", k_norm_weight)
+        _check(q_transform is not None, "k_norm_weight comes with q_transform")
+        _check(tuple(k_norm_weight.shape) == (D,) and k_norm_weight.dtype == torch.bfloat16, "k_norm_weight must be bfloat16 [D]")
+    N = 0
+    if o_weight is not None:
+        _need_device("o_weight", o_weight)
+        _check(o_weight.dtype == torch.bfloat16 and o_weight.dim() == 2 and o_weight.shape[0] == Hq * D,
+               f"o_weight must be bfloat16 [Hq * D = {Hq * D}, N]")
+        N = o_weight.shape[1]
+        _check((Hq * D) % 64 == 0 and N % 8 == 0, f"Hq * D = {Hq * D} must be a multiple of 64 and N = {N} of 8")
+        if o_bias is not None:
+            _need_device("o_bias", o_bias)
+            _check(o_bias.dtype == torch.bfloat16 and tuple(o_bias.shape) == (N,), "o_bias must be bfloat16 [N]")
+        if out is None:
+            out = torch.empty((B, T, N), dtype=torch.bfloat16, device=xq.device)
+        else:
+            _need_device("out", out)
+            _check(tuple(out.shape) == (B, T, N) and out.dtype == torch.bfloat16, f"out must be bfloat16 {(B, T, N)}")
+        if attn_out is not None:
+            _need_device("attn_out", attn_out)
+            _check(attn_out.shape == xq.shape and attn_out.dtype == xq.dtype, "attn_out must match xq in shape and dtype")
+    else:
+        _check(o_bias is None and attn_out is None, "o_bias and attn_out come with o_weight (without it `out` is the attention output)")
+        if out is None:
+            out = torch.empty_like(xq)
+        else:
+            _need_device("out", out)
+            _check(out.shape == xq.shape and out.dtype == xq.dtype, "out must match xq in shape and dtype")
+        attn_out = out
+    _same_device(xq, xk=xk, xv=xv, k_cache=k_cache, v_cache=v_cache, block_tables=block_tables, seq_lens=seq_lens,
+                 query_lens=query_lens, k_scale=k_scale, v_scale=v_scale, out=out, attn_out=attn_out, o_weight=o_weight,
+                 o_bias=o_bias, k_norm_weight=k_norm_weight)
+    key = ("v", B, T, Hq, D, N)
+    need = _decode_step_need.get(key)
+    if need is None:
+        with _on(xq.device):
+            need = _decode_step_need[key] = int(lib.pa_verify_step_workspace_bytes(B, T, Hq, D, N))
+    stream = _stream_ptr(xq.device)
+    if workspace is None:
+        workspace = _workspace(xq.device, need, stream)
+    else:
+        _need_device("workspace", workspace)
+        _check(workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.data_ptr() % 16 == 0,
+               "workspace must be a contiguous, 16-byte aligned uint8 tensor")
+        _check(workspace.numel() >= need, f"workspace needs {need} bytes")
+    qt_keep, qt_ptr = _qt_arg(q_transform, D, xq)
+    addr = lambda t: None if t is None else t.data_ptr()
+    nkv = _lib.NewKvStruct(addr(xk), addr(xv), addr(k_norm_weight), addr(query_lens))
+    proj = None if o_weight is None else _lib.OutProjStruct(addr(o_weight), addr(o_bias), addr(out), N)
+    with _on(xq.device):
+        rc = lib.pa_verify_step(_ptr(xq), ctypes.addressof(nkv), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+                                _ptr(block_tables), _ptr(seq_lens), _ptr(attn_out),
+                                None if proj is None else ctypes.addressof(proj), _ptr(workspace), workspace.numel(),
+                                B, T, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
+                                float(scale), kv_code, _ptr(sinks), win, qt_ptr, stream)
+    _raise_on(rc, "pa_verify_step")
+    return out
 def o_proj_workspace_bytes(M: int, K: int, N: int) -> int:
     """Scratch bytes `o_proj` would use for a call of M rows (0 for shapes that take none)."""
     return int(_lib.load().pa_o_proj_workspace_bytes(int(M), int(K), int(N)))

@@ -325,3 +325,100 @@ def test_argument_errors(pa):
                        o_weight=d["ow"], workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
     with pytest.raises(NotImplementedError):
         pa.decode_step(d["xq"].cpu(), d["xk"], d["xv"], d["k"], d["v"], d["tables"], d["lens"], d["qlens"], scale)
+
+
+# ---- the same for a few tokens per sequence: verify_step -----------------------------------------------------------
+
+def _setup_multi(rng, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, bias, xform, fp8=False):
+    d = _setup(rng, B, Hq, Hkv, D, bs, ctxs, qlens, N, bias, xform, fp8=fp8, poison=not fp8)
+    d["xq"] = bf16_to_dev(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    d["xk"] = bf16_to_dev(rng.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    d["xv"] = bf16_to_dev(rng.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    return d
+
+
+def _verify_three_calls(pa, d, scale, msl, **kw):
+    k, v = d["k"].clone(), d["v"].clone()
+    ks = None if d["ks"] is None else d["ks"].clone()
+    vs = None if d["vs"] is None else d["vs"].clone()
+    if d["qt"] is not None:
+        pa.qk_norm_rope_kv_write(None, d["xk"], d["xv"], k, v, d["tables"], d["lens"], d["qlens"], d["qt"].rope_cos,
+                                 d["qt"].rope_sin, k_norm_weight=d["wk"], eps=d["qt"].eps, k_scale=ks, v_scale=vs)
+    else:
+        pa.kv_write(d["xk"], d["xv"], k, v, d["tables"], d["lens"], d["qlens"], k_scale=ks, v_scale=vs)
+    att = pa.verify(d["xq"], k, v, d["tables"], d["lens"], d["qlens"], scale, k_scale=ks, v_scale=vs, max_seq_len=msl,
+                    q_transform=d["qt"], **kw)
+    out = att if d["ow"] is None else pa.o_proj(att, d["ow"], d["ob"])
+    return out, att, k, v, ks, vs
+
+
+def _verify_step(pa, d, scale, msl, **kw):
+    k, v = d["k"].clone(), d["v"].clone()
+    ks = None if d["ks"] is None else d["ks"].clone()
+    vs = None if d["vs"] is None else d["vs"].clone()
+    out = pa.verify_step(d["xq"], d["xk"], d["xv"], k, v, d["tables"], d["lens"], d["qlens"], scale, k_scale=ks, v_scale=vs,
+                         max_seq_len=msl, q_transform=d["qt"], k_norm_weight=d["wk"], o_weight=d["ow"], o_bias=d["ob"], **kw)
+    return out, k, v, ks, vs
+
+
+VERIFY_CASES = [
+    # B, T, Hq, Hkv, D, bs, contexts (new tokens counted), query lens, N, bias, transform, bound given, fp8
+    (1, 4, 32, 8, 128, 32, [1030], [4], 4096, False, True, True, False),           # the reference's own use: one sequence, K + 1 = 4
+    (8, 4, 32, 8, 128, 32, [1027, 1000, 513, 515, 516, 64, 3, 300], [4, 3, 4, 4, 4, 2, 3, 0], 4096, True, True, True, False),
+    (2, 8, 16, 8, 64, 16, [2050, 700], [8, 5], 512, False, True, True, False),     # head dim 64, five partitions
+    (3, 16, 8, 8, 128, 32, [900, 40, 16], [16, 7, 16], 256, True, False, True, False),   # no GQA: 16 rows per kv head
+    (4, 4, 32, 8, 128, 32, [1500, 600, 90, 5], [4, 4, 1, 4], 1024, False, True, False, False),   # no bound: the balanced schedule
+    (4, 4, 32, 8, 128, 32, [1500, 600, 90, 5], [4, 4, 1, 4], 1024, True, True, True, True),     # fp8 pool
+    (16, 4, 32, 8, 128, 32, [700 + 31 * i for i in range(16)], [4] * 16, 1024, False, True, True, False),   # 64 rows: the projection reads them from memory
+    (2, 8, 32, 8, 128, 32, [1200, 800], [8, 8], 1024, False, True, True, False),   # 32 rows per kv head: not a small call
+]
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,D,bs,ctxs,qlens,N,bias,xform,bounded,fp8", VERIFY_CASES)
+def test_verify_step_equals_the_three_calls(pa, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, bias, xform, bounded, fp8):
+    rng = np.random.default_rng(B * 100 + T * 7 + Hq + D + N)
+    d = _setup_multi(rng, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, bias, xform, fp8=fp8)
+    scale, msl = 1.0 / np.sqrt(D), (int(max(ctxs)) if bounded else None)
+    print(f"verify_step B={B} T={T} Hq={Hq} Hkv={Hkv} D={D} bs={bs} ctx={ctxs[:4]}.. q={qlens[:4]}.. N={N} fp8={fp8}", flush=True)
+    want, att, wk, wv, wks, wvs = _verify_three_calls(pa, d, scale, msl)
+    for fusion in (0, 1):
+        _fusion(fusion)
+        try:
+            got, gk, gv, gks, gvs = _verify_step(pa, d, scale, msl)
+            torch.cuda.synchronize()
+        finally:
+            _fusion(0)
+        _same_bits(got, want, f"projected rows, fusion switch {fusion}")
+        _same_bits(gk, wk, "K pool")
+        _same_bits(gv, wv, "V pool")
+        if fp8:
+            _same_bits(gks, wks, "K scales")
+    a2 = torch.empty_like(d["xq"])
+    got, _, _, _, _ = _verify_step(pa, d, scale, msl, attn_out=a2)
+    _same_bits(got, want, "projected rows with attn_out")
+    _same_bits(a2, att, "attention output beside the projection")
+    got, _, _, _, _ = _verify_step(pa, dict(d, ow=None, ob=None), scale, msl)
+    torch.cuda.synchronize()
+    _same_bits(got, att, "attention output alone")
+    g = dev_to_f32(got)
+    assert not np.isnan(g).any()
+    for b in range(B):
+        assert np.array_equal(g[b, qlens[b]:], np.zeros_like(g[b, qlens[b]:]))     # padding rows
+
+
+def test_verify_step_argument_errors(pa):
+    rng = np.random.default_rng(12)
+    d = _setup_multi(rng, 2, 4, 8, 2, 128, 16, [40, 50], [4, 4], 256, False, True)
+    scale = 1.0 / np.sqrt(128)
+    args = (d["k"], d["v"], d["tables"], d["lens"], d["qlens"], scale)
+    with pytest.raises(ValueError):
+        pa.verify_step(d["xq"], d["xk"][:, :2], d["xv"], *args)
+    with pytest.raises(ValueError):
+        pa.verify_step(d["xq"], d["xk"], d["xv"], *args, k_norm_weight=d["wk"])
+    with pytest.raises(ValueError):
+        pa.verify_step(d["xq"].float(), d["xk"], d["xv"], *args)
+    with pytest.raises(ValueError):
+        big = torch.zeros((2, 65, 8, 128), dtype=torch.bfloat16, device="cuda")
+        pa.verify_step(big, big[:, :, :2], big[:, :, :2], *args)
+    with pytest.raises(NotImplementedError):
+        pa.verify_step(d["xq"].cpu(), d["xk"], d["xv"], *args)
