@@ -527,11 +527,32 @@ int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
 // A caller of verify_launch that can consume the fixed-partition route's split-K partials itself (the projection of
 // pa_verify_step) asks for them here: when the call takes that route with more than one partition, the merge launch
 // is left out and `f` says where the partials are.
+// The same caller hands over the step's cache update: verify_launch either lets it ride on the fixed-partition
+// launch (bf16 pools, all rows of a kv head on one wave) or runs the write launch in front of the attention launch.
 struct VerifyPartials {
   bool want;
   bool left;
   DecodeParams f;
+  const pa_new_kv* new_kv;      // null: the pool already holds the new tokens
+  void* k_cache_w;
+  void* v_cache_w;
+  float* k_scale_w;
+  float* v_scale_w;
+  bool fuse_rows;               // allowed to take the rows on the attention launch
 };
+
+static int verify_write_rows(const VerifyPartials& vp, const pa_q_transform* qt, const int32_t* block_tables,
+                             const int32_t* seq_lens, int B, int T, int Hq, int Hkv, int D, int block_size,
+                             int max_blocks_per_seq, int num_blocks, int kv_dtype, void* stream) {
+  const pa_new_kv* n = vp.new_kv;
+  if (qt)
+    return pa_qk_norm_rope_kv_write(nullptr, n->xk, n->xv, nullptr, nullptr, n->k_norm_weight, qt->norm_eps, qt->rope_cos,
+                                    qt->rope_sin, qt->rope_max_pos, vp.k_cache_w, vp.v_cache_w, vp.k_scale_w, vp.v_scale_w,
+                                    block_tables, seq_lens, n->query_lens, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq,
+                                    num_blocks, kv_dtype, stream);
+  return pa_kv_write(n->xk, n->xv, vp.k_cache_w, vp.v_cache_w, vp.k_scale_w, vp.v_scale_w, block_tables, seq_lens,
+                     n->query_lens, B, T, Hkv, D, block_size, max_blocks_per_seq, num_blocks, kv_dtype, stream);
+}
 
 // Query tokens [t0, t0 + Tc) of the T tokens per sequence through the decode-shaped kernel (pa_verify: all
 // of them in one launch; pa_prefill for shapes the tiled kernel does not take: 64 at a time).
@@ -596,6 +617,22 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
       f.head_major = g_head_major.load();
       f.ws_out = (float*)workspace;
       f.ws_ml = f.ws_out + (size_t)B * Hq * Tc * f.num_partitions * D;
+      if (vp && vp->new_kv) {
+        // (for one or two sequences: B = 1, T = 4 behind 1 K 27.6 -> 25.9 us per layer of a verify step, behind 4 K
+        // 32.5 -> 31.2; with more sequences the start of more workgroups waits for the rows' transform and the write
+        // launch is the faster way: B = 8 34.8 -> 35.6.  Debug switch 10 = 2 takes the rows whatever the batch.)
+        if (vp->fuse_rows && t0 == 0 && Tc == T && decode_new_row_supported(f, PA_BF16, kv_dtype) &&
+            ((long)B * Hkv <= 16 || g_step_fusion.load() == 2)) {
+          f.new_k = vp->new_kv->xk; f.new_v = vp->new_kv->xv; f.new_lens = vp->new_kv->query_lens;
+          if (q_transform) {
+            f.new_kt = f.qt;
+            f.new_kt.norm_weight = (const uint16_t*)vp->new_kv->k_norm_weight;
+          }
+        } else if (int rc = verify_write_rows(*vp, q_transform, block_tables, seq_lens, B, T, Hq, Hkv, D, block_size,
+                                              max_blocks_per_seq, num_blocks, kv_dtype, (void*)s)) {
+          return rc;
+        }
+      }
       profile_begin(s);
       hipError_t e = launch_decode_mfma(f, kv_dtype, 0, s);
       profile_end(s);
@@ -614,6 +651,11 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   const size_t need = decode_balanced_workspace_bytes(B, Hq * Tc, D, p.bal_gv);
   if (!workspace || workspace_bytes < need)
     return fail_arg("%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if (vp && vp->new_kv) {
+    if (int rc = verify_write_rows(*vp, q_transform, block_tables, seq_lens, B, T, Hq, Hkv, D, block_size,
+                                   max_blocks_per_seq, num_blocks, kv_dtype, (void*)s))
+      return rc;
+  }
   p.ws_out = (float*)workspace;
   p.ws_ml = p.ws_out + (size_t)Hq * Tc * ((size_t)B + p.bal_gv) * D;
   p.ws_start = (int32_t*)(p.ws_ml + (size_t)Hq * Tc * ((size_t)B + p.bal_gv) * 2);
@@ -1071,18 +1113,10 @@ int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
       return fail_arg("%s: o_weight, o_bias and out must be 16-byte aligned", who);
   }
   if (!aligned16(workspace) || !aligned16(attn_out)) return fail_arg("%s: workspace and attn_out must be 16-byte aligned", who);
-  // the cache update (argument checks of its own), then the attention, then the projection
   int rc;
-  if (q_transform)
-    rc = pa_qk_norm_rope_kv_write(nullptr, new_kv->xk, new_kv->xv, nullptr, nullptr, new_kv->k_norm_weight,
-                                  q_transform->norm_eps, q_transform->rope_cos, q_transform->rope_sin,
-                                  q_transform->rope_max_pos, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens,
-                                  new_kv->query_lens, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks,
-                                  kv_dtype, stream);
-  else
-    rc = pa_kv_write(new_kv->xk, new_kv->xv, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens,
-                     new_kv->query_lens, B, T, Hkv, D, block_size, max_blocks_per_seq, num_blocks, kv_dtype, stream);
-  if (rc) return rc;
+  if (!new_kv->xk || !new_kv->xv || !new_kv->query_lens) {
+    if (B > 0 && T > 0) return fail_arg("%s: new_kv needs xk, xv and query_lens", who);
+  }
   if (B == 0 || T == 0) return 0;
   if (Hq % Hkv) return fail_arg("%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
   if (kv_dtype != PA_BF16 && kv_dtype != PA_FP8_E4M3FN) return fail_arg("%s: kv_dtype must be bf16 or fp8-e4m3fn", who);
@@ -1110,8 +1144,14 @@ int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
       proj_ws = (float*)(ws + avail);
     }
   }
+  // the cache update (on the attention launch, or a launch with argument checks of its own in front of it), the
+  // attention, the projection
+  const int fusion = g_step_fusion.load();
   VerifyPartials vp;
-  vp.want = proj && !attn_out && g_step_fusion.load() != 1 && g_step_fusion.load() != 2 &&
+  memset(&vp, 0, sizeof(vp));
+  vp.new_kv = new_kv; vp.k_cache_w = k_cache; vp.v_cache_w = v_cache; vp.k_scale_w = k_scale; vp.v_scale_w = v_scale;
+  vp.fuse_rows = fusion != 1 && fusion != 3;
+  vp.want = proj && !attn_out && fusion != 1 && fusion != 2 &&
             o_proj_takes_partials((int)M, K, D, splits, proj_ws != nullptr);
   rc = verify_launch(who, q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, new_kv->query_lens, attn, ws, avail,
                      B, T, 0, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks, max_seq_len, scale, kv_dtype, sinks,

@@ -129,7 +129,7 @@ struct QOperandLayout {
 // same wave stores the row in the pool for the steps to come.
 template <int D, bool FP8, bool MULTI = false, int R = 1, bool LEAN = false, bool SV = false, bool NEWROW = false>
 struct DecodeWave {
-  static_assert(!NEWROW || (!FP8 && !MULTI && R == 1 && !LEAN && !SV), "the new-row form is plain bf16 decode");
+  static_assert(!NEWROW || (!FP8 && R == 1 && !LEAN && !SV), "the new-row forms are bf16, one 16-row operand per wave");
   using KT = KTile<D, FP8>;
   using VT = VTile<D, FP8>;
   static constexpr int VEC = VT::VEC, KLD = KT::KLD, VW = VT::VW;
@@ -165,6 +165,12 @@ struct DecodeWave {
   uint4 knew[NEWROW ? KSTEPS : 1];
   uint32_t vnew[NEWROW ? VW : 1];
   int new_t0, new_from;
+  // NEWROW with MULTI (a few new tokens per sequence): the workgroup keeps the tokens' rows in LDS, row t of
+  // new_k_lds / new_v_lds [T][D] bf16 being token first_new + t of the sequence (K as transformed); patch_new_rows
+  // puts them into the tiles that hold those tokens.  first_new: a position no tile reaches when nothing is to patch.
+  const char* new_k_lds;
+  const char* new_v_lds;
+  int first_new;
 
   __device__ __forceinline__ DecodeWave(const DecodeParams& p_, int head_slot, int lane, uint4* qlds_ = nullptr)
       : p(p_), qlds(qlds_), qlane(lane) {
@@ -185,6 +191,37 @@ struct DecodeWave {
     vbase = (const char*)p.v_cache + (long)hk * D * ESZ;
     new_t0 = -1;
     new_from = 64;
+    new_k_lds = new_v_lds = nullptr;
+    first_new = 0x7fffffff;
+  }
+
+  // NEWROW with MULTI: tile rows of [t0, t0 + 32) that are new tokens (or are redirected to the last one, which is
+  // new) take their K chunks and V elements from the workgroup's LDS copy instead of what the loads brought
+  __device__ __forceinline__ void patch_new_rows(KT& k, VT& v, int t0) const {
+    if constexpr (NEWROW && MULTI) {
+      if (t0 + 31 < first_new) return;                 // wave-uniform: no new token in this tile
+      const int lmax = last - t0;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int tn = t0 + min(16 * u + krow, lmax) - first_new;
+        if (tn >= 0) {
+#pragma unroll
+          for (int s = 0; s < KLD; ++s) {
+            const uint4 c = *(const uint4*)(new_k_lds + ((long)tn * D + (4 * s + g) * 8) * 2);
+            k.k[u][s][0] = c.x; k.k[u][s][1] = c.y; k.k[u][s][2] = c.z; k.k[u][s][3] = c.w;
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int tn = t0 + min(4 * j + g, lmax) - first_new;
+        if (tn >= 0) {
+          const uint32_t* src = (const uint32_t*)(new_v_lds + ((long)tn * D + r * VEC) * 2);
+#pragma unroll
+          for (int dw = 0; dw < VW; ++dw) v.v[j][dw] = src[dw];
+        }
+      }
+    }
   }
 
   // NEWROW: this wave is the one whose tiles include token `pos` (= ctx - 1, the step's new token, whose rows begin()
@@ -253,7 +290,7 @@ struct DecodeWave {
     last = ctx - 1;
     // NEWROW: the new token's rows are requested here, with the Q rows, by every wave (one round trip for all of
     // them; the wave that turns out to hold the token adopts them, see adopt_new_row), and K is transformed behind Q
-    if constexpr (NEWROW) {
+    if constexpr (NEWROW && !MULTI) {
       const uint16_t* krow = (const uint16_t*)p.new_k + ((long)b * p.Hkv + hk) * D;
       const uint16_t* vrow = (const uint16_t*)p.new_v + ((long)b * p.Hkv + hk) * D;
 #pragma unroll
@@ -321,7 +358,7 @@ struct DecodeWave {
       m_run[rg] = -INFINITY;
       l_run[rg] = 0.f;
     }
-    if constexpr (NEWROW) {
+    if constexpr (NEWROW && !MULTI) {
       // the raw K row -> knew, normed and rotated at position ctx - 1 as the write kernel would (same arithmetic,
       // same bits; new_kt.cos null: stored as given)
       if (p.new_kt.cos) {
@@ -661,11 +698,13 @@ struct DecodeWave {
     while (i + 2 < n) {
       if (lockstep) __builtin_amdgcn_s_barrier();
       load_k(kb, t + t_step);
+      patch_new_rows(ka, va, t);
       scores_softmax(ka, va, t, t_end);
       load_v(vb, t + t_step);
       accumulate_pv(va);
       if (lockstep) __builtin_amdgcn_s_barrier();
       load_k(ka, t + 2 * t_step);
+      patch_new_rows(kb, vb, t + t_step);
       scores_softmax(kb, vb, t + t_step, t_end);
       load_v(va, t + 2 * t_step);
       accumulate_pv(vb);
@@ -674,12 +713,15 @@ struct DecodeWave {
     }
     if (i + 1 < n) {
       load_k(kb, t + t_step);
+      patch_new_rows(ka, va, t);
       scores_softmax(ka, va, t, t_end);
       load_v(vb, t + t_step);
       accumulate_pv(va);
+      patch_new_rows(kb, vb, t + t_step);
       scores_softmax(kb, vb, t + t_step, t_end);
       accumulate_pv(vb);
     } else {
+      patch_new_rows(ka, va, t);
       scores_softmax(ka, va, t, t_end);
       accumulate_pv(va);
     }
@@ -810,9 +852,22 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
   const int ctx = sp.ctx;
   int new_len = 0;
   bool takes_new = false;
-  if constexpr (NEWROW) {
+  if constexpr (NEWROW && !MULTI) {
     new_len = min(p.seq_lens[b], p.max_blocks * p.block_size);
     takes_new = new_len >= 1 && (!p.new_lens || p.new_lens[b] >= 1);
+  }
+  // NEWROW with MULTI: the step's new tokens of this sequence, as the write kernel places them: new_n of them from
+  // position new_start on (lengths beyond the table count as its capacity; nothing to write when the lengths are
+  // inconsistent).  The call attends to them only if its own view of the sequence ends with them (no length bound
+  // below the sequence, query tokens = new tokens); otherwise they are stored and the pool rows are read as they are.
+  int new_n = 0, new_start = 0;
+  bool new_seen = false;
+  if constexpr (NEWROW && MULTI) {
+    const int len = min(p.seq_lens[b], p.max_blocks * p.block_size);
+    new_n = min(max(p.new_lens[b], 0), p.T);
+    new_start = len - new_n;
+    if (new_start < 0) new_n = 0;
+    new_seen = new_n > 0 && len == ctx && new_n == sp.tq;
   }
   // where virtual row vr (q head, or (token, head) pair) of sequence b lies in out
   const int n_rep = p.Hq / p.Hkv;
@@ -831,6 +886,40 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
   }
   const int t_end = min(ctx, t_begin + p.partition_size);
   const int ntiles = (t_end - t_begin + 31) >> 5;
+  // NEWROW with MULTI: the workgroup whose partition ends the context (the first one, for tokens the call does not
+  // see) stores the new rows when its tiles are done; it and every workgroup whose partition holds one of the
+  // tokens keep the rows in LDS: K normed and rotated at each token's position by wave 0 (lane (g, r): token r,
+  // chunks 4 s + g; the write kernel's arithmetic, hence its bits), V as given.
+  __shared__ __attribute__((aligned(16))) char sm_new[(NEWROW && MULTI) ? 2 * 16 * D * 2 : 16];
+  bool new_storer = false, new_rows = false;
+  uint4 nk_raw[(NEWROW && MULTI) ? W::KSTEPS : 1], nv_raw = make_uint4(0, 0, 0, 0);
+  NormRopeCoeffs<W::KSTEPS> nk_c;
+  constexpr int CPRW = D / 8;                                // 16-byte chunks per row
+  if constexpr (NEWROW && MULTI) {
+    new_storer = new_n > 0 && w.jbase == 0 && (new_seen ? t_end == ctx : part == 0);
+    const bool new_here = new_seen && new_start < t_end;        // (the tokens end the context: they begin before t_end or not at all)
+    new_rows = new_storer || new_here;
+    if (new_rows) {
+      // the loads first (wave 0: token r's K chunks 4 s + g and what their transform takes from the tables; every
+      // thread: one 16-byte chunk of the V rows, 16 tokens x D / 8 chunks at most); the arithmetic follows behind
+      // the requests of the Q rows and of the first tile
+      if (wave == 0) {
+        const int t = min(w.r, new_n - 1);
+        const uint16_t* krow = (const uint16_t*)p.new_k + (((long)b * p.T + t) * p.Hkv + w.hk) * D;
+#pragma unroll
+        for (int s = 0; s < W::KSTEPS; ++s) nk_raw[s] = *(const uint4*)(krow + (4 * s + w.g) * 8);
+        if (p.new_kt.cos)
+          norm_rope_fetch<D / 8, W::KSTEPS, QOperandLayout<false>>(p.new_kt, min(max(new_start + t, 0), p.new_kt.max_pos - 1), w.g, nk_c);
+      }
+      if (tid < new_n * CPRW) {
+        const int t = tid / CPRW, ch = tid - t * CPRW;
+        nv_raw = *(const uint4*)((const uint16_t*)p.new_v + (((long)b * p.T + t) * p.Hkv + w.hk) * D + ch * 8);
+      }
+      if (new_here) w.first_new = new_start;
+      w.new_k_lds = sm_new;
+      w.new_v_lds = sm_new + 16 * D * 2;
+    }
+  }
   // every load the start needs, then this wave's first tile, then the arithmetic of the start: the first tile is on
   // its way while Q is normed and rotated (one trip to memory less on the path of every workgroup)
   const int t_first = t_begin + 32 * wave, n_mine = (ntiles - wave + NW - 1) / NW;
@@ -842,9 +931,35 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
     w.load_k(k_first, t_first);
     w.load_v(v_first, t_first);
   }
+  if constexpr (NEWROW && MULTI) {
+    if (new_rows) {
+      if (wave == 0) {
+        float x[W::KSTEPS][8];
+#pragma unroll
+        for (int s = 0; s < W::KSTEPS; ++s) {
+          const uint32_t wd[4] = {nk_raw[s].x, nk_raw[s].y, nk_raw[s].z, nk_raw[s].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[s][2 * j] = bf16_bits_to_float(wd[j] & 0xffffu);
+            x[s][2 * j + 1] = bf16_bits_to_float(wd[j] >> 16);
+          }
+        }
+        if (p.new_kt.cos) norm_rope_apply<D / 8, W::KSTEPS, QOperandLayout<false>>(x, p.new_kt, w.g, nk_c);
+        if (w.r < new_n) {
+#pragma unroll
+          for (int s = 0; s < W::KSTEPS; ++s)
+            *(uint4*)(sm_new + ((long)w.r * D + (4 * s + w.g) * 8) * 2) =
+                make_uint4(pack_bf16x2(x[s][0], x[s][1]), pack_bf16x2(x[s][2], x[s][3]),
+                           pack_bf16x2(x[s][4], x[s][5]), pack_bf16x2(x[s][6], x[s][7]));
+        }
+      }
+      if (tid < new_n * CPRW) *(uint4*)(sm_new + 16 * D * 2 + (long)tid * 16) = nv_raw;
+      __syncthreads();
+    }
+  }
   w.finish_q(qp);
   int store_pos = -1;       // NEWROW: this wave stores the new token's rows at this position when its tiles are done
-  if constexpr (NEWROW) {
+  if constexpr (NEWROW && !MULTI) {
     // the new token is number seq_lens[b] - 1, as the write kernel places it (lengths beyond the table count as
     // its capacity); a sequence that takes none this step (new_lens[b] == 0) or is empty is streamed as it is
     if (takes_new) {
@@ -861,10 +976,24 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
     }
   }
   w.stream_from(k_first, v_first, t_first, 32 * NW, n_mine, t_end);
-  if constexpr (NEWROW) {
+  if constexpr (NEWROW && !MULTI) {
     if (store_pos >= 0) {
       if (store_pos != ctx - 1) w.retransform_new_k(b, store_pos);     // K was rotated for position ctx - 1
       w.store_new_row(b, store_pos);
+    }
+  }
+  if constexpr (NEWROW && MULTI) {
+    if (new_storer) {
+      // behind the tile loop, not in front of it: a pending store would make every wait in the loop a wait for all
+      for (int i = tid; i < 2 * new_n * CPRW; i += NW * 64) {
+        const int which = i >= new_n * CPRW, ii = i - which * new_n * CPRW;
+        const int t = ii / CPRW, ch = ii - t * CPRW, pos = new_start + t;
+        const int blk = p.block_tables[(long)b * p.max_blocks + (pos >> p.block_shift)];
+        if (blk < 0 || blk >= p.num_blocks) continue;             // a bad table entry must not redirect the write
+        const long row = (long)blk * p.block_size + (pos & (p.block_size - 1));
+        char* dst = const_cast<char*>(which ? w.vbase : w.kbase) + row * w.row_stride + ch * 16;
+        *(uint4*)dst = *(const uint4*)(sm_new + which * 16 * D * 2 + ((long)t * D + ch * 8) * 2);
+      }
     }
   }
 
@@ -1142,6 +1271,14 @@ hipError_t launch_typed(const DecodeParams& p, int waves, hipStream_t s) {
   if (p.head_major) grid = dim3(slots, p.num_partitions, p.B);
   if (p.query_lens) {      // multi-token rows: the four-wave form
     if (p.rows_per_wave != 16) return hipErrorInvalidValue;
+    if (p.new_k) {
+      if constexpr (FP8) return hipErrorInvalidValue;
+      else {
+        if (slots != p.Hkv || p.T > 16 || !p.new_lens) return hipErrorInvalidValue;     // one 16-row wave per kv head holds all its rows
+        hipLaunchKernelGGL((decode_mfma_kernel<D, false, 4, true, true>), grid, dim3(256), 0, s, p);
+        return hipGetLastError();
+      }
+    }
     hipLaunchKernelGGL((decode_mfma_kernel<D, FP8, 4, true>), grid, dim3(256), 0, s, p);
     return hipGetLastError();
   }
@@ -1200,7 +1337,10 @@ bool decode_mfma_supported(const DecodeParams& p, int q_dtype, int kv_dtype) {
 }
 
 bool decode_new_row_supported(const DecodeParams& p, int q_dtype, int kv_dtype) {
-  return decode_mfma_supported(p, q_dtype, kv_dtype) && kv_dtype == PA_BF16 && p.T == 1 && !p.query_lens;
+  if (!decode_mfma_supported(p, q_dtype, kv_dtype) || kv_dtype != PA_BF16) return false;
+  if (!p.query_lens) return p.T == 1;
+  // multi-token rows: all rows of a kv head on one 16-row wave, at most 16 tokens
+  return p.rows_per_wave == 16 && (p.Hq / p.Hkv) * p.T <= 16 && p.T <= 16;
 }
 
 hipError_t launch_decode_mfma(const DecodeParams& p, int kv_dtype, int waves, hipStream_t s) {

@@ -371,6 +371,9 @@ VERIFY_CASES = [
     (4, 4, 32, 8, 128, 32, [1500, 600, 90, 5], [4, 4, 1, 4], 1024, True, True, True, True),     # fp8 pool
     (16, 4, 32, 8, 128, 32, [700 + 31 * i for i in range(16)], [4] * 16, 1024, False, True, True, False),   # 64 rows: the projection reads them from memory
     (2, 8, 32, 8, 128, 32, [1200, 800], [8, 8], 1024, False, True, True, False),   # 32 rows per kv head: not a small call
+    (6, 4, 32, 8, 128, 16, [514, 513, 515, 34, 4, 1026], [4, 4, 4, 4, 4, 4], 512, False, True, True, False),   # new tokens across a partition, tile, block border; a sequence of only new tokens
+    (3, 16, 8, 8, 64, 32, [530, 16, 1040], [16, 16, 9], 256, True, True, True, False),     # 16 new tokens, head dim 64, across borders
+    (2, 4, 32, 8, 128, 32, [600, 900], [4, 4], 512, False, False, True, False),    # no transform: rows stored as given
 ]
 
 
@@ -381,7 +384,7 @@ def test_verify_step_equals_the_three_calls(pa, B, T, Hq, Hkv, D, bs, ctxs, qlen
     scale, msl = 1.0 / np.sqrt(D), (int(max(ctxs)) if bounded else None)
     print(f"verify_step B={B} T={T} Hq={Hq} Hkv={Hkv} D={D} bs={bs} ctx={ctxs[:4]}.. q={qlens[:4]}.. N={N} fp8={fp8}", flush=True)
     want, att, wk, wv, wks, wvs = _verify_three_calls(pa, d, scale, msl)
-    for fusion in (0, 1):
+    for fusion in (0, 2, 3, 1):
         _fusion(fusion)
         try:
             got, gk, gv, gks, gvs = _verify_step(pa, d, scale, msl)
