@@ -10,7 +10,7 @@ carries, under "configs", one record each for config 3 (paged chunked prefill),
 config 4 (blocksparse prefill) and config 5 (fp8-KV long-context decode), timed in
 the same run with the same protocol: both halves of the headline metric and every
 benchmark-sized configuration, plus "o_proj", the output projection behind config 3's
-attention.  --config N prints that configuration alone (6-13: the kernels and steps around the
+attention.  --config N prints that configuration alone (6-15: the kernels and steps around the
 attention call; their docstrings say what each one is).
 
 value      whole-step throughput: algorithmic HBM bytes / step time for the decode
@@ -709,10 +709,11 @@ def bench_prefill_layer_step(steps, warmup, lib, pa, W):
     }
 
 
-def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound):
+def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound, T=1):
     """Seconds per step of `layers` attention layers, issued call by call and replayed from one HIP graph, on a cache
     whose tables hold `capacity` tokens per sequence; `bound` is the length bound given to `attend` (None: the
-    engine's own choice, which under capture is the longest context the cache admits)."""
+    engine's own choice, which under capture is the longest context the cache admits).  T new tokens per sequence
+    (1: a decode step; more: a speculative verify step) behind `ctx` cached ones."""
     from nkipy_amd.engine import PagedAttention, PagedKVCache
     Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
     nblk = (capacity + bs - 1) // bs
@@ -726,14 +727,14 @@ def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound):
     for pool in cache.k_caches + cache.v_caches:
         pool.copy_(torch.randn(pool.shape, generator=gen, device="cuda", dtype=torch.float32))
     cache.extend(list(range(B)), [ctx] * B)      # contexts of `ctx` tokens (the pool holds whatever it holds)
-    q1 = torch.randn(B, 1, Hq, D, generator=gen, device="cuda").to(torch.bfloat16)
-    k1 = torch.randn(B, 1, Hkv, D, generator=gen, device="cuda").to(torch.bfloat16)
+    q1 = torch.randn(B, T, Hq, D, generator=gen, device="cuda").to(torch.bfloat16)
+    k1 = torch.randn(B, T, Hkv, D, generator=gen, device="cuda").to(torch.bfloat16)
 
     def step():
         for a in att:
             a.attend(q1, k1, k1, max_seq_len=bound)
 
-    cache.begin_step([1] * B, 1)
+    cache.begin_step([T] * B, T)
     sec_eager = _time_steps(step, steps, warmup)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
@@ -773,7 +774,39 @@ def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
                                f"one step = {layers} layers", "algorithmic_bytes_per_layer": byts},
         "roofline": {"bound": "hbm", "achieved": round(byts / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(byts / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "five launches per layer (KV write with K transform, decode + merge, projection + merge)",
+                     "kernel": "three launches per layer (decode with the new row on it, merge, projection with its merge "
+                               "on the load); five without a length bound",
+                     "kernel_avg_ms": round(us * 1e-3, 5), "launches_timed": steps * layers},
+        "cpu_baseline": None,
+    }
+
+
+def bench_verify_layer_step(steps, warmup, lib, pa, W, B=1, T=4, ctx=1024, layers=8):
+    """config 15: a speculative verify step at the reference's operating point (one sequence, K + 1 = 4 tokens), per
+    attention layer through `PagedAttention.attend`: the T tokens' K / V rows into the pool, causal attention of the
+    T tokens over the cache, output projection; tables that end just above the context.  Launch-bound like config
+    13; `batches` repeats it for 4 sequences behind 2 K and 8 behind 1 K."""
+    Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
+    sec, sec_eager, cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, ctx + 96, None, T=T)
+    others = {}
+    for b2, c2 in ((4, 2048), (8, 1024)):
+        s2, e2, _ = _decode_layer_step_times(steps, warmup, b2, c2, layers, c2 + 96, None, T=T)
+        others[f"B{b2}_ctx{c2}"] = {"us_per_layer": round(s2 / layers * 1e6, 2),
+                                    "eager_us_per_layer": round(e2 / layers * 1e6, 2)}
+    byts = 2 * B * (ctx + T) * Hkv * D * 2 + Hq * D * N * 2 + B * T * (2 * Hq * D + 2 * Hkv * D + N) * 2
+    us = sec / layers * 1e6
+    return {
+        "metric": "verify layer step (QK-norm + RoPE + KV write + causal verify + o_proj), layers/s, HIP graph replay",
+        "value": round(1e6 / us, 1), "unit": "layer steps/s",
+        "ms_per_step": round(sec * 1e3, 5), "us_per_layer": round(us, 2),
+        "eager_us_per_layer": round(sec_eager / layers * 1e6, 2), "batches": others,
+        "dtype": "bf16, float32 norm, bf16 rotation, fp32 accumulate",
+        "config": {"workload": f"verify layer step: B={B}, T={T}, context={ctx}, table capacity={cap} tokens per sequence, "
+                               f"layers={layers}, Hq={Hq}, Hkv={Hkv}, D={D}, block_size={bs}, hidden={N}; "
+                               f"one step = {layers} layers", "algorithmic_bytes_per_layer": byts},
+        "roofline": {"bound": "hbm", "achieved": round(byts / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(byts / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "three launches per layer (verify with the new rows on it, merge, projection)",
                      "kernel_avg_ms": round(us * 1e-3, 5), "launches_timed": steps * layers},
         "cpu_baseline": None,
     }
@@ -784,7 +817,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14],
+    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     ap.add_argument("--prefill-impl", type=int, default=0,
@@ -844,6 +877,8 @@ def main():
             res = bench_decode_layer_step(args.steps, args.warmup, lib, pa, W)
         elif cfg == 14:
             res = bench_tile_loop_probe(args.steps, args.warmup)
+        elif cfg == 15:
+            res = bench_verify_layer_step(args.steps, args.warmup, lib, pa, W)
         else:
             res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
         gc.collect()

@@ -1060,30 +1060,66 @@ __device__ __forceinline__ int span_tiles(const DecodeParams& p, int b) {
   return tiles_of(ctx) - first_tile(p, b, ctx);
 }
 
-// Wave-wide: total number of tiles, and (if f >= 0) the sequence holding
-// flattened tile f with the number of tiles before it.
-__device__ __forceinline__ int scan_tiles(const DecodeParams& p, int lane, int f, int* b_out, int* start_out) {
-  int base = 0;
-  bool found = false;
-  for (int bb = 0; bb < p.B; bb += 64) {
-    const int t = (bb + lane < p.B) ? span_tiles(p, bb + lane) : 0;
-    int incl = t;
+// Calls of more than kScanInRegs sequences: the tiles before each sequence (and the total) are laid down in
+// p.ws_start by this one-workgroup launch ahead of the streaming kernel, whose waves then find their first sequence
+// by search instead of each scanning every length (a scan is a chain of a load and six cross-lane steps per 64
+// sequences: at 8 192 sequences of one to three tiles the scans were half of the streaming kernel's time).
+constexpr int kScanInRegs = 512;
+__global__ __launch_bounds__(1024) void decode_tile_prefix_kernel(DecodeParams p) {
+  __shared__ int wave_total[16];
+  __shared__ int carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < p.B; base += 4096) {
+    const int b0 = base + 4 * tid;
+    int t[4], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      t[i] = b0 + i < p.B ? span_tiles(p, b0 + i) : 0;
+      sum += t[i];
+    }
+    int incl = sum;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
       const int v = __shfl_up(incl, off, 64);
       if (lane >= off) incl += v;
     }
-    const int total = __shfl(incl, 63, 64);
-    if (!found && f >= 0 && f < base + total) {
-      const unsigned long long m = __ballot(base + incl > f);
-      const int idx = __ffsll((long long)m) - 1;
-      *b_out = bb + idx;
-      *start_out = base + __shfl(incl - t, idx, 64);
-      found = true;
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    int before = carry;
+    for (int w = 0; w < wave; ++w) before += wave_total[w];
+    int run = before + incl - sum;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (b0 + i < p.B) p.ws_start[b0 + i] = run;
+      run += t[i];
     }
-    base += total;
+    __syncthreads();
+    if (tid == 1023) carry = run;
+    __syncthreads();
   }
-  return base;
+  if (tid == 0) p.ws_start[p.B] = carry;
+}
+
+// Wave-wide: the sequence that holds flattened tile f (0 <= f < ws_start[B]) and the tiles before it, from the
+// prefix sums: 64 probes per round, the last probe not above f wins (equal sums, i.e. sequences without tiles, are
+// thereby skipped)
+__device__ __forceinline__ void find_tile(const DecodeParams& p, int lane, int f, int* b_out, int* start_out) {
+  int lo = 0, hi = p.B, start = 0;
+  while (true) {
+    const int step = (hi - lo + 63) >> 6;
+    const int pos = lo + lane * step;
+    const int v = pos < hi ? p.ws_start[pos] : 0x7fffffff;
+    const unsigned long long m = __ballot(v <= f);
+    const int c = __popcll(m) - 1;                   // lane 0 probes lo, whose sum is not above f
+    start = __shfl(v, c, 64);
+    lo += c * step;
+    hi = min(hi, lo + step);
+    if (step == 1) break;
+  }
+  *b_out = lo;
+  *start_out = start;
 }
 
 template <int D, bool FP8, bool MULTI, int R, bool SV>
@@ -1101,9 +1137,9 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 
   // Total number of tiles and the sequence that holds this wave's first tile.  Up to 512 sequences
   // the lengths are fetched once, all loads in flight together, and scanned in registers; beyond
-  // that, two passes over seq_lens.
-  constexpr int SCAN_STEPS = 8;
-  const bool scan_in_regs = p.B <= 64 * SCAN_STEPS;
+  // that the prefix sums are there already (decode_tile_prefix_kernel).
+  constexpr int SCAN_STEPS = kScanInRegs / 64;
+  const bool scan_in_regs = p.B <= kScanInRegs;
   int N = 0, tl[SCAN_STEPS], incl[SCAN_STEPS];
   if (scan_in_regs) {
 #pragma unroll
@@ -1120,10 +1156,9 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
       N += __shfl(x, 63, 64);
     }
   } else {
-    int dummy_b = 0, dummy_s = 0;
-    N = scan_tiles(p, lane, -1, &dummy_b, &dummy_s);
+    N = p.ws_start[p.B];
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
+  if (scan_in_regs && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
     // tiles before each sequence (and the total), for the merge kernel: it then needs no scan of its own
     int base = 0;
     for (int bb = 0; bb < p.B; bb += 64) {
@@ -1161,7 +1196,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
       base += total;
     }
   } else {
-    scan_tiles(p, lane, f, &b, &start);
+    find_tile(p, lane, f, &b, &start);
   }
   b = __builtin_amdgcn_readfirstlane(b);
   start = __builtin_amdgcn_readfirstlane(start);
@@ -1194,7 +1229,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 template <int D, int G>
 __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParams p) {
   const int b = blockIdx.x;
-  const int start = p.ws_start[b];                   // tiles before this sequence, written by the streaming kernel
+  const int start = p.ws_start[b];                   // tiles before this sequence (streaming kernel, or prefix launch)
   const int T = p.ws_start[b + 1] - start;
   const int N = p.ws_start[p.B];
   constexpr int QUADS = D / 4, VEC = D / 16;
@@ -1313,6 +1348,7 @@ hipError_t launch_balanced_typed(const DecodeParams& p, hipStream_t s) {
   dim3 grid(p.bal_gv / p.bal_ns, (head_slots + p.bal_hsw - 1) / p.bal_hsw);
   const dim3 wg(64 * p.bal_hsw * p.bal_ns);
   const bool one_reader = head_slots == p.Hkv;         // one wave per kv head: it alone reads that head's V rows
+  if (p.B > kScanInRegs) hipLaunchKernelGGL(decode_tile_prefix_kernel, dim3(1), dim3(1024), 0, s, p);
   if (p.query_lens && p.rows_per_wave == 32) {
     if (one_reader) hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 2, true>), grid, wg, 0, s, p);
     else hipLaunchKernelGGL((decode_balanced_kernel<D, FP8, true, 2, false>), grid, wg, 0, s, p);

@@ -130,6 +130,8 @@ def test_bf16_waves_per_workgroup(pa, waves):
     (40, 48, 3, 1, 700),      # head slots do not divide the workgroup evenly
     (9, 32, 16, 100, 1200),   # more head slots than a workgroup holds: two head groups
     (5, 40, 2, 50, 900),      # 20 q heads per kv head: two 16-column chunks per kv head
+    (513, 8, 2, 0, 100),      # more sequences than are scanned in registers: tile sums by a launch of their own
+    (4500, 8, 2, 0, 70),      # ... of more than one pass, searched in three rounds; runs of empty sequences
 ])
 def test_balanced_schedule_shapes(pa, B, Hq, Hkv, lo, hi):
     rng = np.random.default_rng(B * 7 + Hq)
@@ -137,6 +139,10 @@ def test_balanced_schedule_shapes(pa, B, Hq, Hkv, lo, hi):
     if B > 10:
         ctxs[3] = 0
         ctxs[-1] = 0
+    if B > 512:
+        ctxs[:70] = [0] * 70
+        ctxs[300:420] = [0] * 120
+        ctxs[-3:] = [0] * 3
     got, want = _run_bf16(pa, rng, B, Hq, Hkv, 128, 32, ctxs, part=512, impl=3)
     assert_close_abs(got, want, BF16_TOL)
 

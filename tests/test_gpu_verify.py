@@ -62,6 +62,25 @@ def test_verify_matches_oracle(pa, rows, T, Hq, Hkv, D, bs):
         assert np.all(got[b, n:] == 0)          # padding rows
 
 
+def test_verify_of_more_sequences_than_are_scanned_in_registers(pa):
+    """600 sequences: the tiles before each sequence come from the prefix launch and every wave finds its first
+    sequence by search; idle sequences (no query token) at both ends and in a run in the middle."""
+    rng = np.random.default_rng(600)
+    T, Hq, Hkv, D, bs, B = 3, 8, 2, 128, 16, 600
+    qlens = rng.integers(1, T + 1, size=B).tolist()
+    prefixes = rng.integers(0, 60, size=B).tolist()
+    for i in list(range(5)) + list(range(200, 290)) + [B - 1]:
+        qlens[i] = 0
+    q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+    want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.09, q_dtype="bf16")
+    got = pa.verify(bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(ql), 0.09)
+    torch.cuda.synchronize()
+    got = dev_to_f32(got)
+    assert_close_abs(got, want, BF16_TOL)
+    for b, n in enumerate(qlens):
+        assert np.all(got[b, n:] == 0)
+
+
 def test_verify_rows_without_keys_in_the_last_chunk(pa, rows):
     """One long sequence spans every chunk of the schedule; its last 32-token tile holds 3 tokens,
     which the first 5 of 8 query tokens do not see, so their partial of that chunk is empty."""
