@@ -10,7 +10,7 @@ carries, under "configs", one record each for config 3 (paged chunked prefill),
 config 4 (blocksparse prefill) and config 5 (fp8-KV long-context decode), timed in
 the same run with the same protocol: both halves of the headline metric and every
 benchmark-sized configuration, plus "o_proj", the output projection behind config 3's
-attention.  --config N prints that configuration alone (6-15: the kernels and steps around the
+attention.  --config N prints that configuration alone (6-16: the kernels and steps around the
 attention call; their docstrings say what each one is).
 
 value      whole-step throughput: algorithmic HBM bytes / step time for the decode
@@ -709,21 +709,30 @@ def bench_prefill_layer_step(steps, warmup, lib, pa, W):
     }
 
 
-def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound, T=1):
+def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound, T=1, gpt_oss=False):
     """Seconds per step of `layers` attention layers, issued call by call and replayed from one HIP graph, on a cache
     whose tables hold `capacity` tokens per sequence; `bound` is the length bound given to `attend` (None: the
     engine's own choice, which under capture is the longest context the cache admits).  T new tokens per sequence
-    (1: a decode step; more: a speculative verify step) behind `ctx` cached ones."""
+    (1: a decode step; more: a speculative verify step) behind `ctx` cached ones.  gpt_oss: the layer of
+    examples/models/gpt_oss/kernels/attention.py:80-163 instead of qwen3's (64 / 8 heads of 64, hidden 2 880 with a
+    bias, RoPE without QK norm, a sink logit per head, a 128-token window on every other layer)."""
     from nkipy_amd.engine import PagedAttention, PagedKVCache
-    Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
+    Hq, Hkv, D, bs, N = (64, 8, 64, 32, 2880) if gpt_oss else (32, 8, 128, 32, 4096)
     nblk = (capacity + bs - 1) // bs
     cache = PagedKVCache(B * nblk + 8, bs, Hkv, D, max_seqs=B, max_blocks_per_seq=nblk, num_layers=layers)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1313)
     one = torch.ones(D, dtype=torch.bfloat16, device="cuda")
-    att = [PagedAttention(cache, Hq, layer=l, rope_base=1e6, max_positions=nblk * bs, q_norm_weight=one, k_norm_weight=one,
-                          o_weight=(torch.randn(Hq * D, N, generator=gen, device="cuda") / 64).to(torch.bfloat16))
-           for l in range(layers)]
+    if gpt_oss:
+        att = [PagedAttention(cache, Hq, layer=l, rope_base=150000.0, max_positions=nblk * bs,
+                              sinks=torch.randn(Hq, generator=gen, device="cuda"), sliding_window=128 if l % 2 == 0 else None,
+                              o_weight=(torch.randn(Hq * D, N, generator=gen, device="cuda") / 64).to(torch.bfloat16),
+                              o_bias=torch.randn(N, generator=gen, device="cuda").to(torch.bfloat16))
+               for l in range(layers)]
+    else:
+        att = [PagedAttention(cache, Hq, layer=l, rope_base=1e6, max_positions=nblk * bs, q_norm_weight=one, k_norm_weight=one,
+                              o_weight=(torch.randn(Hq * D, N, generator=gen, device="cuda") / 64).to(torch.bfloat16))
+               for l in range(layers)]
     for pool in cache.k_caches + cache.v_caches:
         pool.copy_(torch.randn(pool.shape, generator=gen, device="cuda", dtype=torch.float32))
     cache.extend(list(range(B)), [ctx] * B)      # contexts of `ctx` tokens (the pool holds whatever it holds)
@@ -812,12 +821,47 @@ def bench_verify_layer_step(steps, warmup, lib, pa, W, B=1, T=4, ctx=1024, layer
     }
 
 
+def bench_gpt_oss_layer_step(steps, warmup, lib, pa, W, B=1, ctx=1024, layers=8):
+    """config 16: the decode and verify steps of configs 13 and 15 on the gpt-oss layer, the reference's other model
+    family and its published operating point (one sequence, K + 1 = 4 draft tokens: peagle/speculate.py:137-202):
+    sinks on every layer, a 128-token sliding window on every other one, 64 / 8 heads of 64, output projection to
+    2 880 with a bias.  Launch-bound; microseconds per layer, HIP graph replay and issued call by call."""
+    Hq, Hkv, D, bs, N = 64, 8, 64, 32, 2880
+    sec, sec_eager, cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, ctx + 96, None, gpt_oss=True)
+    others = {}
+    for b2, c2, t2 in ((1, 1024, 4), (8, 1024, 1), (1, 4000, 1), (4, 2048, 4)):
+        s2, e2, _ = _decode_layer_step_times(steps, warmup, b2, c2, layers, c2 + 96, None, T=t2, gpt_oss=True)
+        others[f"B{b2}_ctx{c2}_T{t2}"] = {"us_per_layer": round(s2 / layers * 1e6, 2),
+                                          "eager_us_per_layer": round(e2 / layers * 1e6, 2)}
+    # a windowed layer reads its last 128 tokens, a full one the whole context: the mean of the two
+    kv_bytes = B * ((ctx + 1) + min(ctx + 1, 128)) * Hkv * D * 2
+    byts = kv_bytes + Hq * D * N * 2 + B * (2 * Hq * D + 2 * Hkv * D + N) * 2
+    us = sec / layers * 1e6
+    return {
+        "metric": "gpt-oss decode layer step (RoPE + KV write + paged decode with sinks / window + o_proj), layers/s, HIP graph replay",
+        "value": round(1e6 / us, 1), "unit": "layer steps/s",
+        "ms_per_step": round(sec * 1e3, 5), "us_per_layer": round(us, 2),
+        "eager_us_per_layer": round(sec_eager / layers * 1e6, 2), "other_steps": others,
+        "dtype": "bf16, bf16 rotation, fp32 accumulate",
+        "config": {"workload": f"gpt-oss decode layer step: B={B}, context={ctx}, table capacity={cap} tokens per sequence, "
+                               f"layers={layers} (window 128 on the even ones, sinks on all), Hq={Hq}, Hkv={Hkv}, D={D}, "
+                               f"block_size={bs}, hidden={N} with bias; one step = {layers} layers",
+                   "algorithmic_bytes_per_layer": byts},
+        "roofline": {"bound": "hbm", "achieved": round(byts / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(byts / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "per layer: decode with the new row on it (one partition under the window; else + merge), "
+                               "projection + its merge",
+                     "kernel_avg_ms": round(us * 1e-3, 5), "launches_timed": steps * layers},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15],
+    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     ap.add_argument("--prefill-impl", type=int, default=0,
@@ -879,6 +923,8 @@ def main():
             res = bench_tile_loop_probe(args.steps, args.warmup)
         elif cfg == 15:
             res = bench_verify_layer_step(args.steps, args.warmup, lib, pa, W)
+        elif cfg == 16:
+            res = bench_gpt_oss_layer_step(args.steps, args.warmup, lib, pa, W)
         else:
             res = bench_prefill_layer_step(args.steps, args.warmup, lib, pa, W)
         gc.collect()

@@ -101,12 +101,13 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * partitions; the default MFMA kernel for bf16 / fp8 KV instead cuts the
  * flattened stream of all sequences' 32-token tiles into equal chunks, one per
  * resident wavefront group, so its partition length follows the batch and the
- * device, not partition_size.  Small calls without sinks or a window (by max_seq_len:
- * at most eight partitions per sequence, at most 80 (sequence, kv head) pairs and
- * at most 160 MiB of K and V) take the fixed-partition MFMA kernel, whose fixed cost
- * is lower, on partitions of 256 tokens when those of partition_size would give the
- * device fewer than about 64 workgroups (a single sequence).  The result
- * does not depend on the split beyond the order of float32 sums.
+ * device, not partition_size.  Small calls (by max_seq_len, or by what a sliding window
+ * reaches if that is less: at most eight partitions per sequence, at most 80 (sequence,
+ * kv head) pairs and at most 160 MiB of K and V) take the fixed-partition MFMA kernel,
+ * whose fixed cost is lower, on partitions of 256 tokens when those of partition_size
+ * would give the device fewer than about 64 workgroups (a single sequence); under a
+ * window its partitions count from the first 32-token tile the window reaches.  The
+ * result does not depend on the split beyond the order of float32 sums.
  * max_seq_len: upper bound of seq_lens (sizes the grid and picks the kernel; 0 =
  * max_blocks_per_seq * block_size).  seq_lens[b] == 0 yields zeros.
  * q_dtype / kv_dtype: (F32, F32), (BF16, BF16) or (BF16, FP8_E4M3FN).
@@ -163,8 +164,7 @@ int pa_decode_noalloc(const void* q, const void* k_cache, const void* v_cache,
  *   sinks, sliding_window   as for pa_decode (the window counts back from each query token's own position)
  *   max_seq_len  0, or a host-known upper bound of seq_lens (longer contexts are read up to the bound).  The table
  *                capacity says nothing about the size of a call; with a bound, a small call -- at most eight
- *                512-token partitions per sequence, few sequences and little K and V in all (pa_decode's rule),
- *                no sinks, no window: the
+ *                512-token partitions per sequence, few sequences and little K and V in all (pa_decode's rule): the
  *                reference's own use, one sequence and a handful of draft tokens -- runs on fixed partitions
  *                as a small pa_decode call does, without the balanced schedule's fixed cost.  Same workspace.
  * D in {64, 128}; block_size a power of two >= 16; T <= PA_VERIFY_MAX_TOKENS.
@@ -266,8 +266,9 @@ int pa_o_proj_ws(const void* x, const void* w, const void* bias, void* out, void
  * on the same arguments; what the one call adds is that a small step (the fixed-partition decode kernels, bf16 pool)
  * runs as three launches instead of five: the kernel that reaches a sequence's newest token takes its K / V rows
  * from xk / xv (K transformed on the way) and stores them in the pool itself, and the projection merges the
- * sequence's split-K partials while it forms its rows.  Calls that those kernels do not take (fp8 or fp32 pools,
- * large batches or long contexts, sinks, a window) run the separate launches inside.
+ * sequence's split-K partials while it forms its rows (with sinks or a window the merge stays a launch of its own;
+ * a window that fits one partition needs none).  Calls that those kernels do not take (fp8 or fp32 pools, large
+ * batches or long contexts) run the separate launches inside.
  *   new_kv    the step's new token per sequence: xk, xv [B, Hkv, D] of the pool's source type (bf16; float32 for
  *             an fp32 pool); query_lens [B]: 1 for a sequence that takes a token this step, 0 for one that does
  *             not (its row of xk / xv is ignored); seq_lens counts the new token, as for pa_kv_write;

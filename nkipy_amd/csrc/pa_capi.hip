@@ -256,15 +256,22 @@ size_t pa_decode_workspace_bytes(int B, int Hq, int D, int max_seq_len, int part
 // bytes.  So calls of at most 80 (sequence, kv head) pairs and at most eight partitions per sequence that can touch at
 // most this many bytes of K and V, by the caller's bound on the lengths, take the fixed partitions when nothing
 // needs the balanced kernel.
+// The most tokens the partitions of one sequence cover: the length bound, or, under a sliding window, what the window
+// of the oldest query row reaches back to, rounded out to its 32-token tile (the kernels count partitions from there)
+static int span_bound(const DecodeParams& p) {
+  if (p.window <= 0) return p.max_seq_len;
+  const long reach = (long)p.window + std::max(p.T, 1) - 1 + 31;
+  return (int)std::min<long>(p.max_seq_len, reach);
+}
 constexpr long kDecodeSmallCallBytes = 160L << 20;
 constexpr int kDecodeSmallCallPartitions = 8;
 constexpr long kDecodeSmallCallPairs = 80;
 static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts = kDecodeSmallCallPartitions) {
   const long esz = kv_dtype == PA_FP8_E4M3FN ? 1 : (kv_dtype == PA_BF16 ? 2 : 4);
   if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
-  if (num_partitions_for(p.max_seq_len, p.partition_size) > max_parts) return false;
+  if (num_partitions_for(span_bound(p), p.partition_size) > max_parts) return false;
   if ((long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16) > kDecodeSmallCallPairs) return false;
-  const double bytes = 2.0 * p.B * (double)p.max_seq_len * p.Hkv * p.D * esz;
+  const double bytes = 2.0 * p.B * (double)span_bound(p) * p.Hkv * p.D * esz;
   return bytes <= (double)kDecodeSmallCallBytes;
 }
 // Partitions of 256 tokens instead of the caller's (larger) ones when those would give the device very few
@@ -272,10 +279,10 @@ static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts
 // 28.3 / 27.9; with more workgroups to begin with the finer ones cost more than they bring (8 x 1 K 29.6 / 32.4).
 static int decode_fine_partition(const DecodeParams& p) {
   const int kFine = g_decode_fine.load();
-  if (kFine <= 0 || p.partition_size <= kFine || p.max_seq_len <= kFine) return p.partition_size;
+  if (kFine <= 0 || p.partition_size <= kFine || span_bound(p) <= kFine) return p.partition_size;
   const long slots = (long)p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);      // workgroups per sequence and partition
-  if (p.B * slots * num_partitions_for(p.max_seq_len, p.partition_size) > 64) return p.partition_size;
-  if (num_partitions_for(p.max_seq_len, kFine) > 16) return p.partition_size;
+  if (p.B * slots * num_partitions_for(span_bound(p), p.partition_size) > 64) return p.partition_size;
+  if (num_partitions_for(span_bound(p), kFine) > 16) return p.partition_size;
   return kFine;
 }
 static int decode_kind(const DecodeParams& p, int q_dtype, int kv_dtype, bool needs_balanced = false) {
@@ -313,8 +320,8 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
   plan_decode_balanced(p, current_num_cus());
   const size_t balanced = decode_balanced_workspace_bytes(B, Hq, D, p.bal_gv);
   if (kind == 3) return balanced;
-  // fixed partitions, by choice or by the size of the call: a call with sinks or a window takes the balanced
-  // kernel all the same, so the answer covers both
+  // fixed partitions, by choice or by the size of the call: a forced kernel choice can still send the call to the
+  // balanced kernel, so the answer covers both
   return fixed > balanced ? fixed : balanced;
 }
 
@@ -362,15 +369,17 @@ static int plan_decode(const char* who, DecodePlan& pl, const void* q, const voi
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
   p.block_shift = ilog2_exact(block_size);
   p.partition_size = partition_size;
-  p.num_partitions = num_partitions_for(max_seq_len, partition_size);
   p.max_seq_len = max_seq_len;
+  p.sinks = sinks; p.window = sliding_window;
+  p.num_partitions = num_partitions_for(span_bound(p), partition_size);
   p.scale_log2e = scale * kLog2e;
   p.head_major = g_head_major.load();
   pl.caller_partition = partition_size;
   pl.q_dtype = q_dtype; pl.kv_dtype = kv_dtype;
   if (p.num_partitions > 65535 || B > 65535) return fail_arg("%s: grid too large (partitions=%d B=%d)", who, p.num_partitions, B);
   // kernel choice: 0 automatic, 1 scalar-ALU, 2 MFMA with fixed partitions, 3 MFMA balanced
-  const int kind = pl.kind = decode_kind(p, q_dtype, kv_dtype, sinks != nullptr || sliding_window > 0);
+  // (sinks and a sliding window live in both MFMA kernels; a call forced onto the fixed partitions keeps them)
+  const int kind = pl.kind = decode_kind(p, q_dtype, kv_dtype);
   if (kind < 0) return fail_arg("%s: MFMA kernel forced but shape unsupported", who);
   if (kind == 2 && partition_size % 32) return fail_arg("%s: the fixed-partition MFMA kernel needs partition_size %% 32 == 0", who);
   // a small call of short contexts: the whole context as one partition on eight waves, which merge through LDS, so
@@ -381,20 +390,20 @@ static int plan_decode(const char* who, DecodePlan& pl, const void* q, const voi
   pl.waves = g_decode_waves.load();
   const int single_max = g_decode_single_max.load();
   if (kind == 2 && pl.waves == 0 && g_decode_impl.load() == 0 && p.num_partitions > 1) {
+    const int reach = span_bound(p);
     if (Hq / Hkv <= 8 &&
-        (max_seq_len <= single_max - single_max / 4 || (max_seq_len <= single_max && (long)B * Hkv >= 256))) {
-      p.partition_size = (max_seq_len + 31) & ~31;
+        (reach <= single_max - single_max / 4 || (reach <= single_max && (long)B * Hkv >= 256))) {
+      p.partition_size = (reach + 31) & ~31;
       p.num_partitions = 1;
       pl.waves = 8;
     } else {
       p.partition_size = decode_fine_partition(p);
-      p.num_partitions = num_partitions_for(max_seq_len, p.partition_size);
+      p.num_partitions = num_partitions_for(reach, p.partition_size);
     }
   }
-  if ((sinks || sliding_window > 0) && kind != 3)
-    return fail_arg("%s: sinks and sliding_window need the balanced MFMA kernel (bf16 q, bf16 or fp8 KV, "
+  if ((sinks || sliding_window > 0) && kind == 1)
+    return fail_arg("%s: sinks and sliding_window need the MFMA kernels (bf16 q, bf16 or fp8 KV, "
                     "head_dim 64 or 128, block_size a power of two >= 16)", who);
-  p.sinks = sinks; p.window = sliding_window;
   if (take_q_transform(who, q_transform, kind != 1, p.qt)) return -1;
   return 0;
 }
@@ -429,7 +438,7 @@ static int run_decode(const char* who, DecodePlan& pl, void* workspace, size_t w
     if ((!workspace || workspace_bytes < need) && p.partition_size != pl.caller_partition) {
       // a workspace sized for the caller's partitions only: those, then
       p.partition_size = pl.caller_partition;
-      p.num_partitions = num_partitions_for(p.max_seq_len, p.partition_size);
+      p.num_partitions = num_partitions_for(span_bound(p), p.partition_size);
       need = (size_t)B * Hq * p.num_partitions * ((size_t)D + 2) * sizeof(float);
     }
     if (p.num_partitions > 1) {
@@ -599,18 +608,18 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   // (T = 4, 32 / 8 heads of 128, us per layer replayed from a graph, balanced / fixed partitions): B = 1 behind 4 K
   // 36.0 / 32.9, B = 4 behind 2 K 41.4 / 34.4, B = 4 behind 4 K 47.6 / 38.1, B = 8 behind 2 K 46.8 / 44.0; a single
   // sequence on the finer partitions, B = 1 behind 1 K: 30.5 -> 27.7.  It needs the caller's bound on the lengths (the
-  // table capacity says nothing about the sizes), 16 rows per wave, no sinks and no window, and a workspace that holds
-  // the partitions' partials.
-  if (max_seq_len > 0 && !sinks && sliding_window == 0 && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
+  // table capacity says nothing about the sizes), 16 rows per wave, and a workspace that holds the partitions'
+  // partials.  Under a sliding window the partitions cover what the window reaches, often a single one.
+  if (max_seq_len > 0 && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
     DecodeParams f = p;
     f.partition_size = 512;
     const bool small = decode_small_call(f, kv_dtype);
     if (small) f.partition_size = decode_fine_partition(f);       // a single sequence: finer ones, as for pa_decode
-    f.num_partitions = num_partitions_for(f.max_seq_len, f.partition_size);
+    f.num_partitions = num_partitions_for(span_bound(f), f.partition_size);
     size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
     if (small && f.partition_size != 512 && need_f && !(workspace && workspace_bytes >= need_f)) {
       f.partition_size = 512;
-      f.num_partitions = num_partitions_for(f.max_seq_len, f.partition_size);
+      f.num_partitions = num_partitions_for(span_bound(f), f.partition_size);
     }
     need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
     if (small && (need_f == 0 || (workspace && workspace_bytes >= need_f))) {
@@ -1058,7 +1067,10 @@ int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   // the merge of the decode partitions on the projection's load of its rows, where both kernels are the small-call ones
   // (up to four partitions: the projection requests that many ahead of its weight tiles; with more, the merge's later
   // loads wait behind the tiles and the separate merge launch is faster: B = 8 at 4 K, eight partitions, 45.5 against 43.2 us)
+  // (not with sinks or a window: the projection's merge knows neither the extra term of the denominator nor where a
+  // window's partitions begin)
   const bool merge_on_load = proj && !attn_out && pl.kind == 2 && p.num_partitions > 1 && (p.num_partitions <= 4 || fusion == 3) && fusion != 1 && fusion != 2 &&
+                             !sinks && sliding_window == 0 &&
                              q_dtype == PA_BF16 && o_proj_takes_partials(B, K, D, splits, proj_ws != nullptr);
   if (int rc = run_decode(who, pl, ws, avail, merge_on_load, nullptr, s)) return rc;
   if (!proj) return 0;
@@ -1151,7 +1163,7 @@ int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   memset(&vp, 0, sizeof(vp));
   vp.new_kv = new_kv; vp.k_cache_w = k_cache; vp.v_cache_w = v_cache; vp.k_scale_w = k_scale; vp.v_scale_w = v_scale;
   vp.fuse_rows = fusion != 1 && fusion != 3;
-  vp.want = proj && !attn_out && fusion != 1 && fusion != 2 &&
+  vp.want = proj && !attn_out && fusion != 1 && fusion != 2 && !sinks && sliding_window == 0 &&
             o_proj_takes_partials((int)M, K, D, splits, proj_ws != nullptr);
   rc = verify_launch(who, q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, new_kv->query_lens, attn, ws, avail,
                      B, T, 0, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks, max_seq_len, scale, kv_dtype, sinks,

@@ -150,22 +150,30 @@ __global__ void decode_reduce_kernel(DecodeParams p) {
   int ctx = p.seq_lens[b];
   ctx = min(max(ctx, 0), p.max_seq_len);
   long out_at = ((long)b * p.Hq + vr) * p.D;
+  int tq_rows = 1, head = vr;
   if (multi) {
     // context and rows of this launch as the streaming kernel takes them (query tokens [t0, t0 + T) of T_stride)
     const int qfull = min(min(max(p.query_lens[b], 0), p.T_stride), ctx);
     const int tq = min(max(qfull - p.t0, 0), p.T);
     ctx = tq > 0 ? ctx - qfull + p.t0 + tq : 0;
+    tq_rows = tq;
     const int n_rep = p.Hq / p.Hkv, n_rows = n_rep * p.T;
     const int hk = vr / n_rows, j = vr - hk * n_rows, t = j / n_rep;
-    out_at = (((long)b * p.T_stride + p.t0 + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * p.D;
+    head = hk * n_rep + (j - t * n_rep);
+    out_at = (((long)b * p.T_stride + p.t0 + t) * p.Hq + head) * p.D;
   }
-  const int np = (ctx + p.partition_size - 1) / p.partition_size;
+  // partitions count from the first tile the launch's rows see (a sliding window skips what lies before it)
+  int span = ctx;
+  if (p.window > 0) span -= (max(ctx - tq_rows + 1 - p.window, 0) >> 5) << 5;
+  const int np = (span + p.partition_size - 1) / p.partition_size;
   float mt = -INFINITY;
 #pragma unroll
   for (int i = 0; i < PRE; ++i)
     if (i < np) mt = fmaxf(mt, m_[i]);
   for (int i = PRE; i < np; ++i) mt = fmaxf(mt, p.ws_ml[(base + i) * 2]);
   const float m_ref = mt == -INFINITY ? 0.f : mt;
+  // attention sink: one more term of the denominator, no value
+  const float sink_w = p.sinks ? exp2f(p.sinks[head] * kLog2e - m_ref) : 0.f;
   for (int d = d0; d < p.D; d += blockDim.x) {
     float lt = 0.f, ot = 0.f;
 #pragma unroll
@@ -180,7 +188,7 @@ __global__ void decode_reduce_kernel(DecodeParams p) {
       lt += w;
       ot = __builtin_fmaf(w, p.ws_out[(base + i) * p.D + d], ot);    // (the projection's merge-on-load repeats this arithmetic)
     }
-    Store<QT>::put(p.out, out_at + d, lt > 0.f ? ot / lt : 0.f);
+    Store<QT>::put(p.out, out_at + d, lt > 0.f ? ot / (p.sinks ? lt + sink_w : lt) : 0.f);
   }
 }
 

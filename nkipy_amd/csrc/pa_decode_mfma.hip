@@ -877,7 +877,8 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
     const int hk = vr / n_rows, j = vr - hk * n_rows, t = j / n_rep;
     return (uint16_t*)p.out + (((long)b * p.T_stride + p.t0 + t) * p.Hq + hk * n_rep + (j - t * n_rep)) * D;
   };
-  const int t_begin = part * p.partition_size;
+  // partitions count from the first tile any query row sees (the start of the context, or what a sliding window leaves)
+  const int t_begin = (first_tile(p, b, ctx) << 5) + part * p.partition_size;
   if (t_begin >= ctx) {
     if (ctx == 0 && part == 0 && p.num_partitions == 1) {
       for (int i = tid; i < w.nheads * D; i += NW * 64) out_row(w.hbase + i / D)[i % D] = 0;
@@ -1027,11 +1028,21 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
       lt += sm_l[x][h] * wt;
       ot += sm_o[x][h][pos] * wt;
     }
-    const float o = (MULTI && lt == 0.f) ? 0.f : ot / lt;
     const int vr = w.hbase + h;
     if (p.num_partitions == 1) {
-      out_row(vr)[d] = float_to_bf16_bits(o);
+      // attention sink: one more term of the denominator, no value (as the balanced kernel's store_final)
+      float den = lt;
+      if (p.sinks && lt > 0.f) {
+        int head = vr;
+        if (MULTI) {
+          const int n_rows = n_rep * p.T, hk = vr / n_rows, j = vr - hk * n_rows;
+          head = hk * n_rep + j % n_rep;
+        }
+        den += __builtin_amdgcn_exp2f(p.sinks[head] * kLog2e - mt);
+      }
+      out_row(vr)[d] = float_to_bf16_bits((MULTI && lt == 0.f) ? 0.f : ot / den);
     } else {
+      const float o = (MULTI && lt == 0.f) ? 0.f : ot / lt;
       const long slot = ((long)b * rows_total + vr) * p.num_partitions + part;
       p.ws_out[slot * D + d] = o;
       if (d == 0) { p.ws_ml[slot * 2] = mt; p.ws_ml[slot * 2 + 1] = lt; }
@@ -1161,16 +1172,10 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
   if (scan_in_regs && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
     // tiles before each sequence (and the total), for the merge kernel: it then needs no scan of its own
     int base = 0;
-    for (int bb = 0; bb < p.B; bb += 64) {
-      const int t = (bb + lane < p.B) ? span_tiles(p, bb + lane) : 0;
-      int incl = t;
 #pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int v = __shfl_up(incl, off, 64);
-        if (lane >= off) incl += v;
-      }
-      if (bb + lane < p.B) p.ws_start[bb + lane] = base + incl - t;
-      base += __shfl(incl, 63, 64);
+    for (int i = 0; i < SCAN_STEPS; ++i) {
+      if (64 * i + lane < p.B) p.ws_start[64 * i + lane] = base + incl[i] - tl[i];
+      base += __shfl(incl[i], 63, 64);
     }
     if (lane == 0) p.ws_start[p.B] = base;
   }

@@ -354,7 +354,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     as in `decode`, the window counted back from each query token; so is q_transform, the position of
     row t being seq_lens[b] - query_lens[b] + t.
     max_seq_len: host-known upper bound of seq_lens, as in `decode`; with it a small verify call (a few
-    short sequences, no sinks, no window) takes fixed partitions instead of the balanced schedule, whose
+    short sequences, or a short sliding window) takes fixed partitions instead of the balanced schedule, whose
     fixed cost dominates at that size.  The tiled kernel does not use it.
     """
     lib = _lib.load()

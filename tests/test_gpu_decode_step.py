@@ -63,7 +63,7 @@ def _setup(rng, B, Hq, Hkv, D, bs, ctxs, qlens, N, bias, xform, fp8=False, poiso
     return d
 
 
-def _three_calls(pa, d, scale, psize, msl, attn_only=False):
+def _three_calls(pa, d, scale, psize, msl, attn_only=False, **variant):
     """The sequence decode_step stands for, on copies of the pools."""
     k, v = d["k"].clone(), d["v"].clone()
     ks = None if d["ks"] is None else d["ks"].clone()
@@ -75,7 +75,7 @@ def _three_calls(pa, d, scale, psize, msl, attn_only=False):
     else:
         pa.kv_write(d["xk"][:, None], d["xv"][:, None], k, v, d["tables"], d["lens"], d["qlens"], k_scale=ks, v_scale=vs)
     att = pa.decode(d["xq"], k, v, d["tables"], d["lens"], scale, k_scale=ks, v_scale=vs, partition_size=psize,
-                    max_seq_len=msl, q_transform=d["qt"])
+                    max_seq_len=msl, q_transform=d["qt"], **variant)
     out = att if attn_only or d["ow"] is None else pa.o_proj(att, d["ow"], d["ob"])
     return out, att, k, v, ks, vs
 
@@ -205,14 +205,63 @@ def test_length_bound_below_the_new_token(pa):
     _same_bits(gv, wv, "V pool")
 
 
+SINK_CASES = [
+    # B, Hq, Hkv, D, bs, contexts, N, window, transform
+    (1, 64, 8, 64, 32, [1025], 2880, None, True),            # the gpt-oss layer: sinks on every layer ...
+    (1, 64, 8, 64, 32, [1025], 2880, 128, True),             # ... a 128-token window on every other one: one partition
+    (4, 64, 8, 64, 16, [1500, 129, 128, 1], 2880, 128, True),
+    (3, 32, 8, 128, 32, [2000, 700, 513], 1024, 600, True),  # a window of several partitions
+    (2, 16, 4, 128, 32, [300, 257], 512, 40, False),         # the new token first of a tile, window inside one tile pair
+    (5, 32, 8, 128, 32, [1024, 993, 961, 512, 33], 4096, None, True),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,D,bs,ctxs,N,window,xform", SINK_CASES)
+def test_decode_step_with_sinks_and_window(pa, B, Hq, Hkv, D, bs, ctxs, N, window, xform):
+    """The gpt-oss variant of the layer (examples/models/gpt_oss/kernels/attention.py:117-148) through the one call:
+    sinks and window ride on the small-call kernels, the new row on the decode launch; bit for bit the three calls,
+    and the oracle's values."""
+    rng = np.random.default_rng(B * 100 + Hq + (window or 0))
+    d = _setup(rng, B, Hq, Hkv, D, bs, ctxs, [1] * B, N, True, xform)
+    scale, msl = 1.0 / np.sqrt(D), int(max(ctxs))
+    kw = dict(sinks=torch.from_numpy(rng.standard_normal(Hq).astype(np.float32)).cuda(), sliding_window=window)
+    print(f"decode_step with sinks B={B} Hq={Hq} Hkv={Hkv} D={D} ctx={ctxs} window={window}", flush=True)
+    want, att, wk, wv, _, _ = _three_calls(pa, d, scale, 512, msl, **kw)
+    for fusion in (0, 2, 1):
+        _fusion(fusion)
+        try:
+            got, gk, gv, _, _ = _step(pa, d, scale, 512, msl, **kw)
+            torch.cuda.synchronize()
+        finally:
+            _fusion(0)
+        _same_bits(got, want, f"projected rows, fusion switch {fusion}")
+        _same_bits(gk, wk, f"K pool, fusion switch {fusion}")
+        _same_bits(gv, wv, f"V pool, fusion switch {fusion}")
+    # the attention output against the oracle on the pools the step left
+    a2 = torch.empty_like(d["xq"])
+    _step(pa, d, scale, 512, msl, attn_out=a2, **kw)
+    torch.cuda.synchronize()
+    q = dev_to_f32(d["xq"])
+    if xform:
+        cos, sin = dev_to_f32(d["qt"].rope_cos), dev_to_f32(d["qt"].rope_sin)
+        q = O.qk_norm_rope(q[:, None], dev_to_f32(d["xk"])[:, None], ctxs, [1] * B, cos, sin,
+                           q_norm_weight=dev_to_f32(d["qt"].norm_weight), eps=d["qt"].eps)[0][:, 0]
+    ref = O.paged_decode(O.round_to_bf16(q), dev_to_f32(wk), dev_to_f32(wv), d["tables"].cpu().numpy(), np.asarray(ctxs, np.int32),
+                         scale, q_dtype="bf16", sliding_window=window, sinks=kw["sinks"].cpu().numpy())
+    assert np.abs(dev_to_f32(a2) - ref).max() <= 2e-2
+
+
 @pytest.mark.parametrize("what", ["fp8", "large", "sinks"])
 def test_calls_the_small_step_kernels_do_not_take(pa, what):
-    """fp8 pools (the scale of a block can grow with the new row), calls beyond the small-call bounds and calls with
-    sinks or a window run the separate launches inside the one call: same results."""
+    """fp8 pools (the scale of a block can grow with the new row) and calls beyond the small-call bounds, with sinks
+    and a window too, run the separate launches inside the one call: same results."""
     rng = np.random.default_rng(8)
     if what == "large":
         B, Hq, Hkv, D, bs, N = 48, 32, 8, 128, 32, 1024
         ctxs = [3000 + 13 * i for i in range(B)]
+    elif what == "sinks":
+        B, Hq, Hkv, D, bs, N = 24, 32, 8, 128, 32, 1024
+        ctxs = [1000 + 17 * i for i in range(B)]
     else:
         B, Hq, Hkv, D, bs, N = 4, 32, 8, 128, 32, 1024
         ctxs = [1000, 513, 100, 31]

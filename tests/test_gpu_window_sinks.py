@@ -76,8 +76,8 @@ def test_decode_window_fp8_long_single_sequence(pa):
 
 def test_neutral_options_change_nothing(pa):
     """A window at least as long as every context and sinks of -inf give the plain result bit for bit, in the
-    kernel that implements them (the balanced one).  A plain call this small is served by the fixed-partition
-    kernel by default, whose sums are taken in another order: equal to the tolerance there."""
+    balanced kernel and in the fixed-partition kernel (which serves a call this small by default, and whose sums are
+    taken in another order than the balanced kernel's: equal to the tolerance between the two)."""
     from nkipy_amd import _lib
     lib = _lib.load()
     rng = np.random.default_rng(22)
@@ -94,8 +94,46 @@ def test_neutral_options_change_nothing(pa):
         assert not np.array_equal(dev_bits(pa.decode(*args, sliding_window=2048)), dev_bits(plain))
     finally:
         lib.pa_debug_set(0, 0)
-    assert_close_abs(dev_to_f32(pa.decode(*args)), dev_to_f32(plain), BF16_TOL)
-    assert np.array_equal(dev_bits(pa.decode(*args, sliding_window=2049)), dev_bits(plain))    # options: the balanced kernel
+    small = pa.decode(*args)
+    assert_close_abs(dev_to_f32(small), dev_to_f32(plain), BF16_TOL)
+    assert np.array_equal(dev_bits(pa.decode(*args, sliding_window=2049)), dev_bits(small))
+    assert np.array_equal(dev_bits(pa.decode(*args, sinks=_f32(np.full(Hq, -np.inf)))), dev_bits(small))
+    assert not np.array_equal(dev_bits(pa.decode(*args, sliding_window=2048)), dev_bits(small))
+
+
+@pytest.mark.parametrize("window,part", [(None, 1024), (1, 512), (33, 32), (100, 64), (128, 512), (129, 64), (600, 256),
+                                         (1000, 128), (5000, 1024)])
+@pytest.mark.parametrize("with_sinks", [False, True])
+@pytest.mark.parametrize("D,Hq,Hkv,bs", [(64, 64, 8, 16), (128, 32, 8, 32), (128, 16, 1, 32)])
+def test_decode_window_and_sinks_on_fixed_partitions(pa, window, part, with_sinks, D, Hq, Hkv, bs):
+    """Small calls with a length bound: the fixed-partition kernel, whose partitions count from the first tile the
+    window reaches (one partition on eight waves, one on four, several with the merge launch), forced and by the
+    library's own choice; contexts shorter than the window, ending on tile and partition boundaries."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    if window is None and not with_sinks:
+        pytest.skip("plain decode is covered elsewhere")
+    rng = np.random.default_rng(11 + (window or 0) + D + part)
+    ctxs = [1, 31, 32, 33, 64, 65, 200, 1500, 4097][: 5 if Hkv == 8 else 9] + [part, part + 1, 2 * part + 32]
+    B = len(ctxs)
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    k, v = O.round_to_bf16(k), O.round_to_bf16(v)
+    q = O.round_to_bf16(rng.standard_normal((B, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32) * 2) if with_sinks else None
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_decode(q, k, v, tables, np.asarray(ctxs, np.int32), scale, q_dtype="bf16",
+                          sliding_window=window, sinks=sinks)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), scale)
+    kw = dict(sliding_window=window, sinks=None if sinks is None else bf16_to_dev(sinks), partition_size=part,
+              max_seq_len=max(ctxs))
+    for impl in (2, 0):
+        lib.pa_debug_set(0, impl)
+        try:
+            got = pa.decode(*args, **kw)
+            torch.cuda.synchronize()
+        finally:
+            lib.pa_debug_set(0, 0)
+        assert_close_abs(dev_to_f32(got), want, BF16_TOL)
 
 
 @pytest.fixture(params=[16, 32], ids=["rows16", "rows32"])
@@ -129,6 +167,34 @@ def test_verify_window_and_sinks(pa, rows, window, T, Hq, Hkv, D, bs):
     torch.cuda.synchronize()
     got = dev_to_f32(got)
     assert_close_abs(got, want, BF16_TOL)
+    for b, n in enumerate(qlens):
+        assert np.all(got[b, n:] == 0)
+
+
+@pytest.mark.parametrize("window", [None, 1, 30, 64, 128, 700])
+@pytest.mark.parametrize("T,Hq,Hkv,D,bs", [(4, 64, 8, 64, 16), (4, 32, 8, 128, 32), (3, 8, 2, 128, 32)])
+def test_verify_window_and_sinks_small_calls(pa, window, T, Hq, Hkv, D, bs):
+    """With the caller's length bound a small verify call takes the fixed partitions, sinks and window included:
+    rows of one sequence whose windows begin in different tiles, 16 and 32 rows per kv head."""
+    rng = np.random.default_rng(100 * T + (window or 7) + D)
+    qlens = [T, max(T - 1, 1), 1, T, 0]
+    prefixes = [0, 300, 65, 1533, 40]
+    B = len(qlens)
+    ctxs = [p + t for p, t in zip(prefixes, qlens)]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, [max(c, 1) for c in ctxs])
+    k, v = O.round_to_bf16(k), O.round_to_bf16(v)
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    sinks = O.round_to_bf16(rng.standard_normal(Hq).astype(np.float32))
+    scale = 1.0 / np.sqrt(D)
+    want = O.paged_prefill(q, k, v, tables, np.asarray(ctxs, np.int32), np.asarray(qlens, np.int32), scale,
+                           q_dtype="bf16", sliding_window=window, sinks=sinks)
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(tables), _i32(ctxs), _i32(qlens), scale)
+    got = pa.verify(*args, sliding_window=window, sinks=bf16_to_dev(sinks), max_seq_len=max(ctxs))
+    free = pa.verify(*args, sliding_window=window, sinks=bf16_to_dev(sinks))
+    torch.cuda.synchronize()
+    got = dev_to_f32(got)
+    assert_close_abs(got, want, BF16_TOL)
+    assert_close_abs(dev_to_f32(free), want, BF16_TOL)
     for b, n in enumerate(qlens):
         assert np.all(got[b, n:] == 0)
 
