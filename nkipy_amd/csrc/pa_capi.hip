@@ -1067,10 +1067,9 @@ int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   // the merge of the decode partitions on the projection's load of its rows, where both kernels are the small-call ones
   // (up to four partitions: the projection requests that many ahead of its weight tiles; with more, the merge's later
   // loads wait behind the tiles and the separate merge launch is faster: B = 8 at 4 K, eight partitions, 45.5 against 43.2 us)
-  // (not with sinks or a window: the projection's merge knows neither the extra term of the denominator nor where a
-  // window's partitions begin)
+  // (not under a sliding window: the projection's merge does not know where a window's partitions begin)
   const bool merge_on_load = proj && !attn_out && pl.kind == 2 && p.num_partitions > 1 && (p.num_partitions <= 4 || fusion == 3) && fusion != 1 && fusion != 2 &&
-                             !sinks && sliding_window == 0 &&
+                             sliding_window == 0 &&
                              q_dtype == PA_BF16 && o_proj_takes_partials(B, K, D, splits, proj_ws != nullptr);
   if (int rc = run_decode(who, pl, ws, avail, merge_on_load, nullptr, s)) return rc;
   if (!proj) return 0;
@@ -1082,7 +1081,7 @@ int pa_decode_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   if (merge_on_load && p.num_partitions > 1) {
     o.part_o = p.ws_out; o.part_ml = p.ws_ml; o.part_seq_lens = seq_lens;
     o.part_np = p.num_partitions; o.part_size = p.partition_size; o.part_max_seq_len = p.max_seq_len; o.part_D = D;
-    o.part_T = 1; o.part_n_rep = Hq / Hkv;
+    o.part_T = 1; o.part_n_rep = Hq / Hkv; o.part_sinks = sinks;
   } else {
     o.x = attn;
   }
@@ -1163,7 +1162,7 @@ int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   memset(&vp, 0, sizeof(vp));
   vp.new_kv = new_kv; vp.k_cache_w = k_cache; vp.v_cache_w = v_cache; vp.k_scale_w = k_scale; vp.v_scale_w = v_scale;
   vp.fuse_rows = fusion != 1 && fusion != 3;
-  vp.want = proj && !attn_out && fusion != 1 && fusion != 2 && !sinks && sliding_window == 0 &&
+  vp.want = proj && !attn_out && fusion != 1 && fusion != 2 && sliding_window == 0 &&
             o_proj_takes_partials((int)M, K, D, splits, proj_ws != nullptr);
   rc = verify_launch(who, q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, new_kv->query_lens, attn, ws, avail,
                      B, T, 0, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks, max_seq_len, scale, kv_dtype, sinks,
@@ -1182,7 +1181,7 @@ int pa_verify_step(const void* q, const pa_new_kv* new_kv, void* k_cache, void* 
   if (vp.left) {
     o.part_o = vp.f.ws_out; o.part_ml = vp.f.ws_ml; o.part_seq_lens = seq_lens; o.part_query_lens = new_kv->query_lens;
     o.part_np = vp.f.num_partitions; o.part_size = vp.f.partition_size; o.part_max_seq_len = vp.f.max_seq_len; o.part_D = D;
-    o.part_T = T; o.part_n_rep = Hq / Hkv;
+    o.part_T = T; o.part_n_rep = Hq / Hkv; o.part_sinks = sinks;
   } else {
     o.x = attn;
   }

@@ -326,6 +326,7 @@ struct OProjParams {
   const float* part_ml;     // [B, Hq * T rows, np, 2] (max, sum) of each partial
   const int32_t* part_seq_lens;   // [B] context lengths (clamped to part_max_seq_len as the decode launch did)
   const int32_t* part_query_lens; // multi-token launch: [B] query tokens per sequence; null for decode
+  const float* part_sinks;        // [Hq] sink logits of the attention call (one more term of each row's denominator), or null
   int part_np, part_size, part_max_seq_len, part_D;
   int part_T, part_n_rep;         // tokens per sequence in the launch (x row m is token m % T of sequence m / T), q heads per kv head
 };

@@ -580,16 +580,17 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
   f2_t e_ml[NE][NPRE];
   f4_t e_oa[NE][NPRE], e_ob[NE][NPRE];
   int e_len[NE], e_qlen[NE];
+  float e_sink[NE];
   const int m_items = MERGE ? ktiles * 8 * p.M : 0;
   // x row m is query token m % T of sequence m / T; its q head `head` is row hk n_rep T + t n_rep + j of the sequence's
   // partials, the decode kernels' numbering of (token, head) pairs (T = 1: the q head itself)
-  auto item_place = [&](int item, int& kt, int& m, int& c, int& d, long& base, int& b) __attribute__((always_inline)) {
+  auto item_place = [&](int item, int& kt, int& m, int& c, int& d, long& base, int& b, int& head) __attribute__((always_inline)) {
     const int per_step = 8 * p.M;
     kt = item / per_step;
     const int rem = item - kt * per_step;
     m = rem >> 3; c = rem & 7;
     const int k0 = (kt_begin + kt) * BK + 8 * c;
-    const int head = k0 / p.part_D;
+    head = k0 / p.part_D;
     d = k0 - head * p.part_D;
     const int T = p.part_T, n_rep = p.part_n_rep;
     b = m / T;
@@ -607,10 +608,15 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
   if (MERGE) {
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
-      int kt, m, c, d, b; long base;
-      item_place(min(tid + 256 * e, m_items - 1), kt, m, c, d, base, b);
+      int kt, m, c, d, b, head; long base;
+      item_place(min(tid + 256 * e, m_items - 1), kt, m, c, d, base, b, head);
       const int32_t* plen = p.part_seq_lens + b;
       asm volatile("global_load_dword %0, %1, off" : "=&v"(e_len[e]) : "v"(plen) : "memory");
+      e_sink[e] = 0.f;
+      if (p.part_sinks) {
+        const float* ps = p.part_sinks + head;
+        asm volatile("global_load_dword %0, %1, off" : "=&v"(e_sink[e]) : "v"(ps) : "memory");
+      }
       e_qlen[e] = 1;
       if (p.part_query_lens) {
         const int32_t* pq = p.part_query_lens + b;
@@ -645,7 +651,7 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     // one q head.  Up to NPRE partitions' values are requested before any is used (slots past a sequence's own
     // partition count exist and are loaded, not used).
     const int Dh = p.part_D, np_max = p.part_np;
-    auto finish = [&](int kt, int m, int c, int d, long base, int ctx, const f2_t (&ml)[NPRE], const f4_t (&oa)[NPRE],
+    auto finish = [&](int kt, int m, int c, int d, long base, int ctx, float sink, const f2_t (&ml)[NPRE], const f4_t (&oa)[NPRE],
                       const f4_t (&ob)[NPRE]) __attribute__((always_inline)) {
       const int np = min((ctx + p.part_size - 1) / p.part_size, np_max);
       float mt = -INFINITY;
@@ -672,9 +678,12 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
         const f4_t a = *(const f4_t*)(p.part_o + (base + i) * Dh + d), b = *(const f4_t*)(p.part_o + (base + i) * Dh + d + 4);
         add(p.part_ml[(base + i) * 2], p.part_ml[(base + i) * 2 + 1], a, b);
       }
+      // attention sink: one more term of the denominator (decode_reduce_kernel's expression)
+      const float sink_w = p.part_sinks ? exp2f(sink * kLog2e - m_ref) : 0.f;
+      const float den = p.part_sinks ? lt + sink_w : lt;
       float o[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = lt > 0.f ? ot[j] / lt : 0.f;
+      for (int j = 0; j < 8; ++j) o[j] = lt > 0.f ? ot[j] / den : 0.f;
       *(uint4*)(smem + kt * RS_STAGE + m * 128 + ((c ^ ((m >> 1) & 7)) << 4)) =
           make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
     };
@@ -685,18 +694,18 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
     for (int e = 0; e < NE; ++e) {
 #pragma unroll
       for (int i = 0; i < NPRE; ++i) asm volatile("" : "+v"(e_ml[e][i]), "+v"(e_oa[e][i]), "+v"(e_ob[e][i]));
-      asm volatile("" : "+v"(e_len[e]), "+v"(e_qlen[e]));
+      asm volatile("" : "+v"(e_len[e]), "+v"(e_qlen[e]), "+v"(e_sink[e]));
       const int item = tid + 256 * e;
       if (item < m_items) {
-        int kt, m, c, d, b; long base;
-        item_place(item, kt, m, c, d, base, b);
-        finish(kt, m, c, d, base, context_of(e_len[e], e_qlen[e]), e_ml[e], e_oa[e], e_ob[e]);
+        int kt, m, c, d, b, head; long base;
+        item_place(item, kt, m, c, d, base, b, head);
+        finish(kt, m, c, d, base, context_of(e_len[e], e_qlen[e]), e_sink[e], e_ml[e], e_oa[e], e_ob[e]);
       }
     }
     // more than NE items per thread (more than 8 rows): the rest by ordinary loads
     for (int item = tid + 256 * NE; item < m_items; item += 256) {
-      int kt, m, c, d, b; long base;
-      item_place(item, kt, m, c, d, base, b);
+      int kt, m, c, d, b, head; long base;
+      item_place(item, kt, m, c, d, base, b, head);
       f2_t ml[NPRE];
       f4_t oa[NPRE], ob[NPRE];
 #pragma unroll
@@ -706,7 +715,8 @@ __global__ __launch_bounds__(256) void o_proj_resident_kernel(OProjParams p) {
         oa[i] = *(const f4_t*)(p.part_o + at * Dh + d);
         ob[i] = *(const f4_t*)(p.part_o + at * Dh + d + 4);
       }
-      finish(kt, m, c, d, base, context_of(p.part_seq_lens[b], p.part_query_lens ? p.part_query_lens[b] : 1), ml, oa, ob);
+      finish(kt, m, c, d, base, context_of(p.part_seq_lens[b], p.part_query_lens ? p.part_query_lens[b] : 1),
+             p.part_sinks ? p.part_sinks[head] : 0.f, ml, oa, ob);
     }
   }
   int x_off[4], w_off;

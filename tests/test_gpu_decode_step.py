@@ -227,7 +227,7 @@ def test_decode_step_with_sinks_and_window(pa, B, Hq, Hkv, D, bs, ctxs, N, windo
     kw = dict(sinks=torch.from_numpy(rng.standard_normal(Hq).astype(np.float32)).cuda(), sliding_window=window)
     print(f"decode_step with sinks B={B} Hq={Hq} Hkv={Hkv} D={D} ctx={ctxs} window={window}", flush=True)
     want, att, wk, wv, _, _ = _three_calls(pa, d, scale, 512, msl, **kw)
-    for fusion in (0, 2, 1):
+    for fusion in (0, 2, 3, 1):
         _fusion(fusion)
         try:
             got, gk, gv, _, _ = _step(pa, d, scale, 512, msl, **kw)
@@ -424,6 +424,31 @@ VERIFY_CASES = [
     (3, 16, 8, 8, 64, 32, [530, 16, 1040], [16, 16, 9], 256, True, True, True, False),     # 16 new tokens, head dim 64, across borders
     (2, 4, 32, 8, 128, 32, [600, 900], [4, 4], 512, False, False, True, False),    # no transform: rows stored as given
 ]
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,D,bs,ctxs,qlens,N,window", [
+    (1, 4, 64, 8, 64, 32, [1030], [4], 2880, None),           # the gpt-oss layer at the reference's operating point
+    (1, 4, 64, 8, 64, 32, [1030], [4], 2880, 128),            # ... its windowed layers: one partition
+    (3, 4, 32, 8, 128, 32, [1500, 515, 4], [4, 3, 4], 1024, 600),
+    (2, 4, 32, 8, 128, 16, [700, 258], [4, 4], 512, None),    # two partitions of 512: merged on the projection's load
+])
+def test_verify_step_with_sinks_and_window(pa, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, window):
+    rng = np.random.default_rng(B * 10 + T + Hq + (window or 0))
+    d = _setup_multi(rng, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, True, True)
+    scale, msl = 1.0 / np.sqrt(D), int(max(ctxs))
+    kw = dict(sinks=torch.from_numpy(rng.standard_normal(Hq).astype(np.float32)).cuda(), sliding_window=window)
+    print(f"verify_step with sinks B={B} T={T} Hq={Hq} D={D} ctx={ctxs} window={window}", flush=True)
+    want, att, wk, wv, _, _ = _verify_three_calls(pa, d, scale, msl, **kw)
+    for fusion in (0, 2, 3, 1):
+        _fusion(fusion)
+        try:
+            got, gk, gv, _, _ = _verify_step(pa, d, scale, msl, **kw)
+            torch.cuda.synchronize()
+        finally:
+            _fusion(0)
+        _same_bits(got, want, f"projected rows, fusion switch {fusion}")
+        _same_bits(gk, wk, "K pool")
+        _same_bits(gv, wv, "V pool")
 
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,D,bs,ctxs,qlens,N,bias,xform,bounded,fp8", VERIFY_CASES)
