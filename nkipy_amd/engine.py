@@ -278,6 +278,9 @@ class PagedAttention:
             raise ValueError(f"o_weight must be [{n_heads * cache.head_dim}, hidden], got {tuple(o_weight.shape)}")
         self._out: Dict[int, torch.Tensor] = {}
         self._proj: Dict[int, torch.Tensor] = {}
+        # decode / verify steps prepared once per (T, length bound, storage of xq / xk / xv): a loop that feeds the
+        # layer from the same buffers every step pays the argument checks once (see paged_attn.PreparedStep)
+        self._steps: Dict[tuple, tuple] = {}
 
     def step(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, query_lens: Sequence[int]) -> torch.Tensor:
         if xq.shape[0] != self.cache.max_seqs or len(query_lens) != xq.shape[0]:
@@ -285,6 +288,25 @@ class PagedAttention:
                              f"{len(query_lens)} lengths")
         self.cache.begin_step(query_lens, xq.shape[1])
         return self.attend(xq, xk, xv)
+
+    def reset_steps(self) -> None:
+        """Forget the prepared steps (after replacing a tensor the layer was built with: weights, sinks, norm weights)."""
+        self._steps.clear()
+
+    def _prepared(self, T, bound, xq, xk, xv, make):
+        """The prepared step for these row buffers, built by `make()` on first use.  A step is reused only for the
+        very storage, shapes and strides it was prepared with (it keeps them alive, so an address cannot come back as
+        another tensor's)."""
+        key = (T, bound, xq.data_ptr(), xk.data_ptr(), xv.data_ptr())
+        sig = (xq.shape, xq.stride(), xk.shape, xk.stride(), xv.shape, xv.stride(), xq.dtype, xk.dtype, xv.dtype)
+        hit = self._steps.get(key)
+        if hit is not None and hit[0] == sig:
+            return hit[1]
+        if len(self._steps) >= 4:          # callers that bring fresh tensors every step: nothing to reuse, nothing to hoard
+            self._steps.pop(next(iter(self._steps)))
+        st = make()
+        self._steps[key] = (sig, st)
+        return st
 
     def _q_transform(self):
         """The layer's Q transform for the attention kernels (one object, validated once), None without RoPE."""
@@ -304,7 +326,10 @@ class PagedAttention:
         if B != c.max_seqs or T != c.step_tokens:
             raise ValueError(f"expected [{c.max_seqs}, {c.step_tokens}, ...] as opened by begin_step, got [{B}, {T}, ...]")
         capturing = c.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
-        bound = max_seq_len if max_seq_len is not None else (c.max_model_len if capturing else max(c.max_seq_len, 1))
+        # (the host-known maximum in steps of 256 tokens, the finest partition the kernels choose by it: the bound is part
+        # of what a prepared step is prepared for, and contexts grow by a token a step)
+        bound = max_seq_len if max_seq_len is not None else (
+            c.max_model_len if capturing else min(c.max_model_len, (max(c.max_seq_len, 1) + 255) // 256 * 256))
         if bound < c.max_seq_len:
             raise ValueError(f"max_seq_len {bound} is below a live context of {c.max_seq_len} tokens")
         kc, vc, ks, vs = c.k_caches[l], c.v_caches[l], c.k_scales[l], c.v_scales[l]
@@ -319,41 +344,43 @@ class PagedAttention:
             # being captured into a HIP graph, which will be replayed on longer contexts and so gets the longest
             # sequence the cache admits.  The decode kernels treat every slot as live; idle slots (seq_len 0) come
             # back as zeros (projected: the bias).
-            qt = self._q_transform()
-            if self.o_weight is None:
-                paged_attn.decode_step(xq[:, 0], xk[:, 0], xv[:, 0], kc, vc, c.block_tables, c.seq_lens, c.query_lens,
-                                       self.scale, k_scale=ks, v_scale=vs, partition_size=self.partition_size,
-                                       max_seq_len=bound, q_transform=qt,
-                                       k_norm_weight=None if self.rope is None else self.k_norm_weight, out=out[:, 0],
-                                       sinks=self.sinks, sliding_window=self.sliding_window)
-                return out
-            proj = self._proj.get(T)
-            if proj is None:
-                proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
-            paged_attn.decode_step(xq[:, 0], xk[:, 0], xv[:, 0], kc, vc, c.block_tables, c.seq_lens, c.query_lens,
-                                   self.scale, k_scale=ks, v_scale=vs, partition_size=self.partition_size,
-                                   max_seq_len=bound, q_transform=qt,
-                                   k_norm_weight=None if self.rope is None else self.k_norm_weight,
-                                   o_weight=self.o_weight, o_bias=self.o_bias, out=proj[:, 0],
-                                   sinks=self.sinks, sliding_window=self.sliding_window)
-            return proj
+            proj = None
+            if self.o_weight is not None:
+                proj = self._proj.get(T)
+                if proj is None:
+                    proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
+            res = out if proj is None else proj
+
+            def make():
+                return paged_attn.prepare_decode_step(
+                    xq[:, 0], xk[:, 0], xv[:, 0], kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
+                    k_scale=ks, v_scale=vs, partition_size=self.partition_size, max_seq_len=bound,
+                    q_transform=self._q_transform(), k_norm_weight=None if self.rope is None else self.k_norm_weight,
+                    o_weight=self.o_weight, o_bias=self.o_bias, out=res[:, 0], sinks=self.sinks,
+                    sliding_window=self.sliding_window)
+
+            self._prepared(T, bound, xq, xk, xv, make).launch()
+            return res
         if T > 1 and (self.rope is None or paged_attn.q_transform_supported(T, c.head_dim, c.block_size)) and \
                 paged_attn.prefill_route(B, T, self.n_heads, c.n_kv_heads, c.head_dim, c.block_size, ks is not None,
                                          self.sliding_window or 0) == "verify":
             # a verify step (a few tokens per sequence through the decode-shaped kernel): one call as well
-            qt = self._q_transform()
-            kw = dict(k_scale=ks, v_scale=vs, max_seq_len=bound, q_transform=qt,
-                      k_norm_weight=None if self.rope is None else self.k_norm_weight, sinks=self.sinks,
-                      sliding_window=self.sliding_window)
-            if self.o_weight is None:
-                paged_attn.verify_step(xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale, out=out, **kw)
-                return out
-            proj = self._proj.get(T)
-            if proj is None:
-                proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
-            paged_attn.verify_step(xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale,
-                                   o_weight=self.o_weight, o_bias=self.o_bias, out=proj, **kw)
-            return proj
+            proj = None
+            if self.o_weight is not None:
+                proj = self._proj.get(T)
+                if proj is None:
+                    proj = self._proj[T] = torch.empty((B, T, self.o_weight.shape[1]), dtype=torch.bfloat16, device=c.device)
+            res = out if proj is None else proj
+
+            def make():
+                return paged_attn.prepare_verify_step(
+                    xq, xk, xv, kc, vc, c.block_tables, c.seq_lens, c.query_lens, self.scale, k_scale=ks, v_scale=vs,
+                    max_seq_len=bound, q_transform=self._q_transform(),
+                    k_norm_weight=None if self.rope is None else self.k_norm_weight, o_weight=self.o_weight,
+                    o_bias=self.o_bias, out=res, sinks=self.sinks, sliding_window=self.sliding_window)
+
+            self._prepared(T, bound, xq, xk, xv, make).launch()
+            return res
         qt = None
         if self.rope is not None:
             # the Q half of the norm and rotation rides on the attention kernel's Q load where that

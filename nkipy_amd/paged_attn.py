@@ -698,9 +698,34 @@ def o_proj(x, o_weight, bias=None, *, out=None, workspace=None):
     return out
 
 
-def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
-                partition_size=512, max_seq_len=None, q_transform=None, k_norm_weight=None, o_weight=None, o_bias=None,
-                out=None, attn_out=None, workspace=None, sinks=None, sliding_window=None):
+class PreparedStep:
+    """A `decode_step` / `verify_step` call with its arguments checked and marshalled once, for callers that issue
+    the same step on the same tensors again and again (a layer of a decode loop run without a HIP graph: the call
+    is then bound by the host, and most of the host's time went into re-checking what had not changed).  `launch()`
+    issues it on the current stream and returns `out`.  The step is tied to the storage of every tensor it was
+    prepared with (they are kept alive): new values are copied into them, not passed."""
+    __slots__ = ("fn", "who", "head", "tail", "need", "workspace", "device", "out", "keep")
+
+    def launch(self):
+        stream = _stream_ptr(self.device)
+        ws = self.workspace if self.workspace is not None else _workspace(self.device, self.need, stream)
+        with _on(self.device):
+            rc = self.fn(*self.head, ws.data_ptr(), ws.numel(), *self.tail, stream)
+        _raise_on(rc, self.who)
+        return self.out
+
+    __call__ = launch
+
+
+def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, **kw):
+    """One decode step of an attention layer in one call; arguments and result as `prepare_decode_step`, which this is
+    followed by `launch()`."""
+    return prepare_decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, **kw).launch()
+
+
+def prepare_decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
+                        partition_size=512, max_seq_len=None, q_transform=None, k_norm_weight=None, o_weight=None, o_bias=None,
+                        out=None, attn_out=None, workspace=None, sinks=None, sliding_window=None) -> PreparedStep:
     """One decode step of an attention layer in one call: the cache update, the attention and, with `o_weight`, the
     output projection -- the decode branch of the reference's attention_kernel as a whole
     (examples/models/qwen3/kernels/attention.py:78-147; examples/models/gpt_oss/kernels/attention.py:85-163).
@@ -713,8 +738,9 @@ def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens
     (a `QTransform`: Q's norm weight and the RoPE tables) is given; `k_norm_weight` [D] is K's norm weight (None: K is
     rotated only).  seq_lens counts the new token; query_lens [B] int32 is 1 for the sequences that take one and 0 for
     those that do not.  The pools (and the scales of a float8 pool) are updated in place.
-    Returns the projected rows [B, N] when `o_weight` [Hq * D, N] is given (written to `out` if passed; `attn_out`
-    [B, Hq, D], if passed, also receives the attention output), else the attention output [B, Hq, D] (`out`).
+    The step's result (`PreparedStep.out`, what `launch()` returns) is the projected rows [B, N] when `o_weight`
+    [Hq * D, N] is given (written to `out` if passed; `attn_out` [B, Hq, D], if passed, also receives the attention
+    output), else the attention output [B, Hq, D] (`out`).  Nothing is launched here.
     """
     lib = _lib.load()
     for n, t in (("xq", xq), ("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
@@ -786,10 +812,7 @@ def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens
     if need is None:
         with _on(xq.device):
             need = _decode_step_need[key] = int(lib.pa_decode_step_workspace_bytes(*key))
-    stream = _stream_ptr(xq.device)
-    if workspace is None:
-        workspace = _workspace(xq.device, need, stream)
-    else:
+    if workspace is not None:
         _need_device("workspace", workspace)
         _check(workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.data_ptr() % 16 == 0,
                "workspace must be a contiguous, 16-byte aligned uint8 tensor")
@@ -798,29 +821,37 @@ def decode_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens
     addr = lambda t: None if t is None else t.data_ptr()
     nkv = _lib.NewKvStruct(addr(xk), addr(xv), addr(k_norm_weight), addr(query_lens))
     proj = None if o_weight is None else _lib.OutProjStruct(addr(o_weight), addr(o_bias), addr(out), N)
-    with _on(xq.device):
-        rc = lib.pa_decode_step(_ptr(xq), ctypes.addressof(nkv), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
-                                _ptr(block_tables), _ptr(seq_lens), _ptr(attn_out),
-                                None if proj is None else ctypes.addressof(proj), _ptr(workspace), workspace.numel(),
-                                B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
-                                float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, qt_ptr, stream)
-    _raise_on(rc, "pa_decode_step")
-    return out
+    st = PreparedStep()
+    st.fn, st.who, st.need, st.workspace, st.device, st.out = lib.pa_decode_step, "pa_decode_step", need, workspace, xq.device, out
+    st.head = (_ptr(xq), ctypes.addressof(nkv), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+               _ptr(block_tables), _ptr(seq_lens), _ptr(attn_out), None if proj is None else ctypes.addressof(proj))
+    st.tail = (B, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
+               float(scale), partition_size, q_code, kv_code, _ptr(sinks), win, qt_ptr)
+    # everything an address above points into stays alive with the step
+    st.keep = (nkv, proj, qt_keep, xq, xk, xv, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens,
+               attn_out, out, sinks, k_norm_weight, o_weight, o_bias, q_transform)
+    return st
 
 
 _decode_step_need = {}
 
 
-def verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
-                max_seq_len=None, q_transform=None, k_norm_weight=None, o_weight=None, o_bias=None, out=None,
-                attn_out=None, workspace=None, sinks=None, sliding_window=None):
+def verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, **kw):
+    """A speculative verify step of an attention layer in one call; arguments and result as `prepare_verify_step`,
+    which this is followed by `launch()`."""
+    return prepare_verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, **kw).launch()
+
+
+def prepare_verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k_scale=None, v_scale=None,
+                        max_seq_len=None, q_transform=None, k_norm_weight=None, o_weight=None, o_bias=None, out=None,
+                        attn_out=None, workspace=None, sinks=None, sliding_window=None) -> PreparedStep:
     """A speculative verify step of an attention layer in one call: `decode_step` for up to 64 new tokens per sequence
     (examples/models/gpt_oss/kernels/attention.py:80-163 with seq_len = K + 1; peagle/speculate.py:137-202).
 
     Bit for bit `qk_norm_rope_kv_write(None, xk, xv, ...)` (`kv_write` without `q_transform`), `verify(xq, ...)`,
     `o_proj(...)`.  xq [B, T, Hq, D], xk / xv [B, T, Hkv, D] bfloat16; query_lens [B]: new tokens per sequence (rows
-    t >= query_lens[b] are padding: zero attention output, bias after the projection).  Returns [B, T, N] with
-    `o_weight`, else the attention output [B, T, Hq, D]."""
+    t >= query_lens[b] are padding: zero attention output, bias after the projection).  The step's result is
+    [B, T, N] with `o_weight`, else the attention output [B, T, Hq, D].  Nothing is launched here."""
     lib = _lib.load()
     for n, t in (("xq", xq), ("xk", xk), ("xv", xv), ("k_cache", k_cache), ("v_cache", v_cache),
                  ("block_tables", block_tables), ("seq_lens", seq_lens), ("query_lens", query_lens)):
@@ -889,10 +920,7 @@ def verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens
     if need is None:
         with _on(xq.device):
             need = _decode_step_need[key] = int(lib.pa_verify_step_workspace_bytes(B, T, Hq, D, N))
-    stream = _stream_ptr(xq.device)
-    if workspace is None:
-        workspace = _workspace(xq.device, need, stream)
-    else:
+    if workspace is not None:
         _need_device("workspace", workspace)
         _check(workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.data_ptr() % 16 == 0,
                "workspace must be a contiguous, 16-byte aligned uint8 tensor")
@@ -901,14 +929,15 @@ def verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens
     addr = lambda t: None if t is None else t.data_ptr()
     nkv = _lib.NewKvStruct(addr(xk), addr(xv), addr(k_norm_weight), addr(query_lens))
     proj = None if o_weight is None else _lib.OutProjStruct(addr(o_weight), addr(o_bias), addr(out), N)
-    with _on(xq.device):
-        rc = lib.pa_verify_step(_ptr(xq), ctypes.addressof(nkv), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
-                                _ptr(block_tables), _ptr(seq_lens), _ptr(attn_out),
-                                None if proj is None else ctypes.addressof(proj), _ptr(workspace), workspace.numel(),
-                                B, T, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
-                                float(scale), kv_code, _ptr(sinks), win, qt_ptr, stream)
-    _raise_on(rc, "pa_verify_step")
-    return out
+    st = PreparedStep()
+    st.fn, st.who, st.need, st.workspace, st.device, st.out = lib.pa_verify_step, "pa_verify_step", need, workspace, xq.device, out
+    st.head = (_ptr(xq), ctypes.addressof(nkv), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
+               _ptr(block_tables), _ptr(seq_lens), _ptr(attn_out), None if proj is None else ctypes.addressof(proj))
+    st.tail = (B, T, Hq, Hkv, D, block_size, block_tables.shape[1], num_blocks, msl,
+               float(scale), kv_code, _ptr(sinks), win, qt_ptr)
+    st.keep = (nkv, proj, qt_keep, xq, xk, xv, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens,
+               attn_out, out, sinks, k_norm_weight, o_weight, o_bias, q_transform)
+    return st
 def o_proj_workspace_bytes(M: int, K: int, N: int) -> int:
     """Scratch bytes `o_proj` would use for a call of M rows (0 for shapes that take none)."""
     return int(_lib.load().pa_o_proj_workspace_bytes(int(M), int(K), int(N)))

@@ -288,6 +288,35 @@ def test_calls_the_small_step_kernels_do_not_take(pa, what):
         _same_bits(gvs, vs, "V scales")
 
 
+def test_prepared_step_is_the_call_it_was_prepared_from(pa):
+    """prepare_decode_step / prepare_verify_step check and marshal once; launch() on the same buffers with new contents
+    (rows copied in, lengths advanced in place) gives what a fresh call on those contents gives, bit for bit."""
+    rng = np.random.default_rng(31)
+    B, Hq, Hkv, D, bs, N = 3, 32, 8, 128, 32, 1024
+    ctxs = np.array([700, 513, 31])
+    for T in (1, 3):
+        d = (_setup(rng, B, Hq, Hkv, D, bs, ctxs + 8 * T, [T] * B, N, True, True, poison=False) if T == 1 else
+             _setup_multi(rng, B, T, Hq, Hkv, D, bs, ctxs + 8 * T, [T] * B, N, True, True))
+        scale, msl = 1.0 / np.sqrt(D), 800
+        k, v = d["k"].clone(), d["v"].clone()
+        k2, v2 = k.clone(), v.clone()
+        d["lens"].copy_(_i32(ctxs))
+        kw = dict(max_seq_len=msl, q_transform=d["qt"], k_norm_weight=d["wk"], o_weight=d["ow"], o_bias=d["ob"])
+        prep = (pa.prepare_decode_step if T == 1 else pa.prepare_verify_step)(
+            d["xq"], d["xk"], d["xv"], k, v, d["tables"], d["lens"], d["qlens"], scale, **kw)
+        fresh = pa.decode_step if T == 1 else pa.verify_step
+        for step in range(4):
+            d["lens"].add_(T)
+            for name in ("xq", "xk", "xv"):
+                d[name].copy_(bf16_to_dev(rng.standard_normal(tuple(d[name].shape)).astype(np.float32)))
+            got = prep.launch().clone()
+            want = fresh(d["xq"].clone(), d["xk"].clone(), d["xv"].clone(), k2, v2, d["tables"], d["lens"], d["qlens"], scale, **kw)
+            torch.cuda.synchronize()
+            _same_bits(got, want, f"T={T} step {step}")
+            _same_bits(k, k2, "K pool")
+            _same_bits(v, v2, "V pool")
+
+
 def test_decode_step_in_a_graph(pa):
     """Captured once with a caller-owned workspace, replayed on growing contexts; every replay equals the three calls."""
     rng = np.random.default_rng(9)
