@@ -10,7 +10,7 @@ carries, under "configs", one record each for config 3 (paged chunked prefill),
 config 4 (blocksparse prefill) and config 5 (fp8-KV long-context decode), timed in
 the same run with the same protocol: both halves of the headline metric and every
 benchmark-sized configuration, plus "o_proj", the output projection behind config 3's
-attention.  --config N prints that configuration alone (6-16: the kernels and steps around the
+attention.  --config N prints that configuration alone (6-17: the kernels and steps around the
 attention call; their docstrings say what each one is).
 
 value      whole-step throughput: algorithmic HBM bytes / step time for the decode
@@ -238,7 +238,8 @@ def bench_decode(cfg, steps, warmup, lib, pa, W):
         "roofline": {"bound": "hbm", "achieved": round(ab / (kavg * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(ab / (kavg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": _traffic(cfg)[0], "traffic_source": _traffic(cfg)[1],
-                     "kernel": "decode_balanced_kernel", "kernel_avg_ms": round(kavg, 5),
+                     "kernel": "decode_balanced_kernel" + (" behind decode_tile_prefix_kernel" if B > 512 else ""),
+                     "kernel_avg_ms": round(kavg, 5),
                      "launches_timed": len(kms)},
     }
     if _NO_CPU:
@@ -861,7 +862,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16],
+    ap.add_argument("--config", type=int, default=0, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17],
                     help="0 (default): config 2 as the line, configs 3, 4 and 5 under \"configs\"; N: that configuration alone")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
     ap.add_argument("--prefill-impl", type=int, default=0,
@@ -899,7 +900,7 @@ def main():
         _CONST_DATA = True
 
     def run(cfg):
-        if cfg in (2, 5):
+        if cfg in (2, 5, 17):     # 17: config 2's shape with 8 192 sequences of 10-90 tokens
             res = bench_decode(cfg, args.steps, args.warmup, lib, pa, W)
         elif cfg == 3:
             res = bench_prefill(args.steps, args.warmup, lib, pa, W)

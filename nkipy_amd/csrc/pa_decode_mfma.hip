@@ -1238,9 +1238,17 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int T = p.ws_start[b + 1] - start;
   const int N = p.ws_start[p.B];
   constexpr int QUADS = D / 4, VEC = D / 16;
-  const int item = blockIdx.y * (256 / G) + threadIdx.x / G;
-  const int g = threadIdx.x % G;
   const int rows_total = p.Hq * p.T;                  // virtual heads (p.T = 1 for decode)
+  const int gv = p.bal_gv;
+  const int L = (N + gv - 1) / gv;
+  const int c_first = T ? start / L : 0, c_last = T ? (start + T - 1) / L : 0;
+  if (T != 0 && c_first == c_last) return;            // single piece: written by the streaming kernel
+  // the items of a sequence are spread over gridDim.y workgroups (all of them in one when the call has thousands of
+  // sequences, nearly all of which return above: a fourth of the workgroups to start)
+  const int ny = (rows_total * QUADS * G + 255) / 256;
+  for (int by = blockIdx.y; by < ny; by += gridDim.y) {
+  const int item = by * (256 / G) + threadIdx.x / G;
+  const int g = threadIdx.x % G;
   const bool mine = item < rows_total * QUADS;
   // item = number of a float4 within a piece slot, in the order the streaming kernel lays them out
   // (store_partial): which row and which four d's it is
@@ -1262,12 +1270,9 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   }
   if (T == 0) {
     if (mine && g == 0) *(uint2*)dst = make_uint2(0u, 0u);
-    return;
+    continue;
   }
-  const int gv = p.bal_gv;
-  const int L = (N + gv - 1) / gv;
-  const int c_first = start / L, c_last = (start + T - 1) / L;
-  if (c_first == c_last || !mine) return;   // single piece: written by the streaming kernel
+  if (!mine) continue;                      // (a whole group of G lanes: the butterfly below stays among takers)
   float m = -INFINITY, l = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 4
@@ -1296,11 +1301,12 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
     acc.z = acc.z * a + a2.z * b2; acc.w = acc.w * a + a2.w * b2;
     m = m_new;
   }
-  if (g != 0) return;
+  if (g != 0) continue;
   if (p.sinks && l > 0.f) l += exp2f(p.sinks[head] * kLog2e - m);    // attention sink: denominator only
   const float inv = l == 0.f ? 0.f : 1.f / l;     // padding rows of a multi-token call: zeros
   *(uint2*)dst =
       make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
+  }
 }
 
 template <int D, bool FP8>
@@ -1417,7 +1423,7 @@ hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream
 template <int G>
 static hipError_t launch_reduce_g(const DecodeParams& p, hipStream_t s) {
   const int items = p.Hq * p.T * (p.D / 4);
-  dim3 grid(p.B, (items * G + 255) / 256);
+  dim3 grid(p.B, p.B >= 2048 ? 1 : (items * G + 255) / 256);
   if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, G>), grid, dim3(256), 0, s, p);
   else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, G>), grid, dim3(256), 0, s, p);
   return hipGetLastError();

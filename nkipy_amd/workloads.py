@@ -179,7 +179,8 @@ def quantize_pool_fp8(pool: torch.Tensor):
 def make_decode(config: int, device="cuda", shrink: int = 1) -> DecodeWorkload:
     """config 1: fp32 B=4 8/8 heads D=64 bs=16 ctx U[16,256] pool 128;
     config 2: bf16 B=64 32/8 heads D=128 bs=32 ctx U[512,8192] partition 512;
-    config 5: fp8 KV B=128 64/8 heads D=128 bs=64 ctx logU[1024,32768] partition 1024."""
+    config 5: fp8 KV B=128 64/8 heads D=128 bs=64 ctx logU[1024,32768] partition 1024;
+    config 17: config 2's shape with 8 192 sequences of 10-90 tokens (very many very short contexts)."""
     rng = np.random.default_rng(1000 + config)
     gen = _gen(1000 + config, device)
     if config == 1:
@@ -194,6 +195,10 @@ def make_decode(config: int, device="cuda", shrink: int = 1) -> DecodeWorkload:
         B, Hq, Hkv, D, bs, dtype, part = max(128 // shrink, 1), 64, 8, 128, 64, torch.bfloat16, 1024
         lo, hi = math.log(1024 / shrink), math.log(32768 / shrink)
         ctx = np.floor(np.exp(rng.uniform(lo, hi, size=B))).astype(np.int64)
+        pool_blocks = None
+    elif config == 17:
+        B, Hq, Hkv, D, bs, dtype, part = max(8192 // shrink, 1), 32, 8, 128, 32, torch.bfloat16, 512
+        ctx = rng.integers(10, 91, size=B)
         pool_blocks = None
     else:
         raise ValueError(f"config {config} is not a decode configuration")
