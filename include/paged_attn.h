@@ -199,6 +199,10 @@ int pa_verify(const void* q, const void* k_cache, const void* v_cache,
  * it, a call with too few query tiles to fill the device (one long-context request prefilled in
  * chunks) splits the key tiles of each query tile over up to 16 workgroups and merges their partial
  * results in a second kernel; the result does not depend on the split.
+ * max_seq_len: 0, or a host-known upper bound of seq_lens (a hint for the split: a prompt with little or
+ * nothing cached in front of it -- bound below 3 T -- is bound by its causal diagonal, whose light query
+ * tiles leave the device room anyway, and runs faster unsplit; the table capacity says nothing about
+ * that).  Contexts are not clamped to it by the tiled kernel.
  */
 size_t pa_prefill_workspace_bytes(int B, int T, int Hq, int Hkv, int D, int block_size, int max_blocks_per_seq);
 int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
@@ -206,7 +210,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
-               int max_blocks_per_seq, int num_blocks,
+               int max_blocks_per_seq, int num_blocks, int max_seq_len,
                float scale, int dtype, int kv_dtype, const float* sinks, int sliding_window,
                void* workspace, size_t workspace_bytes, const pa_q_transform* q_transform, void* stream);
 

@@ -47,7 +47,7 @@ SIGNATURES = {
     "pa_verify_workspace_bytes": (c_size_t, [c_int] * 4),
     "pa_verify": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 9 + [c_float, c_int, c_void_p, c_int, c_void_p, c_void_p]),
     "pa_prefill_workspace_bytes": (c_size_t, [c_int] * 7),
-    "pa_prefill": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p, c_void_p]),
+    "pa_prefill": (c_int, [c_void_p] * 9 + [c_int] * 9 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p, c_void_p]),
     "pa_blocksparse_prefill": (c_int, [c_void_p] * 4 + [c_int] * 8 + [c_float, c_int, c_void_p]),
     "pa_o_proj": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
     "pa_o_proj_ws": (c_int, [c_void_p] * 5 + [c_size_t] + [c_int] * 4 + [c_void_p]),

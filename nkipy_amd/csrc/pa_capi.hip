@@ -743,7 +743,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
                const int32_t* block_tables, const int32_t* seq_lens,
                const int32_t* query_lens, void* out,
                int B, int T, int Hq, int Hkv, int D, int block_size,
-               int max_blocks_per_seq, int num_blocks,
+               int max_blocks_per_seq, int num_blocks, int max_seq_len,
                float scale, int dtype, int kv_dtype, const float* sinks, int sliding_window,
                void* workspace, size_t workspace_bytes, const pa_q_transform* q_transform, void* stream) {
   tl_error[0] = 0;
@@ -755,6 +755,8 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
     return fail_arg("pa_prefill: kv_dtype must be bf16 or fp8-e4m3fn (got %d)", kv_dtype);
   const bool fp8 = kv_dtype == PA_FP8_E4M3FN;
   if (block_size <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0) return fail_arg("pa_prefill: bad paging sizes");
+  if (max_seq_len < 0 || (long)max_seq_len > (long)max_blocks_per_seq * block_size)
+    return fail_arg("pa_prefill: max_seq_len=%d outside [0, max_blocks_per_seq * block_size]", max_seq_len);
   if (B == 0 || T == 0) return 0;
   if ((long)num_blocks * block_size > 0x7fffffffL || (long)block_size * Hkv * D * 2 > 0xffffffffL)
     return fail_arg("pa_prefill: pool of %d blocks x %d rows exceeds 2^31 rows (or a block 4 GiB)", num_blocks, block_size);
@@ -785,7 +787,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
       const int tc = T - t0 < PA_VERIFY_MAX_TOKENS ? T - t0 : PA_VERIFY_MAX_TOKENS;
       const int rc = verify_launch("pa_prefill", q, k_cache, v_cache, k_scale, v_scale, block_tables, seq_lens, query_lens,
                                    out, workspace, workspace_bytes, B, T, t0, tc, Hq, Hkv, D, block_size,
-                                   max_blocks_per_seq, num_blocks, 0, scale, kv_dtype, sinks, sliding_window, q_transform,
+                                   max_blocks_per_seq, num_blocks, max_seq_len, scale, kv_dtype, sinks, sliding_window, q_transform,
                                    (hipStream_t)stream);
       if (rc) return rc;
     }
@@ -800,7 +802,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.splits = 1;
   if (workspace) {
     if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
-    const int want = g_prefill_split.load() ? prefill_async_splits(p, current_num_cus()) : 1;
+    const int want = g_prefill_split.load() ? prefill_async_splits(p, current_num_cus(), max_seq_len) : 1;
     if (want > 1 && workspace_bytes >= prefill_split_bytes(p, want)) {
       p.splits = want;
       p.ws_o = (float*)workspace;

@@ -278,7 +278,7 @@ struct PrefillParams {
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);
-int prefill_async_splits(const PrefillParams& p, int num_cus);   // split the launcher would like for this call
+int prefill_async_splits(const PrefillParams& p, int num_cus, int max_seq_len = 0);   // split the launcher would like for this call (max_seq_len: the caller's bound on the lengths, 0 = none)
 bool prefill_supported(const PrefillParams& p);
 hipError_t launch_prefill_async(const PrefillParams& p, int waves, hipStream_t s);
 bool prefill_async_supported(const PrefillParams& p);

@@ -1019,8 +1019,15 @@ static int prefill_waves(const PrefillParams& p, int waves) {
   return waves;
 }
 
-int prefill_async_splits(const PrefillParams& p, int num_cus) {
+int prefill_async_splits(const PrefillParams& p, int num_cus, int max_seq_len) {
   if (p.sparse_stride > 0 || !p.block_tables || !prefill_async_supported(p) || p.impl == 1) return 1;
+  // A prompt with little cached in front of it is bound by its causal diagonal: the query tiles differ in work by
+  // the tile count, the light ones leave room on the device whatever is done, and the split's partials and merge
+  // launch cost more than it gains (one sequence, 32 / 8 heads of 128, us split / unsplit: T = 1 024 alone 34.8 /
+  // 25.1, behind 1 024 cached tokens 48.4 / 44.4, behind 2 048 63.5 / 65.0, behind 4 096 93.9 / 100.6; T = 512 behind
+  // 512 29.1 / 25.7, behind 1 024 35.1 / 34.7, behind 2 048 40.7 / 56.0).  Known only from the caller's bound on the
+  // lengths: the table capacity says nothing about them.
+  if (max_seq_len > 0 && (long)max_seq_len < 3L * p.T) return 1;
   const int waves = prefill_waves(p, p.impl == 4 || p.impl == 8 ? p.impl : 0);
   const long wgs = prefill_workgroups(p, waves, prefill_packs(p));
   const long slots = (long)num_cus * (waves == 4 ? 2 : 1);     // workgroups the device holds at once

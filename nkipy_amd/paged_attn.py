@@ -355,7 +355,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     row t being seq_lens[b] - query_lens[b] + t.
     max_seq_len: host-known upper bound of seq_lens, as in `decode`; with it a small verify call (a few
     short sequences, or a short sliding window) takes fixed partitions instead of the balanced schedule, whose
-    fixed cost dominates at that size.  The tiled kernel does not use it.
+    fixed cost dominates at that size.  For the tiled kernel it is a hint: a chunk with less than twice its own
+    length cached in front of it (max_seq_len < 3 T) runs unsplit, which is faster there.
     """
     lib = _lib.load()
     for n, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_tables", block_tables),
@@ -429,7 +430,7 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
         rc = lib.pa_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale),
                             _ptr(block_tables), _ptr(seq_lens),
                             _ptr(query_lens), _ptr(out), B, T, Hq, Hkv, D, block_size,
-                            block_tables.shape[1], num_blocks, float(scale), BF16, kv_code, _ptr(sinks), win,
+                            block_tables.shape[1], num_blocks, msl, float(scale), BF16, kv_code, _ptr(sinks), win,
                             _ptr(workspace), ws_bytes, qt_ptr, stream)
     _raise_on(rc, "pa_prefill")
     return out

@@ -332,6 +332,39 @@ def test_prefill_split_over_key_tiles(pa, T, Hq, Hkv, window):
         pa.prefill(*args, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"), **kw)
 
 
+def test_prompt_with_a_short_prefix_runs_unsplit_under_a_length_bound(pa):
+    """One prompt of 600 tokens on tables of 8 192: by the table capacity the launcher splits its key tiles; told
+    that no context exceeds 700 tokens (less than three times the chunk) it does not, and gives the unsplit kernel's
+    bits; with a bound of 5 000 tokens the split stays.  All of them the oracle's values."""
+    from nkipy_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(600)
+    B, T, Hq, Hkv, D, bs = 1, 600, 8, 2, 128, 32
+    ctxs, qlens = [T + 100], [T]
+    k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+    wide = np.full((B, 8192 // bs), -1, np.int32)
+    wide[:, :tables.shape[1]] = tables
+    q = O.round_to_bf16(rng.standard_normal((B, T, Hq, D)).astype(np.float32))
+    want = O.paged_prefill(q, O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32),
+                           np.asarray(qlens, np.int32), 0.09, q_dtype="bf16")
+    args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(wide), _i32(ctxs), _i32(qlens), 0.09)
+    assert lib.pa_prefill_workspace_bytes(B, T, Hq, Hkv, D, bs, wide.shape[1]) > 0
+    by_capacity = pa.prefill(*args, route="tiled")
+    bounded = pa.prefill(*args, route="tiled", max_seq_len=700)
+    far_bound = pa.prefill(*args, route="tiled", max_seq_len=5000)
+    lib.pa_debug_set(6, 0)
+    try:
+        unsplit = pa.prefill(*args, route="tiled")
+    finally:
+        lib.pa_debug_set(6, 1)
+    torch.cuda.synchronize()
+    for o in (by_capacity, bounded, far_bound, unsplit):
+        assert_close_abs(dev_to_f32(o), want, BF16_TOL)
+    assert torch.equal(bounded, unsplit)
+    assert torch.equal(far_bound, by_capacity)
+    assert not torch.equal(by_capacity, unsplit)          # (else the comparisons above show nothing)
+
+
 @pytest.mark.parametrize("bs", [16, 64, 24])
 @pytest.mark.parametrize("Hq,Hkv", [(8, 2), (4, 4)])
 def test_prefill_fp8_pool(pa, bs, Hq, Hkv):

@@ -76,9 +76,9 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert dec(B=0) == 0                                        # empty batch is a no-op
     assert lib.pa_blocksparse_prefill(z, z, z, z, 1, 64, 4, 4, 128, 32, 4, 8, 1.0, 1, z) == -1
     assert b"block must be 64" in lib.pa_last_error()
-    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 0, 1, z, 0, z, 0, z, z) == -1
-    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 1, 1, z, -1, z, 0, z, z) == -1 and b"sliding_window" in lib.pa_last_error()
-    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 1.0, 1, 0, z, 0, z, 0, z, z) == -1 and b"kv_dtype" in lib.pa_last_error()
+    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 0, 1.0, 0, 1, z, 0, z, 0, z, z) == -1
+    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 0, 1.0, 1, 1, z, -1, z, 0, z, z) == -1 and b"sliding_window" in lib.pa_last_error()
+    assert lib.pa_prefill(z, z, z, z, z, z, z, z, z, 1, 4, 4, 4, 128, 16, 4, 8, 0, 1.0, 1, 0, z, 0, z, 0, z, z) == -1 and b"kv_dtype" in lib.pa_last_error()
     assert lib.pa_gather_kv(z, z, z, z, 1, 2, 64, 16, 2, 8, 100, 2, z) == -1  # beyond table capacity
     def kvw(**kw):
         a = dict(B=2, T=4, Hkv=2, D=128, bs=16, mb=4, nb=8, kd=1)
