@@ -181,6 +181,42 @@ def decode_step_fp8(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, k_cach
                            sliding_window=_win(sliding_window))
 
 
+# A speculative verify step of a layer in one call (the K + 1 tokens of examples/models/gpt_oss/peagle/speculate.py:137-202
+# through examples/models/gpt_oss/kernels/attention.py:80-163): xq [B, T, Hq, D], xk / xv [B, T, Hkv, D]; `out` is
+# [B, T, N] with o_weight, else [B, T, Hq, D].
+@torch.library.custom_op(f"{_NS}::verify_step", mutates_args=("k_cache", "v_cache", "out"), device_types="cuda")
+def verify_step(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                block_tables: torch.Tensor, seq_lens: torch.Tensor, query_lens: torch.Tensor, scale: float,
+                out: torch.Tensor, max_seq_len: int = 0, rope_cos: Optional[torch.Tensor] = None,
+                rope_sin: Optional[torch.Tensor] = None, q_norm_weight: Optional[torch.Tensor] = None,
+                k_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6,
+                o_weight: Optional[torch.Tensor] = None, o_bias: Optional[torch.Tensor] = None,
+                sinks: Optional[torch.Tensor] = None, sliding_window: int = 0,
+                workspace: Optional[torch.Tensor] = None) -> None:
+    paged_attn.verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale,
+                           max_seq_len=max_seq_len or None,
+                           q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps), k_norm_weight=k_norm_weight,
+                           o_weight=o_weight, o_bias=o_bias, out=out, workspace=workspace, sinks=sinks,
+                           sliding_window=_win(sliding_window))
+
+
+@torch.library.custom_op(f"{_NS}::verify_step_fp8", mutates_args=("k_cache", "v_cache", "k_scale", "v_scale", "out"),
+                         device_types="cuda")
+def verify_step_fp8(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    k_scale: torch.Tensor, v_scale: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                    query_lens: torch.Tensor, scale: float, out: torch.Tensor, max_seq_len: int = 0,
+                    rope_cos: Optional[torch.Tensor] = None, rope_sin: Optional[torch.Tensor] = None,
+                    q_norm_weight: Optional[torch.Tensor] = None, k_norm_weight: Optional[torch.Tensor] = None,
+                    norm_eps: float = 1e-6, o_weight: Optional[torch.Tensor] = None,
+                    o_bias: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
+                    sliding_window: int = 0, workspace: Optional[torch.Tensor] = None) -> None:
+    paged_attn.verify_step(xq, xk, xv, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, k_scale=k_scale,
+                           v_scale=v_scale, max_seq_len=max_seq_len or None,
+                           q_transform=_qt(rope_cos, rope_sin, q_norm_weight, norm_eps), k_norm_weight=k_norm_weight,
+                           o_weight=o_weight, o_bias=o_bias, out=out, workspace=workspace, sinks=sinks,
+                           sliding_window=_win(sliding_window))
+
+
 def _no_cpu(name):
     def impl(*args, **kwargs):
         raise NotImplementedError(f"{_NS}::{name} runs hand-written HIP kernels and has no CPU path; "
@@ -193,10 +229,11 @@ for _op, _name in ((paged_decode, "paged_decode"), (paged_prefill, "paged_prefil
                    (paged_kv_write_fp8, "paged_kv_write_fp8"), (qk_norm_rope_kv_write, "qk_norm_rope_kv_write"),
                    (qk_norm_rope_kv_write_fp8, "qk_norm_rope_kv_write_fp8"),
                    (k_norm_rope_kv_write, "k_norm_rope_kv_write"), (k_norm_rope_kv_write_fp8, "k_norm_rope_kv_write_fp8"),
-                   (o_proj, "o_proj"), (decode_step, "decode_step"), (decode_step_fp8, "decode_step_fp8")):
+                   (o_proj, "o_proj"), (decode_step, "decode_step"), (decode_step_fp8, "decode_step_fp8"),
+                   (verify_step, "verify_step"), (verify_step_fp8, "verify_step_fp8")):
     _op.register_kernel("cpu")(_no_cpu(_name))
     _op.register_fake(lambda *args, **kwargs: None)      # outputs are caller-allocated: nothing to infer
 
 OPS = ("paged_decode", "paged_prefill", "blocksparse_prefill", "paged_kv_write", "paged_kv_write_fp8",
        "qk_norm_rope_kv_write", "qk_norm_rope_kv_write_fp8", "k_norm_rope_kv_write", "k_norm_rope_kv_write_fp8", "o_proj",
-       "decode_step", "decode_step_fp8")
+       "decode_step", "decode_step_fp8", "verify_step", "verify_step_fp8")

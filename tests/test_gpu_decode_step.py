@@ -385,6 +385,35 @@ def test_through_the_dispatcher(pa):
         _same_bits(v, wv, "V pool")
 
 
+def test_verify_step_through_the_dispatcher(pa):
+    """torch.ops.nkipy_amd.verify_step / verify_step_fp8: the same bits as the Python op."""
+    import nkipy_amd.torch_ops  # noqa: F401
+    rng = np.random.default_rng(12)
+    for fp8 in (False, True):
+        B, T, Hq, Hkv, D, bs, N = 2, 4, 16, 4, 128, 32, 512
+        ctxs, qlens = [700, 1031], [4, 3]
+        d = _setup_multi(rng, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, True, True, fp8=fp8)
+        scale = 1.0 / np.sqrt(D)
+        want, wk, wv, wks, wvs = _verify_step(pa, d, scale, max(ctxs))
+        k, v = d["k"].clone(), d["v"].clone()
+        out = torch.empty((B, T, N), dtype=torch.bfloat16, device="cuda")
+        common = dict(max_seq_len=max(ctxs), rope_cos=d["qt"].rope_cos, rope_sin=d["qt"].rope_sin,
+                      q_norm_weight=d["qt"].norm_weight, k_norm_weight=d["wk"], norm_eps=d["qt"].eps, o_weight=d["ow"],
+                      o_bias=d["ob"])
+        if fp8:
+            ks, vs = d["ks"].clone(), d["vs"].clone()
+            torch.ops.nkipy_amd.verify_step_fp8(d["xq"], d["xk"], d["xv"], k, v, ks, vs, d["tables"], d["lens"], d["qlens"],
+                                                scale, out, **common)
+            _same_bits(ks, wks, "K scales")
+        else:
+            torch.ops.nkipy_amd.verify_step(d["xq"], d["xk"], d["xv"], k, v, d["tables"], d["lens"], d["qlens"], scale, out,
+                                            **common)
+        torch.cuda.synchronize()
+        _same_bits(out, want, f"projected rows, fp8={fp8}")
+        _same_bits(k, wk, "K pool")
+        _same_bits(v, wv, "V pool")
+
+
 def test_argument_errors(pa):
     rng = np.random.default_rng(10)
     d = _setup(rng, 2, 8, 2, 128, 16, [40, 50], [1, 1], 256, False, True, poison=False)

@@ -17,6 +17,8 @@ def test_ops_are_registered_with_mutation_schemas():
     assert str(torch.ops.nkipy_amd.paged_kv_write_fp8.default._schema).count("!") == 4    # ... and both scale tables
     assert str(torch.ops.nkipy_amd.decode_step.default._schema).count("!") == 3           # both caches and out
     assert str(torch.ops.nkipy_amd.decode_step_fp8.default._schema).count("!") == 5
+    assert str(torch.ops.nkipy_amd.verify_step.default._schema).count("!") == 3
+    assert str(torch.ops.nkipy_amd.verify_step_fp8.default._schema).count("!") == 5
 
 
 def test_ops_refuse_cpu_tensors_and_trace_with_fake_tensors():
