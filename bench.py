@@ -10,7 +10,8 @@ carries, under "configs", one record each for config 3 (paged chunked prefill),
 config 4 (blocksparse prefill) and config 5 (fp8-KV long-context decode), timed in
 the same run with the same protocol: both halves of the headline metric and every
 benchmark-sized configuration, plus "o_proj", the output projection behind config 3's
-attention.  --config N prints that configuration alone (6-17: the kernels and steps around the
+attention, and under "layer_steps" the microseconds per layer of the small-batch decode and
+verify steps (configs 13, 15, 16).  --config N prints that configuration alone (6-17: the kernels and steps around the
 attention call; their docstrings say what each one is).
 
 value      whole-step throughput: algorithmic HBM bytes / step time for the decode
@@ -955,6 +956,15 @@ def main():
         line["prefill_roofline_frac"] = subs["C3"]["roofline"]["frac"]
         par = [line.get("parity")] + [r.get("parity") for r in subs.values()]
         line["parity_all_pass"] = None if any(x is None for x in par) else all(x["pass"] for x in par)
+        # the launch-bound steps of a small batch (a second each): decode and verify steps of a layer on the qwen3
+        # and gpt-oss shapes, per layer, replayed from a graph and issued call by call
+        steps = {}
+        for cfg, name in ((13, "decode_B8_ctx1K"), (15, "verify_B1_T4_ctx1K"), (16, "gpt_oss_decode_B1_ctx1K")):
+            r = run(cfg)
+            steps[name] = {k: r[k] for k in ("us_per_layer", "eager_us_per_layer", "capacity_8k", "batches", "other_steps")
+                           if k in r}
+            steps[name]["workload"] = r["config"]["workload"]
+        line["layer_steps"] = steps
     if args.prefill_impl:
         line["prefill_impl"] = args.prefill_impl
     if args.const_data:
