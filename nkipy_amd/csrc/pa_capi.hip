@@ -609,8 +609,9 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   // 36.0 / 32.9, B = 4 behind 2 K 41.4 / 34.4, B = 4 behind 4 K 47.6 / 38.1, B = 8 behind 2 K 46.8 / 44.0; a single
   // sequence on the finer partitions, B = 1 behind 1 K: 30.5 -> 27.7.  It needs the caller's bound on the lengths (the
   // table capacity says nothing about the sizes), 16 rows per wave, and a workspace that holds the partitions'
-  // partials.  Under a sliding window the partitions cover what the window reaches, often a single one.
-  if (max_seq_len > 0 && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
+  // partials.  Under a sliding window the partitions cover what the window reaches, often a single one, and the
+  // window is itself a bound.
+  if ((max_seq_len > 0 || sliding_window > 0) && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
     DecodeParams f = p;
     f.partition_size = 512;
     const bool small = decode_small_call(f, kv_dtype);
