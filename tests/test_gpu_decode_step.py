@@ -385,6 +385,66 @@ def test_through_the_dispatcher(pa):
         _same_bits(v, wv, "V pool")
 
 
+def test_random_steps_equal_the_three_calls(pa):
+    """Seeded random decode and verify steps (head shapes, batch, contexts around tile / partition / block borders,
+    idle sequences, sinks, windows, bounds, bias, transform): the one call against the three calls, bit for bit,
+    outputs and pools."""
+    rng = np.random.default_rng(2024)
+    shapes = [(32, 8, 128), (64, 8, 64), (16, 16, 64), (8, 1, 128), (32, 2, 128), (12, 4, 64)]
+    borders = np.array([1, 2, 31, 32, 33, 63, 64, 65, 255, 256, 257, 511, 512, 513, 767, 768, 769, 1023, 1024, 1025, 1500])
+    cases = 0
+    for case in range(40):
+        Hq, Hkv, D = shapes[rng.integers(len(shapes))]
+        bs = int(rng.choice([16, 32, 64]))
+        B = int(rng.choice([1, 2, 3, 5, 9]))
+        T = int(rng.choice([1, 1, 2, 4, 8]))
+        if (Hq // Hkv) * T > 64:
+            T = 1
+        qlens = rng.integers(0 if B > 1 else 1, T + 1, size=B)
+        qlens[rng.integers(B)] = T
+        ctxs = np.maximum(rng.choice(borders, size=B) + rng.integers(0, 3, size=B), qlens)
+        ctxs = np.where(qlens == 0, np.maximum(ctxs, 1), ctxs)
+        N = int(rng.choice([0, 256, 520, 1024]))
+        xform = bool(rng.integers(2))
+        window = [None, None, 1, 40, 128, 600][rng.integers(6)]
+        sinks = torch.from_numpy(rng.standard_normal(Hq).astype(np.float32)).cuda() if rng.integers(2) else None
+        bounded = bool(rng.integers(4))
+        msl = int(ctxs.max()) + int(rng.integers(0, 40)) if bounded else None
+        kw = dict(sinks=sinks, sliding_window=window)
+        tag = f"case {case}: B={B} T={T} Hq={Hq} Hkv={Hkv} D={D} bs={bs} ctx={ctxs.tolist()} q={qlens.tolist()} N={N} xform={xform} window={window} sinks={sinks is not None} msl={msl}"
+        print(tag, flush=True)
+        if T == 1:
+            d = _setup(rng, B, Hq, Hkv, D, bs, ctxs, qlens, N, bool(N) and bool(rng.integers(2)), xform)
+            want, att, wk, wv, _, _ = _three_calls(pa, d, 0.11, 512, msl, **kw)
+            got, gk, gv, _, _ = _step(pa, d, 0.11, 512, msl, **kw)
+        else:
+            d = _setup_multi(rng, B, T, Hq, Hkv, D, bs, ctxs, qlens, N, bool(N) and bool(rng.integers(2)), xform)
+            want, att, wk, wv, _, _ = _verify_three_calls(pa, d, 0.11, msl, **kw)
+            got, gk, gv, _, _ = _verify_step(pa, d, 0.11, msl, **kw)
+        torch.cuda.synchronize()
+        _same_bits(got, want, tag)
+        _same_bits(gk, wk, "K pool, " + tag)
+        _same_bits(gv, wv, "V pool, " + tag)
+        if N == 0:
+            # attention only: the oracle's values too, on the pools the step left
+            q = dev_to_f32(d["xq"]).reshape(B, T, Hq, D)
+            if xform:
+                cos, sin = dev_to_f32(d["qt"].rope_cos), dev_to_f32(d["qt"].rope_sin)
+                q = O.qk_norm_rope(q, dev_to_f32(d["xk"]).reshape(B, T, Hkv, D), ctxs, qlens, cos, sin,
+                                   q_norm_weight=dev_to_f32(d["qt"].norm_weight), eps=d["qt"].eps)[0]
+            lens = np.minimum(ctxs, msl) if msl else ctxs
+            ref = O.paged_prefill(O.round_to_bf16(q), dev_to_f32(wk), dev_to_f32(wv), d["tables"].cpu().numpy(),
+                                  np.asarray(lens, np.int32), np.asarray(qlens, np.int32), 0.11, q_dtype="bf16",
+                                  sliding_window=window, sinks=None if sinks is None else sinks.cpu().numpy())
+            g = dev_to_f32(got).reshape(B, T, Hq, D)
+            if T == 1:                      # decode treats every slot as live: an idle one attends from its last token
+                live = qlens > 0
+                g, ref = g[live], ref[live]
+            assert np.abs(g - ref).max() <= 2e-2, tag
+        cases += 1
+    assert cases == 40
+
+
 def test_verify_step_through_the_dispatcher(pa):
     """torch.ops.nkipy_amd.verify_step / verify_step_fp8: the same bits as the Python op."""
     import nkipy_amd.torch_ops  # noqa: F401
