@@ -48,7 +48,7 @@ extern "C" {
 
 enum { PA_F32 = 0, PA_BF16 = 1, PA_FP8_E4M3FN = 2 };
 
-/* Library version: major * 10000 + minor * 100 + patch. */
+/* Library version: major * 10000 + minor * 100 + patch (a minor step marks a changed or added signature). */
 int pa_version(void);
 
 /* Text of the calling thread's most recent error ("" if none).  Mirrors the

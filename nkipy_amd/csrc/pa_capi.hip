@@ -133,7 +133,7 @@ using namespace pa;
 
 extern "C" {
 
-int pa_version(void) { return 100; }
+int pa_version(void) { return 300; }   // 0.3.0: pa_prefill takes max_seq_len; the one-call steps; sinks and windows on small calls
 
 const char* pa_last_error(void) { return tl_error; }
 
