@@ -1231,7 +1231,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 // G consecutive lanes share one item and take every G-th piece of the sequence; their partial
 // merges are combined with a butterfly.  G = 1 when there are many sequences (each spans a few
 // chunks), 8 or 32 when a sequence spans many.
-template <int D, int G>
+template <int D, int G, bool FOLD = false>
 __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParams p) {
   const int b = blockIdx.x;
   const int start = p.ws_start[b];                   // tiles before this sequence (streaming kernel, or prefix launch)
@@ -1243,10 +1243,10 @@ __global__ __launch_bounds__(256) void decode_balanced_reduce_kernel(DecodeParam
   const int L = (N + gv - 1) / gv;
   const int c_first = T ? start / L : 0, c_last = T ? (start + T - 1) / L : 0;
   if (T != 0 && c_first == c_last) return;            // single piece: written by the streaming kernel
-  // the items of a sequence are spread over gridDim.y workgroups (all of them in one when the call has thousands of
-  // sequences, nearly all of which return above: a fourth of the workgroups to start)
+  // the items of a sequence are spread over gridDim.y workgroups, or (FOLD) all taken by one: for calls of thousands
+  // of sequences, nearly all of which return above, that is a fourth of the workgroups to start
   const int ny = (rows_total * QUADS * G + 255) / 256;
-  for (int by = blockIdx.y; by < ny; by += gridDim.y) {
+  for (int by = FOLD ? 0 : blockIdx.y; by < (FOLD ? ny : (int)blockIdx.y + 1); ++by) {
   const int item = by * (256 / G) + threadIdx.x / G;
   const int g = threadIdx.x % G;
   const bool mine = item < rows_total * QUADS;
@@ -1423,7 +1423,12 @@ hipError_t launch_decode_balanced(const DecodeParams& p, int kv_dtype, hipStream
 template <int G>
 static hipError_t launch_reduce_g(const DecodeParams& p, hipStream_t s) {
   const int items = p.Hq * p.T * (p.D / 4);
-  dim3 grid(p.B, p.B >= 2048 ? 1 : (items * G + 255) / 256);
+  if (G == 1 && p.B >= 2048) {
+    if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, 1, true>), dim3(p.B), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, 1, true>), dim3(p.B), dim3(256), 0, s, p);
+    return hipGetLastError();
+  }
+  dim3 grid(p.B, (items * G + 255) / 256);
   if (p.D == 128) hipLaunchKernelGGL((decode_balanced_reduce_kernel<128, G>), grid, dim3(256), 0, s, p);
   else hipLaunchKernelGGL((decode_balanced_reduce_kernel<64, G>), grid, dim3(256), 0, s, p);
   return hipGetLastError();
