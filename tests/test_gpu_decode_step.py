@@ -189,12 +189,13 @@ def test_sequences_that_take_no_token_and_empty_slots(pa):
     assert np.array_equal(g[2], np.zeros_like(g[2]))
 
 
-def test_length_bound_below_the_new_token(pa):
+@pytest.mark.parametrize("B", [3, 24], ids=["fixed_partitions", "balanced_schedule"])
+def test_length_bound_below_the_new_token(pa, B):
     """A bound that clamps a context below its newest token (pa_decode's rule): the token is stored all the same
     and the attention is over the clamped context."""
     rng = np.random.default_rng(6)
-    B, Hq, Hkv, D, bs, N = 3, 16, 4, 128, 32, 256
-    ctxs = [1000, 1200, 1100]
+    Hq, Hkv, D, bs, N = 16, 4, 128, 32, 256
+    ctxs = ([1000, 1200, 1100] * 8)[:B]
     d = _setup(rng, B, Hq, Hkv, D, bs, ctxs, [1] * B, N, False, True, poison=False)
     scale = 1.0 / np.sqrt(D)
     want, att, wk, wv, _, _ = _three_calls(pa, d, scale, 512, 1100)
@@ -203,6 +204,45 @@ def test_length_bound_below_the_new_token(pa):
     _same_bits(got, want, "projected rows")
     _same_bits(gk, wk, "K pool")
     _same_bits(gv, wv, "V pool")
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,D,bs,lo,hi,window", [
+    (24, 32, 8, 128, 32, 900, 1400, None),     # more (sequence, kv head) pairs than the small-call kernels take
+    (3, 32, 8, 128, 32, 9000, 20000, None),    # few long sequences: every sequence cut into many chunks
+    (70, 8, 2, 64, 16, 1, 300, None),          # many short ones, some of a single token, some idle
+    (6, 40, 2, 128, 64, 3000, 5000, 1000),     # 20 q heads per kv head (two waves per kv head), a window, sinks
+    (600, 8, 2, 128, 32, 1, 90, None),         # more sequences than are scanned in registers
+])
+def test_steps_that_take_the_balanced_schedule(pa, B, Hq, Hkv, D, bs, lo, hi, window):
+    """Steps of more sequences or longer contexts than the small-call kernels take: the write launch, the balanced
+    kernel, its merge and the projection inside the one call; pools poisoned from the new token on (the row must be
+    in the pool before any wave reads it).  Bit for bit the three calls."""
+    rng = np.random.default_rng(B + Hq + hi)
+    ctxs = rng.integers(lo, hi + 1, size=B)
+    ctxs[::5] = (ctxs[::5] // 32) * 32 + 1        # new token first of a tile
+    ctxs[1::5] = np.maximum((ctxs[1::5] // 32) * 32, 1)   # ... last of a tile
+    qlens = np.ones(B, np.int64)
+    if B > 8:
+        qlens[3::7] = 0                           # idle sequences: nothing written, attended to as they are
+    N = 256
+    d = _setup(rng, B, Hq, Hkv, D, bs, ctxs, qlens, N, True, True)
+    scale, msl = 1.0 / np.sqrt(D), int(ctxs.max())
+    kw = {}
+    if window:
+        kw = dict(sinks=torch.from_numpy(rng.standard_normal(Hq).astype(np.float32)).cuda(), sliding_window=window)
+    print(f"balanced decode_step B={B} Hq={Hq} Hkv={Hkv} D={D} bs={bs} ctx={ctxs[:6].tolist()}.. window={window}", flush=True)
+    want, att, wk, wv, _, _ = _three_calls(pa, d, scale, 512, msl, **kw)
+    for fusion in (0, 1):
+        _fusion(fusion)
+        try:
+            got, gk, gv, _, _ = _step(pa, d, scale, 512, msl, **kw)
+            torch.cuda.synchronize()
+        finally:
+            _fusion(0)
+        _same_bits(got, want, f"projected rows, fusion switch {fusion}")
+        _same_bits(gk, wk, f"K pool, fusion switch {fusion}")
+        _same_bits(gv, wv, f"V pool, fusion switch {fusion}")
+    assert not torch.isnan(got.float()).any()
 
 
 SINK_CASES = [
