@@ -124,15 +124,32 @@ class PagedKVCache:
         self.v_scales = [scales() for _ in range(num_layers)]
         self.k_cache, self.v_cache = self.k_caches[0], self.v_caches[0]
         self.k_scale, self.v_scale = self.k_scales[0], self.v_scales[0]
-        # state of the step in flight (begin_step): query lengths on the device, tokens per slot
-        self.query_lens = torch.zeros(max_seqs, dtype=torch.int32, device=device)
         self.step_tokens = 0
         self.allocator = BlockAllocator(num_blocks)
         self.blocks: List[List[int]] = [[] for _ in range(max_seqs)]
         self.lens = [0] * max_seqs
-        self.block_tables = torch.full((max_seqs, max_blocks_per_seq), -1, dtype=torch.int32, device=device)
-        self.seq_lens = torch.zeros(max_seqs, dtype=torch.int32, device=device)
-        self._host_tables = np.full((max_seqs, max_blocks_per_seq), -1, dtype=np.int32)
+        # What the kernels read of the bookkeeping -- table rows, lengths, the query lengths of the step in flight --
+        # lives in ONE device buffer (three views, each starting on a 256-byte boundary) with a host mirror of the same
+        # layout, so that publishing a step is one copy.  The copy is asynchronous: the mirror goes into one of a few
+        # pinned staging buffers, each reused only when the copy that last read it has completed, and the host
+        # never waits for the device's queued work (a decode loop issued call by call stays ahead of the GPU).
+        n_tab = max_seqs * max_blocks_per_seq
+        self._off_lens = (n_tab + 63) // 64 * 64
+        self._off_qlens = self._off_lens + (max_seqs + 63) // 64 * 64
+        self._host_meta = np.zeros(self._off_qlens + max_seqs, dtype=np.int32)
+        self._host_tables = self._host_meta[:n_tab].reshape(max_seqs, max_blocks_per_seq)
+        self._host_tables[:] = -1
+        self._host_lens = self._host_meta[self._off_lens:self._off_lens + max_seqs]
+        self._host_qlens = self._host_meta[self._off_qlens:]
+        self._meta = torch.from_numpy(self._host_meta).to(self.device)
+        self.block_tables = self._meta[:n_tab].view(max_seqs, max_blocks_per_seq)
+        self.seq_lens = self._meta[self._off_lens:self._off_lens + max_seqs]
+        self.query_lens = self._meta[self._off_qlens:]
+        self._stage = self._stage_done = None
+        self._stage_at = 0
+        if self.device.type == "cuda":
+            self._stage = [torch.empty(self._host_meta.size, dtype=torch.int32, pin_memory=True) for _ in range(4)]
+            self._stage_done = [None] * len(self._stage)
 
     # ---- host bookkeeping ----------------------------------------------------------
     def blocks_needed(self, slot: int, n_new: int) -> int:
@@ -201,15 +218,31 @@ class PagedKVCache:
         if any(n < 0 or n > tokens for n in query_lens):
             raise ValueError("query_lens must lie in [0, tokens]")
         active = [s for s in range(self.max_seqs) if query_lens[s] > 0]
-        self.extend(active, [query_lens[s] for s in active])
-        self.query_lens.copy_(torch.tensor(list(query_lens), dtype=torch.int32))
+        before = self._host_qlens.copy()
+        self._host_qlens[:] = query_lens
+        try:
+            self.extend(active, [query_lens[s] for s in active])      # publishes the query lengths with the rest
+        except Exception:
+            self._host_qlens[:] = before
+            raise
         self.step_tokens = tokens
 
     def _publish(self, slots: Sequence[int]) -> None:
-        idx = torch.as_tensor(list(slots), dtype=torch.long, device=self.device)
-        rows = torch.from_numpy(self._host_tables[list(slots)]).to(self.device, non_blocking=False)
-        self.block_tables.index_copy_(0, idx, rows)
-        self.seq_lens.index_copy_(0, idx, torch.tensor([self.lens[s] for s in slots], dtype=torch.int32, device=self.device))
+        """Host mirror -> device (tables, lengths, query lengths: one copy, queued on the current stream)."""
+        for s in slots:
+            self._host_lens[s] = self.lens[s]
+        if self._stage is None:
+            self._meta.copy_(torch.from_numpy(self._host_meta))
+            return
+        i = self._stage_at
+        self._stage_at = (i + 1) % len(self._stage)
+        if self._stage_done[i] is None:
+            self._stage_done[i] = torch.cuda.Event()
+        else:
+            self._stage_done[i].synchronize()         # (long done unless the host is four publications ahead)
+        self._stage[i].numpy()[:] = self._host_meta
+        self._meta.copy_(self._stage[i], non_blocking=True)
+        self._stage_done[i].record()
 
     @property
     def max_seq_len(self) -> int:
