@@ -124,6 +124,47 @@ def test_serving_loop_gpt_oss_variant(rng):
     run(1, [1, 1, 1])
 
 
+def test_steps_published_while_the_device_is_busy():
+    """A loop issued call by call runs ahead of the GPU: the bookkeeping of a dozen later steps is published while the
+    first step's kernels have not started (a long matmul holds the stream).  Every step must still read its own
+    tables, lengths and query lengths: same results as a twin that waits for the device after every step."""
+    from nkipy_amd.engine import PagedAttention, PagedKVCache
+    torch.manual_seed(3)
+    S, Hq, Hkv, D, bs = 3, 8, 2, 128, 16
+
+    def make():
+        cache = PagedKVCache(num_blocks=60, block_size=bs, n_kv_heads=Hkv, head_dim=D, max_seqs=S, max_blocks_per_seq=16)
+        return cache, PagedAttention(cache, Hq, rope_base=10000.0, max_positions=256)
+
+    rows = [(torch.randn(S, 1, Hq, D, device="cuda").to(torch.bfloat16), torch.randn(S, 1, Hkv, D, device="cuda").to(torch.bfloat16),
+             torch.randn(S, 1, Hkv, D, device="cuda").to(torch.bfloat16)) for _ in range(14)]
+    qlens = [[1, 1, 1], [1, 0, 1], [1, 1, 0]]
+    prompt = (torch.randn(S, 20, Hq, D, device="cuda").to(torch.bfloat16), torch.randn(S, 20, Hkv, D, device="cuda").to(torch.bfloat16),
+              torch.randn(S, 20, Hkv, D, device="cuda").to(torch.bfloat16))
+
+    def run(wait):
+        cache, layer = make()
+        layer.step(*prompt, [20, 7, 15])
+        torch.cuda.synchronize()
+        if not wait:
+            big = torch.randn(8192, 8192, device="cuda")
+            for _ in range(6):
+                big = big @ big * 1e-4                 # tens of milliseconds of queued work ahead of the steps
+        outs = []
+        for i, (xq, xk, xv) in enumerate(rows):
+            outs.append(layer.step(xq, xk, xv, qlens[i % 3]).clone())
+            if wait:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        return outs, cache.k_cache.clone()
+
+    a, ka = run(True)
+    b, kb = run(False)
+    for i, (x, y) in enumerate(zip(a, b)):
+        assert torch.equal(x.view(torch.int16), y.view(torch.int16)), f"step {i}"
+    assert torch.equal(ka.view(torch.int16), kb.view(torch.int16))
+
+
 def test_serving_loop_fp8_pool(rng):
     """fp8 pool: the write kernel maintains the scales; attention follows the oracle run on the
     dequantised pool within the fp8 bar."""
