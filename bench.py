@@ -747,12 +747,25 @@ def _decode_layer_step_times(steps, warmup, B, ctx, layers, capacity, bound, T=1
 
     cache.begin_step([T] * B, T)
     sec_eager = _time_steps(step, steps, warmup)
+    global _LAST_STEP_WITH_BOOKKEEPING
+    _LAST_STEP_WITH_BOOKKEEPING = None
+    if T == 1:
+        # the same with the step's bookkeeping in front (tables, lengths and query lengths published to the device):
+        # steps that append nothing, so that the contexts stay what they are; the decode kernels treat every slot as live
+        def full_step():
+            cache.begin_step([0] * B, 1)
+            step()
+        _LAST_STEP_WITH_BOOKKEEPING = _time_steps(full_step, steps, 5)
+        cache.begin_step([1] * B, 1)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step()
     sec = _time_steps(graph.replay, steps, 5)
     del graph
     return sec, sec_eager, nblk * bs
+
+
+_LAST_STEP_WITH_BOOKKEEPING = None
 
 
 def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
@@ -766,6 +779,7 @@ def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
     captured step must serve any length: the balanced kernel) and once with `attend(max_seq_len=1088)`."""
     Hq, Hkv, D, bs, N = 32, 8, 128, 32, 4096
     sec, sec_eager, cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, ctx + 96, None)
+    with_books = _LAST_STEP_WITH_BOOKKEEPING
     big_free, _, big_cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, 8192, None)
     big_bound, _, _ = _decode_layer_step_times(steps, warmup, B, ctx, layers, 8192, ctx + 64)
     kv_bytes = 2 * B * (ctx + 1) * Hkv * D * 2
@@ -776,6 +790,7 @@ def bench_decode_layer_step(steps, warmup, lib, pa, W, B=8, ctx=1024, layers=8):
         "value": round(1e6 / us, 1), "unit": "layer steps/s",
         "ms_per_step": round(sec * 1e3, 5), "us_per_layer": round(us, 2),
         "eager_us_per_layer": round(sec_eager / layers * 1e6, 2),
+        "eager_us_per_step_with_begin_step": round(with_books * 1e6, 1), "eager_us_per_step": round(sec_eager * 1e6, 1),
         "capacity_8k": {"table_capacity_tokens": big_cap,
                         "us_per_layer_no_bound": round(big_free / layers * 1e6, 2),
                         f"us_per_layer_max_seq_len_{ctx + 64}": round(big_bound / layers * 1e6, 2)},
@@ -830,6 +845,7 @@ def bench_gpt_oss_layer_step(steps, warmup, lib, pa, W, B=1, ctx=1024, layers=8)
     2 880 with a bias.  Launch-bound; microseconds per layer, HIP graph replay and issued call by call."""
     Hq, Hkv, D, bs, N = 64, 8, 64, 32, 2880
     sec, sec_eager, cap = _decode_layer_step_times(steps, warmup, B, ctx, layers, ctx + 96, None, gpt_oss=True)
+    with_books = _LAST_STEP_WITH_BOOKKEEPING
     others = {}
     for b2, c2, t2 in ((1, 1024, 4), (8, 1024, 1), (1, 4000, 1), (4, 2048, 4)):
         s2, e2, _ = _decode_layer_step_times(steps, warmup, b2, c2, layers, c2 + 96, None, T=t2, gpt_oss=True)
@@ -844,6 +860,7 @@ def bench_gpt_oss_layer_step(steps, warmup, lib, pa, W, B=1, ctx=1024, layers=8)
         "value": round(1e6 / us, 1), "unit": "layer steps/s",
         "ms_per_step": round(sec * 1e3, 5), "us_per_layer": round(us, 2),
         "eager_us_per_layer": round(sec_eager / layers * 1e6, 2), "other_steps": others,
+        "eager_us_per_step_with_begin_step": round(with_books * 1e6, 1), "eager_us_per_step": round(sec_eager * 1e6, 1),
         "dtype": "bf16, bf16 rotation, fp32 accumulate",
         "config": {"workload": f"gpt-oss decode layer step: B={B}, context={ctx}, table capacity={cap} tokens per sequence, "
                                f"layers={layers} (window 128 on the even ones, sinks on all), Hq={Hq}, Hkv={Hkv}, D={D}, "
@@ -961,7 +978,8 @@ def main():
         steps = {}
         for cfg, name in ((13, "decode_B8_ctx1K"), (15, "verify_B1_T4_ctx1K"), (16, "gpt_oss_decode_B1_ctx1K")):
             r = run(cfg)
-            steps[name] = {k: r[k] for k in ("us_per_layer", "eager_us_per_layer", "capacity_8k", "batches", "other_steps")
+            steps[name] = {k: r[k] for k in ("us_per_layer", "eager_us_per_layer", "eager_us_per_step", "eager_us_per_step_with_begin_step",
+                                             "capacity_8k", "batches", "other_steps")
                            if k in r}
             steps[name]["workload"] = r["config"]["workload"]
         line["layer_steps"] = steps
