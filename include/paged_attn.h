@@ -103,7 +103,8 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * resident wavefront group, so its partition length follows the batch and the
  * device, not partition_size.  Small calls (by max_seq_len, or by what a sliding window
  * reaches if that is less: at most eight partitions per sequence, at most 80 (sequence,
- * kv head) pairs and at most 160 MiB of K and V) take the fixed-partition MFMA kernel,
+ * kv head) pairs -- 320 at head dim 64, 1 024 under a window that fits one partition --
+ * and at most 160 MiB of K and V) take the fixed-partition MFMA kernel,
  * whose fixed cost is lower, on partitions of 256 tokens when those of partition_size
  * would give the device fewer than about 64 workgroups (a single sequence); under a
  * window its partitions count from the first 32-token tile the window reaches.  The
@@ -397,7 +398,8 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * pa_decode call runs as one partition per sequence on eight wavefronts (default 1024; 0 = never); key 10: what
  * pa_decode_step lets ride on its decode and projection launches (0 = the new row and the merge, the default; 1 = neither:
  * the separate launches; 2 = the new row only; 3 = the merge only); key 11: tokens per partition that the smallest
- * fixed-partition decode calls take instead of the caller's larger ones (default 256; 0 = the caller's always). */
+ * fixed-partition decode calls take instead of the caller's larger ones (default 256; 0 = the caller's always);
+ * key 12: the most (sequence, kv head) pairs a small call may have (0 = the rule described at pa_decode). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

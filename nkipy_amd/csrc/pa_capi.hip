@@ -58,6 +58,7 @@ static std::atomic<int> g_d64_tiled_from{PA_VERIFY_MAX_TOKENS + 1};   // query t
 // (the waves merge through LDS, so there is no split-K workspace and no merge launch): debug switch 9, 0 = never.
 static std::atomic<int> g_decode_single_max{1024};
 static std::atomic<int> g_decode_fine{256};     // tokens per partition of the smallest fixed-partition calls (0: the caller's always)
+static std::atomic<long> g_small_call_pairs{0};  // debug switch 12: the (sequence, kv head) pair limit of small calls (0: the rule in decode_small_call)
 static std::atomic<int> g_step_fusion{0};       // pa_decode_step, debug switch 10
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
@@ -165,6 +166,7 @@ int pa_debug_set(int key, int value) {
   if (key == 9) { g_decode_single_max = value < 0 ? 0 : value; return 0; }
   if (key == 10) { g_step_fusion = value; return 0; }
   if (key == 11) { g_decode_fine = value < 0 ? 0 : value & ~31; return 0; }
+  if (key == 12) { g_small_call_pairs = value < 0 ? 0 : value; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -266,11 +268,21 @@ static int span_bound(const DecodeParams& p) {
 constexpr long kDecodeSmallCallBytes = 160L << 20;
 constexpr int kDecodeSmallCallPartitions = 8;
 constexpr long kDecodeSmallCallPairs = 80;
+// The same comparison on the gpt-oss layer (64 / 8 heads of 64, whose rows are half as long; us per layer, fixed /
+// balanced, contexts of 1 K): B = 12 27.4 / 30.3, 16 29.0 / 31.2, 24 31.1 / 35.7, 32 33.5 / 38.2, 64 55.3 / 48.8; B = 16 at
+// 4 K 47.2 / 47.9: at head dim 64 the fixed partitions stay ahead up to four times as many pairs.  And a sliding window
+// that fits one partition leaves every sequence a handful of tiles, which one workgroup per (sequence, kv head) reads
+// in one go, without partials or a merge (window 128: B = 16 17.3 / 26.0, B = 64 23.8 / 31.7).
+constexpr long kDecodeSmallCallPairsD64 = 320;
+constexpr long kDecodeSmallCallPairsOnePartition = 1024;
 static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts = kDecodeSmallCallPartitions) {
   const long esz = kv_dtype == PA_FP8_E4M3FN ? 1 : (kv_dtype == PA_BF16 ? 2 : 4);
   if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
   if (num_partitions_for(span_bound(p), p.partition_size) > max_parts) return false;
-  if ((long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16) > kDecodeSmallCallPairs) return false;
+  long pairs_max = p.D <= 64 ? kDecodeSmallCallPairsD64 : kDecodeSmallCallPairs;
+  if (p.window > 0 && span_bound(p) <= p.partition_size) pairs_max = kDecodeSmallCallPairsOnePartition;
+  if (g_small_call_pairs.load() > 0) pairs_max = g_small_call_pairs.load();
+  if ((long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16) > pairs_max) return false;
   const double bytes = 2.0 * p.B * (double)span_bound(p) * p.Hkv * p.D * esz;
   return bytes <= (double)kDecodeSmallCallBytes;
 }
