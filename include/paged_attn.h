@@ -103,7 +103,8 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * resident wavefront group, so its partition length follows the batch and the
  * device, not partition_size.  Small calls (by max_seq_len, or by what a sliding window
  * reaches if that is less: at most eight partitions per sequence, at most 80 (sequence,
- * kv head) pairs -- 320 at head dim 64, 1 024 under a window that fits one partition --
+ * kv head) pairs -- 320 at head dim 64, 1 024 when a sequence is one partition's worth
+ * (a bound of at most 768 tokens, or a sliding window that fits a partition) --
  * and at most 160 MiB of K and V) take the fixed-partition MFMA kernel,
  * whose fixed cost is lower, on partitions of 256 tokens when those of partition_size
  * would give the device fewer than about 64 workgroups (a single sequence); under a

@@ -280,7 +280,10 @@ static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts
   if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
   if (num_partitions_for(span_bound(p), p.partition_size) > max_parts) return false;
   long pairs_max = p.D <= 64 ? kDecodeSmallCallPairsD64 : kDecodeSmallCallPairs;
-  if (p.window > 0 && span_bound(p) <= p.partition_size) pairs_max = kDecodeSmallCallPairsOnePartition;
+  // ... and so do contexts of at most 768 tokens, which decode reads as one partition on eight waves (head dim 128,
+  // contexts of 600, fixed / balanced: B = 16 27.6 / 35.9, 32 31.4 / 42.0, 48 47.4 / 47.9; verify, T = 4: B = 16
+  // 39.8 / 46.0, 32 53.0 / 60.2)
+  if ((p.window > 0 && span_bound(p) <= p.partition_size) || span_bound(p) <= 768) pairs_max = kDecodeSmallCallPairsOnePartition;
   if (g_small_call_pairs.load() > 0) pairs_max = g_small_call_pairs.load();
   if ((long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16) > pairs_max) return false;
   const double bytes = 2.0 * p.B * (double)span_bound(p) * p.Hkv * p.D * esz;
