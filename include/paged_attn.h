@@ -102,13 +102,15 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * flattened stream of all sequences' 32-token tiles into equal chunks, one per
  * resident wavefront group, so its partition length follows the batch and the
  * device, not partition_size.  Small calls (by max_seq_len, or by what a sliding window
- * reaches if that is less: at most eight partitions per sequence, at most 80 (sequence,
+ * reaches if that is less: at most eight partitions per sequence, at most 256 (sequence,
  * kv head) pairs -- 320 at head dim 64, 1 024 when a sequence is one partition's worth
  * (a bound of at most 768 tokens, or a sliding window that fits a partition) --
  * and at most 160 MiB of K and V) take the fixed-partition MFMA kernel,
- * whose fixed cost is lower, on partitions of 256 tokens when those of partition_size
- * would give the device fewer than about 64 workgroups (a single sequence); under a
- * window its partitions count from the first 32-token tile the window reaches.  The
+ * whose fixed cost is lower: on partitions of 256 tokens when those of partition_size
+ * would give the device fewer than about 64 workgroups (a single sequence), and on
+ * partitions sized to give one workgroup per CU (256-1 152 tokens) when those of
+ * partition_size would give it more workgroups than it has CUs; under a
+ * window the partitions count from the first 32-token tile the window reaches.  The
  * result does not depend on the split beyond the order of float32 sums.
  * max_seq_len: upper bound of seq_lens (sizes the grid and picks the kernel; 0 =
  * max_blocks_per_seq * block_size).  seq_lens[b] == 0 yields zeros.

@@ -267,7 +267,7 @@ static int span_bound(const DecodeParams& p) {
 }
 constexpr long kDecodeSmallCallBytes = 160L << 20;
 constexpr int kDecodeSmallCallPartitions = 8;
-constexpr long kDecodeSmallCallPairs = 80;
+constexpr long kDecodeSmallCallPairs = 256;     // (80 while every call took partitions of 512; see decode_sized_partition)
 // The same comparison on the gpt-oss layer (64 / 8 heads of 64, whose rows are half as long; us per layer, fixed /
 // balanced, contexts of 1 K): B = 12 27.4 / 30.3, 16 29.0 / 31.2, 24 31.1 / 35.7, 32 33.5 / 38.2, 64 55.3 / 48.8; B = 16 at
 // 4 K 47.2 / 47.9: at head dim 64 the fixed partitions stay ahead up to four times as many pairs.  And a sliding window
@@ -299,6 +299,26 @@ static int decode_fine_partition(const DecodeParams& p) {
   if (p.B * slots * num_partitions_for(span_bound(p), p.partition_size) > 64) return p.partition_size;
   if (num_partitions_for(span_bound(p), kFine) > 16) return p.partition_size;
   return kFine;
+}
+// Many (sequence, kv head) pairs: partitions sized to the device instead.  Two of these workgroups on one CU slow each
+// other by a third (B = 8 / 10 / 11 sequences behind 1 K on partitions of 512, 192-264 workgroups of which a third
+// trivial: kernel 15.4 / 16.1 / 16.7 us; B = 12: 21.3), so the context is cut into as many partitions as keep the
+// workgroups at one per CU -- not finer than 256 tokens, not longer than 1 152 -- and, where that cannot be had, at two
+// per CU.  us per layer of a decode step, balanced / partitions of 512 / sized this way, contexts of 1 K: B = 12 35.9 /
+// 35.6 / 31.0, 16 38.4 / 37.6 / 33.8, 24 44.5 / 46.2 / 39.2, 32 49.5 / 54.6 / 44.2; of 2 K: B = 16 47.6 / 52.8 / 46.4.
+// Returns the partition size, or 0 when the call is too large for the fixed partitions altogether.
+static int decode_sized_partition(const DecodeParams& p, int num_cus) {
+  const long pairs = (long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);
+  const int reach = span_bound(p);
+  const int np_min = (reach + 1151) / 1152;
+  for (int per_cu = 1; per_cu <= 2; ++per_cu) {
+    const long room = (long)per_cu * num_cus / pairs;                  // partitions per pair that fit
+    if (room < np_min) continue;
+    const int finest = (reach + (per_cu == 1 ? 255 : 511)) / (per_cu == 1 ? 256 : 512);
+    const int np = (int)std::max<long>(np_min, std::min<long>(room, finest));
+    return (((reach + np - 1) / np) + 31) & ~31;
+  }
+  return 0;
 }
 static int decode_kind(const DecodeParams& p, int q_dtype, int kv_dtype, bool needs_balanced = false) {
   const int impl = g_decode_impl.load();
@@ -412,7 +432,9 @@ static int plan_decode(const char* who, DecodePlan& pl, const void* q, const voi
       p.num_partitions = 1;
       pl.waves = 8;
     } else {
-      p.partition_size = decode_fine_partition(p);
+      const long pairs = (long)B * Hkv * ((Hq / Hkv + 15) / 16);
+      const int sized = pairs * p.num_partitions > current_num_cus() ? decode_sized_partition(p, current_num_cus()) : 0;
+      p.partition_size = sized > 0 ? sized : decode_fine_partition(p);
       p.num_partitions = num_partitions_for(reach, p.partition_size);
     }
   }
@@ -630,7 +652,13 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     DecodeParams f = p;
     f.partition_size = 512;
     const bool small = decode_small_call(f, kv_dtype);
-    if (small) f.partition_size = decode_fine_partition(f);       // a single sequence: finer ones, as for pa_decode
+    if (small) {
+      // a single sequence: finer partitions; many (sequence, kv head) pairs: partitions sized to the device (as pa_decode)
+      const long pairs = (long)B * Hkv * (((Hq / Hkv) * Tc + 15) / 16);
+      const int sized = pairs * num_partitions_for(span_bound(f), 512) > current_num_cus()
+                            ? decode_sized_partition(f, current_num_cus()) : 0;
+      f.partition_size = sized > 0 ? sized : decode_fine_partition(f);
+    }
     f.num_partitions = num_partitions_for(span_bound(f), f.partition_size);
     size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);
     if (small && f.partition_size != 512 && need_f && !(workspace && workspace_bytes >= need_f)) {
