@@ -1065,6 +1065,18 @@ __global__ __launch_bounds__(NW * 64, NW > 4 ? 1 : 2) void decode_mfma_kernel(De
 // [q head][b + chunk], merged by decode_balanced_reduce_kernel.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ int tiles_of(int ctx) { return (ctx + 31) >> 5; }
+
+// Inclusive prefix sum over the 64 lanes of a wave on DPP adds: shifts by 1, 2, 4 and 8 inside each row of 16 lanes
+// (a lane without a source adds 0), then lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into rows 2 and 3.
+__device__ __forceinline__ int wave_inclusive_sum(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111 /* row_shr:1 */, 0xf, 0xf, true);
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112 /* row_shr:2 */, 0xf, 0xf, true);
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114 /* row_shr:4 */, 0xf, 0xf, true);
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118 /* row_shr:8 */, 0xf, 0xf, true);
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142 /* row_bcast:15 */, 0xa, 0xf, false);
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143 /* row_bcast:31 */, 0xc, 0xf, false);
+  return x;
+}
 // Tiles of sequence b that the schedule streams: all of them, or those the window reaches
 __device__ __forceinline__ int span_tiles(const DecodeParams& p, int b) {
   const int ctx = clamp_ctx(p, b);
@@ -1090,12 +1102,7 @@ __global__ __launch_bounds__(1024) void decode_tile_prefix_kernel(DecodeParams p
       t[i] = b0 + i < p.B ? span_tiles(p, b0 + i) : 0;
       sum += t[i];
     }
-    int incl = sum;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const int v = __shfl_up(incl, off, 64);
-      if (lane >= off) incl += v;
-    }
+    const int incl = wave_inclusive_sum(sum);
     if (lane == 63) wave_total[wave] = incl;
     __syncthreads();
     int before = carry;
@@ -1157,14 +1164,11 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
     for (int i = 0; i < SCAN_STEPS; ++i) tl[i] = (64 * i + lane < p.B) ? span_tiles(p, 64 * i + lane) : 0;
 #pragma unroll
     for (int i = 0; i < SCAN_STEPS; ++i) {
-      int x = tl[i];
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int v = __shfl_up(x, off, 64);
-        if (lane >= off) x += v;
+      incl[i] = 0;
+      if (64 * i < p.B) {                    // (wave-uniform: steps past the last sequence cost nothing)
+        incl[i] = wave_inclusive_sum(tl[i]);
+        N += __builtin_amdgcn_readlane(incl[i], 63);
       }
-      incl[i] = x;
-      N += __shfl(x, 63, 64);
     }
   } else {
     N = p.ws_start[p.B];
@@ -1175,7 +1179,7 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
 #pragma unroll
     for (int i = 0; i < SCAN_STEPS; ++i) {
       if (64 * i + lane < p.B) p.ws_start[64 * i + lane] = base + incl[i] - tl[i];
-      base += __shfl(incl[i], 63, 64);
+      base += __builtin_amdgcn_readlane(incl[i], 63);
     }
     if (lane == 0) p.ws_start[p.B] = base;
   }
@@ -1190,12 +1194,12 @@ __global__ __launch_bounds__(512, 2) void decode_balanced_kernel(DecodeParams p)
     bool found = false;
 #pragma unroll
     for (int i = 0; i < SCAN_STEPS; ++i) {
-      const int total = __shfl(incl[i], 63, 64);
+      const int total = __builtin_amdgcn_readlane(incl[i], 63);
       if (!found && f < base + total) {
         const unsigned long long m = __ballot(base + incl[i] > f);
         const int idx = __ffsll((long long)m) - 1;
         b = 64 * i + idx;
-        start = base + __shfl(incl[i] - tl[i], idx, 64);
+        start = base + __builtin_amdgcn_readlane(incl[i] - tl[i], idx);
         found = true;
       }
       base += total;
