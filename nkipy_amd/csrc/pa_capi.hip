@@ -60,6 +60,7 @@ static std::atomic<int> g_decode_single_max{1024};
 static std::atomic<int> g_decode_fine{256};     // tokens per partition of the smallest fixed-partition calls (0: the caller's always)
 static std::atomic<long> g_small_call_pairs{0};  // debug switch 12: the (sequence, kv head) pair limit of small calls (0: the rule in decode_small_call)
 static std::atomic<int> g_step_fusion{0};       // pa_decode_step, debug switch 10
+static std::atomic<int> g_d64_wide{1};          // debug switch 13: partitions counted in bytes at head dim 64 (see token_scale)
 
 // ---- profiling: event pairs around the main kernel of each op ----------------
 // Events come from a free list that pa_profile_collect refills, so that a timed pass which follows a collected
@@ -167,6 +168,7 @@ int pa_debug_set(int key, int value) {
   if (key == 10) { g_step_fusion = value; return 0; }
   if (key == 11) { g_decode_fine = value < 0 ? 0 : value & ~31; return 0; }
   if (key == 12) { g_small_call_pairs = value < 0 ? 0 : value; return 0; }
+  if (key == 13) { g_d64_wide = value != 0; return 0; }
   return fail_arg("pa_debug_set: unknown key %d", key);
 }
 
@@ -265,8 +267,20 @@ static int span_bound(const DecodeParams& p) {
   const long reach = (long)p.window + std::max(p.T, 1) - 1 + 31;
   return (int)std::min<long>(p.max_seq_len, reach);
 }
-constexpr long kDecodeSmallCallBytes = 160L << 20;
+// The partition sizes below were found at head dim 128; what they measure is the bytes a workgroup streams, and a
+// token of head dim 64 is half of them.  Where a limit in tokens would send a call of head dim 64 to more partitions
+// than pay (or to the balanced kernel), the partitions are twice the tokens instead: the caller's partition_size
+// when it gives more than eight partitions, the finer partitions of a single sequence likewise, and the longest
+// partition the sized ones may have.  (64 / 8 heads of 64, us per call replayed, before / after: B = 1 behind 4 K 12.6 /
+// 11.3, behind 8 K 15.8 / 14.0; B = 2 behind 8 K 17.6 / 14.5; B = 4 behind 6 K 19.6 / 18.0; B = 32 behind 2 K 35.3 /
+// 30.5.  Doubling everything at head dim 64 cost where the tokens' count was fine: B = 8 behind 1 K 9.7 -> 10.6.)
+static int token_scale(const DecodeParams& p) { return g_d64_wide.load() && p.D <= 64 ? 2 : 1; }
 constexpr int kDecodeSmallCallPartitions = 8;
+static int base_partition(const DecodeParams& p) {
+  if (num_partitions_for(span_bound(p), p.partition_size) <= kDecodeSmallCallPartitions) return p.partition_size;
+  return p.partition_size * token_scale(p);
+}
+constexpr long kDecodeSmallCallBytes = 160L << 20;
 constexpr long kDecodeSmallCallPairs = 256;     // (80 while every call took partitions of 512; see decode_sized_partition)
 // The same comparison on the gpt-oss layer (64 / 8 heads of 64, whose rows are half as long; us per layer, fixed /
 // balanced, contexts of 1 K): B = 12 27.4 / 30.3, 16 29.0 / 31.2, 24 31.1 / 35.7, 32 33.5 / 38.2, 64 55.3 / 48.8; B = 16 at
@@ -278,7 +292,7 @@ constexpr long kDecodeSmallCallPairsOnePartition = 1024;
 static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts = kDecodeSmallCallPartitions) {
   const long esz = kv_dtype == PA_FP8_E4M3FN ? 1 : (kv_dtype == PA_BF16 ? 2 : 4);
   if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
-  if (num_partitions_for(span_bound(p), p.partition_size) > max_parts) return false;
+  if (num_partitions_for(span_bound(p), base_partition(p)) > max_parts) return false;
   long pairs_max = p.D <= 64 ? kDecodeSmallCallPairsD64 : kDecodeSmallCallPairs;
   // ... and so do contexts of at most 768 tokens, which decode reads as one partition on eight waves (head dim 128,
   // contexts of 600, fixed / balanced: B = 16 27.6 / 35.9, 32 31.4 / 42.0, 48 47.4 / 47.9; verify, T = 4: B = 16
@@ -293,28 +307,30 @@ static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts
 // workgroups (a single sequence, mostly): same units, partitions of 512 / of 256: 1 x 1 K 25.8 / 22.9, 1 x 4 K
 // 28.3 / 27.9; with more workgroups to begin with the finer ones cost more than they bring (8 x 1 K 29.6 / 32.4).
 static int decode_fine_partition(const DecodeParams& p) {
-  const int kFine = g_decode_fine.load();
-  if (kFine <= 0 || p.partition_size <= kFine || span_bound(p) <= kFine) return p.partition_size;
+  const int base = base_partition(p);
+  int kFine = g_decode_fine.load();
+  if (kFine > 0 && num_partitions_for(span_bound(p), kFine) > 12) kFine *= token_scale(p);    // (9 of 256 behind 2 K: 9.1 us, 5 of 512: 9.2-9.3)
+  if (kFine <= 0 || base <= kFine || span_bound(p) <= kFine) return base;
   const long slots = (long)p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);      // workgroups per sequence and partition
-  if (p.B * slots * num_partitions_for(span_bound(p), p.partition_size) > 64) return p.partition_size;
-  if (num_partitions_for(span_bound(p), kFine) > 16) return p.partition_size;
+  if (p.B * slots * num_partitions_for(span_bound(p), base) > 64) return base;
+  if (num_partitions_for(span_bound(p), kFine) > 16) return base;
   return kFine;
 }
 // Many (sequence, kv head) pairs: partitions sized to the device instead.  Two of these workgroups on one CU slow each
 // other by a third (B = 8 / 10 / 11 sequences behind 1 K on partitions of 512, 192-264 workgroups of which a third
 // trivial: kernel 15.4 / 16.1 / 16.7 us; B = 12: 21.3), so the context is cut into as many partitions as keep the
-// workgroups at one per CU -- not finer than 256 tokens, not longer than 1 152 -- and, where that cannot be had, at two
-// per CU.  us per layer of a decode step, balanced / partitions of 512 / sized this way, contexts of 1 K: B = 12 35.9 /
+// workgroups at one per CU -- not finer than 256 tokens, not longer than 1 152 (twice that at head dim 64, see
+// token_scale) -- and, where that cannot be had, at two per CU.  us per layer of a decode step, balanced / partitions of 512 / sized this way, contexts of 1 K: B = 12 35.9 /
 // 35.6 / 31.0, 16 38.4 / 37.6 / 33.8, 24 44.5 / 46.2 / 39.2, 32 49.5 / 54.6 / 44.2; of 2 K: B = 16 47.6 / 52.8 / 46.4.
 // Returns the partition size, or 0 when the call is too large for the fixed partitions altogether.
 static int decode_sized_partition(const DecodeParams& p, int num_cus) {
   const long pairs = (long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);
-  const int reach = span_bound(p);
-  const int np_min = (reach + 1151) / 1152;
+  const int reach = span_bound(p), ts = token_scale(p);
+  const int np_min = (reach + 1152 * ts - 1) / (1152 * ts);
   for (int per_cu = 1; per_cu <= 2; ++per_cu) {
     const long room = (long)per_cu * num_cus / pairs;                  // partitions per pair that fit
     if (room < np_min) continue;
-    const int finest = (reach + (per_cu == 1 ? 255 : 511)) / (per_cu == 1 ? 256 : 512);
+    const int finest = num_partitions_for(reach, per_cu == 1 ? 256 : 512);
     const int np = (int)std::max<long>(np_min, std::min<long>(room, finest));
     return (((reach + np - 1) / np) + 31) & ~31;
   }
@@ -440,7 +456,8 @@ static int plan_decode(const char* who, DecodePlan& pl, const void* q, const voi
       pl.waves = 8;
     } else {
       const long pairs = (long)B * Hkv * ((Hq / Hkv + 15) / 16);
-      const int sized = pairs * p.num_partitions > current_num_cus() ? decode_sized_partition(p, current_num_cus()) : 0;
+      const int np_base = num_partitions_for(reach, base_partition(p));
+      const int sized = pairs * np_base > current_num_cus() ? decode_sized_partition(p, current_num_cus()) : 0;
       p.partition_size = equal_partitions(reach, sized > 0 ? sized : decode_fine_partition(p));
       p.num_partitions = num_partitions_for(reach, p.partition_size);
     }
@@ -662,7 +679,7 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     if (small) {
       // a single sequence: finer partitions; many (sequence, kv head) pairs: partitions sized to the device (as pa_decode)
       const long pairs = (long)B * Hkv * (((Hq / Hkv) * Tc + 15) / 16);
-      const int sized = pairs * num_partitions_for(span_bound(f), 512) > current_num_cus()
+      const int sized = pairs * num_partitions_for(span_bound(f), base_partition(f)) > current_num_cus()
                             ? decode_sized_partition(f, current_num_cus()) : 0;
       f.partition_size = equal_partitions(span_bound(f), sized > 0 ? sized : decode_fine_partition(f));
     }

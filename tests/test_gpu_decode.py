@@ -208,6 +208,56 @@ def test_small_calls_take_the_fixed_partition_kernel(pa):
     assert np.array_equal(dev_bits(run(0, wide, sinks=sinks)), dev_bits(run(3, wide)))
 
 
+def test_head_dim_64_partitions_are_counted_in_bytes(pa):
+    """Head dim 64: a call whose bound gives more than eight partitions of partition_size still takes the
+    fixed-partition kernel when twice as long partitions give at most eight (the bits of that kernel forced onto
+    partitions of 1 024 tokens), a single sequence behind 4 K runs on 512-token partitions instead of sixteen of 256,
+    and the results are the oracle's; with debug switch 13 off the first call is the balanced kernel's."""
+    from nkipy_amd import _lib
+    rng = np.random.default_rng(64)
+    Hq, Hkv, D, bs = 16, 4, 64, 32
+
+    def make(ctxs, cap):
+        B = len(ctxs)
+        k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+        wide = np.full((B, cap // bs), -1, np.int32)
+        wide[:, :tables.shape[1]] = tables
+        q = rng.standard_normal((B, Hq, D)).astype(np.float32)
+        want = O.paged_decode(O.round_to_bf16(q), O.round_to_bf16(k), O.round_to_bf16(v), tables, np.asarray(ctxs, np.int32),
+                              0.125, q_dtype="bf16")
+        return bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(wide), _i32(ctxs), want
+
+    def run(args, impl=0, **kw):
+        _set_impl(impl)
+        try:
+            o = pa.decode(*args[:5], 0.125, **kw)
+            torch.cuda.synchronize()
+        finally:
+            _set_impl(0)
+        return o
+
+    two = make([7000, 300, 5000, 8100], 8192)           # bound 8 192: sixteen partitions of 512, eight of 1 024
+    got = run(two, partition_size=512)
+    assert_close_abs(dev_to_f32(got), two[5], BF16_TOL)
+    assert np.array_equal(dev_bits(got), dev_bits(run(two, impl=2, partition_size=1024)))
+    assert not np.array_equal(dev_bits(got), dev_bits(run(two, impl=3, partition_size=512)))
+    lib = _lib.load()
+    lib.pa_debug_set(13, 0)
+    try:
+        assert np.array_equal(dev_bits(run(two, partition_size=512)), dev_bits(run(two, impl=3, partition_size=512)))
+    finally:
+        lib.pa_debug_set(13, 1)
+    one = make([3900], 4096)                            # a single sequence: the finer partitions, 512 tokens here
+    got = run(one, partition_size=512)
+    assert_close_abs(dev_to_f32(got), one[5], BF16_TOL)
+    assert np.array_equal(dev_bits(got), dev_bits(run(one, impl=2, partition_size=512)))
+    assert not np.array_equal(dev_bits(got), dev_bits(run(one, impl=2, partition_size=256)))
+    many = make([2100] * 3 + [1, 900] + [1800] * 59, 2176)      # 256 (sequence, kv head) pairs: one partition of 2 176
+    got = run(many, partition_size=512)
+    assert_close_abs(dev_to_f32(got), many[5], BF16_TOL)
+    assert np.array_equal(dev_bits(got), dev_bits(run(many, impl=2, partition_size=2176)))
+
+
 def test_identity_table_equals_dense_cache(pa):
     """A dense (B, S, Hkv, D) cache viewed as a pool with an identity table."""
     rng = np.random.default_rng(5)
