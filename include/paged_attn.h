@@ -111,9 +111,10 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
  * partitions sized to give one workgroup per CU (256-1 152 tokens) when those of
  * partition_size would give it more workgroups than it has CUs; under a
  * window the partitions count from the first 32-token tile the window reaches.  At head
- * dim 64, whose tokens are half the bytes, a call that would exceed eight partitions is
- * counted on partitions of twice partition_size, a single sequence that would exceed twelve
- * of the finer partitions takes them at 512 tokens, and the sized ones may be 2 304 long.
+ * dim 64 and on fp8 pools, whose tokens are half the bytes, a call that would exceed eight
+ * partitions is counted on partitions of twice partition_size (not an fp8 pool of head dim
+ * 64), a single sequence that would exceed twelve of the finer partitions takes them at 512
+ * tokens, and the sized ones may be 2 304 long.
  * The result does not depend on the split beyond the order of float32 sums.
  * max_seq_len: upper bound of seq_lens (sizes the grid and picks the kernel; 0 =
  * max_blocks_per_seq * block_size).  seq_lens[b] == 0 yields zeros.
@@ -406,7 +407,7 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * the separate launches; 2 = the new row only; 3 = the merge only); key 11: tokens per partition that the smallest
  * fixed-partition decode calls take instead of the caller's larger ones (default 256; 0 = the caller's always);
  * key 12: the most (sequence, kv head) pairs a small call may have (0 = the rule described at pa_decode).
- * key 13: 0 = partitions of small calls counted in tokens at head dim 64 too (1, the default: see pa_decode). */
+ * key 13: 0 = partitions of small calls counted in tokens at head dim 64 and on fp8 pools too (1, the default: see pa_decode). */
 int pa_debug_set(int key, int value);
 
 /* Kernel timing for benchmarks: when enabled, every launch of the main kernel

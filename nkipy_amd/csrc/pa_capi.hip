@@ -267,18 +267,25 @@ static int span_bound(const DecodeParams& p) {
   const long reach = (long)p.window + std::max(p.T, 1) - 1 + 31;
   return (int)std::min<long>(p.max_seq_len, reach);
 }
-// The partition sizes below were found at head dim 128; what they measure is the bytes a workgroup streams, and a
-// token of head dim 64 is half of them.  Where a limit in tokens would send a call of head dim 64 to more partitions
-// than pay (or to the balanced kernel), the partitions are twice the tokens instead: the caller's partition_size
-// when it gives more than eight partitions, the finer partitions of a single sequence likewise, and the longest
-// partition the sized ones may have.  (64 / 8 heads of 64, us per call replayed, before / after: B = 1 behind 4 K 12.6 /
-// 11.3, behind 8 K 15.8 / 14.0; B = 2 behind 8 K 17.6 / 14.5; B = 4 behind 6 K 19.6 / 18.0; B = 32 behind 2 K 35.3 /
-// 30.5.  Doubling everything at head dim 64 cost where the tokens' count was fine: B = 8 behind 1 K 9.7 -> 10.6.)
-static int token_scale(const DecodeParams& p) { return g_d64_wide.load() && p.D <= 64 ? 2 : 1; }
+// The partition sizes below were found on bf16 pools of head dim 128; what they measure is the bytes a workgroup
+// streams, and a token of head dim 64, or of an fp8 pool, is half of them.  Where a limit in tokens would send such a
+// call to more partitions than pay (or to the balanced kernel), the partitions are twice the tokens instead: the
+// caller's partition_size when it gives more than eight partitions, the finer partitions of a single sequence
+// likewise, and the longest partition the sized ones may have.  (us per call replayed, before / after.  64 / 8 heads of
+// 64, bf16: B = 1 behind 4 K 12.6 / 11.3, behind 8 K 15.8 / 14.0; B = 2 behind 8 K 17.6 / 14.5; B = 4 behind 6 K 19.6 /
+// 18.0; B = 32 behind 2 K 35.3 / 30.5.  64 / 8 heads of 128, fp8: B = 1 behind 8 K 18.4 / 16.5, B = 4 behind 6 K 22.1 /
+// 19.2, B = 32 behind 2 K 37.2 / 29.1.  Doubling everything cost where the tokens' count was fine: head dim 64, B = 8
+// behind 1 K 9.7 -> 10.6.)
+static int token_scale(const DecodeParams& p, int kv_dtype) {
+  return g_d64_wide.load() && (p.D <= 64 || kv_dtype == PA_FP8_E4M3FN) ? 2 : 1;
+}
 constexpr int kDecodeSmallCallPartitions = 8;
-static int base_partition(const DecodeParams& p) {
+static int base_partition(const DecodeParams& p, int kv_dtype) {
   if (num_partitions_for(span_bound(p), p.partition_size) <= kDecodeSmallCallPartitions) return p.partition_size;
-  return p.partition_size * token_scale(p);
+  // (not for fp8 pools of head dim 64, which are better off on the balanced kernel there: B = 2 behind 8 K 15.4
+  // against 16.6 us, B = 4 behind 6 K 15.6 against 16.4)
+  if (p.D <= 64 && kv_dtype == PA_FP8_E4M3FN) return p.partition_size;
+  return p.partition_size * token_scale(p, kv_dtype);
 }
 constexpr long kDecodeSmallCallBytes = 160L << 20;
 constexpr long kDecodeSmallCallPairs = 256;     // (80 while every call took partitions of 512; see decode_sized_partition)
@@ -292,7 +299,7 @@ constexpr long kDecodeSmallCallPairsOnePartition = 1024;
 static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts = kDecodeSmallCallPartitions) {
   const long esz = kv_dtype == PA_FP8_E4M3FN ? 1 : (kv_dtype == PA_BF16 ? 2 : 4);
   if (p.max_seq_len <= 0 || p.partition_size <= 0 || p.partition_size % 32) return false;
-  if (num_partitions_for(span_bound(p), base_partition(p)) > max_parts) return false;
+  if (num_partitions_for(span_bound(p), base_partition(p, kv_dtype)) > max_parts) return false;
   long pairs_max = p.D <= 64 ? kDecodeSmallCallPairsD64 : kDecodeSmallCallPairs;
   // ... and so do contexts of at most 768 tokens, which decode reads as one partition on eight waves (head dim 128,
   // contexts of 600, fixed / balanced: B = 16 27.6 / 35.9, 32 31.4 / 42.0, 48 47.4 / 47.9; verify, T = 4: B = 16
@@ -306,10 +313,10 @@ static bool decode_small_call(const DecodeParams& p, int kv_dtype, int max_parts
 // Partitions of 256 tokens instead of the caller's (larger) ones when those would give the device very few
 // workgroups (a single sequence, mostly): same units, partitions of 512 / of 256: 1 x 1 K 25.8 / 22.9, 1 x 4 K
 // 28.3 / 27.9; with more workgroups to begin with the finer ones cost more than they bring (8 x 1 K 29.6 / 32.4).
-static int decode_fine_partition(const DecodeParams& p) {
-  const int base = base_partition(p);
+static int decode_fine_partition(const DecodeParams& p, int kv_dtype) {
+  const int base = base_partition(p, kv_dtype);
   int kFine = g_decode_fine.load();
-  if (kFine > 0 && num_partitions_for(span_bound(p), kFine) > 12) kFine *= token_scale(p);    // (9 of 256 behind 2 K: 9.1 us, 5 of 512: 9.2-9.3)
+  if (kFine > 0 && num_partitions_for(span_bound(p), kFine) > 12) kFine *= token_scale(p, kv_dtype);    // (9 of 256 behind 2 K: 9.1 us, 5 of 512: 9.2-9.3)
   if (kFine <= 0 || base <= kFine || span_bound(p) <= kFine) return base;
   const long slots = (long)p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);      // workgroups per sequence and partition
   if (p.B * slots * num_partitions_for(span_bound(p), base) > 64) return base;
@@ -323,9 +330,9 @@ static int decode_fine_partition(const DecodeParams& p) {
 // token_scale) -- and, where that cannot be had, at two per CU.  us per layer of a decode step, balanced / partitions of 512 / sized this way, contexts of 1 K: B = 12 35.9 /
 // 35.6 / 31.0, 16 38.4 / 37.6 / 33.8, 24 44.5 / 46.2 / 39.2, 32 49.5 / 54.6 / 44.2; of 2 K: B = 16 47.6 / 52.8 / 46.4.
 // Returns the partition size, or 0 when the call is too large for the fixed partitions altogether.
-static int decode_sized_partition(const DecodeParams& p, int num_cus) {
+static int decode_sized_partition(const DecodeParams& p, int kv_dtype, int num_cus) {
   const long pairs = (long)p.B * p.Hkv * ((p.Hq / p.Hkv * std::max(p.T, 1) + 15) / 16);
-  const int reach = span_bound(p), ts = token_scale(p);
+  const int reach = span_bound(p), ts = token_scale(p, kv_dtype);
   const int np_min = (reach + 1152 * ts - 1) / (1152 * ts);
   for (int per_cu = 1; per_cu <= 2; ++per_cu) {
     const long room = (long)per_cu * num_cus / pairs;                  // partitions per pair that fit
@@ -362,7 +369,7 @@ size_t pa_decode_workspace_bytes_for(int B, int Hq, int Hkv, int D, int block_si
   p.max_seq_len = max_seq_len; p.partition_size = partition_size;
   const int kind = decode_kind(p, q_dtype, kv_dtype);
   int np = num_partitions_for(max_seq_len, partition_size);
-  if (kind == 2 && max_seq_len > 0) np = std::max(np, num_partitions_for(max_seq_len, decode_fine_partition(p)));
+  if (kind == 2 && max_seq_len > 0) np = std::max(np, num_partitions_for(max_seq_len, decode_fine_partition(p, kv_dtype)));
   const size_t fixed = np <= 1 ? 0 : (size_t)B * Hq * np * ((size_t)D + 2) * sizeof(float);
   if (max_seq_len <= 0) {
     // no bound given: pa_decode then takes the table capacity, which this function is not told.  The answer covers
@@ -456,9 +463,9 @@ static int plan_decode(const char* who, DecodePlan& pl, const void* q, const voi
       pl.waves = 8;
     } else {
       const long pairs = (long)B * Hkv * ((Hq / Hkv + 15) / 16);
-      const int np_base = num_partitions_for(reach, base_partition(p));
-      const int sized = pairs * np_base > current_num_cus() ? decode_sized_partition(p, current_num_cus()) : 0;
-      p.partition_size = equal_partitions(reach, sized > 0 ? sized : decode_fine_partition(p));
+      const int np_base = num_partitions_for(reach, base_partition(p, kv_dtype));
+      const int sized = pairs * np_base > current_num_cus() ? decode_sized_partition(p, kv_dtype, current_num_cus()) : 0;
+      p.partition_size = equal_partitions(reach, sized > 0 ? sized : decode_fine_partition(p, kv_dtype));
       p.num_partitions = num_partitions_for(reach, p.partition_size);
     }
   }
@@ -679,9 +686,9 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     if (small) {
       // a single sequence: finer partitions; many (sequence, kv head) pairs: partitions sized to the device (as pa_decode)
       const long pairs = (long)B * Hkv * (((Hq / Hkv) * Tc + 15) / 16);
-      const int sized = pairs * num_partitions_for(span_bound(f), base_partition(f)) > current_num_cus()
-                            ? decode_sized_partition(f, current_num_cus()) : 0;
-      f.partition_size = equal_partitions(span_bound(f), sized > 0 ? sized : decode_fine_partition(f));
+      const int sized = pairs * num_partitions_for(span_bound(f), base_partition(f, kv_dtype)) > current_num_cus()
+                            ? decode_sized_partition(f, kv_dtype, current_num_cus()) : 0;
+      f.partition_size = equal_partitions(span_bound(f), sized > 0 ? sized : decode_fine_partition(f, kv_dtype));
     }
     f.num_partitions = num_partitions_for(span_bound(f), f.partition_size);
     size_t need_f = f.num_partitions <= 1 ? 0 : (size_t)B * Hq * Tc * f.num_partitions * ((size_t)D + 2) * sizeof(float);

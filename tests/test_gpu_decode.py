@@ -258,6 +258,43 @@ def test_head_dim_64_partitions_are_counted_in_bytes(pa):
     assert np.array_equal(dev_bits(got), dev_bits(run(many, impl=2, partition_size=2176)))
 
 
+def test_fp8_pool_partitions_are_counted_in_bytes(pa):
+    """An fp8 pool of head dim 128 (tokens of 128 bytes, like bf16 ones of head dim 64): a bound of sixteen partitions
+    of 512 tokens is taken as eight of 1 024 on the fixed-partition kernel; an fp8 pool of head dim 64 stays with the
+    balanced kernel there.  Both the oracle's values."""
+    rng = np.random.default_rng(8)
+    for D, want_fixed in ((128, True), (64, False)):
+        Hq, Hkv, bs = 8, 4, 32
+        ctxs = [7000, 300, 5000, 8100]
+        B = len(ctxs)
+        k, v, tables = make_paged(rng, B, Hkv, D, bs, ctxs)
+        wide = np.full((B, 8192 // bs), -1, np.int32)
+        wide[:, :tables.shape[1]] = tables
+        kq, ks = O.quantize_kv_fp8(k)
+        vq, vs = O.quantize_kv_fp8(v)
+        q = O.round_to_bf16(rng.standard_normal((B, Hq, D)).astype(np.float32))
+        scale = 1.0 / np.sqrt(D)
+        want = O.paged_decode(q, kq, vq, tables, np.asarray(ctxs, np.int32), scale, k_scale=ks, v_scale=vs, q_dtype="bf16")
+        args = (bf16_to_dev(q), torch.from_numpy(kq).cuda().view(torch.float8_e4m3fn),
+                torch.from_numpy(vq).cuda().view(torch.float8_e4m3fn), _i32(wide), _i32(ctxs), scale)
+        kw = dict(k_scale=torch.from_numpy(ks).cuda(), v_scale=torch.from_numpy(vs).cuda())
+
+        def run(impl, part):
+            _set_impl(impl)
+            try:
+                o = pa.decode(*args, partition_size=part, **kw)
+                torch.cuda.synchronize()
+            finally:
+                _set_impl(0)
+            return o
+
+        got = run(0, 512)
+        assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+        fixed, balanced = run(2, 1024), run(3, 512)
+        assert not np.array_equal(dev_bits(fixed), dev_bits(balanced))
+        assert np.array_equal(dev_bits(got), dev_bits(fixed if want_fixed else balanced))
+
+
 def test_identity_table_equals_dense_cache(pa):
     """A dense (B, S, Hkv, D) cache viewed as a pool with an identity table."""
     rng = np.random.default_rng(5)
