@@ -396,7 +396,7 @@ class PagedAttention:
             return res
         if T > 1 and (self.rope is None or paged_attn.q_transform_supported(T, c.head_dim, c.block_size)) and \
                 paged_attn.prefill_route(B, T, self.n_heads, c.n_kv_heads, c.head_dim, c.block_size, ks is not None,
-                                         self.sliding_window or 0) == "verify":
+                                         self.sliding_window or 0, bound) == "verify":
             # a verify step (a few tokens per sequence through the decode-shaped kernel): one call as well
             proj = None
             if self.o_weight is not None:

@@ -314,10 +314,21 @@ def decode(q, k_cache, v_cache, block_tables, seq_lens, scale, *, k_scale=None, 
 # the grid is small) lies between 16 and 48 rows for batches of 1 to 64 sequences
 VERIFY_MAX_ROWS = 32
 VERIFY_MAX_ROWS_FP8 = 256     # fp8 pools: the tiled kernel has no packed-rows form for them (B = 64, 4 K prefix: T = 64 718 vs 810 us)
+# bf16 pools of head dim 128, more than 16 rows per kv head.  Up to VERIFY_MAX_ROWS rows the verify kernel gives a kv
+# head two 16-row waves, each of which streams every tile, and from this many (sequence x bound) tokens on the tiled
+# kernel's packed rows are ahead (32 / 8 heads, T = 8, ragged contexts up to the bound, us verify / tiled: B = 8 behind
+# 2 K 22.9 / 23.5, behind 4 K 41.0 / 31.3; B = 16 behind 1 K 20.2 / 22.6, behind 2 K 43.0 / 30.1; B = 32 behind 1 K 35.8 /
+# 29.5; B = 64 behind 2 K 90.3 / 72.0).  Beyond VERIFY_MAX_ROWS a small call -- few sequences, a bound of a few thousand
+# tokens -- is still faster on the verify kernel's fixed partitions (T = 16, us verify / tiled: B = 1 behind 1 K 14.1 /
+# 21.0, behind 4 K 20.9 / 25.1; B = 2 behind 2 K 19.7 / 22.4; B = 4 behind 500 15.9 / 18.9), up to this many
+# (sequence x row x bound) products.
+TILED_FROM_TOKENS = 20_000
+VERIFY_SMALL_CALL = 300_000
 
 
-def prefill_route(B, T, Hq, Hkv, D, block_size, fp8=False, window=0) -> str:
-    """Which kernel `prefill` takes for a shape: "verify" (the decode-shaped kernel) or "tiled"."""
+def prefill_route(B, T, Hq, Hkv, D, block_size, fp8=False, window=0, bound=None) -> str:
+    """Which kernel `prefill` takes for a shape: "verify" (the decode-shaped kernel) or "tiled".  bound: what the
+    caller knows of the longest context (None: nothing)."""
     can_verify = verify_supported(T, D, block_size)
     # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
     rows = T * (Hq // Hkv)
@@ -325,8 +336,19 @@ def prefill_route(B, T, Hq, Hkv, D, block_size, fp8=False, window=0) -> str:
         # the tiled kernel takes head dim 64 two kv heads at a time (not a single kv head); below 320 rows per kv head, and for small
         # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself)
         return "tiled" if not can_verify or (Hkv >= 2 and B >= 8 and rows >= 320) else "verify"
-    return "verify" if can_verify and (D != 128 or rows <= VERIFY_MAX_ROWS
-                                       or (fp8 and (window > 0 or rows <= VERIFY_MAX_ROWS_FP8))) else "tiled"
+    if not can_verify:
+        return "tiled"
+    if D != 128:
+        return "verify"
+    if fp8:
+        return "verify" if window > 0 or rows <= VERIFY_MAX_ROWS_FP8 else "tiled"
+    if rows <= 16 or (window > 0 and rows <= VERIFY_MAX_ROWS):
+        return "verify"
+    if rows <= VERIFY_MAX_ROWS:
+        if bound is None:
+            return "tiled" if B >= 16 else "verify"
+        return "tiled" if B >= 8 and B * bound >= TILED_FROM_TOKENS else "verify"
+    return "verify" if bound is not None and window == 0 and B * rows * bound <= VERIFY_SMALL_CALL else "tiled"
 
 
 def verify_supported(T, D, block_size) -> bool:
@@ -344,8 +366,10 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     j <= seq_lens[b] - query_lens[b] + i of the paged context, which already
     contains the new tokens' K/V.
 
-    Two kernels stand behind it.  Short query runs -- speculative verify: T * (Hq / Hkv) <=
-    VERIFY_MAX_ROWS -- go through the decode kernel with the (token, head) pairs as its query rows
+    Two kernels stand behind it.  Short query runs -- speculative verify: up to 16 (token, q head) rows per
+    kv head always, up to VERIFY_MAX_ROWS for small batches and short bounds, more for a handful of sequences
+    under a bound of a few thousand tokens (`prefill_route`) -- go through the decode kernel with the
+    (token, head) pairs as its query rows
     (HBM-bound: the context is read once per kv head); everything else through the tiled
     matrix-core prefill kernel (head_dim 128, and 64 with two or more kv heads; long query runs
     at head_dim 64 over a single kv head go through the verify kernel 64 tokens at a time).
@@ -385,7 +409,8 @@ def prefill(q, k_cache, v_cache, block_tables, seq_lens, query_lens, scale, *, k
     sinks, win = _check_variant(sinks, sliding_window, Hq, q)
     can_verify = verify_supported(T, D, block_size)
     if route is None:
-        route = prefill_route(B, T, Hq, Hkv, D, block_size, kv_code == FP8, win)
+        route = prefill_route(B, T, Hq, Hkv, D, block_size, kv_code == FP8, win,
+                              None if max_seq_len is None else int(max_seq_len))
     if route == "verify":
         _check(can_verify, f"the verify kernel needs T <= 64, head_dim 64 or 128 and a power-of-two block size >= 16 "
                            f"(T={T}, D={D}, block_size={block_size})")

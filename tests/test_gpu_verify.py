@@ -94,6 +94,38 @@ def test_verify_rows_without_keys_in_the_last_chunk(pa, rows):
         assert_close_abs(dev_to_f32(got), want, BF16_TOL)
 
 
+def test_prefill_picks_the_route_by_rows_batch_and_bound(pa):
+    """32 rows per kv head: a batch of 16 sequences under a bound of 2 K takes the tiled kernel, the same batch under a
+    bound of 1 K and a single sequence the verify kernel; 64 rows of one sequence under a bound of 2 K the verify
+    kernel, without a bound the tiled one.  Whatever the route, the oracle's values."""
+    rng = np.random.default_rng(21)
+    Hq, Hkv, D, bs = 16, 4, 128, 32
+
+    def check(B, T, hi, bound, expect):
+        qlens = [T] * B
+        qlens[-1] = max(T - 3, 1)
+        prefixes = [int(x) for x in rng.integers(hi // 4, hi - T, size=B)]
+        q, k, v, tables, ctxs, ql = _case(rng, T, qlens, prefixes, Hq, Hkv, bs, D)
+        wide = np.full((B, max(tables.shape[1], (bound or 0) // bs)), -1, np.int32)     # table capacity >= the bound
+        wide[:, :tables.shape[1]] = tables
+        args = (bf16_to_dev(q), bf16_to_dev(k), bf16_to_dev(v), _i32(wide), _i32(ctxs), _i32(ql), 0.09)
+        kw = {} if bound is None else {"max_seq_len": bound}
+        got = pa.prefill(*args, **kw)
+        torch.cuda.synchronize()
+        want = O.paged_prefill(q, k, v, tables, ctxs, ql, 0.09, q_dtype="bf16")
+        assert_close_abs(dev_to_f32(got), want, BF16_TOL)
+        forced = {r: pa.prefill(*args, route=r, **kw) for r in ("verify", "tiled")}
+        torch.cuda.synchronize()
+        assert not np.array_equal(dev_to_f32(forced["verify"]), dev_to_f32(forced["tiled"]))
+        assert np.array_equal(dev_to_f32(got), dev_to_f32(forced[expect])), (B, T, hi, bound, expect)
+
+    check(16, 8, 600, 2048, "tiled")
+    check(16, 8, 600, 1024, "verify")
+    check(1, 8, 1500, 2048, "verify")
+    check(1, 16, 1500, 2048, "verify")
+    check(1, 16, 1500, None, "tiled")
+
+
 def test_verify_agrees_with_tiled_prefill_and_decode(pa):
     rng = np.random.default_rng(12)
     T, Hq, Hkv, D, bs = 4, 32, 8, 128, 32

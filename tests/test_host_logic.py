@@ -132,6 +132,27 @@ def test_c_abi_argument_errors_without_gpu(lib):
     assert lib.pa_decode_step_workspace_bytes(0, 32, 8, 128, 32, 100, 512, 4096, 1, 1) == 0
 
 
+def test_prefill_route_by_rows_batch_and_bound():
+    """Which kernel `prefill` picks for runs of a few tokens (bf16 pools, head dim 128): up to 16 rows per kv head the
+    verify kernel; 17-32 rows the tiled kernel from 8 sequences and 20 000 (sequence x bound) tokens on; beyond, the
+    tiled kernel but for small calls; windows, fp8 pools and head dim 64 as before."""
+    from nkipy_amd.paged_attn import prefill_route as route
+    assert route(64, 4, 32, 8, 128, 32, bound=8192) == "verify"                 # 16 rows
+    assert route(1, 8, 32, 8, 128, 32, bound=32768) == "verify"                  # 32 rows, one sequence
+    assert route(8, 8, 32, 8, 128, 32, bound=2048) == "verify"
+    assert route(8, 8, 32, 8, 128, 32, bound=4096) == "tiled"
+    assert route(16, 8, 32, 8, 128, 32, bound=1024) == "verify"
+    assert route(16, 4, 64, 8, 128, 32, bound=2048) == "tiled"
+    assert route(16, 8, 32, 8, 128, 32) == "tiled" and route(8, 8, 32, 8, 128, 32) == "verify"      # no bound
+    assert route(32, 8, 32, 8, 128, 32, window=128, bound=4096) == "verify"
+    assert route(1, 16, 32, 8, 128, 32, bound=4096) == "verify"                  # 64 rows, a small call
+    assert route(1, 16, 32, 8, 128, 32) == "tiled" and route(8, 16, 32, 8, 128, 32, bound=4096) == "tiled"
+    assert route(4, 16, 32, 8, 128, 32, bound=1024, window=64) == "tiled"
+    assert route(64, 8, 32, 8, 128, 32, fp8=True, bound=4096) == "verify"        # fp8 pools: by rows alone
+    assert route(64, 64, 64, 8, 64, 32, bound=4096) == "tiled" and route(4, 64, 64, 8, 64, 32, bound=4096) == "verify"
+    assert route(4, 65, 32, 8, 128, 32, bound=512) == "tiled"                    # more tokens than the verify kernel takes
+
+
 def test_ops_refuse_host_arrays():
     import nkipy_amd
     a = np.zeros((1, 1, 64), np.float32)
