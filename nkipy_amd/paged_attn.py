@@ -341,6 +341,11 @@ def prefill_route(B, T, Hq, Hkv, D, block_size, fp8=False, window=0, bound=None)
     if D != 128:
         return "verify"
     if fp8:
+        # (a few sequences with many rows behind short contexts are ahead on the tiled kernel all the same: 32 / 8
+        # heads, us verify / tiled, T = 32: B = 1 behind 1 K 34.2 / 21.7, B = 4 behind 2 K 44.5 / 38.1; T = 64: B = 4
+        # behind 2 K 61.4 / 42.8; B = 8 behind 4 K 83.3 / 99.2 is not)
+        if window == 0 and bound is not None and rows >= 128 and B * bound <= 80 * rows:
+            return "tiled"
         return "verify" if window > 0 or rows <= VERIFY_MAX_ROWS_FP8 else "tiled"
     if rows <= 16 or (window > 0 and rows <= VERIFY_MAX_ROWS):
         return "verify"
