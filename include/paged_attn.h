@@ -398,7 +398,7 @@ int pa_qk_norm_rope_kv_write(const void* xq, const void* xk, const void* xv, voi
  * workgroup packed over the q heads of a kv head, which is what short chunks get by default); key 4:
  * per-tile barrier that keeps the kv-head wavefronts of a balanced decode workgroup on
  * the same tile (1 = automatic, the default: on for bf16 pools, off for fp8 pools; 0 = never; 2 = always); key 5: query rows per wavefront of pa_verify (0 =
- * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never);
+ * automatic, 16 or 32 = forced); key 6: split form of pa_prefill (1 = when useful, the default; 0 = never; 2-16 = that many shares);
  * key 7: query tokens from which pa_prefill at head dim 64 takes the tiled kernel (0 = the default, 65);
  * key 3 value 6: one q head per wave at head dim 64; key 8: pa_o_proj takes 256 x 256 tiles
  * also where it would take 128 x 128 ones (1 = on); key 9: the longest length bound (tokens) up to which a small

@@ -877,7 +877,8 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.splits = 1;
   if (workspace) {
     if (!aligned16(workspace)) return fail_arg("pa_prefill: workspace must be 16-byte aligned");
-    const int want = g_prefill_split.load() ? prefill_async_splits(p, current_num_cus(), max_seq_len) : 1;
+    const int forced = g_prefill_split.load();       // 1: the rule; 0: never; 2-16: that many shares
+    const int want = forced == 1 ? prefill_async_splits(p, current_num_cus(), max_seq_len) : forced <= 0 ? 1 : std::min(forced, 16);
     if (want > 1 && workspace_bytes >= prefill_split_bytes(p, want)) {
       p.splits = want;
       p.ws_o = (float*)workspace;

@@ -1032,9 +1032,16 @@ int prefill_async_splits(const PrefillParams& p, int num_cus, int max_seq_len) {
   const long wgs = prefill_workgroups(p, waves, prefill_packs(p));
   const long slots = (long)num_cus * (waves == 4 ? 2 : 1);     // workgroups the device holds at once
   if (wgs >= slots) return 1;                         // enough workgroups to fill the chip
-  const long cap_tiles = ((long)p.max_blocks * p.block_size + 63) / 64;
+  // key tiles a workgroup may have to walk: by the caller's bound, else by the table capacity
+  const long tiles = ((max_seq_len > 0 ? (long)max_seq_len : (long)p.max_blocks * p.block_size) + 63) / 64;
   long s = (2L * num_cus + wgs - 1) / wgs;            // aim at two workgroups per CU
-  if (s > cap_tiles / 8) s = cap_tiles / 8;           // ... of at least 8 key tiles each at table capacity
+  // ... of at least 8 key tiles each; the more workgroups there are to begin with, the longer a share must be to
+  // pay for its partials (a float32 row per query row and share) and the merge launch: 16 tiles from one workgroup
+  // per two CUs on, 40 from one per CU on (32 / 8 heads of 128, us unsplit / two shares: 2 x 512 tokens behind 1 K
+  // 36.6 / 46.7, 4 x 256 behind 1 K 32.1 / 41.4, 2 x 256 behind 1 K 30.2 / 32.7; 1 x 256 behind 1 K 30.0 / 27.3 and
+  // 1 x 1 024 behind 4 K 98.2 / 93.1 keep their two)
+  const long min_tiles = wgs >= num_cus ? 40 : 2 * wgs >= num_cus ? 16 : 8;
+  if (s > tiles / min_tiles) s = tiles / min_tiles;
   if (s > 16) s = 16;
   return s < 2 ? 1 : (int)s;
 }
