@@ -845,6 +845,7 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   p.q = q; p.k = k_cache; p.v = v_cache; p.block_tables = block_tables; p.seq_lens = seq_lens;
   p.query_lens = query_lens; p.out = out;
   fill_prefill_shape(p, B, T, Hq, Hkv, D, block_size, max_blocks_per_seq, num_blocks);
+  p.len_bound = max_seq_len;
   p.scale_log2e = scale * kLog2e;
   p.kv_fp8 = fp8 ? 1 : 0; p.k_scale = k_scale; p.v_scale = v_scale;
   // head_dim 64: the tiled kernel takes two or more kv heads (two heads share its 256-byte rows); short

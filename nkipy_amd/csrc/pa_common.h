@@ -275,6 +275,7 @@ struct PrefillParams {
   float* ws_ml;             // splits > 1: [B * T * Hq, splits, 2] partial (max, sum)
   QTransform qt;            // asynchronous kernel only: Q rows are normed and rotated as they are loaded
   int num_cus;              // CUs of the device the call runs on (0: unknown, taken as 256); steers the workgroup shape
+  int len_bound;            // the caller's bound on the sequence lengths (0: none); steers the workgroup shape as well
 };
 
 hipError_t launch_prefill(const PrefillParams& p, hipStream_t s);

@@ -1014,7 +1014,14 @@ static int prefill_waves(const PrefillParams& p, int waves) {
     // fewer 256-row workgroups than CUs (one request's chunk of up to a few thousand tokens): the call is bound by
     // its longest workgroup, and twice as many of half the size, two per CU, finish sooner (B = 1: T = 512 behind
     // a 4 K prefix 66 -> 55 us, T = 1 024 37.5 -> 33.5 us; with the device full the 8-wave form is ~7 % ahead)
-    if (waves == 8 && p.block_tables && (long)p.B * p.Hq * ((p.T + 255) / 256) < (p.num_cus > 0 ? p.num_cus : 256)) waves = 4;
+    const long wgs8 = (long)p.B * p.Hq * ((p.T + 255) / 256), cus = p.num_cus > 0 ? p.num_cus : 256;
+    if (waves == 8 && p.block_tables && wgs8 < cus) waves = 4;
+    // short contexts by the caller's bound (prompts of a batch with little cached in front: at most 16 key tiles per
+    // workgroup) with the device full twice over: a workgroup's start and end weigh as much as its tiles, and the two
+    // 4-wave workgroups of a CU overlap them (32 / 8 heads, no prefix, us 8 / 4 waves: 32 x 256 tokens 56.8 / 49.0, 16 x
+    // 512 69.7 / 65.6, 8 x 1 024 97.7 / 95.1, 4 x 1 024 57.2 / 52.6; with the device full once the 8-wave form stays: 2 x
+    // 1 024 31.5 / 35.3, 4 x 512 21.2 / 22.5)
+    if (waves == 8 && p.block_tables && p.len_bound > 0 && p.len_bound <= 1024 && wgs8 >= 2 * cus) waves = 4;
   }
   return waves;
 }
