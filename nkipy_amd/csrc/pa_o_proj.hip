@@ -902,8 +902,12 @@ hipError_t launch_o_proj(const OProjParams& p, hipStream_t s) {
   if (p.M <= 64) return launch_skinny<2>(p, s);
   if (p.M <= 128) return launch_skinny<4>(p, s);
   // a few hundred rows: the 128-row form over several row blocks as long as its workgroups (N / 64 per block) fit
-  // the device in one go; measured against the other forms at K = N = 4096
-  if (!g_o_proj_force_large && (long)((p.M + 127) / 128) * ((p.N + 63) / 64) <= 256 && (long)p.M * p.K * 2 < 0x7fffffffL)
+  // the device in one go; measured against the other forms at K = N = 4096.  With a longer K two of them per CU
+  // are still ahead of the 128 x 128 form, whose one wave per SIMD pays a latency per k-step (us few rows / 128 x 128:
+  // K = 8 192 N = 5 120 M = 512 111.8 / 146.9, M = 768 115.1 / 150.0; K = N = 5 120 M = 512 72.0 / 96.5; K = N = 8 192 M = 384
+  // 113.3 / 150.0; at K = 4 096 it is the other way round: N = 4 096 M = 640 48.6 / 41.5, N = 2 880 M = 768 51.3 / 34.8)
+  const long few_rows_wgs = p.K >= 5120 ? 512 : 256;
+  if (!g_o_proj_force_large && (long)((p.M + 127) / 128) * ((p.N + 63) / 64) <= few_rows_wgs && (long)p.M * p.K * 2 < 0x7fffffffL)
     return launch_skinny<4>(p, s);
   if (p.M <= 256) return launch_skinny<8>(p, s);
   {

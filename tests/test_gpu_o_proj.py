@@ -72,7 +72,9 @@ def test_o_proj_tile_forms(pa, M, K, N, bias, force_large):
 
 @pytest.mark.parametrize("M,K,N,bias", [(4352, 4096, 4096, True),      # 256 x 256 tiles: 17 row tiles (so row tiles 8.. of an XCD's walk), 64 k-steps
                                         (1024, 4096, 4096, False),     # 128 x 128 tiles, deep ring (one workgroup per CU)
-                                        (2048, 4096, 2880, True)])     # 128 x 128 tiles, two-stage ring, ragged last column tile
+                                        (2048, 4096, 2880, True),      # 128 x 128 tiles, two-stage ring, ragged last column tile
+                                        (600, 8192, 5120, True),       # the 128-row few-rows form, two workgroups per CU (K >= 5 120), ragged last row block
+                                        (1024, 8192, 5120, False)])    # 128 x 128 tiles at 128 k-steps
 def test_o_proj_long_k_every_row_tile(pa, M, K, N, bias):
     """The tiled forms at the projection's real depth (K = 4096: 64 steps through the ring, far more than the
     ring is deep or the loop is rotated by), rows checked in every row tile: 16 per 128 rows, at in-tile
