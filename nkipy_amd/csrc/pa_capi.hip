@@ -655,8 +655,21 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     // (which spills a little) only from four 16-row groups on.
     const int n_rows = (Hq / Hkv) * Tc, forced = g_verify_rows.load();
     // (not under a sliding window: the few tiles a launch then sees are better spread over more waves)
-    const bool wide = n_rows > 16 && (B >= 16 || (n_rows >= 128 && sliding_window == 0)) &&
-                      (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
+    bool wide = n_rows > 16 && (B >= (D == 64 ? 8 : 16) || (n_rows >= 128 && sliding_window == 0)) &&
+                (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
+    // fp8 pools at head dim 128: the two-operand wave no longer fits the registers (it spills some fifty) and only
+    // pays on the largest calls (32 / 8 heads, ragged contexts, us 16 / 32 rows per wave: B = 32 behind 4 K T = 8 63.5 /
+    // 86.7, T = 16 98.9 / 103.2, T = 32 178.6 / 159.1; B = 64 behind 1 K T = 8 42.4 / 59.5, T = 32 109.2 / 112.8)
+    // ... and at head dim 128 over bf16 pools, where it spills as many (32 / 8 heads, T = 16: B = 16 behind 1 K 30.7 / 55.8,
+    // B = 32 behind 2 K 80.7 / 90.4; T = 32, B = 16 behind 4 K 122.5 / 114.7).  At head dim 64 it fits, and is ahead once the
+    // call is large enough for its half as many waves (64 / 8 heads, on the balanced schedule: T = 4 B = 32 behind 1 K
+    // 24.3 / 34.2, B = 64 behind 1 K 39.9 / 36.1, B = 16 behind 4 K 47.5 / 37.4; T = 8 B = 16 behind 1 K 25.2 / 29.5, B = 8
+    // behind 4 K 41.2 / 31.3).  The measure is sequences x rows per kv head x length bound.
+    if (wide) {
+      const long bound = max_seq_len > 0 ? std::min<long>(max_seq_len, cap) : cap;
+      const long work = (long)B * n_rows * bound;
+      wide = work >= (D == 64 ? 1200000L : kv_dtype == PA_FP8_E4M3FN ? 12L << 20 : 8L << 20);
+    }
     p.rows_per_wave = forced == 16 || forced == 32 ? forced : (wide ? 32 : 16);
   }
   p.block_size = block_size; p.max_blocks = max_blocks_per_seq; p.num_blocks = num_blocks;
@@ -679,10 +692,23 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
   // table capacity says nothing about the sizes), 16 rows per wave, and a workspace that holds the partitions'
   // partials.  Under a sliding window the partitions cover what the window reaches, often a single one, and the
   // window is itself a bound.
-  if ((max_seq_len > 0 || sliding_window > 0) && p.rows_per_wave == 16 && g_decode_impl.load() == 0) {
+  // The fixed partitions take 16 rows per wave, so a call that would take 32 on the balanced schedule is asked first
+  // whether it is a small one: it mostly is better off here (64 / 8 heads of 64, T = 4, us fixed partitions / balanced
+  // with 32 rows: B = 16 behind 1 K 14.1 / 24.1, B = 32 behind 1 K 23.2 / 33.1; fp8 pool, 32 / 8 heads of 128, T = 8:
+  // B = 16 behind 1 K 18.0 / 42.5, behind 4 K 53.6 / 62.3).  Not when every kv head has several 16-row waves, each of
+  // which reads its partitions, over long contexts: at head dim 64 (where the two-operand wave fits) from 80 000
+  // (sequence x wave x bound) products on the balanced schedule with 32 rows is ahead (B = 8 behind 4 K T = 8 35.6 /
+  // 29.4, B = 12 behind 4 K T = 4 45.2 / 35.2; B = 8 behind 4 K T = 4 21.8 / 29.2 is not).
+  if ((max_seq_len > 0 || sliding_window > 0) && g_verify_rows.load() != 32 && g_decode_impl.load() == 0) {
     DecodeParams f = p;
+    f.rows_per_wave = 16;
     f.partition_size = 512;
-    const bool small = decode_small_call(f, kv_dtype);
+    bool small = decode_small_call(f, kv_dtype);
+    {
+      const int n_rows = (Hq / Hkv) * Tc;
+      if (small && D == 64 && n_rows > 16 && p.rows_per_wave == 32 &&
+          (long)B * ((n_rows + 15) / 16) * span_bound(f) > 80000) small = false;
+    }
     if (small) {
       // a single sequence: finer partitions; many (sequence, kv head) pairs: partitions sized to the device (as pa_decode)
       const long pairs = (long)B * Hkv * (((Hq / Hkv) * Tc + 15) / 16);
@@ -851,9 +877,9 @@ int pa_prefill(const void* q, const void* k_cache, const void* v_cache,
   // head_dim 64: the tiled kernel takes two or more kv heads (two heads share its 256-byte rows); short
   // query runs and a single kv head go to the decode-shaped kernel, 64 query tokens per launch, each
   // launch reading the context up to its last token once per kv head
-  // (measured crossover for runs of up to 64 tokens: 320 query rows per kv head in a batch of 8 or more)
+  // (measured crossover for runs of up to 64 tokens: 384 query rows per kv head in a batch of 8 or more)
   const int from64 = g_d64_tiled_from.load();
-  const bool many_rows = from64 == PA_VERIFY_MAX_TOKENS + 1 && B >= 8 && (long)T * (Hq / Hkv) >= 320;
+  const bool many_rows = from64 == PA_VERIFY_MAX_TOKENS + 1 && B >= 8 && (long)T * (Hq / Hkv) >= 384;
   const bool tiled64 = D == 64 && (T >= from64 || many_rows) && p.impl != 1 && prefill_async_supported(p);
   if (!prefill_supported(p) && !tiled64) {
     if (D != 64) return fail_arg("pa_prefill: unsupported shape (D=%d block_size=%d)", D, block_size);

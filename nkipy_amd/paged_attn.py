@@ -333,19 +333,15 @@ def prefill_route(B, T, Hq, Hkv, D, block_size, fp8=False, window=0, bound=None)
     # the tiled kernel is built for bf16 pools and head_dim 128; what it cannot take goes to the verify kernel
     rows = T * (Hq // Hkv)
     if D == 64:
-        # the tiled kernel takes head dim 64 two kv heads at a time (not a single kv head); below 320 rows per kv head, and for small
-        # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself)
-        return "tiled" if not can_verify or (Hkv >= 2 and B >= 8 and rows >= 320) else "verify"
+        # the tiled kernel takes head dim 64 two kv heads at a time (not a single kv head); below 384 rows per kv head, and for small
+        # batches, the verify kernel is faster (measured crossover, as in pa_prefill itself: 64 / 8 heads, us verify /
+        # tiled, T = 40: B = 8 behind 1 K 30.5 / 39.9, behind 4 K 58.0 / 74.6; T = 48: B = 8 behind 2 K 48.2 / 45.1)
+        return "tiled" if not can_verify or (Hkv >= 2 and B >= 8 and rows >= 384) else "verify"
     if not can_verify:
         return "tiled"
     if D != 128:
         return "verify"
     if fp8:
-        # (a few sequences with many rows behind short contexts are ahead on the tiled kernel all the same: 32 / 8
-        # heads, us verify / tiled, T = 32: B = 1 behind 1 K 34.2 / 21.7, B = 4 behind 2 K 44.5 / 38.1; T = 64: B = 4
-        # behind 2 K 61.4 / 42.8; B = 8 behind 4 K 83.3 / 99.2 is not)
-        if window == 0 and bound is not None and rows >= 128 and B * bound <= 80 * rows:
-            return "tiled"
         return "verify" if window > 0 or rows <= VERIFY_MAX_ROWS_FP8 else "tiled"
     if rows <= 16 or (window > 0 and rows <= VERIFY_MAX_ROWS):
         return "verify"

@@ -148,10 +148,9 @@ def test_prefill_route_by_rows_batch_and_bound():
     assert route(1, 16, 32, 8, 128, 32, bound=4096) == "verify"                  # 64 rows, a small call
     assert route(1, 16, 32, 8, 128, 32) == "tiled" and route(8, 16, 32, 8, 128, 32, bound=4096) == "tiled"
     assert route(4, 16, 32, 8, 128, 32, bound=1024, window=64) == "tiled"
-    assert route(64, 8, 32, 8, 128, 32, fp8=True, bound=4096) == "verify"        # fp8 pools: by rows, but for a few
-    assert route(1, 32, 32, 8, 128, 32, fp8=True, bound=1024) == "tiled"         # sequences with many rows behind short
-    assert route(8, 64, 32, 8, 128, 32, fp8=True, bound=4096) == "verify"        # contexts
-    assert route(1, 32, 32, 8, 128, 32, fp8=True) == "verify"
+    assert route(64, 8, 32, 8, 128, 32, fp8=True, bound=4096) == "verify"        # fp8 pools: by rows alone
+    assert route(1, 32, 32, 8, 128, 32, fp8=True, bound=1024) == "verify"
+    assert route(4, 65, 32, 8, 128, 32, fp8=True, bound=1024) == "tiled"
     assert route(64, 64, 64, 8, 64, 32, bound=4096) == "tiled" and route(4, 64, 64, 8, 64, 32, bound=4096) == "verify"
     assert route(4, 65, 32, 8, 128, 32, bound=512) == "tiled"                    # more tokens than the verify kernel takes
 
