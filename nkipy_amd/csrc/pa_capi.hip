@@ -657,10 +657,12 @@ static int verify_launch(const char* who, const void* q, const void* k_cache, co
     // (not under a sliding window: the few tiles a launch then sees are better spread over more waves)
     bool wide = n_rows > 16 && (B >= (D == 64 ? 8 : 16) || (n_rows >= 128 && sliding_window == 0)) &&
                 (D == 64 || kv_dtype == PA_FP8_E4M3FN || n_rows > 48);
-    // fp8 pools at head dim 128: the two-operand wave no longer fits the registers (it spills some fifty) and only
-    // pays on the largest calls (32 / 8 heads, ragged contexts, us 16 / 32 rows per wave: B = 32 behind 4 K T = 8 63.5 /
+    // fp8 pools at head dim 128: the two-operand wave is the lean form (Q fragments from LDS, V single-buffered; its
+    // some fifty spilled registers lie in the start and end of a sequence, not in the tile loop), which the 16-row
+    // wave with K and V streamed two tiles deep has overtaken; it only pays on the largest calls (32 / 8 heads,
+    // ragged contexts, us 16 / 32 rows per wave: B = 32 behind 4 K T = 8 63.5 /
     // 86.7, T = 16 98.9 / 103.2, T = 32 178.6 / 159.1; B = 64 behind 1 K T = 8 42.4 / 59.5, T = 32 109.2 / 112.8)
-    // ... and at head dim 128 over bf16 pools, where it spills as many (32 / 8 heads, T = 16: B = 16 behind 1 K 30.7 / 55.8,
+    // ... and at head dim 128 over bf16 pools, the same lean form (32 / 8 heads, T = 16: B = 16 behind 1 K 30.7 / 55.8,
     // B = 32 behind 2 K 80.7 / 90.4; T = 32, B = 16 behind 4 K 122.5 / 114.7).  At head dim 64 it fits, and is ahead once the
     // call is large enough for its half as many waves (64 / 8 heads, on the balanced schedule: T = 4 B = 32 behind 1 K
     // 24.3 / 34.2, B = 64 behind 1 K 39.9 / 36.1, B = 16 behind 4 K 47.5 / 37.4; T = 8 B = 16 behind 1 K 25.2 / 29.5, B = 8
